@@ -1,0 +1,322 @@
+"""ctypes loader for the CPU oracle (oracle/flexllm_oracle.c).
+
+TEST INFRASTRUCTURE ONLY: imported by tests/, by the smoke run and by the
+benchmark's cpu_baseline leg, never by the shipped package.
+"""
+import ctypes as C
+import os
+import subprocess
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_SO = os.path.join(_HERE, "libflexllm_oracle.so")
+
+
+def build(force=False):
+    """Compile the oracle with gcc (no GPU toolchain involved)."""
+    if force or not os.path.exists(_SO):
+        subprocess.check_call(["make", "-B", "-C", _HERE, "libflexllm_oracle.so"],
+                              stdout=subprocess.DEVNULL)
+    return _SO
+
+
+_lib = None
+
+
+def lib():
+    global _lib
+    if _lib is None:
+        build()
+        _lib = C.CDLL(_SO)
+        _lib.fxo_half_to_float.restype = C.c_float
+        _lib.fxo_half_to_float.argtypes = [C.c_uint16]
+        _lib.fxo_argmax.restype = C.c_int
+    return _lib
+
+
+def _p(a):
+    return a.ctypes.data_as(C.c_void_p) if a is not None else None
+
+
+def _f32(a):
+    return np.ascontiguousarray(a, dtype=np.float32)
+
+
+def _f(v):
+    return C.c_float(float(v))
+
+
+def quant_sym(x, bits=8):
+    x = _f32(x)
+    rows, dim = x.reshape(-1, x.shape[-1]).shape
+    q = np.empty(x.shape, np.int8)
+    s = np.empty(rows, np.float32)
+    lib().fxo_quant_sym(_p(x), rows, dim, bits, _p(q), _p(s))
+    return q, s.reshape(x.shape[:-1])
+
+
+def quant_asym(x, bits=4):
+    x = _f32(x)
+    rows, dim = x.reshape(-1, x.shape[-1]).shape
+    q = np.empty(x.shape, np.uint8)
+    s = np.empty(rows, np.float32)
+    b = np.empty(rows, np.float32)
+    lib().fxo_quant_asym(_p(x), rows, dim, bits, _p(q), _p(s), _p(b))
+    return q, s, b
+
+
+def dequant(acc, s_x, w_s, b_x=None, w_sum=None):
+    acc = np.ascontiguousarray(acc, np.int32)
+    rows, n = acc.shape
+    s_x = _f32(np.reshape(s_x, -1)); w_s = _f32(w_s)
+    b_x = _f32(np.reshape(b_x, -1)) if b_x is not None else None
+    w_sum = _f32(w_sum) if w_sum is not None else None
+    y = np.empty((rows, n), np.float32)
+    lib().fxo_dequant(_p(acc), rows, n, _p(s_x), _p(b_x), _p(w_s), _p(w_sum), _p(y))
+    return y
+
+
+def static_quant(x, scale, factor=1.0, signed=True, bits=8):
+    """x [rows][heads][dim] -> int8 (signed) / uint8 (unsigned)."""
+    x = _f32(x)
+    rows, heads, dim = x.shape
+    scale = _f32(scale)
+    assert scale.shape == (heads,)
+    q = np.empty(x.shape, np.int8)
+    lib().fxo_static_quant(_p(x), rows, heads, dim, _p(scale), _f(factor), int(signed), bits, _p(q))
+    return q if signed else q.view(np.uint8)
+
+
+def static_dequant(acc, a_s, w_s):
+    acc = np.ascontiguousarray(acc, np.int32)
+    rows, ah, dim = acc.shape
+    a_s = _f32(a_s); w_s = _f32(w_s)
+    y = np.empty(acc.shape, np.float32)
+    lib().fxo_static_dequant(_p(acc), rows, ah, w_s.shape[0], dim, _p(a_s), _p(w_s), _p(y))
+    return y
+
+
+def head_quant_sym(x, bits=8):
+    x = _f32(x)
+    rows, heads, dim = x.shape
+    q = np.empty(x.shape, np.int8)
+    s = np.empty((rows, heads), np.float32)
+    lib().fxo_head_quant_sym(_p(x), rows, heads, dim, bits, _p(q), _p(s))
+    return q, s
+
+
+def linear_i8(a, w):
+    a = np.ascontiguousarray(a); w = np.ascontiguousarray(w, np.int8)
+    m, k = a.shape
+    n = w.shape[0]
+    assert w.shape[1] == k
+    c = np.empty((m, n), np.int32)
+    if a.dtype == np.uint8:
+        lib().fxo_linear_u8i8(_p(a), _p(w), m, k, n, _p(c))
+    else:
+        assert a.dtype == np.int8
+        lib().fxo_linear_i8(_p(a), _p(w), m, k, n, _p(c))
+    return c
+
+
+def fht(x, scale=1.0):
+    x = _f32(x)
+    rows, n = x.reshape(-1, x.shape[-1]).shape
+    y = np.empty(x.shape, np.float32)
+    lib().fxo_fht(_p(x), rows, n, _f(scale), _p(y))
+    return y
+
+
+def rmsnorm_pref(x, gamma, eps=1e-5):
+    x = _f32(x); gamma = _f32(gamma)
+    rows, dim = x.shape
+    y = np.empty(x.shape, np.float32)
+    lib().fxo_rmsnorm_pref(_p(x), _p(gamma), rows, dim, _f(eps), _p(y))
+    return y
+
+
+def rmsnorm_dec(x, gamma, block_parallel=8, eps=1e-5):
+    x = _f32(x); gamma = _f32(gamma)
+    y = np.empty(x.shape, np.float32)
+    lib().fxo_rmsnorm_dec(_p(x), _p(gamma), x.shape[-1], block_parallel, _f(eps), _p(y))
+    return y
+
+
+def rope_table(max_pos, head_dim=64, theta=500000.0, factor=32, low=1, high=4, orig=8192):
+    s = np.empty((max_pos, head_dim // 2), np.float32)
+    c = np.empty((max_pos, head_dim // 2), np.float32)
+    lib().fxo_rope_table(max_pos, head_dim, _f(theta), factor, low, high, orig, _p(s), _p(c))
+    return s, c
+
+
+def rope(x, sin_t, cos_t, pos0=0):
+    x = _f32(x)
+    tokens, heads, hd = x.shape
+    y = np.empty(x.shape, np.float32)
+    lib().fxo_rope(_p(x), tokens, heads, hd, _p(_f32(sin_t)), _p(_f32(cos_t)), pos0, _p(y))
+    return y
+
+
+def swish(x):
+    x = _f32(x); y = np.empty(x.shape, np.float32)
+    lib().fxo_swish(_p(x), x.size, _p(y)); return y
+
+
+def gate(a, b):
+    a = _f32(a); b = _f32(b); y = np.empty(a.shape, np.float32)
+    lib().fxo_gate(_p(a), _p(b), a.size, _p(y)); return y
+
+
+def residual(a, b):
+    a = _f32(a); b = _f32(b); y = np.empty(a.shape, np.float32)
+    lib().fxo_residual(_p(a), _p(b), a.size, _p(y)); return y
+
+
+def softmax(x):
+    x = _f32(x)
+    rows, dim = x.reshape(-1, x.shape[-1]).shape
+    y = np.empty(x.shape, np.float32)
+    lib().fxo_softmax(_p(x), rows, dim, _p(y)); return y
+
+
+def causal_mask(x):
+    x = _f32(x)
+    rows, heads, dim = x.shape
+    y = np.empty(x.shape, np.float32)
+    lib().fxo_causal_mask(_p(x), rows, heads, dim, _p(y)); return y
+
+
+class MhaScales(C.Structure):
+    _fields_ = [("q_s", C.c_void_p), ("k_s", C.c_void_p), ("v_s", C.c_void_p), ("a_s", C.c_void_p)]
+
+
+def _scales(q_s, k_s, v_s, a_s):
+    keep = [_f32(q_s), _f32(k_s), _f32(v_s), _f32(a_s)]
+    sc = MhaScales(*[a.ctypes.data for a in keep])
+    return sc, keep
+
+
+def mha_prefill(q, k, v, q_s, k_s, v_s, a_s, want_p=False):
+    """q [s][qh][hd], k/v [s][kvh][hd] fp32 -> dict(q8,k8,v8,p8,o)."""
+    q = _f32(q); k = _f32(k); v = _f32(v)
+    s, qh, hd = q.shape
+    kvh = k.shape[1]
+    sc, keep = _scales(q_s, k_s, v_s, a_s)
+    q8 = np.empty(q.shape, np.int8); k8 = np.empty(k.shape, np.int8); v8 = np.empty(v.shape, np.int8)
+    p8 = np.empty((qh, s, s), np.uint8) if want_p else None
+    o = np.empty(q.shape, np.float32)
+    lib().fxo_mha_prefill(_p(q), _p(k), _p(v), s, qh, kvh, hd, C.byref(sc), _p(q8), _p(k8), _p(v8), _p(p8), _p(o))
+    return dict(q8=q8, k8=k8, v8=v8, p8=p8, o=o)
+
+
+def mha_decode(q8, k_cache, v_cache, q_s, k_s, v_s, a_s, want_p=False):
+    """q8 [qh][hd] int8, caches [len][kvh][hd] int8 -> (o [qh][hd] fp32, p8 [qh][len])."""
+    q8 = np.ascontiguousarray(q8, np.int8)
+    k_cache = np.ascontiguousarray(k_cache, np.int8); v_cache = np.ascontiguousarray(v_cache, np.int8)
+    qh, hd = q8.shape
+    ln, kvh, _ = k_cache.shape
+    sc, keep = _scales(q_s, k_s, v_s, a_s)
+    p8 = np.empty((qh, ln), np.uint8) if want_p else None
+    o = np.empty((qh, hd), np.float32)
+    lib().fxo_mha_decode(_p(q8), _p(k_cache), _p(v_cache), ln, qh, kvh, hd, C.byref(sc), _p(p8), _p(o))
+    return o, p8
+
+
+def half_to_float(h):
+    return lib().fxo_half_to_float(int(h))
+
+
+def lm_head(table_u16, n):
+    table_u16 = np.ascontiguousarray(table_u16, np.uint16)
+    vocab, hidden = table_u16.shape
+    n = _f32(n)
+    logits = np.empty(vocab, np.float32)
+    lib().fxo_lm_head(_p(table_u16), vocab, hidden, _p(n), _p(logits))
+    return logits
+
+
+def pack_pref(x, tp):
+    x = _f32(x); tokens, dim = x.shape
+    out = np.empty((tokens // tp, dim, tp), np.float32)
+    lib().fxo_pack_pref(_p(x), tokens, dim, tp, _p(out)); return out
+
+
+def unpack_pref(packed, tp):
+    packed = _f32(packed); blocks, dim, _ = packed.shape
+    x = np.empty((blocks * tp, dim), np.float32)
+    lib().fxo_unpack_pref(_p(packed), blocks * tp, dim, tp, _p(x)); return x
+
+
+def pack_dec(x, bp):
+    x = _f32(x); dim = x.shape[0]
+    out = np.empty((dim // bp, bp), np.float32)
+    lib().fxo_pack_dec(_p(x), dim, bp, _p(out)); return out
+
+
+def unpack_dec(packed, bp):
+    packed = _f32(packed); dim = packed.size
+    x = np.empty(dim, np.float32)
+    lib().fxo_unpack_dec(_p(packed), dim, bp, _p(x)); return x
+
+
+# ---------------------------------------------------------------- model level
+
+class Model(C.Structure):
+    _fields_ = [(n, C.c_int) for n in
+                ("layers", "hidden", "kv_hidden", "inter", "q_heads", "kv_heads", "head_dim", "vocab", "max_pos")] + \
+               [("eps", C.c_float), ("fht_scale", C.c_float)] + \
+               [(n, C.c_void_p) for n in
+                ("wq", "wk", "wv", "wo", "wg", "wu", "wd", "sq", "sk", "sv", "so", "sg", "su", "sd",
+                 "gamma", "q_s", "k_s", "v_s", "a_s", "rope_sin", "rope_cos", "embed")]
+
+
+class OracleModel:
+    """Wraps numpy weight arrays (see flexllm_amd.llama.synth_weights) for the oracle's model functions."""
+
+    def __init__(self, cfg, w):
+        self.cfg = cfg
+        self.w = w
+        self._keep = []
+        L = cfg["layers"]
+
+        def ptr_array(name):
+            arrs = [np.ascontiguousarray(w[name][l]) for l in range(L)]
+            self._keep.append(arrs)
+            pa = (C.c_void_p * L)(*[a.ctypes.data for a in arrs])
+            self._keep.append(pa)
+            return C.cast(pa, C.c_void_p)
+
+        m = Model()
+        for n in ("layers", "hidden", "kv_hidden", "inter", "q_heads", "kv_heads", "head_dim", "vocab", "max_pos"):
+            setattr(m, n, int(cfg[n]))
+        m.eps = float(cfg["eps"]); m.fht_scale = float(cfg["fht_scale"])
+        for n in ("wq", "wk", "wv", "wo", "wg", "wu", "wd", "sq", "sk", "sv", "so", "sg", "su", "sd"):
+            setattr(m, n, ptr_array(n))
+        for n, dt in (("gamma", np.float32), ("q_s", np.float32), ("k_s", np.float32), ("v_s", np.float32),
+                      ("a_s", np.float32), ("rope_sin", np.float32), ("rope_cos", np.float32), ("embed", np.uint16)):
+            a = np.ascontiguousarray(w[n], dt)
+            self._keep.append(a)
+            setattr(m, n, a.ctypes.data)
+        self.m = m
+
+    def new_caches(self):
+        c = self.cfg
+        shape = (c["layers"], c["max_pos"], c["kv_hidden"])
+        return np.zeros(shape, np.int8), np.zeros(shape, np.int8)
+
+    def decode_token(self, x_in, pos, k_cache, v_cache, want_logits=True):
+        c = self.cfg
+        x_in = _f32(x_in)
+        hidden = np.empty(c["hidden"], np.float32)
+        logits = np.empty(c["vocab"], np.float32) if want_logits else None
+        lib().fxo_llama_decode_token(C.byref(self.m), _p(x_in), int(pos), _p(k_cache), _p(v_cache),
+                                     _p(hidden), _p(logits))
+        return hidden, logits
+
+    def prefill(self, x_in, k_cache, v_cache):
+        x_in = _f32(x_in)
+        s = x_in.shape[0]
+        hidden = np.empty(x_in.shape, np.float32)
+        lib().fxo_llama_prefill(C.byref(self.m), _p(x_in), s, _p(k_cache), _p(v_cache), _p(hidden))
+        return hidden

@@ -1,0 +1,286 @@
+"""Pins the CPU oracle (oracle/flexllm_oracle.c) against facts that do not come from
+the oracle's own formulas: closed forms, invariants, special cases, textbook routines
+and brute force.  The reference ships no stored golden vectors for this path (its
+testbenches synthesise inputs and compute goldens in-process), so these checks plus the
+testbench-style float64 "fake-quant" goldens below are what anchors the oracle."""
+import numpy as np
+import pytest
+import scipy.linalg
+import scipy.special
+
+rng = np.random.default_rng(1234)
+
+
+# ------------------------------------------------------------------ quant
+def test_quant_sym_special_cases(oracle):
+    x = np.zeros((3, 16), np.float32)
+    x[1, 3] = -2.54; x[1, 5] = 1.0
+    x[2] = np.linspace(-1, 1, 16)
+    q, s = oracle.quant_sym(x)
+    assert s[0] == 1.0 and not q[0].any()              # all-zero row: scale 1, zeros
+    assert q[1, 3] == -127 and s[1] == np.float32(2.54) / np.float32(127)
+    assert q[2, 0] == -127 and q[2, -1] == 127         # absmax maps to +-127 exactly
+    # dequantised error bounded by half a step
+    assert np.all(np.abs(q[2] * s[2] - x[2]) <= s[2] * 0.5 * (1 + 1e-6))
+
+
+def test_quant_sym_ties_round_away_from_zero(oracle):
+    # scale = 127/127 = 1 exactly, so x/s = x and .5 values are exact ties
+    x = np.array([[127.0, 0.5, -0.5, 1.5, -1.5, 2.5, -2.5, 0.49999997]], np.float32)
+    q, s = oracle.quant_sym(x)
+    assert s[0] == 1.0
+    assert q[0].tolist() == [127, 1, -1, 2, -2, 3, -3, 0]
+
+
+def test_quant_sym_matches_numpy_float32(oracle):
+    x = rng.standard_normal((64, 2048)).astype(np.float32)
+    q, s = oracle.quant_sym(x)
+    s_np = (np.abs(x).max(axis=1) / np.float32(127)).astype(np.float32)
+    t = (x / s_np[:, None]).astype(np.float32)
+    q_np = (np.sign(t) * np.floor(np.abs(t) + np.float32(0.5))).astype(np.int8)
+    assert np.array_equal(s, s_np) and np.array_equal(q, q_np)
+
+
+def test_quant_asym_range_and_endpoints(oracle):
+    x = rng.uniform(-1, 1, (8, 256)).astype(np.float32)
+    q, s, b = oracle.quant_asym(x, bits=4)
+    assert q.min() == 0 and q.max() == 15
+    assert np.array_equal(b, x.min(axis=1))
+    assert np.all(q[np.arange(8), x.argmax(axis=1)] == 15)
+    assert np.all(np.abs(q * s[:, None] + b[:, None] - x) <= s[:, None] * 0.5 * (1 + 1e-5))
+
+
+def test_dequant_order_and_asym_term(oracle):
+    acc = rng.integers(-2**20, 2**20, (4, 32)).astype(np.int32)
+    s_x = rng.uniform(1e-3, 1e-2, 4).astype(np.float32)
+    w_s = rng.uniform(1e-3, 1e-2, 32).astype(np.float32)
+    y = oracle.dequant(acc, s_x, w_s)
+    ref = (acc.astype(np.float32) * s_x[:, None]).astype(np.float32) * w_s[None, :]
+    assert np.array_equal(y, ref.astype(np.float32))
+    b = rng.uniform(-1, 1, 4).astype(np.float32); ws = rng.uniform(-5, 5, 32).astype(np.float32)
+    y2 = oracle.dequant(acc, s_x, w_s, b, ws)
+    np.testing.assert_allclose(y2, ref.astype(np.float64) + b[:, None].astype(np.float64) * ws[None, :], rtol=1e-6, atol=1e-7)
+
+
+def test_static_quant_clamps(oracle):
+    x = np.array([[[1000.0, -1000.0, 0.26, -0.26, 0.25, 127.49 * 0.5]]], np.float32)
+    q = oracle.static_quant(x, np.array([0.5], np.float32), factor=1.0, signed=True)
+    assert q[0, 0].tolist() == [127, -128, 1, -1, 1, 127]
+    p = np.array([[[1.0, 0.5, 0.0, 1.5 / 256, 200.0 / 256]]], np.float32)
+    u = oracle.static_quant(p, np.array([1.0 / 256], np.float32), signed=False)
+    assert u.dtype == np.uint8 and u[0, 0].tolist() == [255, 128, 0, 2, 200]
+    # unsigned branch clamps high only at 2^8-1
+    u2 = oracle.static_quant(np.array([[[3.0]]], np.float32), np.array([1.0 / 255], np.float32), signed=False)
+    assert u2[0, 0, 0] == 255
+    # q uses factor*scale as the divisor (sqrt(head_dim) folded into the Q scale)
+    q2 = oracle.static_quant(np.array([[[8.0]]], np.float32), np.array([0.5], np.float32), factor=8.0)
+    assert q2[0, 0, 0] == 2
+
+
+# ------------------------------------------------------------------ integer GEMM
+def test_linear_i8_exact(oracle):
+    a = rng.integers(-128, 128, (5, 300)).astype(np.int8)
+    w = rng.integers(-128, 128, (7, 300)).astype(np.int8)
+    assert np.array_equal(oracle.linear_i8(a, w), a.astype(np.int64) @ w.astype(np.int64).T)
+    au = rng.integers(0, 256, (5, 300)).astype(np.uint8)
+    assert np.array_equal(oracle.linear_i8(au, w), au.astype(np.int64) @ w.astype(np.int64).T)
+    # extreme values at K=8192 stay inside int32
+    a = np.full((1, 8192), -128, np.int8); w = np.full((1, 8192), -128, np.int8)
+    assert oracle.linear_i8(a, w)[0, 0] == 8192 * 128 * 128
+
+
+# ------------------------------------------------------------------ FHT
+@pytest.mark.parametrize("n", [2, 4, 8, 16, 64])
+def test_fht_equals_sylvester_matrix_exactly_on_integers(oracle, n):
+    x = rng.integers(-50, 50, (6, n)).astype(np.float32)
+    H = scipy.linalg.hadamard(n).astype(np.float64)
+    assert np.array_equal(oracle.fht(x), (x.astype(np.float64) @ H.T).astype(np.float32))
+
+
+@pytest.mark.parametrize("n", [2048, 8192])
+def test_fht_large_vs_float64_and_involution(oracle, n):
+    x = rng.standard_normal((3, n)).astype(np.float32)
+    H = scipy.linalg.hadamard(n).astype(np.float64)
+    scale = np.float32(np.sqrt(n))
+    y = oracle.fht(x, scale)
+    np.testing.assert_allclose(y, x.astype(np.float64) @ H.T / np.float64(scale), rtol=0, atol=2e-5)
+    np.testing.assert_allclose(oracle.fht(y, scale), x, atol=1e-5)              # H(Hx)/n = x
+    np.testing.assert_allclose((y.astype(np.float64) ** 2).sum(1), (x.astype(np.float64) ** 2).sum(1), rtol=1e-5)
+
+
+def test_fht_stage_order_is_bits_1_to_m_minus_1_then_0(oracle):
+    """The omega network equals an in-place butterfly network whose stage s pairs indices that
+    differ in bit (s+1) mod m, bit-clear element first; same float result bit for bit."""
+    n, m = 256, 8
+    x = (rng.standard_normal((4, n)) * 1e3).astype(np.float32)
+    d = x.copy()
+    idx = np.arange(n)
+    for s in range(m):
+        bit = 1 << ((s + 1) % m)
+        lo = idx[(idx & bit) == 0]
+        u, v = d[:, lo].copy(), d[:, lo | bit].copy()
+        d[:, lo] = u + v
+        d[:, lo | bit] = u - v
+    assert np.array_equal(oracle.fht(x), d)
+
+
+# ------------------------------------------------------------------ norms / activations
+def test_rmsnorm_vs_float64(oracle):
+    x = rng.standard_normal((16, 2048)).astype(np.float32) * 3
+    g = rng.uniform(0.5, 1.5, 2048).astype(np.float32)
+    x64 = x.astype(np.float64)
+    ref = x64 / np.sqrt((x64 ** 2).mean(1, keepdims=True) + 1e-5) * g
+    np.testing.assert_allclose(oracle.rmsnorm_pref(x, g), ref, rtol=2e-6)
+    for bp in (4, 8, 16):
+        np.testing.assert_allclose(oracle.rmsnorm_dec(x[0], g, bp), ref[0], rtol=2e-6)
+    # unit-gamma output has unit mean square
+    y = oracle.rmsnorm_pref(x, np.ones(2048, np.float32))
+    np.testing.assert_allclose((y.astype(np.float64) ** 2).mean(1), 1.0, rtol=1e-4)
+
+
+def test_swish_gate_residual(oracle):
+    x = rng.standard_normal(4096).astype(np.float32) * 4
+    np.testing.assert_allclose(oracle.swish(x), x.astype(np.float64) * scipy.special.expit(x.astype(np.float64)), rtol=1e-6, atol=1e-9)
+    assert oracle.swish(np.zeros(1, np.float32))[0] == 0
+    a = rng.standard_normal(64).astype(np.float32); b = rng.standard_normal(64).astype(np.float32)
+    assert np.array_equal(oracle.gate(a, b), a * b) and np.array_equal(oracle.residual(a, b), a + b)
+
+
+def test_softmax_vs_scipy_and_ragged(oracle):
+    for dim in (1, 3, 5, 64, 1023, 4096):
+        x = (rng.standard_normal((3, dim)) * 5).astype(np.float32)
+        y = oracle.softmax(x)
+        np.testing.assert_allclose(y, scipy.special.softmax(x.astype(np.float64), axis=1), rtol=3e-6, atol=1e-12)
+        np.testing.assert_allclose(y.astype(np.float64).sum(1), 1.0, rtol=1e-5)
+    # masked entries (-1e32) become exact zeros and do not disturb the rest
+    x = (rng.standard_normal((1, 64))).astype(np.float32)
+    xm = x.copy(); xm[0, 40:] = np.float32(-1e32)
+    ym = oracle.softmax(xm)
+    assert not ym[0, 40:].any()
+    assert np.array_equal(ym[0, :40], oracle.softmax(x[:, :40])[0])
+
+
+def test_causal_mask(oracle):
+    x = rng.standard_normal((8, 2, 8)).astype(np.float32)
+    y = oracle.causal_mask(x)
+    for r in range(8):
+        assert np.array_equal(y[r, :, :r + 1], x[r, :, :r + 1])
+        assert np.all(y[r, :, r + 1:] == np.float32(-1e32))
+
+
+# ------------------------------------------------------------------ RoPE
+def _hf_llama3_inv_freq(head_dim=64, theta=500000.0, factor=32.0, low=1.0, high=4.0, orig=8192):
+    """Llama-3 rope scaling as published with the model (float64)."""
+    inv_freq = 1.0 / theta ** (np.arange(0, head_dim, 2, dtype=np.float64) / head_dim)
+    low_wl, high_wl = orig / low, orig / high
+    wl = 2 * np.pi / inv_freq
+    out = np.where(wl > low_wl, inv_freq / factor, inv_freq)
+    smooth = (orig / wl - low) / (high - low)
+    mid = (1 - smooth) * inv_freq / factor + smooth * inv_freq
+    is_mid = (wl >= high_wl) & (wl <= low_wl)
+    return np.where(is_mid, mid, out)
+
+
+def test_rope_table_vs_published_llama3_scaling(oracle):
+    s, c = oracle.rope_table(2048)
+    inv = _hf_llama3_inv_freq()
+    pos = np.arange(2048, dtype=np.float64)[:, None]
+    # float32 angle pos*freq carries ~1e-7 relative error -> absolute error grows with the angle
+    np.testing.assert_allclose(s, np.sin(pos * inv), atol=3e-4)
+    np.testing.assert_allclose(c, np.cos(pos * inv), atol=3e-4)
+    np.testing.assert_allclose(s[:64], np.sin(pos[:64] * inv), atol=1e-5)
+    assert np.all(s[0] == 0) and np.all(c[0] == 1)
+
+
+def test_rope_rotation_properties(oracle):
+    s, c = oracle.rope_table(128)
+    x = rng.standard_normal((100, 4, 64)).astype(np.float32)
+    y = oracle.rope(x, s, c, pos0=7)
+    # pairs (k, k+32) are rotated: norms preserved
+    np.testing.assert_allclose(y[..., :32] ** 2 + y[..., 32:] ** 2, x[..., :32] ** 2 + x[..., 32:] ** 2, rtol=1e-5, atol=1e-6)
+    z = (x[..., :32] + 1j * x[..., 32:]) * (c[7:107, None, :] + 1j * s[7:107, None, :])
+    np.testing.assert_allclose(y[..., :32], z.real, rtol=1e-5, atol=1e-6)
+    np.testing.assert_allclose(y[..., 32:], z.imag, rtol=1e-5, atol=1e-6)
+    assert np.array_equal(oracle.rope(x[:1], s, c, pos0=0), x[:1])       # position 0 is the identity
+
+
+# ------------------------------------------------------------------ attention
+def _scales(qh=8, kvh=2):
+    q_s = (0.02 + 0.002 * np.arange(qh)).astype(np.float32)
+    k_s = (0.03 + 0.003 * np.arange(kvh)).astype(np.float32)
+    v_s = (0.025 + 0.002 * np.arange(kvh)).astype(np.float32)
+    a_s = np.full(qh, 1.0 / 255, np.float32)
+    return q_s, k_s, v_s, a_s
+
+
+def test_mha_prefill_vs_testbench_style_fake_quant_golden(oracle):
+    """Golden built the way SpinQuant_Llama_32_1B/MHA_i8xi8_prefilling_tb.cpp:26-218 builds it:
+    fake-quant q/k/v, float matmuls, masked softmax, fake-quant P, float PV; 5e-3 relative (tb :251)."""
+    S, qh, kvh, hd = 64, 8, 2, 64
+    q = rng.uniform(-2.8, 2.8, (S, qh, hd)).astype(np.float32)
+    k = rng.uniform(-2.8, 2.8, (S, kvh, hd)).astype(np.float32)
+    v = rng.uniform(-2.8, 2.8, (S, kvh, hd)).astype(np.float32)
+    q_s, k_s, v_s, a_s = _scales(qh, kvh)
+    out = oracle.mha_prefill(q, k, v, q_s, k_s, v_s, a_s, want_p=True)
+    rnd = lambda t: np.sign(t) * np.floor(np.abs(t) + 0.5)
+    qf = np.clip(rnd(q.astype(np.float64) / 8 / q_s[None, :, None]), -128, 127)
+    kf = np.clip(rnd(k.astype(np.float64) / k_s[None, :, None]), -128, 127)
+    vf = np.clip(rnd(v.astype(np.float64) / v_s[None, :, None]), -128, 127)
+    assert np.array_equal(out["q8"], qf) and np.array_equal(out["k8"], kf) and np.array_equal(out["v8"], vf)
+    o_ref = np.zeros((S, qh, hd))
+    for h in range(qh):
+        kh = h // (qh // kvh)
+        a = (qf[:, h] * q_s[h]) @ (kf[:, kh] * k_s[kh]).T
+        a[np.triu_indices(S, 1)] = -np.inf
+        p = scipy.special.softmax(a, axis=1)
+        pq = np.minimum(255, rnd(p / a_s[h]))
+        # P may differ by one step where p/a_s sits on a rounding tie in float32 vs float64
+        assert np.abs(out["p8"][h].astype(np.int64) - pq).max() <= 1
+        assert (out["p8"][h] != pq).mean() < 2e-3
+        assert not np.triu(out["p8"][h], 1).any()
+        o_ref[:, h] = (out["p8"][h].astype(np.float64) * a_s[h]) @ (vf[:, kh] * v_s[kh])
+    np.testing.assert_allclose(out["o"], o_ref, rtol=5e-3, atol=1e-5)
+    np.testing.assert_allclose(out["o"], o_ref, rtol=1e-5, atol=1e-6)
+
+
+def test_mha_decode_equals_prefill_rows_bit_for_bit(oracle):
+    """Decode of query i over i+1 cached keys must reproduce prefill row i exactly: masked scores
+    contribute exact zeros to the same four partial sums."""
+    S, qh, kvh, hd = 37 + 3, 8, 2, 64
+    q = rng.uniform(-3, 3, (S, qh, hd)).astype(np.float32)
+    k = rng.uniform(-3, 3, (S, kvh, hd)).astype(np.float32)
+    v = rng.uniform(-3, 3, (S, kvh, hd)).astype(np.float32)
+    sc = _scales(qh, kvh)
+    out = oracle.mha_prefill(q, k, v, *sc, want_p=True)
+    for i in (0, 1, 2, 3, 4, 17, S - 1):
+        o, p = oracle.mha_decode(out["q8"][i], out["k8"][:i + 1], out["v8"][:i + 1], *sc, want_p=True)
+        assert np.array_equal(o, out["o"][i])
+        assert np.array_equal(p, out["p8"][:, i, :i + 1])
+
+
+# ------------------------------------------------------------------ layouts
+def test_prefill_and_decode_stream_layouts_roundtrip_and_index_formula(oracle):
+    tokens, dim, tp = 16, 24, 8
+    x = rng.standard_normal((tokens, dim)).astype(np.float32)
+    p = oracle.pack_pref(x, tp)
+    # MHA_i8xi8_prefilling_tb.cpp:38-40: idx = (i/TP)*dim + j ; sub = i%TP
+    for i in (0, 7, 8, 15):
+        for j in (0, 5, 23):
+            assert p.reshape(-1, tp)[(i // tp) * dim + j, i % tp] == x[i, j]
+    assert np.array_equal(oracle.unpack_pref(p, tp), x)
+    bp, d = 8, 64
+    t = rng.standard_normal(d).astype(np.float32)
+    pd = oracle.pack_dec(t, bp)
+    # Linear_Layer_Decoding_tb.cpp:148: [j % (dim/BP)][j / (dim/BP)]
+    for j in (0, 7, 8, 63):
+        assert pd[j % (d // bp), j // (d // bp)] == t[j]
+    assert np.array_equal(oracle.unpack_dec(pd, bp), t)
+
+
+def test_half_to_float_and_lm_head(oracle):
+    vals = np.array([0.0, -0.0, 1.0, -2.5, 65504.0, 6.1e-5, 5.96e-8, 3e-6, 0.333], np.float16)
+    for h in vals:
+        assert np.float32(oracle.half_to_float(h.view(np.uint16))) == np.float32(h)
+    E = rng.standard_normal((50, 128)).astype(np.float16)
+    n = rng.standard_normal(128).astype(np.float32)
+    np.testing.assert_allclose(oracle.lm_head(E.view(np.uint16), n), E.astype(np.float64) @ n, rtol=1e-4, atol=1e-4)
