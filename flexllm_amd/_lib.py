@@ -1,0 +1,52 @@
+"""ctypes binding of libflexllm_hip.so.  The library must have been built (python -m flexllm_amd.build);
+there is deliberately no fallback path."""
+import ctypes as C
+import os
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(HERE, "libflexllm_hip.so")
+
+
+class LibraryMissing(RuntimeError):
+    pass
+
+
+class FlexLLMError(RuntimeError):
+    pass
+
+
+class MhaScales(C.Structure):
+    _fields_ = [("q_s", C.c_void_p), ("k_s", C.c_void_p), ("v_s", C.c_void_p), ("a_s", C.c_void_p)]
+
+
+class LlamaConfig(C.Structure):
+    _fields_ = [(n, C.c_int) for n in
+                ("layers", "hidden", "kv_hidden", "inter", "q_heads", "kv_heads", "head_dim", "vocab", "max_pos")] + \
+               [("eps", C.c_float), ("fht_scale", C.c_float)]
+
+
+class LlamaWeights(C.Structure):
+    _fields_ = [(n, C.c_void_p) for n in
+                ("wq", "wk", "wv", "wo", "wg", "wu", "wd", "sq", "sk", "sv", "so", "sg", "su", "sd",
+                 "gamma", "q_s", "k_s", "v_s", "a_s", "rope_sin", "rope_cos", "embed")]
+
+
+_lib = None
+
+
+def lib():
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise LibraryMissing(
+                "%s not found: build it with `python -m flexllm_amd.build` (hipcc, gfx950). "
+                "There is no CPU fallback." % LIB_PATH)
+        _lib = C.CDLL(LIB_PATH)
+        _lib.flexllm_last_error.restype = C.c_char_p
+        _lib.flexllm_build_info.restype = C.c_char_p
+    return _lib
+
+
+def check(rc):
+    if rc != 0:
+        raise FlexLLMError("flexllm error %d: %s" % (rc, lib().flexllm_last_error().decode()))

@@ -1,0 +1,159 @@
+// Shared device helpers and host-side error plumbing for libflexllm_hip (gfx950 only).
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <stdio.h>
+#include "../../include/flexllm_hip.h"
+
+namespace fx {
+
+constexpr int kWave = 64;
+
+using i32x4 = int __attribute__((ext_vector_type(4)));
+using i32x16 = int __attribute__((ext_vector_type(16)));
+using f32x4 = float __attribute__((ext_vector_type(4)));
+
+void set_error(const char* fmt, ...);
+
+#define FX_REQUIRE(cond, ...)                                   \
+    do {                                                        \
+        if (!(cond)) {                                          \
+            fx::set_error(__VA_ARGS__);                         \
+            return FLEXLLM_EINVAL;                              \
+        }                                                       \
+    } while (0)
+
+#define FX_HIP(call)                                                                   \
+    do {                                                                               \
+        hipError_t e_ = (call);                                                        \
+        if (e_ != hipSuccess) {                                                        \
+            fx::set_error("%s failed: %s (%s:%d)", #call, hipGetErrorString(e_), __FILE__, __LINE__); \
+            return FLEXLLM_EHIP;                                                       \
+        }                                                                              \
+    } while (0)
+
+#define FX_LAUNCH_CHECK()                                                              \
+    do {                                                                               \
+        hipError_t e_ = hipGetLastError();                                             \
+        if (e_ != hipSuccess) {                                                        \
+            fx::set_error("kernel launch failed: %s (%s:%d)", hipGetErrorString(e_), __FILE__, __LINE__); \
+            return FLEXLLM_EHIP;                                                       \
+        }                                                                              \
+    } while (0)
+
+inline hipStream_t as_stream(void* s) { return reinterpret_cast<hipStream_t>(s); }
+
+// ---------------------------------------------------------------- cross-lane exchange
+// Value held by lane (lane ^ MASK).  1,2: DPP quad_perm; 4,8,16: ds_swizzle bit mode (no LDS
+// traffic, crossbar only); 32: bpermute.
+template <int MASK>
+__device__ __forceinline__ int lane_xor_i(int v) {
+    if constexpr (MASK == 1) {
+        return __builtin_amdgcn_mov_dpp(v, 0xB1, 0xF, 0xF, true);   // quad_perm [1,0,3,2]
+    } else if constexpr (MASK == 2) {
+        return __builtin_amdgcn_mov_dpp(v, 0x4E, 0xF, 0xF, true);   // quad_perm [2,3,0,1]
+    } else if constexpr (MASK == 4 || MASK == 8 || MASK == 16) {
+        return __builtin_amdgcn_ds_swizzle(v, (MASK << 10) | 0x1F); // and=0x1f or=0 xor=MASK
+    } else {
+        static_assert(MASK == 32, "lane_xor mask");
+        return __builtin_amdgcn_ds_bpermute(((int)(threadIdx.x & 63) ^ 32) << 2, v);
+    }
+}
+template <int MASK>
+__device__ __forceinline__ float lane_xor_f(float v) {
+    return __int_as_float(lane_xor_i<MASK>(__float_as_int(v)));
+}
+
+__device__ __forceinline__ float wave_max(float v) {
+    v = fmaxf(v, lane_xor_f<1>(v));
+    v = fmaxf(v, lane_xor_f<2>(v));
+    v = fmaxf(v, lane_xor_f<4>(v));
+    v = fmaxf(v, lane_xor_f<8>(v));
+    v = fmaxf(v, lane_xor_f<16>(v));
+    v = fmaxf(v, lane_xor_f<32>(v));
+    return v;
+}
+__device__ __forceinline__ float wave_min(float v) {
+    v = fminf(v, lane_xor_f<1>(v));
+    v = fminf(v, lane_xor_f<2>(v));
+    v = fminf(v, lane_xor_f<4>(v));
+    v = fminf(v, lane_xor_f<8>(v));
+    v = fminf(v, lane_xor_f<16>(v));
+    v = fminf(v, lane_xor_f<32>(v));
+    return v;
+}
+__device__ __forceinline__ float wave_sum(float v) {
+    v += lane_xor_f<1>(v);
+    v += lane_xor_f<2>(v);
+    v += lane_xor_f<4>(v);
+    v += lane_xor_f<8>(v);
+    v += lane_xor_f<16>(v);
+    v += lane_xor_f<32>(v);
+    return v;
+}
+__device__ __forceinline__ int wave_sum_i(int v) {
+    v += lane_xor_i<1>(v);
+    v += lane_xor_i<2>(v);
+    v += lane_xor_i<4>(v);
+    v += lane_xor_i<8>(v);
+    v += lane_xor_i<16>(v);
+    v += lane_xor_i<32>(v);
+    return v;
+}
+
+// Block-wide reductions for blocks of NW waves; `red` is NW floats of LDS.  Every thread gets the result.
+template <int NW>
+__device__ __forceinline__ float block_max(float v, float* red) {
+    v = wave_max(v);
+    if constexpr (NW == 1) return v;
+    const int w = threadIdx.x >> 6;
+    __syncthreads();
+    if ((threadIdx.x & 63) == 0) red[w] = v;
+    __syncthreads();
+    float r = red[0];
+#pragma unroll
+    for (int i = 1; i < NW; i++) r = fmaxf(r, red[i]);
+    return r;
+}
+template <int NW>
+__device__ __forceinline__ float block_min(float v, float* red) {
+    v = wave_min(v);
+    if constexpr (NW == 1) return v;
+    const int w = threadIdx.x >> 6;
+    __syncthreads();
+    if ((threadIdx.x & 63) == 0) red[w] = v;
+    __syncthreads();
+    float r = red[0];
+#pragma unroll
+    for (int i = 1; i < NW; i++) r = fminf(r, red[i]);
+    return r;
+}
+template <int NW>
+__device__ __forceinline__ float block_sum(float v, float* red) {
+    v = wave_sum(v);
+    if constexpr (NW == 1) return v;
+    const int w = threadIdx.x >> 6;
+    __syncthreads();
+    if ((threadIdx.x & 63) == 0) red[w] = v;
+    __syncthreads();
+    float r = red[0];
+#pragma unroll
+    for (int i = 1; i < NW; i++) r += red[i];
+    return r;
+}
+
+// ---------------------------------------------------------------- quantisation arithmetic
+// round half away from zero of x/s with IEEE division, wrapped to 8 bits like (ap_int<8>)round(x/s).
+__device__ __forceinline__ int quant_round(float x, float s) { return (int)roundf(x / s); }
+
+__device__ __forceinline__ uint32_t pack4_i8(int a, int b, int c, int d) {
+    return (uint32_t)(a & 0xff) | ((uint32_t)(b & 0xff) << 8) | ((uint32_t)(c & 0xff) << 16) | ((uint32_t)(d & 0xff) << 24);
+}
+
+// symmetric scale from a row's absmax: absmax/127, 0 -> 1
+__device__ __forceinline__ float sym_scale(float absmax, float scale_base) {
+    float s = absmax / scale_base;
+    return s == 0.0f ? 1.0f : s;
+}
+
+}  // namespace fx

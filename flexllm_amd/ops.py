@@ -1,0 +1,234 @@
+"""Python wrappers over the C ABI operators.  Arguments are DeviceArrays; outputs are allocated here
+unless passed in.  Names follow the reference's module names (quant, Linear_Layer, FHT, LayerNorm, RoPE,
+Swish, Residual_Layer, Softmax, MHA_i8xi8)."""
+import ctypes as C
+
+import numpy as np
+
+from ._lib import lib, check, MhaScales
+from .device import DeviceArray, _s, to_device
+
+
+def _p(a):
+    return C.c_void_p(a.ptr) if a is not None else None
+
+
+def _rows(a):
+    return int(np.prod(a.shape[:-1], dtype=np.int64))
+
+
+# ---------------------------------------------------------------- quant.h
+def quant_sym_i8(x, stream=None):
+    q = DeviceArray(x.shape, np.int8)
+    s = DeviceArray(x.shape[:-1] or (1,), np.float32)
+    check(lib().flexllm_quant_sym_i8(_p(x), _p(q), _p(s), _rows(x), x.shape[-1], _s(stream)))
+    return q, s
+
+
+def quant_asym_u8(x, bits=4, stream=None):
+    q = DeviceArray(x.shape, np.uint8)
+    s = DeviceArray(x.shape[:-1] or (1,), np.float32)
+    b = DeviceArray(x.shape[:-1] or (1,), np.float32)
+    check(lib().flexllm_quant_asym_u8(_p(x), _p(q), _p(s), _p(b), bits, _rows(x), x.shape[-1], _s(stream)))
+    return q, s, b
+
+
+def dequant_i32_f32(acc, s_x, w_s, b_x=None, w_sum=None, stream=None):
+    y = DeviceArray(acc.shape, np.float32)
+    check(lib().flexllm_dequant_i32_f32(_p(acc), _p(s_x), _p(b_x), _p(w_s), _p(w_sum), _p(y), _rows(acc),
+                                        acc.shape[-1], _s(stream)))
+    return y
+
+
+def static_quant_i8(x, scale, factor=1.0, signed=True, stream=None):
+    rows, heads, dim = x.shape
+    q = DeviceArray(x.shape, np.int8 if signed else np.uint8)
+    check(lib().flexllm_static_quant_i8(_p(x), _p(q), _p(scale), C.c_float(factor), int(signed), rows, heads, dim,
+                                        _s(stream)))
+    return q
+
+
+def static_dequant_i32_f32(acc, a_s, w_s, stream=None):
+    rows, ah, dim = acc.shape
+    y = DeviceArray(acc.shape, np.float32)
+    check(lib().flexllm_static_dequant_i32_f32(_p(acc), _p(y), _p(a_s), _p(w_s), rows, ah, w_s.shape[0], dim, _s(stream)))
+    return y
+
+
+def head_quant_sym_i8(x, stream=None):
+    rows, heads, dim = x.shape
+    q = DeviceArray(x.shape, np.int8)
+    s = DeviceArray((rows, heads), np.float32)
+    check(lib().flexllm_head_quant_sym_i8(_p(x), _p(q), _p(s), rows, heads, dim, _s(stream)))
+    return q, s
+
+
+# ---------------------------------------------------------------- Linear_Layer.h
+def linear_i8_gemv(x, w, stream=None, out=None):
+    n, k = w.shape
+    acc = out if out is not None else DeviceArray((n,), np.int32)
+    check(lib().flexllm_linear_i8_gemv(_p(x), _p(w), _p(acc), k, n, _s(stream)))
+    return acc
+
+
+def linear_i8_gemv_dequant(x, s_x, w, w_s, residual=None, stream=None, out=None):
+    n, k = w.shape
+    y = out if out is not None else DeviceArray((n,), np.float32)
+    check(lib().flexllm_linear_i8_gemv_dequant(_p(x), _p(s_x), _p(w), _p(w_s), _p(residual), _p(y), k, n, _s(stream)))
+    return y
+
+
+def linear_i8_gemm(a, w, stream=None, out=None):
+    m, k = a.shape
+    n = w.shape[0]
+    acc = out if out is not None else DeviceArray((m, n), np.int32)
+    check(lib().flexllm_linear_i8_gemm(_p(a), _p(w), _p(acc), m, k, n, _s(stream)))
+    return acc
+
+
+def linear_i8_gemm_dequant(a, s_x, w, w_s, residual=None, stream=None, out=None):
+    m, k = a.shape
+    n = w.shape[0]
+    y = out if out is not None else DeviceArray((m, n), np.float32)
+    check(lib().flexllm_linear_i8_gemm_dequant(_p(a), _p(s_x), _p(w), _p(w_s), _p(residual), _p(y), m, k, n, _s(stream)))
+    return y
+
+
+# ---------------------------------------------------------------- FHT.h
+def fht_f32(x, scale=1.0, stream=None, out=None):
+    y = out if out is not None else DeviceArray(x.shape, np.float32)
+    check(lib().flexllm_fht_f32(_p(x), _p(y), _rows(x), x.shape[-1], C.c_float(scale), _s(stream)))
+    return y
+
+
+def fht_quant_i8(x, scale=1.0, stream=None):
+    q = DeviceArray(x.shape, np.int8)
+    s = DeviceArray(x.shape[:-1] or (1,), np.float32)
+    check(lib().flexllm_fht_quant_i8(_p(x), _p(q), _p(s), _rows(x), x.shape[-1], C.c_float(scale), _s(stream)))
+    return q, s
+
+
+# ---------------------------------------------------------------- LayerNorm.h
+def rmsnorm_f32(x, gamma, eps=1e-5, stream=None):
+    y = DeviceArray(x.shape, np.float32)
+    check(lib().flexllm_rmsnorm_f32(_p(x), _p(gamma), _p(y), _rows(x), x.shape[-1], C.c_float(eps), _s(stream)))
+    return y
+
+
+def rmsnorm_quant_i8(x, gamma, eps=1e-5, stream=None):
+    q = DeviceArray(x.shape, np.int8)
+    s = DeviceArray(x.shape[:-1] or (1,), np.float32)
+    check(lib().flexllm_rmsnorm_quant_i8(_p(x), _p(gamma), _p(q), _p(s), _rows(x), x.shape[-1], C.c_float(eps), _s(stream)))
+    return q, s
+
+
+# ---------------------------------------------------------------- RoPE.h
+def rope_table(max_pos, head_dim=64, theta=500000.0, factor=32, low=1, high=4, orig=8192):
+    s = np.empty((max_pos, head_dim // 2), np.float32)
+    c = np.empty((max_pos, head_dim // 2), np.float32)
+    check(lib().flexllm_rope_table_host(s.ctypes.data_as(C.c_void_p), c.ctypes.data_as(C.c_void_p), max_pos, head_dim,
+                                        C.c_float(theta), factor, low, high, orig))
+    return s, c
+
+
+def rope_f32(x, sin_t, cos_t, pos0=0, stream=None):
+    tokens, heads, hd = x.shape
+    y = DeviceArray(x.shape, np.float32)
+    check(lib().flexllm_rope_f32(_p(x), _p(y), _p(sin_t), _p(cos_t), tokens, heads, hd, pos0, _s(stream)))
+    return y
+
+
+# ---------------------------------------------------------------- Swish.h / gate / Residual_Layer.h
+def swish_f32(x, stream=None):
+    y = DeviceArray(x.shape, np.float32)
+    check(lib().flexllm_swish_f32(_p(x), _p(y), C.c_size_t(x.size), _s(stream)))
+    return y
+
+
+def swiglu_f32(gate, up, stream=None):
+    y = DeviceArray(gate.shape, np.float32)
+    check(lib().flexllm_swiglu_f32(_p(gate), _p(up), _p(y), C.c_size_t(gate.size), _s(stream)))
+    return y
+
+
+def residual_add_f32(a, b, stream=None):
+    y = DeviceArray(a.shape, np.float32)
+    check(lib().flexllm_residual_add_f32(_p(a), _p(b), _p(y), C.c_size_t(a.size), _s(stream)))
+    return y
+
+
+def softmax_f32(x, stream=None):
+    y = DeviceArray(x.shape, np.float32)
+    check(lib().flexllm_softmax_f32(_p(x), _p(y), _rows(x), x.shape[-1], _s(stream)))
+    return y
+
+
+# ---------------------------------------------------------------- MHA_i8xi8.h
+class Scales:
+    """Device copies of one layer's static attention scales."""
+
+    def __init__(self, q_s, k_s, v_s, a_s):
+        self.arrays = [to_device(np.asarray(a, np.float32)) for a in (q_s, k_s, v_s, a_s)]
+        self.struct = MhaScales(*[a.ptr for a in self.arrays])
+
+    def ref(self):
+        return C.byref(self.struct)
+
+
+def kv_cache(kv_heads, max_pos, head_dim=64):
+    assert max_pos % 64 == 0
+    k = DeviceArray((kv_heads, max_pos, head_dim), np.int8).zero_()
+    v = DeviceArray((kv_heads, max_pos // 64, head_dim, 64), np.int8).zero_()
+    return k, v
+
+
+def kv_append_i8(k, v, k_cache, v_cache, scales, pos0, stream=None):
+    tokens, kvh, hd = k.shape
+    max_pos = k_cache.shape[1]
+    check(lib().flexllm_kv_append_i8(_p(k), _p(v), _p(k_cache), _p(v_cache), scales.ref(), tokens, kvh, hd, max_pos, pos0,
+                                     _s(stream)))
+
+
+def kv_store_i8(k8, v8, k_cache, v_cache, pos0, stream=None):
+    tokens, kvh, hd = k8.shape
+    max_pos = k_cache.shape[1]
+    check(lib().flexllm_kv_store_i8(_p(k8), _p(v8), _p(k_cache), _p(v_cache), tokens, kvh, hd, max_pos, pos0, _s(stream)))
+
+
+def mha_i8_decode(q8, k_cache, v_cache, scales, length, want_p=False, stream=None):
+    qh, hd = q8.shape
+    kvh, max_pos, _ = k_cache.shape
+    o = DeviceArray((qh, hd), np.float32)
+    p8 = DeviceArray((qh, length), np.uint8) if want_p else None
+    check(lib().flexllm_mha_i8_decode(_p(q8), _p(k_cache), _p(v_cache), scales.ref(), _p(o), _p(p8), length, qh, kvh, hd,
+                                      max_pos, _s(stream)))
+    return o, p8
+
+
+def mha_i8_prefill(q8, k8, v8, scales, want_p=False, stream=None):
+    s, qh, hd = q8.shape
+    kvh = k8.shape[1]
+    o = DeviceArray((s, qh, hd), np.float32)
+    p8 = DeviceArray((qh, s, s), np.uint8) if want_p else None
+    check(lib().flexllm_mha_i8_prefill(_p(q8), _p(k8), _p(v8), scales.ref(), _p(o), _p(p8), s, qh, kvh, hd, _s(stream)))
+    return o, p8
+
+
+# ---------------------------------------------------------------- Logits.h (greedy)
+def embed_f16(table, token, stream=None):
+    y = DeviceArray((table.shape[1],), np.float32)
+    check(lib().flexllm_embed_f16(_p(table), _p(token), _p(y), table.shape[1], _s(stream)))
+    return y
+
+
+def lm_head_f16(table, n, stream=None):
+    vocab, hidden = table.shape
+    logits = DeviceArray((vocab,), np.float32)
+    check(lib().flexllm_lm_head_f16(_p(table), _p(n), _p(logits), vocab, hidden, _s(stream)))
+    return logits
+
+
+def argmax_f32(x, stream=None):
+    r = DeviceArray((1,), np.int32)
+    check(lib().flexllm_argmax_f32(_p(x), x.size, _p(r), _s(stream)))
+    return r

@@ -1,0 +1,241 @@
+/*
+ * flexllm_hip.h - C ABI of libflexllm_hip.so: the FlexLLM quantized-transformer
+ * datapath (Modules/ + MHA_i8xi8.h of Crazy-James26/FlexLLM) on one MI355X (gfx950).
+ *
+ * Conventions
+ *  - Every tensor pointer is DEVICE memory, dense row-major, token-major
+ *    (x[token][feature]); weights are int8 [out_features][in_features].
+ *  - `stream` is a hipStream_t passed as void* (NULL = default stream).  Calls only
+ *    enqueue work; nothing synchronises unless stated.
+ *  - Return value: 0 on success, a negative FLEXLLM_E* code otherwise (the reference
+ *    functions return void and print; errors here never print).  flexllm_last_error()
+ *    gives the message of the last failure on the calling thread.
+ *  - Integer results (int32 accumulators, int8/uint8 tensors) are bit-exact functions of
+ *    their inputs.  fp32 results follow the reference's operation order except for
+ *    reductions over a row (sum of squares, sum of exponentials), whose association
+ *    differs; those agree to <=1e-3 relative.
+ *
+ * Reference citations are relative to the reference tree root.
+ */
+#ifndef FLEXLLM_HIP_H
+#define FLEXLLM_HIP_H
+#include <stddef.h>
+#include <stdint.h>
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define FLEXLLM_OK 0
+#define FLEXLLM_EINVAL (-1)   /* bad shape / null pointer / unsupported size */
+#define FLEXLLM_EHIP (-2)     /* a HIP runtime call failed */
+#define FLEXLLM_ENOMEM (-3)
+
+const char* flexllm_last_error(void);
+/* Library version and the offload architecture the kernels were built for ("gfx950"). */
+const char* flexllm_build_info(void);
+
+/* ---- minimal runtime plumbing for hosts without a HIP binding (ctypes, cgo ...) ---- */
+int flexllm_rt_device_count(int* count);
+int flexllm_rt_device_name(char* buf, int buflen);
+int flexllm_rt_malloc(void** dptr, size_t bytes);
+int flexllm_rt_free(void* dptr);
+int flexllm_rt_memcpy_h2d(void* dst, const void* src, size_t bytes, void* stream);
+int flexllm_rt_memcpy_d2h(void* dst, const void* src, size_t bytes, void* stream);
+int flexllm_rt_memcpy_d2d(void* dst, const void* src, size_t bytes, void* stream);
+int flexllm_rt_memset(void* dst, int value, size_t bytes, void* stream);
+int flexllm_rt_stream_create(void** stream);
+int flexllm_rt_stream_destroy(void* stream);
+int flexllm_rt_stream_sync(void* stream);
+int flexllm_rt_device_sync(void);
+int flexllm_rt_event_create(void** event);
+int flexllm_rt_event_destroy(void* event);
+int flexllm_rt_event_record(void* event, void* stream);
+int flexllm_rt_event_sync(void* event);
+int flexllm_rt_event_elapsed_ms(void* start, void* stop, float* ms);
+/* Fill with a counter-based PRNG (SplitMix64 of seed+index): int8 uniform in [lo,hi], fp32
+ * uniform in [lo,hi), fp32 standard normal (Box-Muller).  Bit-identical to
+ * flexllm_amd.synth on the host. */
+int flexllm_rt_fill_i8(int8_t* dst, size_t n, uint64_t seed, int lo, int hi, void* stream);
+int flexllm_rt_fill_uniform_f32(float* dst, size_t n, uint64_t seed, float lo, float hi, void* stream);
+int flexllm_rt_fill_uniform_f16(uint16_t* dst, size_t n, uint64_t seed, float lo, float hi, void* stream);
+
+/* ---- quant.h ------------------------------------------------------------------------ */
+/* Per-token symmetric int8 quantisation: s=absmax/127 (0 -> 1), q=round_half_away(x/s).
+ * Replaces pref_quant_layer_fp32_qint<8,false,...> (Modules/quant.h:6-112) and
+ * dec_quant_layer_fp32_qint<8,false,...> (Modules/quant.h:332-431).  x [rows][dim] fp32,
+ * q [rows][dim] int8, s [rows] fp32.  dim % 4 == 0. */
+int flexllm_quant_sym_i8(const float* x, int8_t* q, float* s, int rows, int dim, void* stream);
+/* Per-token asymmetric unsigned quantisation (bits in 2..8): s=(max-min)/(2^bits-1), b=min,
+ * q=round((x-b)/s) stored one value per byte.  Modules/quant.h:53-82, :382-405. */
+int flexllm_quant_asym_u8(const float* x, uint8_t* q, float* s, float* b, int bits, int rows, int dim, void* stream);
+/* y[r][n] = (float(acc[r][n]) * s_x[r]) * w_s[n]  [+ b_x[r] * w_sum[n]] ; b_x and w_sum may both be NULL.
+ * Replaces pref_dequant_layer_qint_fp32 (Modules/quant.h:115-164) and
+ * dec_dequant_layer_qint_fp32(_bandwidth) (Modules/quant.h:434-524). */
+int flexllm_dequant_i32_f32(const int32_t* acc, const float* s_x, const float* b_x, const float* w_s,
+                            const float* w_sum, float* y, int rows, int n, void* stream);
+/* Static per-head quantisation: q=clamp(round(x/(factor*scale[h]))); x [rows][heads][dim].
+ * is_signed=1: clamp to [-128,127]; 0: clamp high to 255, stored as uint8 bit pattern.
+ * Replaces pref_static_sym_per_tensor_quant_layer_fp32_qint (Modules/quant.h:252-293) and
+ * dec_MHA_static_sym_per_tensor_quant_layer_fp32_qint (Modules/quant.h:716-755). */
+int flexllm_static_quant_i8(const float* x, int8_t* q, const float* scale, float factor, int is_signed,
+                            int rows, int heads, int dim, void* stream);
+/* y=(float(acc)*a_s[h])*w_s[h/(act_heads/w_heads)]; acc [rows][act_heads][dim].
+ * Replaces pref_static_sym_per_tensor_dequant_layer_qint_fp32 (Modules/quant.h:296-326) and the
+ * decode form (Modules/quant.h:758-805). */
+int flexllm_static_dequant_i32_f32(const int32_t* acc, float* y, const float* a_s, const float* w_s,
+                                   int rows, int act_heads, int w_heads, int dim, void* stream);
+/* Dynamic per-(token,head) symmetric int8 quantisation, x [rows][heads][dim], s [rows][heads].
+ * Replaces dec_MHA_quant_layer_fp32_qint<8,false,...> (Modules/quant.h:527-617). */
+int flexllm_head_quant_sym_i8(const float* x, int8_t* q, float* s, int rows, int heads, int dim, void* stream);
+
+/* ---- Linear_Layer.h ------------------------------------------------------------------- */
+/* Decode GEMV, exact: acc[n] = sum_k x[k]*W[n][k].  Replaces dec_Linear_Layer_i4xi4
+ * (Modules/Linear_Layer.h:862-923) instantiated with the int8 PEs (Modules/PE.h:793-830,
+ * Modules/MHA.h:564-611).  k % 16 == 0, k <= 16384. */
+int flexllm_linear_i8_gemv(const int8_t* x, const int8_t* w, int32_t* acc, int k, int n, void* stream);
+/* Fused decode linear: y[n] = (float(acc[n])*s_x[0])*w_s[n] (+ residual[n] if residual != NULL).
+ * = GEMV above + dec_dequant_layer_qint_fp32_bandwidth (Modules/quant.h:470-524)
+ * (+ dec_Residual_Layer, Modules/Residual_Layer.h:69-87). */
+int flexllm_linear_i8_gemv_dequant(const int8_t* x, const float* s_x, const int8_t* w, const float* w_s,
+                                   const float* residual, float* y, int k, int n, void* stream);
+/* Prefill GEMM, exact: acc[m][n] = sum_k a[m][k]*W[n][k] on int8 MFMA tiles.  Replaces
+ * pref_Linear_Layer_i4xi4 (Modules/Linear_Layer.h:293-341) with the int8 systolic array
+ * (Modules/MHA.h:113-187, Modules/PE.h:526-583).  k % 64 == 0. */
+int flexllm_linear_i8_gemm(const int8_t* a, const int8_t* w, int32_t* acc, int m, int k, int n, void* stream);
+/* Fused prefill linear: y[m][n] = (float(acc)*s_x[m])*w_s[n] (+ residual[m][n]).
+ * = GEMM + pref_dequant_layer_qint_fp32 (Modules/quant.h:115-164) (+ pref_Residual_Layer). */
+int flexllm_linear_i8_gemm_dequant(const int8_t* a, const float* s_x, const int8_t* w, const float* w_s,
+                                   const float* residual, float* y, int m, int k, int n, void* stream);
+
+/* ---- FHT.h ---------------------------------------------------------------------------- */
+/* y = H_n x / scale (Sylvester order, butterfly stage order of the reference's omega network, so
+ * the fp32 result is bit-identical).  Replaces pref_FHT (Modules/FHT.h:7-67) and dec_FHT
+ * (Modules/FHT.h:69-129).  n is a power of two, 1024 <= n <= 8192. In-place allowed. */
+int flexllm_fht_f32(const float* x, float* y, int rows, int n, float scale, void* stream);
+/* FHT followed by flexllm_quant_sym_i8 on each transformed row, without the fp32 round trip. */
+int flexllm_fht_quant_i8(const float* x, int8_t* q, float* s, int rows, int n, float scale, void* stream);
+
+/* ---- LayerNorm.h ---------------------------------------------------------------------- */
+/* RMSNorm: y = (x * (1/sqrt(mean(x^2)+eps))) * gamma.  Replaces pref_Layer_Norm
+ * (Modules/LayerNorm.h:28-183) and dec_Layer_Norm (Modules/LayerNorm.h:210-370), beta disabled. */
+int flexllm_rmsnorm_f32(const float* x, const float* gamma, float* y, int rows, int dim, float eps, void* stream);
+/* RMSNorm followed by flexllm_quant_sym_i8 on each row. */
+int flexllm_rmsnorm_quant_i8(const float* x, const float* gamma, int8_t* q, float* s, int rows, int dim,
+                             float eps, void* stream);
+
+/* ---- RoPE.h --------------------------------------------------------------------------- */
+/* Rotate-half RoPE from tables sin_t/cos_t [max_pos][head_dim/2]; x,y [tokens][heads][head_dim];
+ * token t sits at position pos0+t.  Replaces pref_RoPE_layer (Modules/RoPE.h:8-94) and
+ * dec_RoPE_layer (Modules/RoPE.h:96-173). */
+int flexllm_rope_f32(const float* x, float* y, const float* sin_t, const float* cos_t, int tokens, int heads,
+                     int head_dim, int pos0, void* stream);
+/* Host-side table builder (Llama-3 frequency scaling, formula kept in Modules/RoPE.h:28-50);
+ * sin_t/cos_t are HOST pointers [max_pos][head_dim/2]. */
+int flexllm_rope_table_host(float* sin_t, float* cos_t, int max_pos, int head_dim, float theta, int factor,
+                            int low_freq_factor, int high_freq_factor, int original_max_pe);
+
+/* ---- Swish.h / gate / Residual_Layer.h --------------------------------------------------- */
+/* y = x/(1+exp(-x)).  pref_Swish / dec_Swish (Modules/Swish.h:5-41). */
+int flexllm_swish_f32(const float* x, float* y, size_t n, void* stream);
+/* y = up * (gate/(1+exp(-gate))).  Swish + pref/dec_Gate_Layer_fp32xfp32
+ * (Modules/Linear_Layer.h:612-630, :1103-1121). */
+int flexllm_swiglu_f32(const float* gate, const float* up, float* y, size_t n, void* stream);
+/* y = a + b.  pref/dec_Residual_Layer (Modules/Residual_Layer.h:47-87). */
+int flexllm_residual_add_f32(const float* a, const float* b, float* y, size_t n, void* stream);
+
+/* ---- Softmax.h / MHA.h --------------------------------------------------------------- */
+/* Row softmax with max subtraction.  pref_Softmax (Modules/Softmax.h:6-163), dec_MHA_Softmax
+ * (Modules/Softmax.h:456-635). */
+int flexllm_softmax_f32(const float* x, float* y, int rows, int dim, void* stream);
+
+/* Static per-head attention scales of one layer (device pointers): Q_s[q_heads], K_s[kv_heads],
+ * V_s[kv_heads], A_s[q_heads] (parameters/{Q,K,V,A}_s.h rows, SpinQuant_Llama_32_1B/MHA_i8xi8.h:11-14). */
+typedef struct {
+    const float* q_s;
+    const float* k_s;
+    const float* v_s;
+    const float* a_s;
+} flexllm_mha_scales;
+
+/* int8 KV cache of one layer, head-major so that one head's keys are contiguous:
+ *   K: [kv_heads][max_pos][64]              V: [kv_heads][max_pos/64][64 channels][64 positions]
+ * (max_pos % 64 == 0).  The reference's 16/32-token line layouts (Modules/MHA.h:74-109, :299-336,
+ * :447-515, :741-804) are converted by the host adapter. */
+/* Append: quantise k (post-RoPE) and v fp32 [tokens][kv_heads][head_dim] with K_s / V_s and store at
+ * positions pos0.. ; replaces the static quant + dec_K/V_cache_buffer/manager write path. */
+int flexllm_kv_append_i8(const float* k, const float* v, int8_t* k_cache, int8_t* v_cache,
+                         const flexllm_mha_scales* sc, int tokens, int kv_heads, int head_dim, int max_pos,
+                         int pos0, void* stream);
+/* Same for already-quantised int8 k8/v8 [tokens][kv_heads][head_dim] (pure relayout). */
+int flexllm_kv_store_i8(const int8_t* k8, const int8_t* v8, int8_t* k_cache, int8_t* v_cache, int tokens,
+                        int kv_heads, int head_dim, int max_pos, int pos0, void* stream);
+/* Decode attention for one query token against `len` cached positions (new token already appended):
+ * scores=q8.K8 (int32) -> *Q_s*K_s -> softmax -> P=min(255,round(p/A_s)) (uint8) -> P.V8 (int32) -> *A_s*V_s.
+ * Replaces the dec_MHA_i8xi8_qxk / dec_MHA_Softmax / quant / dec_MHA_i8xi8_axv chain of
+ * SpinQuant_Llama_32_1B/MHA_i8xi8.h:1027-1114.  q8 [q_heads][head_dim]; o fp32 [q_heads][head_dim];
+ * p8_out (optional, may be NULL) uint8 [q_heads][len].  head_dim == 64, len <= 8192, q_heads/kv_heads <= 4.
+ * Uses a library-owned scratch buffer (allocated on first use, grown with a device synchronisation). */
+int flexllm_mha_i8_decode(const int8_t* q8, const int8_t* k_cache, const int8_t* v_cache,
+                          const flexllm_mha_scales* sc, float* o, uint8_t* p8_out, int len, int q_heads,
+                          int kv_heads, int head_dim, int max_pos, void* stream);
+/* Prefill causal attention over s tokens: q8 [s][q_heads][64], k8/v8 [s][kv_heads][64] int8 (already
+ * quantised), o fp32 [s][q_heads][64].  Replaces SpinQuant_Llama_32_1B/MHA_i8xi8.h:369-427 from the
+ * qxk stage on.  s % 64 == 0.  p8_out optional uint8 [q_heads][s][s]. */
+int flexllm_mha_i8_prefill(const int8_t* q8, const int8_t* k8, const int8_t* v8, const flexllm_mha_scales* sc,
+                           float* o, uint8_t* p8_out, int s, int q_heads, int kv_heads, int head_dim, void* stream);
+
+/* ---- Logits.h (greedy) ---------------------------------------------------------------- */
+/* logits[v] = sum_k fp16(E[v][k]) * n[k] (fp32 accumulate): tied fp16 lm_head GEMV. */
+int flexllm_lm_head_f16(const uint16_t* embed, const float* n, float* logits, int vocab, int hidden, void* stream);
+/* Index of the maximum (lowest index on ties); result is a device int. */
+int flexllm_argmax_f32(const float* x, int n, int* result, void* stream);
+/* y = fp32(E[token]) with the token id read from device memory. */
+int flexllm_embed_f16(const uint16_t* embed, const int* token, float* y, int hidden, void* stream);
+
+/* ---- whole model: Llama-3.2-1B W8A8 SpinQuant graph ------------------------------------- */
+/* Layer order of SpinQuant_Llama_32_1B/SpinQuant_Prefilling.h:940-1049 and
+ * SpinQuant_Decoding_mem_opt.h:1050-1126 with int8 symmetric linear layers. */
+typedef struct {
+    int layers, hidden, kv_hidden, inter, q_heads, kv_heads, head_dim, vocab, max_pos;
+    float eps, fht_scale;
+} flexllm_llama_config;
+
+typedef struct {
+    /* arrays of `layers` device pointers (host arrays of device pointers) */
+    const int8_t* const* wq; const int8_t* const* wk; const int8_t* const* wv; const int8_t* const* wo;
+    const int8_t* const* wg; const int8_t* const* wu; const int8_t* const* wd;
+    const float* const* sq; const float* const* sk; const float* const* sv; const float* const* so;
+    const float* const* sg; const float* const* su; const float* const* sd;
+    const float* gamma;                 /* device [2*layers+1][hidden] */
+    const float* q_s; const float* k_s; const float* v_s; const float* a_s; /* device [layers][heads] */
+    const float* rope_sin; const float* rope_cos;                           /* device [max_pos][head_dim/2] */
+    const uint16_t* embed;              /* device fp16 [vocab][hidden] */
+} flexllm_llama_weights;
+
+typedef struct flexllm_llama flexllm_llama;
+
+/* Copies/repacks the weights into the library's own device layout (fused qkv and gate/up rows) and
+ * allocates the int8 KV cache [layers][max_pos][kv_hidden] x2 and the activation workspace. */
+int flexllm_llama_create(flexllm_llama** out, const flexllm_llama_config* cfg, const flexllm_llama_weights* w);
+int flexllm_llama_destroy(flexllm_llama* m);
+/* Device pointers to the int8 caches ([layers][max_pos][kv_hidden]) for inspection / pre-filling. */
+int flexllm_llama_kv_cache(flexllm_llama* m, int8_t** k_cache, int8_t** v_cache);
+/* One decode step at position pos from fp32 embedding x_in (device, [hidden]); writes the residual
+ * stream after the last layer to hidden_out (device, may be NULL) and, if logits != NULL, the fp32
+ * logits [vocab]. */
+int flexllm_llama_decode_hidden(flexllm_llama* m, const float* x_in, int pos, float* hidden_out, float* logits,
+                                void* stream);
+/* Greedy generation loop on the device: starting from token id *token_io (device int) at position pos0,
+ * runs `steps` decode steps (embedding lookup -> 16 layers -> final norm -> lm_head -> argmax), writes the
+ * generated ids to tokens_out (device int[steps]).  With use_graph != 0 one step is captured in a HIP graph
+ * and replayed. */
+int flexllm_llama_decode_greedy(flexllm_llama* m, int* token_io, int pos0, int steps, int* tokens_out,
+                                int use_graph, void* stream);
+/* Prefill s tokens at positions 0..s-1 from fp32 embeddings x_in (device [s][hidden]); fills the KV cache,
+ * writes the residual stream to hidden_out (device [s][hidden], may be NULL). */
+int flexllm_llama_prefill_hidden(flexllm_llama* m, const float* x_in, int s, float* hidden_out, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif
