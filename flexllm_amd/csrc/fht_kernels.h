@@ -1,0 +1,138 @@
+// Fast Walsh-Hadamard transform of fp32 rows (SpinQuant online rotation), optionally fused with the
+// per-token int8 quantisation that follows it.
+//
+// The reference runs an omega network: log2(n) x (perfect shuffle, butterfly on adjacent pairs).  That is
+// the in-place butterfly network whose stage s pairs the elements whose indices differ in bit
+// (s+1) mod log2(n), the bit-clear element receiving u+v and the bit-set element u-v.  Running the
+// stages in that order (bits 1,2,...,log2(n)-1, then 0) reproduces the reference's fp32 result bit for
+// bit, so the int8 tensor quantised from it is exact as well.
+//
+// One workgroup of 256 threads transforms one row:
+//   layout A: element i = j*1024 + t*4 + e   (float4 loads, e = bits 0-1, lane = bits 2-7, wave = bits 8-9,
+//             j = bits 10+)      -> stage bit 1 in registers, bits 2..7 as cross-lane butterflies (DPP
+//             quad_perm / ds_swizzle / bpermute), no memory traffic
+//   one transpose through LDS
+//   layout B: element i = r*256 + t          (r = bits 8+, t = bits 0-7)
+//                                -> stages bits 8.. in registers, then bit 0 as a DPP butterfly.
+#pragma once
+#include "common.h"
+
+namespace fx {
+
+constexpr int kFhtBlock = 256;
+
+template <int MASK>
+__device__ __forceinline__ float lane_butterfly(float a, bool bit_set) {
+    const float p = lane_xor_f<MASK>(a);
+    return bit_set ? (p - a) : (a + p);
+}
+
+template <int LOG2N, bool QUANT>
+__global__ __launch_bounds__(kFhtBlock) void fht_kernel(const float* __restrict__ x, float* __restrict__ y,
+                                                        int8_t* __restrict__ q, float* __restrict__ s, float scale) {
+    constexpr int N = 1 << LOG2N;
+    constexpr int NJ = N / 1024;   // float4 vectors per thread in layout A
+    constexpr int NR = N / 256;    // floats per thread in layout B
+    __shared__ float lds[N];
+    __shared__ float red[kFhtBlock / kWave];
+    const int t = threadIdx.x;
+    const int lane = t & 63;
+    const size_t row = blockIdx.x;
+    const float4* xr = reinterpret_cast<const float4*>(x + row * N);
+
+    float4 a[NJ];
+#pragma unroll
+    for (int j = 0; j < NJ; j++) a[j] = xr[j * 256 + t];
+
+    // stage: bit 1 (elements e and e^2 of each float4)
+#pragma unroll
+    for (int j = 0; j < NJ; j++) {
+        const float u0 = a[j].x, v0 = a[j].z, u1 = a[j].y, v1 = a[j].w;
+        a[j].x = u0 + v0; a[j].z = u0 - v0;
+        a[j].y = u1 + v1; a[j].w = u1 - v1;
+    }
+    // stages: bits 2..7 = lane bits 0..5
+#define FX_LANE_STAGE(MASK)                                             \
+    {                                                                   \
+        const bool hi = (lane & MASK) != 0;                             \
+        _Pragma("unroll") for (int j = 0; j < NJ; j++) {                \
+            a[j].x = lane_butterfly<MASK>(a[j].x, hi);                  \
+            a[j].y = lane_butterfly<MASK>(a[j].y, hi);                  \
+            a[j].z = lane_butterfly<MASK>(a[j].z, hi);                  \
+            a[j].w = lane_butterfly<MASK>(a[j].w, hi);                  \
+        }                                                               \
+    }
+    FX_LANE_STAGE(1)
+    FX_LANE_STAGE(2)
+    FX_LANE_STAGE(4)
+    FX_LANE_STAGE(8)
+    FX_LANE_STAGE(16)
+    FX_LANE_STAGE(32)
+#undef FX_LANE_STAGE
+
+    // transpose A -> B through LDS
+#pragma unroll
+    for (int j = 0; j < NJ; j++) reinterpret_cast<float4*>(lds)[j * 256 + t] = a[j];
+    __syncthreads();
+    float b[NR];
+#pragma unroll
+    for (int r = 0; r < NR; r++) b[r] = lds[r * 256 + t];
+
+    // stages: bits 8..LOG2N-1 = register index bits 0..
+#pragma unroll
+    for (int bit = 1; bit < NR; bit <<= 1) {
+#pragma unroll
+        for (int r = 0; r < NR; r++) {
+            if ((r & bit) == 0) {
+                const float u = b[r], v = b[r | bit];
+                b[r] = u + v;
+                b[r | bit] = u - v;
+            }
+        }
+    }
+    // last stage: bit 0 = lane bit 0
+    {
+        const bool hi = (lane & 1) != 0;
+#pragma unroll
+        for (int r = 0; r < NR; r++) b[r] = lane_butterfly<1>(b[r], hi);
+    }
+
+    float amax = 0.0f;
+#pragma unroll
+    for (int r = 0; r < NR; r++) {
+        b[r] = b[r] / scale;
+        if constexpr (QUANT) amax = fmaxf(amax, fabsf(b[r]));
+    }
+    if constexpr (!QUANT) {
+        float* yr = y + row * N;
+#pragma unroll
+        for (int r = 0; r < NR; r++) yr[r * 256 + t] = b[r];
+    } else {
+        amax = block_max<kFhtBlock / kWave>(amax, red);   // its leading barrier also retires the lds reads above
+        const float sc = sym_scale(amax, 127.0f);
+        if (t == 0) s[row] = sc;
+        int8_t* lds_q = reinterpret_cast<int8_t*>(lds);
+#pragma unroll
+        for (int r = 0; r < NR; r++) lds_q[r * 256 + t] = (int8_t)quant_round(b[r], sc);
+        __syncthreads();
+        i32x4* qr = reinterpret_cast<i32x4*>(q + row * N);
+        for (int c = t; c < N / 16; c += kFhtBlock) qr[c] = reinterpret_cast<const i32x4*>(lds_q)[c];
+    }
+}
+
+template <bool QUANT>
+static int launch_fht(const float* x, float* y, int8_t* q, float* s, int rows, int n, float scale, hipStream_t st) {
+    switch (n) {
+        case 1024: fht_kernel<10, QUANT><<<rows, kFhtBlock, 0, st>>>(x, y, q, s, scale); break;
+        case 2048: fht_kernel<11, QUANT><<<rows, kFhtBlock, 0, st>>>(x, y, q, s, scale); break;
+        case 4096: fht_kernel<12, QUANT><<<rows, kFhtBlock, 0, st>>>(x, y, q, s, scale); break;
+        case 8192: fht_kernel<13, QUANT><<<rows, kFhtBlock, 0, st>>>(x, y, q, s, scale); break;
+        default:
+            set_error("fht: n=%d must be a power of two in [1024, 8192]", n);
+            return FLEXLLM_EINVAL;
+    }
+    FX_LAUNCH_CHECK();
+    return FLEXLLM_OK;
+}
+
+}  // namespace fx

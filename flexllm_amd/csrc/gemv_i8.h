@@ -67,4 +67,81 @@ __device__ __forceinline__ void wave_gemv_rows(const int8_t* __restrict__ w, con
     }
 }
 
+constexpr int kGemvBlock = 256;
+constexpr int kGemvWaves = kGemvBlock / kWave;
+
+enum GemvEpi { kEpiRaw = 0, kEpiDequant = 1, kEpiSwiglu = 2 };
+
+__device__ __forceinline__ float silu_f(float v) { return v / (1.0f + expf(-v)); }
+
+// rows_per_wave consecutive rows per wave; grid covers ceil(n / (4*rows_per_wave)) blocks.
+//   kEpiRaw:     acc_out[row] = sum
+//   kEpiDequant: y[row] = (float(sum)*s_x)*w_s[row] (+ residual[row])
+//   kEpiSwiglu:  rows are interleaved (2i = gate_i, 2i+1 = up_i); y[i] = up_i * silu(gate_i), both dequantised
+//                as above.  rows_per_wave is even, so a pair never straddles two waves.
+template <int NCH, int U, int EPI>
+__global__ __launch_bounds__(kGemvBlock) void gemv_i8_kernel(const int8_t* __restrict__ x, const int8_t* __restrict__ w,
+                                                             int32_t* __restrict__ acc_out, const float* __restrict__ s_x,
+                                                             const float* __restrict__ w_s,
+                                                             const float* __restrict__ residual, float* __restrict__ y,
+                                                             int k, int n, int rows_per_wave) {
+    const int lane = threadIdx.x & 63;
+    const int gw = blockIdx.x * kGemvWaves + (threadIdx.x >> 6);
+    const int row0 = gw * rows_per_wave;
+    if (row0 >= n) return;
+    const int nrows = min(rows_per_wave, n - row0);
+    const int nchunks = k >> 4;
+    i32x4 xr[NCH];
+    load_x_chunks<NCH>(x, nchunks, lane, xr);
+    if constexpr (EPI == kEpiDequant) {
+        const float sx = s_x[0];
+        wave_gemv_rows<NCH, U>(w, xr, k, nchunks, row0, nrows, lane, [&](int row, int sum) {
+            if (lane == 0) {
+                float v = (float)sum * sx * w_s[row];
+                if (residual) v = v + residual[row];
+                y[row] = v;
+            }
+        });
+    } else if constexpr (EPI == kEpiSwiglu) {
+        const float sx = s_x[0];
+        float gate = 0.0f;
+        wave_gemv_rows<NCH, U>(w, xr, k, nchunks, row0, nrows, lane, [&](int row, int sum) {
+            const float v = (float)sum * sx * w_s[row];
+            if ((row & 1) == 0) gate = v;
+            else if (lane == 0) y[row >> 1] = v * silu_f(gate);
+        });
+    } else {
+        wave_gemv_rows<NCH, U>(w, xr, k, nchunks, row0, nrows, lane, [&](int row, int sum) {
+            if (lane == 0) acc_out[row] = sum;
+        });
+    }
+}
+
+// Picks rows per wave so that the chip holds ~8 waves per CU while each wave still streams several KiB.
+static inline int pick_rows_per_wave(int k, int n) {
+    const int target_waves = 256 * 8;  // 256 CUs x 8 waves
+    int rpw = (n + target_waves - 1) / target_waves;
+    if (rpw < 2) rpw = 2;
+    return (rpw + 1) & ~1;
+}
+
+template <int EPI>
+inline int launch_gemv(const int8_t* x, const int8_t* w, int32_t* acc, const float* s_x, const float* w_s,
+                       const float* residual, float* y, int k, int n, hipStream_t st) {
+    const int nch = (k / 16 + 63) / 64;
+    const int rpw = pick_rows_per_wave(k, n);
+    const int waves = (n + rpw - 1) / rpw;
+    const int grid = (waves + kGemvWaves - 1) / kGemvWaves;
+#define FX_GEMV_CASE(NCH, U)                                                                                     \
+    gemv_i8_kernel<NCH, U, EPI><<<grid, kGemvBlock, 0, st>>>(x, w, acc, s_x, w_s, residual, y, k, n, rpw)
+    if (nch <= 1) FX_GEMV_CASE(1, 4);
+    else if (nch <= 2) FX_GEMV_CASE(2, 4);
+    else if (nch <= 4) FX_GEMV_CASE(4, 2);
+    else if (nch <= 8) FX_GEMV_CASE(8, 2);
+    else FX_GEMV_CASE(16, 2);
+#undef FX_GEMV_CASE
+    FX_LAUNCH_CHECK();
+    return FLEXLLM_OK;
+}
+
 }  // namespace fx

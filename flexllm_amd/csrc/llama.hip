@@ -1,0 +1,395 @@
+// Llama-3.2-1B W8A8 SpinQuant graph on one GPU: owns the repacked weights, the int8 KV cache and the
+// activation workspace, and strings the kernels together in the reference's layer order
+// (RMSNorm -> quant -> q/k/v -> RoPE -> static int8 quant -> KV append -> int8 attention -> o_proj -> residual
+//  -> RMSNorm -> quant -> gate/up -> SiLU*up -> Hadamard R4 -> quant -> down -> residual).
+//
+// Decode keeps every per-step quantity that changes between steps (position, current token) in device
+// memory so that one captured HIP graph can be replayed for every generated token.
+#include "attn_decode_kernels.h"
+#include "elementwise_kernels.h"
+#include "fht_kernels.h"
+#include "gemv_i8.h"
+#include "logits_kernels.h"
+#include "prefill.h"
+#include <vector>
+
+struct flexllm_llama {
+    flexllm_llama_config cfg;
+    std::vector<fx::LayerW> layers;
+    float* gamma = nullptr;
+    float *q_s = nullptr, *k_s = nullptr, *v_s = nullptr, *a_s = nullptr;
+    float *rope_sin = nullptr, *rope_cos = nullptr;
+    uint16_t* embed = nullptr;
+    int8_t *k_cache = nullptr, *v_cache = nullptr;   // [layers] x per-layer cache
+    size_t cache_layer_bytes = 0;
+    // decode workspace
+    float *x = nullptr, *x2 = nullptr, *qkv = nullptr, *h = nullptr, *nrm = nullptr, *logits = nullptr;
+    int8_t *xq = nullptr, *q8 = nullptr;
+    float* xs = nullptr;
+    float* scores = nullptr;
+    float2* stats = nullptr;
+    int32_t* o_acc = nullptr;
+    int* state = nullptr;           // [0] position of the token being processed, [1] step index
+    float* am_v = nullptr;
+    int* am_i = nullptr;
+    hipGraphExec_t graph_exec = nullptr;
+    int* graph_token_io = nullptr;
+    int* graph_tokens_out = nullptr;
+    hipStream_t graph_stream = nullptr;
+    std::vector<void*> owned;
+    fx::PrefillWorkspace pws;
+};
+
+namespace fx {
+
+// ---- small fused decode kernels ------------------------------------------------------------------
+// RoPE on q and k, static int8 quantisation of q/k/v, append of k/v at the current position.
+// qkv is fp32 [H + 2*KV] = [q | k | v]; one block.
+static __global__ __launch_bounds__(256) void dec_qkv_post_kernel(const float* __restrict__ qkv, const float* __restrict__ sin_t,
+                                                                  const float* __restrict__ cos_t, const float* __restrict__ q_s,
+                                                                  const float* __restrict__ k_s, const float* __restrict__ v_s,
+                                                                  int8_t* __restrict__ q8, int8_t* __restrict__ kc,
+                                                                  int8_t* __restrict__ vc, const int* __restrict__ state,
+                                                                  int q_heads, int kv_heads, int max_pos) {
+    const int pos = state[0];
+    const int half = kHd / 2;
+    const float* sn = sin_t + (size_t)pos * half;
+    const float* cs = cos_t + (size_t)pos * half;
+    const int H = q_heads * kHd, KV = kv_heads * kHd;
+    const int q_pairs = q_heads * half, k_pairs = kv_heads * half;
+    for (int i = threadIdx.x; i < q_pairs + k_pairs + KV; i += 256) {
+        if (i < q_pairs) {
+            const int hd = i / half, k = i % half;
+            const float t0 = qkv[hd * kHd + k], t1 = qkv[hd * kHd + k + half];
+            const float o0 = t0 * cs[k] - t1 * sn[k];
+            const float o1 = t0 * sn[k] + t1 * cs[k];
+            const float div = 8.0f * q_s[hd];      // sqrt(head_dim) folded into the Q scale
+            q8[hd * kHd + k] = (int8_t)static_q8(o0, div);
+            q8[hd * kHd + k + half] = (int8_t)static_q8(o1, div);
+        } else if (i < q_pairs + k_pairs) {
+            const int j = i - q_pairs;
+            const int hd = j / half, k = j % half;
+            const float t0 = qkv[H + hd * kHd + k], t1 = qkv[H + hd * kHd + k + half];
+            const float o0 = t0 * cs[k] - t1 * sn[k];
+            const float o1 = t0 * sn[k] + t1 * cs[k];
+            const float div = 1.0f * k_s[hd];
+            int8_t* dst = kc + k_index(hd, pos, max_pos);
+            dst[k] = (int8_t)static_q8(o0, div);
+            dst[k + half] = (int8_t)static_q8(o1, div);
+        } else {
+            const int j = i - q_pairs - k_pairs;
+            const int hd = j / kHd, d = j % kHd;
+            vc[v_index(hd, pos, d, max_pos)] = (int8_t)static_q8(qkv[H + KV + j], 1.0f * v_s[hd]);
+        }
+    }
+}
+
+// Dequantise the attention accumulators and quantise the 2048-vector per token for o_proj; one block.
+template <int VPT>
+static __global__ __launch_bounds__(256) void dec_out_quant_kernel(const int32_t* __restrict__ o_acc, const float* __restrict__ a_s,
+                                                                   const float* __restrict__ v_s, int8_t* __restrict__ q,
+                                                                   float* __restrict__ s, int n, int group) {
+    __shared__ float red[4];
+    float v[VPT];
+    float amax = 0.0f;
+#pragma unroll
+    for (int i = 0; i < VPT; i++) {
+        const int idx = threadIdx.x + i * 256;
+        v[i] = 0.0f;
+        if (idx < n) {
+            const int qh = idx / kHd;
+            v[i] = (float)o_acc[idx] * a_s[qh] * v_s[qh / group];
+            amax = fmaxf(amax, fabsf(v[i]));
+        }
+    }
+    amax = block_max<4>(amax, red);
+    const float sc = sym_scale(amax, 127.0f);
+    if (threadIdx.x == 0) s[0] = sc;
+#pragma unroll
+    for (int i = 0; i < VPT; i++) {
+        const int idx = threadIdx.x + i * 256;
+        if (idx < n) q[idx] = (int8_t)quant_round(v[i], sc);
+    }
+}
+
+static __global__ void set_state_kernel(int* state, int pos, int step) { state[0] = pos; state[1] = step; }
+
+static __global__ __launch_bounds__(64) void argmax_final_advance_kernel(const float* __restrict__ pv, const int* __restrict__ pi,
+                                                                         int nparts, int* __restrict__ token_io,
+                                                                         int* __restrict__ tokens_out, int* __restrict__ state) {
+    float best = -INFINITY;
+    int bi = 0x7fffffff;
+    for (int i = threadIdx.x; i < nparts; i += 64) {
+        const float v = pv[i];
+        const int idx = pi[i];
+        if (v > best || (v == best && idx < bi)) { best = v; bi = idx; }
+    }
+#pragma unroll
+    for (int m = 1; m < 64; m <<= 1) {
+        const float ov = __shfl_xor(best, m);
+        const int oi = __shfl_xor(bi, m);
+        if (ov > best || (ov == best && oi < bi)) { best = ov; bi = oi; }
+    }
+    if (threadIdx.x == 0) {
+        const int tok = bi == 0x7fffffff ? 0 : bi;
+        token_io[0] = tok;
+        tokens_out[state[1]] = tok;
+        state[0] += 1;
+        state[1] += 1;
+    }
+}
+
+static int dev_alloc(flexllm_llama* m, void** p, size_t bytes) {
+    hipError_t e = hipMalloc(p, bytes ? bytes : 1);
+    if (e != hipSuccess) {
+        set_error("hipMalloc(%zu) failed: %s", bytes, hipGetErrorString(e));
+        return e == hipErrorOutOfMemory ? FLEXLLM_ENOMEM : FLEXLLM_EHIP;
+    }
+    m->owned.push_back(*p);
+    return FLEXLLM_OK;
+}
+#define FX_ALLOC(m, ptr, bytes)                                    \
+    do {                                                           \
+        int rc_ = dev_alloc(m, (void**)&(ptr), (bytes));           \
+        if (rc_) return rc_;                                       \
+    } while (0)
+
+// All decode kernels of one layer, enqueued on `st`.
+static int decode_layer(flexllm_llama* m, int l, hipStream_t st) {
+    const flexllm_llama_config& c = m->cfg;
+    const LayerW& w = m->layers[l];
+    const int H = c.hidden, KV = c.kv_hidden, I = c.inter;
+    const int group = c.q_heads / c.kv_heads;
+    const float* g0 = m->gamma + (size_t)(2 * l) * H;
+    const float* g1 = m->gamma + (size_t)(2 * l + 1) * H;
+    const float* q_s = m->q_s + (size_t)l * c.q_heads;
+    const float* k_s = m->k_s + (size_t)l * c.kv_heads;
+    const float* v_s = m->v_s + (size_t)l * c.kv_heads;
+    const float* a_s = m->a_s + (size_t)l * c.q_heads;
+    int8_t* kc = m->k_cache + (size_t)l * m->cache_layer_bytes;
+    int8_t* vc = m->v_cache + (size_t)l * m->cache_layer_bytes;
+    int rc;
+    // attention block
+    rmsnorm_kernel<2, true><<<1, kBlock, 0, st>>>(m->x, g0, nullptr, m->xq, m->xs, H, c.eps);
+    if ((rc = launch_gemv<kEpiDequant>(m->xq, w.wqkv, nullptr, m->xs, w.sqkv, nullptr, m->qkv, H, H + 2 * KV, st))) return rc;
+    dec_qkv_post_kernel<<<1, 256, 0, st>>>(m->qkv, m->rope_sin, m->rope_cos, q_s, k_s, v_s, m->q8, kc, vc, m->state,
+                                           c.q_heads, c.kv_heads, c.max_pos);
+    dim3 grid(c.max_pos / kChunk, c.kv_heads);
+    dec_scores_kernel<<<grid, 64 * group, 0, st>>>(m->q8, kc, q_s, k_s, m->scores, m->stats, m->o_acc, m->state, 0,
+                                                   c.max_pos, group, c.max_pos);
+    dec_pv_kernel<<<grid, 64 * group, 0, st>>>(m->scores, m->stats, vc, a_s, m->o_acc, nullptr, m->state, 0, c.max_pos,
+                                               group, c.max_pos);
+    dec_out_quant_kernel<8><<<1, 256, 0, st>>>(m->o_acc, a_s, v_s, m->xq, m->xs, H, group);
+    if ((rc = launch_gemv<kEpiDequant>(m->xq, w.wo, nullptr, m->xs, w.so, m->x, m->x2, H, H, st))) return rc;
+    // feed-forward block
+    rmsnorm_kernel<2, true><<<1, kBlock, 0, st>>>(m->x2, g1, nullptr, m->xq, m->xs, H, c.eps);
+    if ((rc = launch_gemv<kEpiSwiglu>(m->xq, w.wgu, nullptr, m->xs, w.sgu, nullptr, m->h, H, 2 * I, st))) return rc;
+    fht_kernel<13, true><<<1, kFhtBlock, 0, st>>>(m->h, nullptr, m->xq, m->xs, c.fht_scale);
+    if ((rc = launch_gemv<kEpiDequant>(m->xq, w.wd, nullptr, m->xs, w.sd, m->x2, m->x, I, H, st))) return rc;
+    FX_LAUNCH_CHECK();
+    return FLEXLLM_OK;
+}
+
+static int decode_head(flexllm_llama* m, float* logits, hipStream_t st) {
+    const flexllm_llama_config& c = m->cfg;
+    rmsnorm_kernel<2, false><<<1, kBlock, 0, st>>>(m->x, m->gamma + (size_t)(2 * c.layers) * c.hidden, m->nrm, nullptr,
+                                                   nullptr, c.hidden, c.eps);
+    return lm_head_launch(m->embed, m->nrm, logits, c.vocab, c.hidden, st);
+}
+
+// One greedy step: embedding of *token_io -> layers -> head -> argmax -> *token_io, tokens_out[step], pos++.
+static int greedy_step(flexllm_llama* m, int* token_io, int* tokens_out, hipStream_t st) {
+    const flexllm_llama_config& c = m->cfg;
+    embed_kernel<<<(c.hidden + 255) / 256, 256, 0, st>>>(reinterpret_cast<const __half*>(m->embed), token_io, m->x, c.hidden);
+    int rc;
+    for (int l = 0; l < c.layers; l++)
+        if ((rc = decode_layer(m, l, st))) return rc;
+    if ((rc = decode_head(m, m->logits, st))) return rc;
+    argmax_partial_kernel<<<kArgmaxParts, 256, 0, st>>>(m->logits, c.vocab, m->am_v, m->am_i);
+    argmax_final_advance_kernel<<<1, 64, 0, st>>>(m->am_v, m->am_i, kArgmaxParts, token_io, tokens_out, m->state);
+    FX_LAUNCH_CHECK();
+    return FLEXLLM_OK;
+}
+
+}  // namespace fx
+
+using namespace fx;
+
+extern "C" {
+
+int flexllm_llama_create(flexllm_llama** out, const flexllm_llama_config* cfg, const flexllm_llama_weights* w) {
+    FX_REQUIRE(out && cfg && w, "llama_create: null pointer");
+    const flexllm_llama_config& c = *cfg;
+    FX_REQUIRE(c.head_dim == kHd, "llama_create: head_dim=%d (only 64)", c.head_dim);
+    FX_REQUIRE(c.layers > 0 && c.hidden == c.q_heads * c.head_dim && c.kv_hidden == c.kv_heads * c.head_dim,
+               "llama_create: hidden=%d q_heads=%d kv_hidden=%d kv_heads=%d inconsistent", c.hidden, c.q_heads, c.kv_hidden, c.kv_heads);
+    FX_REQUIRE(c.hidden == 2048 && c.inter == 8192, "llama_create: hidden=%d inter=%d (kernels are instantiated for 2048/8192)", c.hidden, c.inter);
+    FX_REQUIRE(c.q_heads % c.kv_heads == 0 && c.q_heads / c.kv_heads <= 4, "llama_create: GQA group %d > 4", c.q_heads / c.kv_heads);
+    FX_REQUIRE(c.max_pos > 0 && c.max_pos % kChunk == 0 && c.max_pos <= kChunk * kMaxChunks,
+               "llama_create: max_pos=%d must be a multiple of 128, <= 8192", c.max_pos);
+    FX_REQUIRE(c.vocab > 0, "llama_create: vocab=%d", c.vocab);
+    flexllm_llama* m = new flexllm_llama();
+    m->cfg = c;
+    const int H = c.hidden, KV = c.kv_hidden, I = c.inter, L = c.layers;
+    auto fail = [&](int rc) { flexllm_llama_destroy(m); return rc; };
+#define FX_TRY(expr)                          \
+    do {                                      \
+        int rc__ = (expr);                    \
+        if (rc__) return fail(rc__);          \
+    } while (0)
+#define FX_TRY_HIP(call)                                                               \
+    do {                                                                               \
+        hipError_t e_ = (call);                                                        \
+        if (e_ != hipSuccess) {                                                        \
+            set_error("%s failed: %s", #call, hipGetErrorString(e_));                  \
+            return fail(FLEXLLM_EHIP);                                                 \
+        }                                                                              \
+    } while (0)
+    m->layers.resize(L);
+    for (int l = 0; l < L; l++) {
+        LayerW& lw = m->layers[l];
+        FX_TRY(dev_alloc(m, (void**)&lw.wqkv, (size_t)(H + 2 * KV) * H));
+        FX_TRY(dev_alloc(m, (void**)&lw.wo, (size_t)H * H));
+        FX_TRY(dev_alloc(m, (void**)&lw.wgu, (size_t)2 * I * H));
+        FX_TRY(dev_alloc(m, (void**)&lw.wd, (size_t)H * I));
+        FX_TRY(dev_alloc(m, (void**)&lw.sqkv, sizeof(float) * (H + 2 * KV)));
+        FX_TRY(dev_alloc(m, (void**)&lw.so, sizeof(float) * H));
+        FX_TRY(dev_alloc(m, (void**)&lw.sgu, sizeof(float) * 2 * I));
+        FX_TRY(dev_alloc(m, (void**)&lw.sd, sizeof(float) * H));
+        FX_TRY_HIP(hipMemcpy(lw.wqkv, w->wq[l], (size_t)H * H, hipMemcpyDeviceToDevice));
+        FX_TRY_HIP(hipMemcpy(lw.wqkv + (size_t)H * H, w->wk[l], (size_t)KV * H, hipMemcpyDeviceToDevice));
+        FX_TRY_HIP(hipMemcpy(lw.wqkv + (size_t)(H + KV) * H, w->wv[l], (size_t)KV * H, hipMemcpyDeviceToDevice));
+        FX_TRY_HIP(hipMemcpy(lw.wo, w->wo[l], (size_t)H * H, hipMemcpyDeviceToDevice));
+        FX_TRY_HIP(hipMemcpy2D(lw.wgu, (size_t)2 * H, w->wg[l], H, H, I, hipMemcpyDeviceToDevice));
+        FX_TRY_HIP(hipMemcpy2D(lw.wgu + H, (size_t)2 * H, w->wu[l], H, H, I, hipMemcpyDeviceToDevice));
+        FX_TRY_HIP(hipMemcpy(lw.wd, w->wd[l], (size_t)H * I, hipMemcpyDeviceToDevice));
+        FX_TRY_HIP(hipMemcpy(lw.sqkv, w->sq[l], sizeof(float) * H, hipMemcpyDeviceToDevice));
+        FX_TRY_HIP(hipMemcpy(lw.sqkv + H, w->sk[l], sizeof(float) * KV, hipMemcpyDeviceToDevice));
+        FX_TRY_HIP(hipMemcpy(lw.sqkv + H + KV, w->sv[l], sizeof(float) * KV, hipMemcpyDeviceToDevice));
+        FX_TRY_HIP(hipMemcpy(lw.so, w->so[l], sizeof(float) * H, hipMemcpyDeviceToDevice));
+        FX_TRY_HIP(hipMemcpy2D(lw.sgu, 2 * sizeof(float), w->sg[l], sizeof(float), sizeof(float), I, hipMemcpyDeviceToDevice));
+        FX_TRY_HIP(hipMemcpy2D(lw.sgu + 1, 2 * sizeof(float), w->su[l], sizeof(float), sizeof(float), I, hipMemcpyDeviceToDevice));
+        FX_TRY_HIP(hipMemcpy(lw.sd, w->sd[l], sizeof(float) * H, hipMemcpyDeviceToDevice));
+    }
+    auto dup = [&](void** dst, const void* src, size_t bytes) -> int {
+        int rc = dev_alloc(m, dst, bytes);
+        if (rc) return rc;
+        hipError_t e = hipMemcpy(*dst, src, bytes, hipMemcpyDeviceToDevice);
+        if (e != hipSuccess) { set_error("hipMemcpy failed: %s", hipGetErrorString(e)); return FLEXLLM_EHIP; }
+        return FLEXLLM_OK;
+    };
+    FX_TRY(dup((void**)&m->gamma, w->gamma, sizeof(float) * (size_t)(2 * L + 1) * H));
+    FX_TRY(dup((void**)&m->q_s, w->q_s, sizeof(float) * (size_t)L * c.q_heads));
+    FX_TRY(dup((void**)&m->k_s, w->k_s, sizeof(float) * (size_t)L * c.kv_heads));
+    FX_TRY(dup((void**)&m->v_s, w->v_s, sizeof(float) * (size_t)L * c.kv_heads));
+    FX_TRY(dup((void**)&m->a_s, w->a_s, sizeof(float) * (size_t)L * c.q_heads));
+    FX_TRY(dup((void**)&m->rope_sin, w->rope_sin, sizeof(float) * (size_t)c.max_pos * (kHd / 2)));
+    FX_TRY(dup((void**)&m->rope_cos, w->rope_cos, sizeof(float) * (size_t)c.max_pos * (kHd / 2)));
+    FX_TRY(dup((void**)&m->embed, w->embed, sizeof(uint16_t) * (size_t)c.vocab * H));
+    m->cache_layer_bytes = (size_t)c.kv_heads * c.max_pos * kHd;
+    FX_TRY(dev_alloc(m, (void**)&m->k_cache, m->cache_layer_bytes * L));
+    FX_TRY(dev_alloc(m, (void**)&m->v_cache, m->cache_layer_bytes * L));
+    FX_TRY_HIP(hipMemset(m->k_cache, 0, m->cache_layer_bytes * L));
+    FX_TRY_HIP(hipMemset(m->v_cache, 0, m->cache_layer_bytes * L));
+    FX_TRY(dev_alloc(m, (void**)&m->x, sizeof(float) * H));
+    FX_TRY(dev_alloc(m, (void**)&m->x2, sizeof(float) * H));
+    FX_TRY(dev_alloc(m, (void**)&m->nrm, sizeof(float) * H));
+    FX_TRY(dev_alloc(m, (void**)&m->qkv, sizeof(float) * (H + 2 * KV)));
+    FX_TRY(dev_alloc(m, (void**)&m->h, sizeof(float) * I));
+    FX_TRY(dev_alloc(m, (void**)&m->logits, sizeof(float) * c.vocab));
+    FX_TRY(dev_alloc(m, (void**)&m->xq, (size_t)I));
+    FX_TRY(dev_alloc(m, (void**)&m->q8, (size_t)H));
+    FX_TRY(dev_alloc(m, (void**)&m->xs, sizeof(float) * 4));
+    FX_TRY(dev_alloc(m, (void**)&m->scores, sizeof(float) * (size_t)c.q_heads * c.max_pos));
+    FX_TRY(dev_alloc(m, (void**)&m->stats, sizeof(float2) * (size_t)c.q_heads * kMaxChunks));
+    FX_TRY(dev_alloc(m, (void**)&m->o_acc, sizeof(int32_t) * H));
+    FX_TRY(dev_alloc(m, (void**)&m->state, sizeof(int) * 4));
+    FX_TRY(dev_alloc(m, (void**)&m->am_v, sizeof(float) * kArgmaxParts));
+    FX_TRY(dev_alloc(m, (void**)&m->am_i, sizeof(int) * kArgmaxParts));
+    FX_TRY_HIP(hipDeviceSynchronize());
+#undef FX_TRY
+#undef FX_TRY_HIP
+    *out = m;
+    return FLEXLLM_OK;
+}
+
+int flexllm_llama_destroy(flexllm_llama* m) {
+    if (!m) return FLEXLLM_OK;
+    (void)hipDeviceSynchronize();
+    if (m->graph_exec) (void)hipGraphExecDestroy(m->graph_exec);
+    prefill_workspace_free(&m->pws);
+    for (void* p : m->owned) (void)hipFree(p);
+    delete m;
+    return FLEXLLM_OK;
+}
+
+int flexllm_llama_kv_cache(flexllm_llama* m, int8_t** k_cache, int8_t** v_cache) {
+    FX_REQUIRE(m && k_cache && v_cache, "llama_kv_cache: null pointer");
+    *k_cache = m->k_cache;
+    *v_cache = m->v_cache;
+    return FLEXLLM_OK;
+}
+
+int flexllm_llama_decode_hidden(flexllm_llama* m, const float* x_in, int pos, float* hidden_out, float* logits,
+                                void* stream) {
+    FX_REQUIRE(m && x_in, "llama_decode_hidden: null pointer");
+    FX_REQUIRE(pos >= 0 && pos < m->cfg.max_pos, "llama_decode_hidden: pos=%d outside [0,%d)", pos, m->cfg.max_pos);
+    hipStream_t st = as_stream(stream);
+    const int H = m->cfg.hidden;
+    set_state_kernel<<<1, 1, 0, st>>>(m->state, pos, 0);
+    FX_HIP(hipMemcpyAsync(m->x, x_in, sizeof(float) * H, hipMemcpyDeviceToDevice, st));
+    for (int l = 0; l < m->cfg.layers; l++) {
+        int rc = decode_layer(m, l, st);
+        if (rc) return rc;
+    }
+    if (hidden_out) FX_HIP(hipMemcpyAsync(hidden_out, m->x, sizeof(float) * H, hipMemcpyDeviceToDevice, st));
+    if (logits) {
+        int rc = decode_head(m, logits, st);
+        if (rc) return rc;
+    }
+    return FLEXLLM_OK;
+}
+
+int flexllm_llama_decode_greedy(flexllm_llama* m, int* token_io, int pos0, int steps, int* tokens_out, int use_graph,
+                                void* stream) {
+    FX_REQUIRE(m && token_io && tokens_out, "llama_decode_greedy: null pointer");
+    FX_REQUIRE(steps >= 0 && pos0 >= 0 && pos0 + steps <= m->cfg.max_pos,
+               "llama_decode_greedy: pos0=%d steps=%d exceed max_pos=%d", pos0, steps, m->cfg.max_pos);
+    hipStream_t st = as_stream(stream);
+    set_state_kernel<<<1, 1, 0, st>>>(m->state, pos0, 0);
+    FX_LAUNCH_CHECK();
+    if (!use_graph) {
+        for (int s = 0; s < steps; s++) {
+            int rc = greedy_step(m, token_io, tokens_out, st);
+            if (rc) return rc;
+        }
+        return FLEXLLM_OK;
+    }
+    FX_REQUIRE(st != nullptr, "llama_decode_greedy: graph replay needs a non-default stream");
+    if (!m->graph_exec || m->graph_token_io != token_io || m->graph_tokens_out != tokens_out || m->graph_stream != st) {
+        if (m->graph_exec) { (void)hipGraphExecDestroy(m->graph_exec); m->graph_exec = nullptr; }
+        FX_HIP(hipStreamSynchronize(st));
+        hipGraph_t graph;
+        FX_HIP(hipStreamBeginCapture(st, hipStreamCaptureModeThreadLocal));
+        int rc = greedy_step(m, token_io, tokens_out, st);
+        hipError_t e = hipStreamEndCapture(st, &graph);
+        if (rc) { if (e == hipSuccess) (void)hipGraphDestroy(graph); return rc; }
+        FX_HIP(e);
+        e = hipGraphInstantiate(&m->graph_exec, graph, nullptr, nullptr, 0);
+        (void)hipGraphDestroy(graph);
+        FX_HIP(e);
+        m->graph_token_io = token_io;
+        m->graph_tokens_out = tokens_out;
+        m->graph_stream = st;
+    }
+    for (int s = 0; s < steps; s++) FX_HIP(hipGraphLaunch(m->graph_exec, st));
+    return FLEXLLM_OK;
+}
+
+int flexllm_llama_prefill_hidden(flexllm_llama* m, const float* x_in, int s, float* hidden_out, void* stream) {
+    FX_REQUIRE(m && x_in, "llama_prefill_hidden: null pointer");
+    return llama_prefill_run(m->cfg, m->layers.data(), m->gamma, m->q_s, m->k_s, m->v_s, m->a_s, m->rope_sin, m->rope_cos,
+                             m->k_cache, m->v_cache, m->cache_layer_bytes, &m->pws, x_in, s, hidden_out, as_stream(stream));
+}
+
+}  // extern "C"

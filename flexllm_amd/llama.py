@@ -1,0 +1,136 @@
+"""Llama-3.2-1B W8A8 SpinQuant graph: configuration, seeded synthetic weights (host and device, bit-identical)
+and the wrapper over the C ABI model object (flexllm_llama_*)."""
+import ctypes as C
+import math
+
+import numpy as np
+
+from . import synth
+from ._lib import lib, check, LlamaConfig, LlamaWeights
+from .device import DeviceArray, to_device, _s
+from .ops import rope_table
+
+# Model constants of the reference (Modules/config.h:19-44 of the reference tree).
+LLAMA32_1B = dict(layers=16, hidden=2048, kv_hidden=512, inter=8192, q_heads=32, kv_heads=8, head_dim=64,
+                  vocab=128256, max_pos=4096, eps=1e-5, fht_scale=90.50966799)
+
+_PROJ = dict(q=("hidden", "hidden"), k=("kv_hidden", "hidden"), v=("kv_hidden", "hidden"), o=("hidden", "hidden"),
+             g=("inter", "hidden"), u=("inter", "hidden"), d=("hidden", "inter"))
+
+
+def make_config(**over):
+    cfg = dict(LLAMA32_1B)
+    cfg.update(over)
+    return cfg
+
+
+def _seed(base, layer, tensor):
+    return (base * 1000003 + layer * 101 + tensor) & 0xFFFFFFFFFFFF
+
+
+def synth_weights(cfg, seed=1, device=False):
+    """Random-init int8 weights U[-127,127] with per-channel scales sized so that activations stay O(1),
+    RMSNorm gains U[0.5,1.5], static attention scales with a seeded +-20% jitter per head, fp16 embedding.
+    device=False -> numpy arrays (for the oracle); device=True -> DeviceArrays filled on the GPU by the
+    same counter-based generator."""
+    i8 = synth.device_i8 if device else synth.host_i8
+    f32 = synth.device_uniform_f32 if device else synth.host_uniform_f32
+    f16 = synth.device_uniform_f16 if device else synth.host_uniform_f16
+    w = {}
+    for t, (name, (n_key, k_key)) in enumerate(_PROJ.items()):
+        n, k = cfg[n_key], cfg[k_key]
+        base = 1.0 / (73.0 * math.sqrt(k))
+        w["w" + name] = [i8((n, k), _seed(seed, l, t)) for l in range(cfg["layers"])]
+        w["s" + name] = [f32((n,), _seed(seed, l, 20 + t), 0.5 * base, 1.5 * base) for l in range(cfg["layers"])]
+    L = cfg["layers"]
+    w["gamma"] = f32((2 * L + 1, cfg["hidden"]), _seed(seed, 99, 1), 0.5, 1.5)
+    w["q_s"] = f32((L, cfg["q_heads"]), _seed(seed, 99, 2), 0.8 * 0.004, 1.2 * 0.004)
+    w["k_s"] = f32((L, cfg["kv_heads"]), _seed(seed, 99, 3), 0.8 * 0.03, 1.2 * 0.03)
+    w["v_s"] = f32((L, cfg["kv_heads"]), _seed(seed, 99, 4), 0.8 * 0.03, 1.2 * 0.03)
+    w["a_s"] = f32((L, cfg["q_heads"]), _seed(seed, 99, 5), 1.0 / 255, 1.0 / 255)
+    w["embed"] = f16((cfg["vocab"], cfg["hidden"]), _seed(seed, 99, 6), -1.7, 1.7)
+    sin_t, cos_t = rope_table(cfg["max_pos"], cfg["head_dim"])
+    if device:
+        w["rope_sin"], w["rope_cos"] = to_device(sin_t), to_device(cos_t)
+    else:
+        w["rope_sin"], w["rope_cos"] = sin_t, cos_t
+        w["embed"] = w["embed"].view(np.uint16)
+    return w
+
+
+class Llama:
+    """Device model object.  `weights` holds DeviceArrays (see synth_weights(device=True))."""
+
+    def __init__(self, cfg, weights):
+        self.cfg = cfg
+        c = LlamaConfig()
+        for n in ("layers", "hidden", "kv_hidden", "inter", "q_heads", "kv_heads", "head_dim", "vocab", "max_pos"):
+            setattr(c, n, int(cfg[n]))
+        c.eps = float(cfg["eps"]); c.fht_scale = float(cfg["fht_scale"])
+        L = cfg["layers"]
+        keep = []
+        w = LlamaWeights()
+        for n in ("wq", "wk", "wv", "wo", "wg", "wu", "wd", "sq", "sk", "sv", "so", "sg", "su", "sd"):
+            arr = (C.c_void_p * L)(*[weights[n][l].ptr for l in range(L)])
+            keep.append(arr)
+            setattr(w, n, C.cast(arr, C.c_void_p))
+        for n in ("gamma", "q_s", "k_s", "v_s", "a_s", "rope_sin", "rope_cos", "embed"):
+            setattr(w, n, weights[n].ptr)
+        h = C.c_void_p()
+        check(lib().flexllm_llama_create(C.byref(h), C.byref(c), C.byref(w)))
+        self.handle = h
+        cache_shape_k = (L, cfg["kv_heads"], cfg["max_pos"], cfg["head_dim"])
+        cache_shape_v = (L, cfg["kv_heads"], cfg["max_pos"] // 64, cfg["head_dim"], 64)
+        kp, vp = C.c_void_p(), C.c_void_p()
+        check(lib().flexllm_llama_kv_cache(self.handle, C.byref(kp), C.byref(vp)))
+        self.k_cache = _borrow(kp.value, cache_shape_k, np.int8)
+        self.v_cache = _borrow(vp.value, cache_shape_v, np.int8)
+
+    def decode_hidden(self, x_in, pos, want_logits=False, stream=None):
+        hidden = DeviceArray((self.cfg["hidden"],), np.float32)
+        logits = DeviceArray((self.cfg["vocab"],), np.float32) if want_logits else None
+        check(lib().flexllm_llama_decode_hidden(self.handle, C.c_void_p(x_in.ptr), int(pos), C.c_void_p(hidden.ptr),
+                                                C.c_void_p(logits.ptr) if logits else None, _s(stream)))
+        return hidden, logits
+
+    def decode_greedy(self, token_io, pos0, steps, tokens_out, use_graph=True, stream=None):
+        check(lib().flexllm_llama_decode_greedy(self.handle, C.c_void_p(token_io.ptr), int(pos0), int(steps),
+                                                C.c_void_p(tokens_out.ptr), int(use_graph), _s(stream)))
+
+    def prefill_hidden(self, x_in, stream=None):
+        s = x_in.shape[0]
+        hidden = DeviceArray((s, self.cfg["hidden"]), np.float32)
+        check(lib().flexllm_llama_prefill_hidden(self.handle, C.c_void_p(x_in.ptr), s, C.c_void_p(hidden.ptr), _s(stream)))
+        return hidden
+
+    def caches_token_major(self):
+        """int8 caches as numpy [layer][pos][kv_hidden] (the oracle's layout)."""
+        c = self.cfg
+        k = self.k_cache.numpy().transpose(0, 2, 1, 3).reshape(c["layers"], c["max_pos"], c["kv_hidden"])
+        v = self.v_cache.numpy().transpose(0, 2, 4, 1, 3).reshape(c["layers"], c["max_pos"], c["kv_hidden"])
+        return k, v
+
+    def load_caches_token_major(self, k, v):
+        c = self.cfg
+        L, P, KH, HD = c["layers"], c["max_pos"], c["kv_heads"], c["head_dim"]
+        self.k_cache.copy_from(np.ascontiguousarray(k.reshape(L, P, KH, HD).transpose(0, 2, 1, 3)))
+        self.v_cache.copy_from(np.ascontiguousarray(v.reshape(L, P // 64, 64, KH, HD).transpose(0, 3, 1, 4, 2)))
+
+    def close(self):
+        if self.handle:
+            lib().flexllm_llama_destroy(self.handle)
+            self.handle = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+
+def _borrow(ptr, shape, dtype):
+    a = DeviceArray.__new__(DeviceArray)
+    a.shape = tuple(shape); a.dtype = np.dtype(dtype)
+    a.nbytes = int(np.prod(shape, dtype=np.int64)) * a.dtype.itemsize
+    a.ptr = ptr; a._owner = False
+    return a

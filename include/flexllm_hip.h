@@ -98,6 +98,11 @@ int flexllm_linear_i8_gemv(const int8_t* x, const int8_t* w, int32_t* acc, int k
  * (+ dec_Residual_Layer, Modules/Residual_Layer.h:69-87). */
 int flexllm_linear_i8_gemv_dequant(const int8_t* x, const float* s_x, const int8_t* w, const float* w_s,
                                    const float* residual, float* y, int k, int n, void* stream);
+/* Fused gate/up projection + SwiGLU: w_gu is int8 [2n][k] with rows interleaved (row 2i = gate_i, row 2i+1 = up_i),
+ * w_s_gu the matching 2n scales; y[i] = up_i * (gate_i/(1+exp(-gate_i))), gate_i/up_i dequantised as above.
+ * = two GEMVs + dec_Swish (Modules/Swish.h:26-41) + dec_Gate_Layer_fp32xfp32 (Modules/Linear_Layer.h:1103-1121). */
+int flexllm_linear_i8_gemv_swiglu(const int8_t* x, const float* s_x, const int8_t* w_gu, const float* w_s_gu, float* y,
+                                  int k, int n, void* stream);
 /* Prefill GEMM, exact: acc[m][n] = sum_k a[m][k]*W[n][k] on int8 MFMA tiles.  Replaces
  * pref_Linear_Layer_i4xi4 (Modules/Linear_Layer.h:293-341) with the int8 systolic array
  * (Modules/MHA.h:113-187, Modules/PE.h:526-583).  k % 64 == 0. */

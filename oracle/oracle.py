@@ -227,6 +227,13 @@ def half_to_float(h):
     return lib().fxo_half_to_float(int(h))
 
 
+def embed(table_u16, token):
+    table_u16 = np.ascontiguousarray(table_u16, np.uint16)
+    y = np.empty(table_u16.shape[1], np.float32)
+    lib().fxo_embed(_p(table_u16), table_u16.shape[1], int(token), _p(y))
+    return y
+
+
 def lm_head(table_u16, n):
     table_u16 = np.ascontiguousarray(table_u16, np.uint16)
     vocab, hidden = table_u16.shape
