@@ -1,0 +1,183 @@
+#!/usr/bin/env python3
+"""Headline benchmark: full 16-layer Llama-3.2-1B W8A8 SpinQuant greedy decode, batch 1, int8 KV cache
+pre-filled so that the context grows to 4096 positions; plus the 1024-token prefill time.
+
+A "step" is one generated token (embedding -> 16 layers -> final norm -> fp16 lm_head -> argmax), replayed
+as one HIP graph.  Inputs (weights, caches) are resident in HBM before the timed region.  Prints ONE JSON
+line.  One GPU only.
+"""
+import argparse
+import ctypes as C
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0          # MI355X published HBM3E bandwidth
+INT8_PEAK_TOPS = 5000.0        # MI355X published dense int8 MFMA rate
+
+
+def bytes_per_token(cfg, mean_len):
+    """Algorithmic HBM bytes of one decode step at context length mean_len."""
+    H, KV, I, L, V = cfg["hidden"], cfg["kv_hidden"], cfg["inter"], cfg["layers"], cfg["vocab"]
+    w = L * (H * H + 2 * KV * H + H * H + 2 * I * H + H * I)            # int8 weights
+    scales = 4 * L * (H + 2 * KV + H + 2 * I + H)
+    gamma = 4 * (2 * L + 1) * H
+    lm_head = 2 * V * H
+    kv_read = L * 2 * KV * mean_len
+    kv_write = L * 2 * KV
+    return w + scales + gamma + lm_head + kv_read + kv_write
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=64)
+    ap.add_argument("--warmup", type=int, default=8)
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-prefill", action="store_true", help="skip the prefill timing")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on one GPU only (no collectives, no sharding); use --gpus 1", file=sys.stderr)
+        sys.exit(2)
+
+    import flexllm_amd as fx
+    from flexllm_amd import llama, synth, ops
+    from flexllm_amd.device import Event, device_sync
+
+    lib = fx.lib()
+    cfg = llama.make_config()
+    K, W = args.steps, args.warmup
+    assert K + W < cfg["max_pos"]
+    dev_w = llama.synth_weights(cfg, seed=1, device=True)
+    model = llama.Llama(cfg, dev_w)
+    # cache pre-filled with seeded int8 values directly in cache layout, as the reference's decode harness does
+    C_fill = lib.flexllm_rt_fill_i8
+    fx.check(C_fill(C.c_void_p(model.k_cache.ptr), C.c_size_t(model.k_cache.size), C.c_uint64(901), -100, 100, None))
+    fx.check(C_fill(C.c_void_p(model.v_cache.ptr), C.c_size_t(model.v_cache.size), C.c_uint64(902), -100, 100, None))
+    stream = fx.Stream()
+    pos_end = cfg["max_pos"]
+    pos_timed = pos_end - K
+    pos_warm = pos_timed - W
+    tok = fx.to_device(np.array([12345], np.int32))
+    out_w = fx.zeros((max(W, 1),), np.int32)
+    out = fx.zeros((K,), np.int32)
+    device_sync()
+
+    # ---- decode: W warm-up steps (also captures the graph), then exactly K timed steps -----------------
+    model.decode_greedy(tok, pos_warm, W, out, use_graph=True, stream=stream) if W else None
+    stream.sync()
+    e0, e1 = Event(), Event()
+    device_sync()
+    t0 = time.perf_counter()
+    e0.record(stream)
+    model.decode_greedy(tok, pos_timed, K, out, use_graph=True, stream=stream)
+    e1.record(stream)
+    e1.sync()
+    device_sync()
+    wall_ms = (time.perf_counter() - t0) * 1e3
+    ev_ms = e0.elapsed_ms(e1)
+    ms_per_step = wall_ms / K
+    tok_s = 1e3 / ms_per_step
+    mean_len = (pos_timed + 1 + pos_end) / 2.0
+    bpt = bytes_per_token(cfg, mean_len)
+    token_gbs = bpt / (ms_per_step * 1e-3) / 1e9
+
+    # ---- dominant kernel: the fused gate/up GEMV (+SwiGLU), 33.6 MB of int8 weights per launch ---------
+    H, I, L = cfg["hidden"], cfg["inter"], cfg["layers"]
+    wgu = [synth.device_i8((2 * I, H), 7000 + l) for l in range(L)]            # 16 distinct buffers = 537 MB: streams from HBM
+    sgu = synth.device_uniform_f32((2 * I,), 7100, 1e-4, 3e-4)
+    xq = synth.device_i8((H,), 7200)
+    xs = fx.to_device(np.array([0.02], np.float32))
+    y = fx.empty((I,), np.float32)
+    reps = 20
+    for l in range(L):
+        fx.check(lib.flexllm_linear_i8_gemv_swiglu(C.c_void_p(xq.ptr), C.c_void_p(xs.ptr), C.c_void_p(wgu[l].ptr),
+                                                   C.c_void_p(sgu.ptr), C.c_void_p(y.ptr), H, I, stream.handle))
+    k0, k1 = Event(), Event()
+    k0.record(stream)
+    for _ in range(reps):
+        for l in range(L):
+            lib.flexllm_linear_i8_gemv_swiglu(C.c_void_p(xq.ptr), C.c_void_p(xs.ptr), C.c_void_p(wgu[l].ptr),
+                                              C.c_void_p(sgu.ptr), C.c_void_p(y.ptr), H, I, stream.handle)
+    k1.record(stream)
+    k1.sync()
+    kern_ms = k0.elapsed_ms(k1) / (reps * L)
+    kern_bytes = 2 * I * H + 4 * 2 * I + H + 4 + 4 * I            # weights + scales + x + s_x + y
+    kern_gbs = kern_bytes / (kern_ms * 1e-3) / 1e9
+    del wgu
+
+    # ---- prefill: 1024 synthetic tokens through the 16 layers ------------------------------------------
+    prefill_ms = None
+    if not args.no_prefill:
+        try:
+            S = 1024
+            x_in = synth.device_uniform_f32((S, H), 4243, -1.7, 1.7)
+            model.prefill_hidden(x_in, stream=stream)
+            stream.sync()
+            p0, p1 = Event(), Event()
+            p0.record(stream)
+            for _ in range(3):
+                model.prefill_hidden(x_in, stream=stream)
+            p1.record(stream)
+            p1.sync()
+            prefill_ms = p0.elapsed_ms(p1) / 3
+        except Exception as e:  # prefill path not available in this build
+            print("prefill leg skipped: %s" % e, file=sys.stderr)
+
+    # ---- CPU baseline: the oracle (scalar C port of the reference modules), bounded sample --------------
+    cpu = None
+    if not args.no_cpu:
+        from oracle import oracle
+        Ls = 2                                                       # layers in the sample
+        cfg_s = llama.make_config(layers=Ls, vocab=8192)
+        dw = llama.synth_weights(cfg_s, seed=1, device=True)
+        hw = {k: ([a.numpy() for a in v] if isinstance(v, list) else v.numpy()) for k, v in dw.items()}
+        hw["embed"] = hw["embed"].view(np.uint16)
+        om = oracle.OracleModel(cfg_s, hw)
+        kc, vc = om.new_caches()
+        kc[:] = synth.host_i8(kc.shape, 903, -100, 100)
+        vc[:] = synth.host_i8(vc.shape, 904, -100, 100)
+        x = synth.host_normal_f32((H,), 905)
+        n_tok = 3
+        t0 = time.perf_counter()
+        for i in range(n_tok):
+            om.decode_token(x, cfg["max_pos"] - n_tok + i, kc, vc, want_logits=False)
+        t_layers = (time.perf_counter() - t0) / n_tok / Ls                     # seconds per layer per token
+        t0 = time.perf_counter()
+        oracle.lm_head(hw["embed"], x)
+        t_head = (time.perf_counter() - t0) * cfg["vocab"] / cfg_s["vocab"]   # scaled to the full vocabulary
+        cpu_tok_s = 1.0 / (t_layers * cfg["layers"] + t_head)
+        cpu = {"value": round(cpu_tok_s, 4), "unit": "tok/s", "cores": 1, "kind": "port",
+               "sample": "%d tokens x %d of 16 layers at context 4096 + lm_head over %d of %d rows, scaled linearly to "
+                         "16 layers and the full vocabulary (scalar C oracle, host cores=%d)"
+                         % (n_tok, Ls, cfg_s["vocab"], cfg["vocab"], os.cpu_count())}
+
+    result = {
+        "metric": "decode tok/s + prefill ms (1024 tok), Llama-3.2-1B W8A8, % HBM/MFMA roofline",
+        "value": round(tok_s, 2), "unit": "tok/s", "n_gpus": 1, "steps": K, "warmup": W,
+        "ms_per_step": round(ms_per_step, 5), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "int8", "data": "synthetic",
+        "config": {"workload": "Llama-3.2-1B W8A8 SpinQuant greedy decode, batch 1, int8 KV cache, context %d..%d, "
+                               "fp16 tied lm_head, HIP graph replay" % (pos_timed + 1, pos_end),
+                   "layers": cfg["layers"], "context": pos_end, "device": fx.device.device_name()},
+        "decode": {"bytes_per_token": int(bpt), "achieved_GBs": round(token_gbs, 1),
+                   "hbm_frac": round(token_gbs / HBM_PEAK_GBS, 4), "event_ms_per_step": round(ev_ms / K, 5),
+                   "last_tokens": out.numpy()[-4:].tolist()},
+        "prefill_ms_1024": None if prefill_ms is None else round(prefill_ms, 3),
+        "roofline": {"bound": "hbm", "kernel": "gemv_i8_kernel<2,4,swiglu> (gate/up 2048->2x8192)",
+                     "achieved": round(kern_gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(kern_gbs / HBM_PEAK_GBS, 4), "traffic": None,
+                     "bytes_per_launch": int(kern_bytes), "avg_us": round(kern_ms * 1e3, 3)},
+        "cpu_baseline": cpu,
+    }
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()
