@@ -64,6 +64,50 @@ static __global__ __launch_bounds__(256) void kv_store_kernel(const int8_t* __re
     }
 }
 
+// RoPE on q and k, static int8 quantisation of q/k/v, append of k/v to the cache.  One block per token:
+// qkv is fp32 [tokens][H + 2*KV] = [q | k | v]; token t sits at position state[0] (decode, device-side
+// position) or pos0 + t (prefill).  q8 is [tokens][H].
+static __global__ __launch_bounds__(256) void qkv_post_kernel(const float* __restrict__ qkv_all, const float* __restrict__ sin_t,
+                                                              const float* __restrict__ cos_t, const float* __restrict__ q_s,
+                                                              const float* __restrict__ k_s, const float* __restrict__ v_s,
+                                                              int8_t* __restrict__ q8_all, int8_t* __restrict__ kc,
+                                                              int8_t* __restrict__ vc, const int* __restrict__ state, int pos0,
+                                                              int q_heads, int kv_heads, int max_pos) {
+    const int pos = state ? state[0] : pos0 + (int)blockIdx.x;
+    const int half = kHd / 2;
+    const float* sn = sin_t + (size_t)pos * half;
+    const float* cs = cos_t + (size_t)pos * half;
+    const int H = q_heads * kHd, KV = kv_heads * kHd;
+    const float* qkv = qkv_all + (size_t)blockIdx.x * (H + 2 * KV);
+    int8_t* q8 = q8_all + (size_t)blockIdx.x * H;
+    const int q_pairs = q_heads * half, k_pairs = kv_heads * half;
+    for (int i = threadIdx.x; i < q_pairs + k_pairs + KV; i += 256) {
+        if (i < q_pairs) {
+            const int hd = i / half, k = i % half;
+            const float t0 = qkv[hd * kHd + k], t1 = qkv[hd * kHd + k + half];
+            const float o0 = t0 * cs[k] - t1 * sn[k];
+            const float o1 = t0 * sn[k] + t1 * cs[k];
+            const float div = 8.0f * q_s[hd];      // sqrt(head_dim) folded into the Q scale
+            q8[hd * kHd + k] = (int8_t)static_q8(o0, div);
+            q8[hd * kHd + k + half] = (int8_t)static_q8(o1, div);
+        } else if (i < q_pairs + k_pairs) {
+            const int j = i - q_pairs;
+            const int hd = j / half, k = j % half;
+            const float t0 = qkv[H + hd * kHd + k], t1 = qkv[H + hd * kHd + k + half];
+            const float o0 = t0 * cs[k] - t1 * sn[k];
+            const float o1 = t0 * sn[k] + t1 * cs[k];
+            const float div = 1.0f * k_s[hd];
+            int8_t* dst = kc + k_index(hd, pos, max_pos);
+            dst[k] = (int8_t)static_q8(o0, div);
+            dst[k + half] = (int8_t)static_q8(o1, div);
+        } else {
+            const int j = i - q_pairs - k_pairs;
+            const int hd = j / kHd, d = j % kHd;
+            vc[v_index(hd, pos, d, max_pos)] = (int8_t)static_q8(qkv[H + KV + j], 1.0f * v_s[hd]);
+        }
+    }
+}
+
 // ---- phase A ------------------------------------------------------------------------------
 // grid (nchunks, kv_heads); block 64*group threads: wave g = query head kvh*group+g, lane = key.
 static __global__ __launch_bounds__(256) void dec_scores_kernel(const int8_t* __restrict__ q8, const int8_t* __restrict__ kc,

@@ -1,0 +1,145 @@
+// Causal int8 prefill attention (GQA) on MFMA, reading K and V from the layer's int8 cache.
+//
+// One wave owns 32 consecutive queries of one head and walks the key tiles (32 keys) up to its diagonal.
+// The score tile is computed TRANSPOSED, S^T = K_tile . Q_tile^T, so that in the 32x32 accumulator layout a
+// lane holds 16 scores of ONE query (column l%32; keys 8a+4g+b for register 4a+b, g = l/32).  That is also
+// the A-operand shape of the second matrix product P.V (row = query l%32, 16 k-values for k-group g), so the
+// quantised probabilities never leave the registers; V's B operand is gathered in the same key order from
+// the cache's transposed 64-position blocks ([channel][position]: four 4-byte runs per lane).
+//
+// The reference normalises by the full-row sum BEFORE rounding the probabilities to uint8, so the wave makes
+// two passes over its key tiles: pass 1 keeps a running max / running sum of exponentials per query, pass 2
+// recomputes the scores (64-deep dot products: cheap), forms p = exp(s-max)*(1/sum), P = min(255,
+// round(p/A_s)) and accumulates P.V.  P is unsigned and the MFMA is signed x signed: (P-128).V is
+// accumulated and 128*colsum(V) over the same keys is added at the end, both exact in int32.
+#pragma once
+#include "attn_decode_kernels.h"
+
+namespace fx {
+
+constexpr int kPfTile = 32;
+
+__device__ __forceinline__ i32x16 zero16() {
+    i32x16 z;
+#pragma unroll
+    for (int r = 0; r < 16; r++) z[r] = 0;
+    return z;
+}
+
+// grid (ceil(s/128), q_heads), 256 threads: wave w handles queries [(4*blockIdx.x + w)*32, +32)
+static __global__ __launch_bounds__(256) void pf_attention_kernel(const int8_t* __restrict__ q8, const int8_t* __restrict__ kc,
+                                                                  const int8_t* __restrict__ vc, const float* __restrict__ q_s,
+                                                                  const float* __restrict__ k_s, const float* __restrict__ v_s,
+                                                                  const float* __restrict__ a_s, float* __restrict__ o,
+                                                                  uint8_t* __restrict__ p8_out, int s, int q_heads, int group,
+                                                                  int max_pos) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int qb = blockIdx.x * 4 + wave;
+    const int q0 = qb * kPfTile;
+    if (q0 >= s) return;
+    const int h = blockIdx.y, kvh = h / group;
+    const int col = lane & 31, g = lane >> 5;
+    const int query = q0 + col;
+    const float sq = q_s[h], sk = k_s[kvh], as = 1.0f * a_s[h];
+
+    // B operand of S^T = K.Q^T: this lane's query row, 16 d-bytes of k-group g, two k-steps (d 0..31, 32..63)
+    const int8_t* qrow = q8 + ((size_t)query * q_heads + h) * kHd;
+    const i32x4 qf0 = *reinterpret_cast<const i32x4*>(qrow + g * 16);
+    const i32x4 qf1 = *reinterpret_cast<const i32x4*>(qrow + 32 + g * 16);
+
+    auto score_tile = [&](int k0, float (&sc)[16]) {
+        const int8_t* krow = kc + k_index(kvh, k0 + col, max_pos);
+        const i32x4 kf0 = *reinterpret_cast<const i32x4*>(krow + g * 16);
+        const i32x4 kf1 = *reinterpret_cast<const i32x4*>(krow + 32 + g * 16);
+        i32x16 acc = zero16();
+        acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(kf0, qf0, acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(kf1, qf1, acc, 0, 0, 0);
+#pragma unroll
+        for (int r = 0; r < 16; r++) {
+            const int key = k0 + (r >> 2) * 8 + g * 4 + (r & 3);
+            const float v = (float)acc[r] * sq * sk;
+            sc[r] = key <= query ? v : -1e32f;
+        }
+    };
+
+    const int ntiles = qb + 1;
+    // ---- pass 1: row max and row sum of exponentials ----
+    float m_run = -1e32f, l_run = 0.0f;
+    for (int kt = 0; kt < ntiles; kt++) {
+        float sc[16];
+        score_tile(kt * kPfTile, sc);
+        float mt = sc[0];
+#pragma unroll
+        for (int r = 1; r < 16; r++) mt = fmaxf(mt, sc[r]);
+        const float m_new = fmaxf(m_run, mt);
+        float sum = 0.0f;
+#pragma unroll
+        for (int r = 0; r < 16; r++) sum += expf(sc[r] - m_new);
+        l_run = l_run * expf(m_run - m_new) + sum;
+        m_run = m_new;
+    }
+    // merge the two lanes that share a query
+    const float m_o = lane_xor_f<32>(m_run), l_o = lane_xor_f<32>(l_run);
+    const float mx = fmaxf(m_run, m_o);
+    const float total = l_run * expf(m_run - mx) + l_o * expf(m_o - mx);
+    const float cd = 1.0f / total;
+
+    // ---- pass 2: probabilities, P.V ----
+    i32x16 oacc0 = zero16(), oacc1 = zero16();
+    int vsum0 = 0, vsum1 = 0;
+    for (int kt = 0; kt < ntiles; kt++) {
+        const int k0 = kt * kPfTile;
+        float sc[16];
+        score_tile(k0, sc);
+        i32x4 pf;
+#pragma unroll
+        for (int a = 0; a < 4; a++) {
+            uint32_t packed = 0;
+#pragma unroll
+            for (int b = 0; b < 4; b++) {
+                const float p = expf(sc[a * 4 + b] - mx) * cd;
+                int p8 = (int)roundf(p / as);
+                p8 = p8 > 255 ? 255 : p8;
+                if (p8_out) {
+                    const int key = k0 + a * 8 + g * 4 + b;
+                    p8_out[((size_t)h * s + query) * s + key] = (uint8_t)p8;
+                }
+                packed |= (uint32_t)((p8 ^ 0x80) & 0xff) << (8 * b);
+            }
+            pf[a] = (int)packed;
+        }
+        // B operand: V[key][d] for this lane's channel d = col (+32) and the same 16 keys, from [d][64 pos] blocks
+        const int8_t* vblk = vc + v_index(kvh, k0, 0, max_pos);       // start of (block, d=0) row, at position k0%64
+        i32x4 vf0, vf1;
+#pragma unroll
+        for (int a = 0; a < 4; a++) {
+            vf0[a] = *reinterpret_cast<const int*>(vblk + (size_t)col * kVBlock + a * 8 + g * 4);
+            vf1[a] = *reinterpret_cast<const int*>(vblk + (size_t)(col + 32) * kVBlock + a * 8 + g * 4);
+            vsum0 = __builtin_amdgcn_sdot4(0x01010101, vf0[a], vsum0, false);
+            vsum1 = __builtin_amdgcn_sdot4(0x01010101, vf1[a], vsum1, false);
+        }
+        oacc0 = __builtin_amdgcn_mfma_i32_32x32x32_i8(pf, vf0, oacc0, 0, 0, 0);
+        oacc1 = __builtin_amdgcn_mfma_i32_32x32x32_i8(pf, vf1, oacc1, 0, 0, 0);
+    }
+    vsum0 += lane_xor_i<32>(vsum0);
+    vsum1 += lane_xor_i<32>(vsum1);
+    const float sv = v_s[kvh], sa = a_s[h];
+#pragma unroll
+    for (int r = 0; r < 16; r++) {
+        const int row = q0 + (r >> 2) * 8 + g * 4 + (r & 3);
+        float* orow = o + ((size_t)row * q_heads + h) * kHd;
+        orow[col] = (float)(oacc0[r] + 128 * vsum0) * sa * sv;
+        orow[col + 32] = (float)(oacc1[r] + 128 * vsum1) * sa * sv;
+    }
+}
+
+inline int mha_prefill_launch(const int8_t* q8, const int8_t* kc, const int8_t* vc, const float* q_s, const float* k_s,
+                              const float* v_s, const float* a_s, float* o, uint8_t* p8_out, int s, int q_heads,
+                              int kv_heads, int max_pos, hipStream_t st) {
+    dim3 grid((s + 127) / 128, q_heads);
+    pf_attention_kernel<<<grid, 256, 0, st>>>(q8, kc, vc, q_s, k_s, v_s, a_s, o, p8_out, s, q_heads, q_heads / kv_heads, max_pos);
+    FX_LAUNCH_CHECK();
+    return FLEXLLM_OK;
+}
+
+}  // namespace fx

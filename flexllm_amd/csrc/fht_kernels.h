@@ -27,7 +27,7 @@ __device__ __forceinline__ float lane_butterfly(float a, bool bit_set) {
     return bit_set ? (p - a) : (a + p);
 }
 
-template <int LOG2N, bool QUANT>
+template <int LOG2N, bool QUANT, bool SWIGLU = false>
 __global__ __launch_bounds__(kFhtBlock) void fht_kernel(const float* __restrict__ x, float* __restrict__ y,
                                                         int8_t* __restrict__ q, float* __restrict__ s, float scale) {
     constexpr int N = 1 << LOG2N;
@@ -38,11 +38,23 @@ __global__ __launch_bounds__(kFhtBlock) void fht_kernel(const float* __restrict_
     const int t = threadIdx.x;
     const int lane = t & 63;
     const size_t row = blockIdx.x;
-    const float4* xr = reinterpret_cast<const float4*>(x + row * N);
-
     float4 a[NJ];
+    if constexpr (SWIGLU) {
+        // input row is [2N] interleaved (gate_i, up_i); element i = up_i * silu(gate_i)
+        const float4* xr = reinterpret_cast<const float4*>(x + row * (2 * N));
 #pragma unroll
-    for (int j = 0; j < NJ; j++) a[j] = xr[j * 256 + t];
+        for (int j = 0; j < NJ; j++) {
+            const float4 p0 = xr[(j * 256 + t) * 2], p1 = xr[(j * 256 + t) * 2 + 1];
+            a[j].x = p0.y * (p0.x / (1.0f + expf(-p0.x)));
+            a[j].y = p0.w * (p0.z / (1.0f + expf(-p0.z)));
+            a[j].z = p1.y * (p1.x / (1.0f + expf(-p1.x)));
+            a[j].w = p1.w * (p1.z / (1.0f + expf(-p1.z)));
+        }
+    } else {
+        const float4* xr = reinterpret_cast<const float4*>(x + row * N);
+#pragma unroll
+        for (int j = 0; j < NJ; j++) a[j] = xr[j * 256 + t];
+    }
 
     // stage: bit 1 (elements e and e^2 of each float4)
 #pragma unroll

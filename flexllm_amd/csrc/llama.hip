@@ -43,47 +43,6 @@ struct flexllm_llama {
 namespace fx {
 
 // ---- small fused decode kernels ------------------------------------------------------------------
-// RoPE on q and k, static int8 quantisation of q/k/v, append of k/v at the current position.
-// qkv is fp32 [H + 2*KV] = [q | k | v]; one block.
-static __global__ __launch_bounds__(256) void dec_qkv_post_kernel(const float* __restrict__ qkv, const float* __restrict__ sin_t,
-                                                                  const float* __restrict__ cos_t, const float* __restrict__ q_s,
-                                                                  const float* __restrict__ k_s, const float* __restrict__ v_s,
-                                                                  int8_t* __restrict__ q8, int8_t* __restrict__ kc,
-                                                                  int8_t* __restrict__ vc, const int* __restrict__ state,
-                                                                  int q_heads, int kv_heads, int max_pos) {
-    const int pos = state[0];
-    const int half = kHd / 2;
-    const float* sn = sin_t + (size_t)pos * half;
-    const float* cs = cos_t + (size_t)pos * half;
-    const int H = q_heads * kHd, KV = kv_heads * kHd;
-    const int q_pairs = q_heads * half, k_pairs = kv_heads * half;
-    for (int i = threadIdx.x; i < q_pairs + k_pairs + KV; i += 256) {
-        if (i < q_pairs) {
-            const int hd = i / half, k = i % half;
-            const float t0 = qkv[hd * kHd + k], t1 = qkv[hd * kHd + k + half];
-            const float o0 = t0 * cs[k] - t1 * sn[k];
-            const float o1 = t0 * sn[k] + t1 * cs[k];
-            const float div = 8.0f * q_s[hd];      // sqrt(head_dim) folded into the Q scale
-            q8[hd * kHd + k] = (int8_t)static_q8(o0, div);
-            q8[hd * kHd + k + half] = (int8_t)static_q8(o1, div);
-        } else if (i < q_pairs + k_pairs) {
-            const int j = i - q_pairs;
-            const int hd = j / half, k = j % half;
-            const float t0 = qkv[H + hd * kHd + k], t1 = qkv[H + hd * kHd + k + half];
-            const float o0 = t0 * cs[k] - t1 * sn[k];
-            const float o1 = t0 * sn[k] + t1 * cs[k];
-            const float div = 1.0f * k_s[hd];
-            int8_t* dst = kc + k_index(hd, pos, max_pos);
-            dst[k] = (int8_t)static_q8(o0, div);
-            dst[k + half] = (int8_t)static_q8(o1, div);
-        } else {
-            const int j = i - q_pairs - k_pairs;
-            const int hd = j / kHd, d = j % kHd;
-            vc[v_index(hd, pos, d, max_pos)] = (int8_t)static_q8(qkv[H + KV + j], 1.0f * v_s[hd]);
-        }
-    }
-}
-
 // Dequantise the attention accumulators and quantise the 2048-vector per token for o_proj; one block.
 template <int VPT>
 static __global__ __launch_bounds__(256) void dec_out_quant_kernel(const int32_t* __restrict__ o_acc, const float* __restrict__ a_s,
@@ -172,8 +131,8 @@ static int decode_layer(flexllm_llama* m, int l, hipStream_t st) {
     // attention block
     rmsnorm_kernel<2, true><<<1, kBlock, 0, st>>>(m->x, g0, nullptr, m->xq, m->xs, H, c.eps);
     if ((rc = launch_gemv<kEpiDequant>(m->xq, w.wqkv, nullptr, m->xs, w.sqkv, nullptr, m->qkv, H, H + 2 * KV, st))) return rc;
-    dec_qkv_post_kernel<<<1, 256, 0, st>>>(m->qkv, m->rope_sin, m->rope_cos, q_s, k_s, v_s, m->q8, kc, vc, m->state,
-                                           c.q_heads, c.kv_heads, c.max_pos);
+    qkv_post_kernel<<<1, 256, 0, st>>>(m->qkv, m->rope_sin, m->rope_cos, q_s, k_s, v_s, m->q8, kc, vc, m->state, 0,
+                                       c.q_heads, c.kv_heads, c.max_pos);
     dim3 grid(c.max_pos / kChunk, c.kv_heads);
     dec_scores_kernel<<<grid, 64 * group, 0, st>>>(m->q8, kc, q_s, k_s, m->scores, m->stats, m->o_acc, m->state, 0,
                                                    c.max_pos, group, c.max_pos);

@@ -1,11 +1,101 @@
-// Prefill path (placeholder until the MFMA GEMM and the causal attention kernel land).
+// Prefill path of the Llama graph: M tokens at once through int8 MFMA GEMMs and causal int8 attention,
+// plus the C ABI entry point of the stand-alone prefill attention.
 #include "prefill.h"
+#include "attn_prefill.h"
+#include "elementwise_kernels.h"
+#include "fht_kernels.h"
+#include "gemm_i8.h"
 
 namespace fx {
-int llama_prefill_run(const flexllm_llama_config&, const LayerW*, const float*, const float*, const float*, const float*,
-                      const float*, const float*, const float*, int8_t*, int8_t*, size_t, PrefillWorkspace*, const float*,
-                      int, float*, hipStream_t) {
-    set_error("prefill: not built yet");
-    return FLEXLLM_EINVAL;
+
+struct PrefillBuffers {
+    float *x, *x2, *qkv, *att, *gu;
+    int8_t *xq, *q8;
+    float* xs;
+};
+
+static int prefill_workspace_get(PrefillWorkspace* ws, const flexllm_llama_config& c, int s, PrefillBuffers* b) {
+    const size_t H = c.hidden, KV = c.kv_hidden, I = c.inter;
+    auto up = [](size_t v) { return (v + 255) & ~(size_t)255; };
+    const size_t sz_x = up(sizeof(float) * s * H), sz_qkv = up(sizeof(float) * s * (H + 2 * KV));
+    const size_t sz_gu = up(sizeof(float) * s * 2 * I), sz_xq = up((size_t)s * I), sz_q8 = up((size_t)s * H);
+    const size_t sz_xs = up(sizeof(float) * s);
+    const size_t total = 3 * sz_x + sz_qkv + sz_gu + sz_xq + sz_q8 + sz_xs;
+    if (ws->tokens < s) {
+        FX_HIP(hipDeviceSynchronize());
+        prefill_workspace_free(ws);
+        hipError_t e = hipMalloc(&ws->base, total);
+        if (e != hipSuccess) { set_error("prefill workspace hipMalloc(%zu) failed: %s", total, hipGetErrorString(e)); return FLEXLLM_ENOMEM; }
+        ws->tokens = s;
+    }
+    char* p = (char*)ws->base;
+    b->x = (float*)p; p += sz_x;
+    b->x2 = (float*)p; p += sz_x;
+    b->att = (float*)p; p += sz_x;
+    b->qkv = (float*)p; p += sz_qkv;
+    b->gu = (float*)p; p += sz_gu;
+    b->xq = (int8_t*)p; p += sz_xq;
+    b->q8 = (int8_t*)p; p += sz_q8;
+    b->xs = (float*)p;
+    return FLEXLLM_OK;
 }
+
+int llama_prefill_run(const flexllm_llama_config& c, const LayerW* layers, const float* gamma, const float* q_s_all,
+                      const float* k_s_all, const float* v_s_all, const float* a_s_all, const float* rope_sin,
+                      const float* rope_cos, int8_t* k_cache, int8_t* v_cache, size_t cache_layer_bytes,
+                      PrefillWorkspace* ws, const float* x_in, int s, float* hidden_out, hipStream_t st) {
+    FX_REQUIRE(s > 0 && s % kPfTile == 0 && s <= c.max_pos, "prefill: s=%d must be a positive multiple of 32, <= max_pos=%d", s, c.max_pos);
+    PrefillBuffers b;
+    int rc = prefill_workspace_get(ws, c, s, &b);
+    if (rc) return rc;
+    const int H = c.hidden, KV = c.kv_hidden, I = c.inter;
+    FX_HIP(hipMemcpyAsync(b.x, x_in, sizeof(float) * (size_t)s * H, hipMemcpyDeviceToDevice, st));
+    for (int l = 0; l < c.layers; l++) {
+        const LayerW& w = layers[l];
+        const float* g0 = gamma + (size_t)(2 * l) * H;
+        const float* g1 = gamma + (size_t)(2 * l + 1) * H;
+        const float* q_s = q_s_all + (size_t)l * c.q_heads;
+        const float* k_s = k_s_all + (size_t)l * c.kv_heads;
+        const float* v_s = v_s_all + (size_t)l * c.kv_heads;
+        const float* a_s = a_s_all + (size_t)l * c.q_heads;
+        int8_t* kc = k_cache + (size_t)l * cache_layer_bytes;
+        int8_t* vc = v_cache + (size_t)l * cache_layer_bytes;
+        // attention block
+        rmsnorm_kernel<2, true><<<s, kBlock, 0, st>>>(b.x, g0, nullptr, b.xq, b.xs, H, c.eps);
+        if ((rc = launch_gemm<kGemmDequant>(b.xq, w.wqkv, nullptr, b.xs, w.sqkv, nullptr, b.qkv, s, H, H + 2 * KV, st))) return rc;
+        qkv_post_kernel<<<s, 256, 0, st>>>(b.qkv, rope_sin, rope_cos, q_s, k_s, v_s, b.q8, kc, vc, nullptr, 0, c.q_heads,
+                                           c.kv_heads, c.max_pos);
+        if ((rc = mha_prefill_launch(b.q8, kc, vc, q_s, k_s, v_s, a_s, b.att, nullptr, s, c.q_heads, c.kv_heads, c.max_pos, st))) return rc;
+        quant_sym_kernel<2><<<s, kBlock, 0, st>>>(b.att, b.xq, b.xs, H);
+        if ((rc = launch_gemm<kGemmDequant>(b.xq, w.wo, nullptr, b.xs, w.so, b.x, b.x2, s, H, H, st))) return rc;
+        // feed-forward block
+        rmsnorm_kernel<2, true><<<s, kBlock, 0, st>>>(b.x2, g1, nullptr, b.xq, b.xs, H, c.eps);
+        if ((rc = launch_gemm<kGemmDequant>(b.xq, w.wgu, nullptr, b.xs, w.sgu, nullptr, b.gu, s, H, 2 * I, st))) return rc;
+        fht_kernel<13, true, true><<<s, kFhtBlock, 0, st>>>(b.gu, nullptr, b.xq, b.xs, c.fht_scale);
+        if ((rc = launch_gemm<kGemmDequant>(b.xq, w.wd, nullptr, b.xs, w.sd, b.x2, b.x, s, I, H, st))) return rc;
+    }
+    FX_LAUNCH_CHECK();
+    if (hidden_out) FX_HIP(hipMemcpyAsync(hidden_out, b.x, sizeof(float) * (size_t)s * H, hipMemcpyDeviceToDevice, st));
+    return FLEXLLM_OK;
+}
+
 }  // namespace fx
+
+using namespace fx;
+
+extern "C" {
+
+int flexllm_mha_i8_prefill(const int8_t* q8, const int8_t* k_cache, const int8_t* v_cache, const flexllm_mha_scales* sc,
+                           float* o, uint8_t* p8_out, int s, int q_heads, int kv_heads, int head_dim, int max_pos,
+                           void* stream) {
+    FX_REQUIRE(q8 && k_cache && v_cache && sc && o, "mha_prefill: null pointer");
+    FX_REQUIRE(sc->q_s && sc->k_s && sc->v_s && sc->a_s, "mha_prefill: null scale table");
+    FX_REQUIRE(head_dim == kHd, "mha_prefill: head_dim=%d (only 64)", head_dim);
+    FX_REQUIRE(kv_heads > 0 && q_heads % kv_heads == 0, "mha_prefill: q_heads=%d kv_heads=%d", q_heads, kv_heads);
+    FX_REQUIRE(s > 0 && s % kPfTile == 0 && s <= max_pos && max_pos % kVBlock == 0,
+               "mha_prefill: s=%d max_pos=%d (s a positive multiple of 32, s <= max_pos, max_pos %% 64 == 0)", s, max_pos);
+    return mha_prefill_launch(q8, k_cache, v_cache, sc->q_s, sc->k_s, sc->v_s, sc->a_s, o, p8_out, s, q_heads, kv_heads,
+                              max_pos, as_stream(stream));
+}
+
+}  // extern "C"

@@ -31,7 +31,7 @@ def _seed(base, layer, tensor):
 def synth_weights(cfg, seed=1, device=False):
     """Random-init int8 weights U[-127,127] with per-channel scales sized so that activations stay O(1),
     RMSNorm gains U[0.5,1.5], static attention scales with a seeded +-20% jitter per head, fp16 embedding.
-    device=False -> numpy arrays (for the oracle); device=True -> DeviceArrays filled on the GPU by the
+    device=False -> numpy arrays on the host; device=True -> DeviceArrays filled on the GPU by the
     same counter-based generator."""
     i8 = synth.device_i8 if device else synth.host_i8
     f32 = synth.device_uniform_f32 if device else synth.host_uniform_f32
@@ -104,7 +104,7 @@ class Llama:
         return hidden
 
     def caches_token_major(self):
-        """int8 caches as numpy [layer][pos][kv_hidden] (the oracle's layout)."""
+        """int8 caches as numpy [layer][pos][kv_hidden] (token-major)."""
         c = self.cfg
         k = self.k_cache.numpy().transpose(0, 2, 1, 3).reshape(c["layers"], c["max_pos"], c["kv_hidden"])
         v = self.v_cache.numpy().transpose(0, 2, 4, 1, 3).reshape(c["layers"], c["max_pos"], c["kv_hidden"])

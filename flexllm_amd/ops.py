@@ -205,12 +205,13 @@ def mha_i8_decode(q8, k_cache, v_cache, scales, length, want_p=False, stream=Non
     return o, p8
 
 
-def mha_i8_prefill(q8, k8, v8, scales, want_p=False, stream=None):
+def mha_i8_prefill(q8, k_cache, v_cache, scales, want_p=False, stream=None):
     s, qh, hd = q8.shape
-    kvh = k8.shape[1]
+    kvh, max_pos, _ = k_cache.shape
     o = DeviceArray((s, qh, hd), np.float32)
-    p8 = DeviceArray((qh, s, s), np.uint8) if want_p else None
-    check(lib().flexllm_mha_i8_prefill(_p(q8), _p(k8), _p(v8), scales.ref(), _p(o), _p(p8), s, qh, kvh, hd, _s(stream)))
+    p8 = DeviceArray((qh, s, s), np.uint8).zero_() if want_p else None
+    check(lib().flexllm_mha_i8_prefill(_p(q8), _p(k_cache), _p(v_cache), scales.ref(), _p(o), _p(p8), s, qh, kvh, hd,
+                                       max_pos, _s(stream)))
     return o, p8
 
 

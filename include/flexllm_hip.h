@@ -183,11 +183,15 @@ int flexllm_kv_store_i8(const int8_t* k8, const int8_t* v8, int8_t* k_cache, int
 int flexllm_mha_i8_decode(const int8_t* q8, const int8_t* k_cache, const int8_t* v_cache,
                           const flexllm_mha_scales* sc, float* o, uint8_t* p8_out, int len, int q_heads,
                           int kv_heads, int head_dim, int max_pos, void* stream);
-/* Prefill causal attention over s tokens: q8 [s][q_heads][64], k8/v8 [s][kv_heads][64] int8 (already
- * quantised), o fp32 [s][q_heads][64].  Replaces SpinQuant_Llama_32_1B/MHA_i8xi8.h:369-427 from the
- * qxk stage on.  s % 64 == 0.  p8_out optional uint8 [q_heads][s][s]. */
-int flexllm_mha_i8_prefill(const int8_t* q8, const int8_t* k8, const int8_t* v8, const flexllm_mha_scales* sc,
-                           float* o, uint8_t* p8_out, int s, int q_heads, int kv_heads, int head_dim, void* stream);
+/* Prefill causal attention over s tokens (positions 0..s-1): q8 [s][q_heads][64] int8; K and V are read from
+ * the cache layouts above (filled by flexllm_kv_append_i8 / flexllm_kv_store_i8); o fp32 [s][q_heads][64].
+ * Replaces SpinQuant_Llama_32_1B/MHA_i8xi8.h:369-427 from the qxk stage on (pref_MHA_i8xi8_qxk_template,
+ * pref_causal_mask_template, pref_Softmax, uint8 P quant, pref_MHA_i8xi8_axv_template, dequant).
+ * s % 32 == 0.  p8_out optional uint8 [q_heads][s][s], zero-filled by the caller (only the causal tiles are
+ * written). */
+int flexllm_mha_i8_prefill(const int8_t* q8, const int8_t* k_cache, const int8_t* v_cache,
+                           const flexllm_mha_scales* sc, float* o, uint8_t* p8_out, int s, int q_heads,
+                           int kv_heads, int head_dim, int max_pos, void* stream);
 
 /* ---- Logits.h (greedy) ---------------------------------------------------------------- */
 /* logits[v] = sum_k fp16(E[v][k]) * n[k] (fp32 accumulate): tied fp16 lm_head GEMV. */
