@@ -1,0 +1,535 @@
+// One persistent kernel per decoded token: all 16 layers, the final norm and the fp16 lm_head.
+//
+// Why: at batch 1 a decode step is ~100 dependent phases of 0.3-4 us of HBM streaming each; as separate
+// kernels every phase pays a launch plus a cold start, and the chip idles between them.  Here 256 workgroups
+// (one per CU, 512 threads) stay resident and walk the phases together:
+//   per layer  1 RMSNorm+quant (redundantly in every workgroup) -> q/k/v GEMV rows
+//              2 RoPE + static int8 quant + KV append, int8 scores of a 128-key chunk, chunk max / sum-exp
+//              3 row statistics from the chunk statistics, uint8 probabilities, partial P.V (int32 atomics)
+//              4 attention dequant + per-token quant (redundant) -> o_proj rows + residual
+//              5 RMSNorm+quant (redundant) -> gate/up rows + SiLU*up
+//              6 Hadamard R4 + quant (redundant) -> down rows + residual
+//   then       final RMSNorm (redundant) -> lm_head rows, per-workgroup argmax candidates.
+// Phases are separated by a grid barrier built from device-scope relaxed atomics (two-level arrive, one
+// broadcast flag).  The weights a workgroup needs in the NEXT phase do not depend on the activations, so
+// they are loaded into registers BEFORE waiting on the barrier: HBM keeps streaming while the barrier's
+// round trips are in flight.
+//
+// Memory-model discipline (no cache flushes inside the kernel): every value that crosses workgroups between
+// barriers (x, x2, qkv, h, chunk statistics, attention accumulators) is written and read with device-scope
+// relaxed atomic stores/loads, which bypass the per-XCD L2 for coherence; each thread drains its outstanding
+// stores (s_waitcnt 0) before the workgroup arrives at the barrier.  Weights and the old KV cache are
+// read-only inside a step and use ordinary loads; the new token's K/V row is used from LDS by the workgroup
+// that owns its chunk and written to the cache for later steps (visible after the kernel boundary).
+// Every spin is bounded: on a timeout the kernel sets an error flag and runs to completion.
+#pragma once
+#include "attn_decode_kernels.h"
+#include "gemv_i8.h"
+#include "prefill.h"
+#include <hip/hip_fp16.h>
+
+namespace fx {
+
+constexpr int kMegaWG = 256;       // workgroups (persistent, one per CU)
+constexpr int kMegaT = 512;        // threads per workgroup
+constexpr int kMegaWaves = kMegaT / 64;
+constexpr int kMegaGroup = 32;     // workgroups per first-level barrier counter
+constexpr int kMegaSpinLimit = 1 << 22;
+
+struct MegaParams {
+    const LayerW* layers;          // device array [layers]
+    const float *gamma, *q_s, *k_s, *v_s, *a_s, *rope_sin, *rope_cos;
+    const __half* embed;
+    int8_t *k_cache, *v_cache;
+    size_t cache_layer_bytes;
+    float *x, *x2, *qkv, *h, *logits;
+    float2* stats;                 // [q_heads][32]
+    int32_t* o_acc;                // [H]
+    int* state;                    // [0] pos, [1] step, [2] barrier epoch base, [3] error flag
+    unsigned* bar;                 // [0] flag, [64] top counter, [128+64g] group counters
+    const int* token;              // current token id (device), used when x_in == NULL
+    const float* x_in;             // optional fp32 input embedding
+    float* am_v;                   // [kMegaWG] argmax candidates
+    int* am_i;
+    int n_layers, max_pos, vocab, want_head;
+    float eps, fht_scale;
+    long long* timeline;           // optional [n_layers*6+2][2] wall-clock stamps of workgroup 0 (after wait, before arrive)
+};
+
+__device__ __forceinline__ float ld_f(const float* p) { return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
+__device__ __forceinline__ void st_f(float* p, float v) { __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
+__device__ __forceinline__ int ld_i(const int* p) { return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
+__device__ __forceinline__ void st_i(int* p, int v) { __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
+
+// Grid barrier from device-scope relaxed atomics: workgroup w adds 1 to group counter w/32 (8 counters on
+// separate 256-byte lines, so at most 32 atomics serialise on one address); the last arriver of a group adds 1
+// to the top counter, the last of those publishes the epoch in a flag that everybody polls.  (Polling the
+// group counters directly costs more: 256 pollers then contend with the arriving atomics on the same lines.)
+struct GridBarrier {
+    unsigned* mem;                              // [0] flag, [64] top counter, [128 + 64*g] group counters
+    unsigned epoch;
+    int* err;
+    __device__ __forceinline__ void arrive() {
+        __builtin_amdgcn_s_waitcnt(0);          // this thread's stores have been acknowledged
+        __syncthreads();
+        epoch++;
+        if (threadIdx.x == 0) {
+            const int g = blockIdx.x / kMegaGroup;
+            const unsigned old = __hip_atomic_fetch_add(&mem[128 + 64 * g], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            if (old == epoch * kMegaGroup - 1) {
+                const unsigned o2 = __hip_atomic_fetch_add(&mem[64], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                if (o2 == epoch * (kMegaWG / kMegaGroup) - 1)
+                    __hip_atomic_store(&mem[0], epoch, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            }
+        }
+    }
+    __device__ __forceinline__ void wait() {
+        if (threadIdx.x == 0) {
+            int it = 0;
+            // signed distance so that the comparison survives counter wrap-around
+            while ((int)(__hip_atomic_load(&mem[0], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) - epoch) < 0) {
+                if (++it > kMegaSpinLimit) { st_i(err, 1); break; }
+            }
+        }
+        __syncthreads();
+    }
+};
+
+struct MegaLds {
+    __attribute__((aligned(16))) float f[8192];        // FHT buffer / fp32 staging (32 KiB)
+    __attribute__((aligned(16))) int8_t xq[8192];      // quantised activation vector of the current GEMV
+    float red[kMegaWaves];
+    float sc[4][kChunk];                               // scores of this chunk, 4 query heads
+    __attribute__((aligned(16))) int8_t q8[4][kHd];
+    __attribute__((aligned(16))) int8_t knew[kHd];
+    __attribute__((aligned(16))) int8_t vnew[kHd];
+    __attribute__((aligned(16))) uint8_t pb[4][kChunk];
+    float rowmax[4], rowcd[4];
+    int osum[4][kHd];
+    float bestv[kMegaWaves];
+    int besti[kMegaWaves];
+};
+
+template <int NW>
+__device__ __forceinline__ float mega_block_max(float v, float* red) { return block_max<NW>(v, red); }
+
+// RMSNorm (optional) + per-token int8 quantisation of a 2048-vector held as 4 values per thread; result in L.xq.
+// Returns the quantisation scale to every thread.
+__device__ __forceinline__ float norm_quant_2048(float (&v)[4], const float* __restrict__ gamma, bool do_norm, float eps,
+                                                 MegaLds& L) {
+    const int t = threadIdx.x;
+    if (do_norm) {
+        float ss = (v[0] * v[0] + v[1] * v[1]) + (v[2] * v[2] + v[3] * v[3]);
+        ss = block_sum<kMegaWaves>(ss, L.red);
+        const float rms = 1.0f / sqrtf(ss / 2048.0f + eps);
+        const float4 g = reinterpret_cast<const float4*>(gamma)[t];
+        v[0] = v[0] * rms * g.x; v[1] = v[1] * rms * g.y; v[2] = v[2] * rms * g.z; v[3] = v[3] * rms * g.w;
+    }
+    float amax = fmaxf(fmaxf(fabsf(v[0]), fabsf(v[1])), fmaxf(fabsf(v[2]), fabsf(v[3])));
+    amax = block_max<kMegaWaves>(amax, L.red);
+    const float sc = sym_scale(amax, 127.0f);
+    reinterpret_cast<uint32_t*>(L.xq)[t] = pack4_i8(quant_round(v[0], sc), quant_round(v[1], sc), quant_round(v[2], sc),
+                                                    quant_round(v[3], sc));
+    __syncthreads();
+    return sc;
+}
+
+template <int NCH>
+__device__ __forceinline__ void mega_load_rows(const int8_t* __restrict__ w, int k, int row, int lane, i32x4 (&wr)[NCH]) {
+    const i32x4* p = reinterpret_cast<const i32x4*>(w + (size_t)row * k);
+#pragma unroll
+    for (int i = 0; i < NCH; i++) wr[i] = __builtin_nontemporal_load(p + lane + 64 * i);
+}
+template <int NCH>
+__device__ __forceinline__ int mega_dot_row(const i32x4 (&wr)[NCH], const int8_t* xq_lds, int lane) {
+    int acc = 0;
+#pragma unroll
+    for (int i = 0; i < NCH; i++) acc = dot16(wr[i], reinterpret_cast<const i32x4*>(xq_lds)[lane + 64 * i], acc);
+    return wave_sum_i(acc);
+}
+
+__global__ __launch_bounds__(kMegaT, 1) void decode_mega_kernel(MegaParams p) {
+    __shared__ MegaLds L;
+    const int t = threadIdx.x, lane = t & 63, wave = t >> 6, wg = blockIdx.x;
+    constexpr int H = 2048, KV = 512, I = 8192, QH = 32, KVH = 8, GROUP = 4;
+    const int pos = p.state[0];
+    const int len = pos + 1;
+    GridBarrier bar{p.bar, (unsigned)p.state[2], &p.state[3]};
+    int stamp_i = 0;
+    auto stamp = [&]() { if (p.timeline && wg == 0 && t == 0) p.timeline[stamp_i] = wall_clock64(); stamp_i++; };
+    const int tok = p.x_in ? 0 : p.token[0];
+
+    // attention work item of this workgroup
+    const int a_h = wg / 32, a_c = wg % 32;
+    const bool a_active = a_c * kChunk < len && a_c * kChunk < p.max_pos;
+    const bool a_owner = a_active && (pos / kChunk == a_c);       // this chunk holds the new token
+
+    for (int l = 0; l < p.n_layers; l++) {
+        const LayerW w = p.layers[l];
+        const float* g0 = p.gamma + (size_t)(2 * l) * H;
+        const float* g1 = p.gamma + (size_t)(2 * l + 1) * H;
+        const float* q_s = p.q_s + l * QH;
+        const float* k_s = p.k_s + l * KVH;
+        const float* v_s = p.v_s + l * KVH;
+        const float* a_s = p.a_s + l * QH;
+        int8_t* kc = p.k_cache + (size_t)l * p.cache_layer_bytes;
+        int8_t* vc = p.v_cache + (size_t)l * p.cache_layer_bytes;
+
+        // ================= phase 1: RMSNorm + quant -> q/k/v rows (12 rows per workgroup) =================
+        {
+            i32x4 wr[2][2];
+            const int r0 = wg * 12 + wave, r1 = r0 + 8;
+            const bool has1 = wave < 4;
+            mega_load_rows<2>(w.wqkv, H, r0, lane, wr[0]);
+            if (has1) mega_load_rows<2>(w.wqkv, H, r1, lane, wr[1]);
+            if (l > 0) bar.wait();                                   // x of the previous layer is complete
+            stamp();
+            float v[4];
+            if (l == 0) {
+                if (p.x_in) { const float4 q = reinterpret_cast<const float4*>(p.x_in)[t]; v[0] = q.x; v[1] = q.y; v[2] = q.z; v[3] = q.w; }
+                else {
+#pragma unroll
+                    for (int i = 0; i < 4; i++) v[i] = __half2float(p.embed[(size_t)tok * H + 4 * t + i]);
+                }
+            } else {
+#pragma unroll
+                for (int i = 0; i < 4; i++) v[i] = ld_f(&p.x[4 * t + i]);
+            }
+            const float sx = norm_quant_2048(v, g0, true, p.eps, L);
+            const int a0 = mega_dot_row<2>(wr[0], L.xq, lane);
+            if (lane == 0) st_f(&p.qkv[r0], (float)a0 * sx * w.sqkv[r0]);
+            if (has1) {
+                const int a1 = mega_dot_row<2>(wr[1], L.xq, lane);
+                if (lane == 0) st_f(&p.qkv[r1], (float)a1 * sx * w.sqkv[r1]);
+            }
+            stamp();
+            bar.arrive();
+        }
+
+        // ================= phase 2: RoPE/quant/append, scores of this chunk, chunk statistics =================
+        {
+            i32x4 kreg = {0, 0, 0, 0};
+            const int key = t >> 2, part = t & 3;
+            const int kpos = a_c * kChunk + key;
+            if (a_active) kreg = *reinterpret_cast<const i32x4*>(kc + k_index(a_h, min(kpos, p.max_pos - 1), p.max_pos) + part * 16);
+            bar.wait();
+            stamp();
+            if (a_active) {
+                const float* sn = p.rope_sin + (size_t)pos * 32;
+                const float* cs = p.rope_cos + (size_t)pos * 32;
+                if (t < 128) {                                        // q: 4 heads x 32 pairs
+                    const int g = t >> 5, k = t & 31, qh = a_h * GROUP + g;
+                    const float t0 = ld_f(&p.qkv[qh * kHd + k]), t1 = ld_f(&p.qkv[qh * kHd + k + 32]);
+                    const float o0 = t0 * cs[k] - t1 * sn[k], o1 = t0 * sn[k] + t1 * cs[k];
+                    const float div = 8.0f * q_s[qh];
+                    L.q8[g][k] = (int8_t)static_q8(o0, div);
+                    L.q8[g][k + 32] = (int8_t)static_q8(o1, div);
+                } else if (t < 160) {                                 // k of the new token: 32 pairs
+                    const int k = t - 128;
+                    const float t0 = ld_f(&p.qkv[H + a_h * kHd + k]), t1 = ld_f(&p.qkv[H + a_h * kHd + k + 32]);
+                    const float o0 = t0 * cs[k] - t1 * sn[k], o1 = t0 * sn[k] + t1 * cs[k];
+                    const float div = 1.0f * k_s[a_h];
+                    const int8_t b0 = (int8_t)static_q8(o0, div), b1 = (int8_t)static_q8(o1, div);
+                    L.knew[k] = b0; L.knew[k + 32] = b1;
+                    if (a_owner) { int8_t* dst = kc + k_index(a_h, pos, p.max_pos); dst[k] = b0; dst[k + 32] = b1; }
+                } else if (t < 224) {                                 // v of the new token
+                    const int d = t - 160;
+                    const int8_t b = (int8_t)static_q8(ld_f(&p.qkv[H + KV + a_h * kHd + d]), 1.0f * v_s[a_h]);
+                    L.vnew[d] = b;
+                    if (a_owner) vc[v_index(a_h, pos, d, p.max_pos)] = b;
+                }
+                __syncthreads();
+                if (kpos == pos) kreg = reinterpret_cast<const i32x4*>(L.knew)[part];
+                float s_mine = 0.0f;
+#pragma unroll
+                for (int g = 0; g < GROUP; g++) {
+                    int acc = dot16(kreg, reinterpret_cast<const i32x4*>(L.q8[g])[part], 0);
+                    acc += lane_xor_i<1>(acc);
+                    acc += lane_xor_i<2>(acc);
+                    const float s = (float)acc * q_s[a_h * GROUP + g] * k_s[a_h];
+                    if (part == g) s_mine = s;
+                }
+                L.sc[part][key] = kpos < len ? s_mine : -1e32f;
+                __syncthreads();
+                if (wave < GROUP) {
+                    const float s0 = L.sc[wave][lane], s1 = L.sc[wave][lane + 64];
+                    const float m = wave_max(fmaxf(s0, s1));
+                    float sum = (a_c * kChunk + lane < len ? expf(s0 - m) : 0.0f) + (a_c * kChunk + lane + 64 < len ? expf(s1 - m) : 0.0f);
+                    sum = wave_sum(sum);
+                    if (lane == 0) {
+                        st_f(&p.stats[(a_h * GROUP + wave) * 32 + a_c].x, m);
+                        st_f(&p.stats[(a_h * GROUP + wave) * 32 + a_c].y, sum);
+                    }
+                }
+            }
+            stamp();
+            bar.arrive();
+        }
+
+        // ================= phase 3: row statistics, uint8 probabilities, partial P.V =================
+        {
+            i32x4 vreg = {0, 0, 0, 0};
+            const int blk = t >> 8, d = (t >> 2) & 63, part = t & 3;
+            const int bpos = a_c * kChunk + blk * kVBlock;
+            if (a_active && bpos < p.max_pos)
+                vreg = *reinterpret_cast<const i32x4*>(vc + v_index(a_h, bpos, d, p.max_pos) + part * 16);
+            bar.wait();
+            stamp();
+            if (a_active) {
+                const int nchunks = (len + kChunk - 1) / kChunk;
+                if (wave < GROUP) {
+                    float m_c = -1e32f, l_c = 0.0f;
+                    if (lane < nchunks) {
+                        m_c = ld_f(&p.stats[(a_h * GROUP + wave) * 32 + lane].x);
+                        l_c = ld_f(&p.stats[(a_h * GROUP + wave) * 32 + lane].y);
+                    }
+                    const float mx = wave_max(m_c);
+                    const float sum = wave_sum(lane < nchunks ? l_c * expf(m_c - mx) : 0.0f);
+                    if (lane == 0) { L.rowmax[wave] = mx; L.rowcd[wave] = 1.0f / sum; }
+                }
+                __syncthreads();
+                {
+                    const int g = t >> 7, key = t & 127;
+                    const float pr = expf(L.sc[g][key] - L.rowmax[g]) * L.rowcd[g];
+                    int p8 = (int)roundf(pr / (1.0f * a_s[a_h * GROUP + g]));
+                    p8 = p8 > 255 ? 255 : p8;
+                    if (a_c * kChunk + key >= len) p8 = 0;
+                    L.pb[g][key] = (uint8_t)(p8 ^ 0x80);
+                }
+                // the new token's V row is not in the cache yet: patch it into the prefetched registers
+                if (pos >= bpos + part * 16 && pos < bpos + part * 16 + 16) {
+                    const int byte = pos & 15;
+                    int wsel = vreg[byte >> 2];
+                    const int sh = (byte & 3) * 8;
+                    wsel = (wsel & ~(0xff << sh)) | (((int)(uint8_t)L.vnew[d]) << sh);
+                    vreg[byte >> 2] = wsel;
+                }
+                __syncthreads();
+                const i32x4 ones = {0x01010101, 0x01010101, 0x01010101, 0x01010101};
+                int vsum = dot16(ones, vreg, 0);
+                int tot[GROUP];
+#pragma unroll
+                for (int g = 0; g < GROUP; g++) {
+                    int acc = dot16(reinterpret_cast<const i32x4*>(L.pb[g])[blk * 4 + part], vreg, 0) + 128 * vsum;
+                    acc += lane_xor_i<1>(acc);
+                    acc += lane_xor_i<2>(acc);
+                    tot[g] = acc;
+                }
+                if (blk == 1 && part == 0) {
+#pragma unroll
+                    for (int g = 0; g < GROUP; g++) L.osum[g][d] = tot[g];
+                }
+                __syncthreads();
+                if (blk == 0 && part == 0) {
+#pragma unroll
+                    for (int g = 0; g < GROUP; g++)
+                        __hip_atomic_fetch_add(&p.o_acc[(a_h * GROUP + g) * kHd + d], tot[g] + L.osum[g][d], __ATOMIC_RELAXED,
+                                               __HIP_MEMORY_SCOPE_AGENT);
+                }
+            }
+            stamp();
+            bar.arrive();
+        }
+
+        // ================= phase 4: attention dequant + quant -> o_proj rows (8 per workgroup) + residual =================
+        {
+            i32x4 wr[2];
+            const int row = wg * 8 + wave;
+            mega_load_rows<2>(w.wo, H, row, lane, wr);
+            bar.wait();
+            stamp();
+            float v[4];
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                const int idx = 4 * t + i, qh = idx / kHd;
+                v[i] = (float)ld_i(&p.o_acc[idx]) * a_s[qh] * v_s[qh / GROUP];
+            }
+            const float sx = norm_quant_2048(v, nullptr, false, p.eps, L);
+            const int a0 = mega_dot_row<2>(wr, L.xq, lane);
+            if (lane == 0) {
+                float xr;
+                if (l == 0) xr = p.x_in ? p.x_in[row] : __half2float(p.embed[(size_t)tok * H + row]);
+                else xr = ld_f(&p.x[row]);
+                st_f(&p.x2[row], (float)a0 * sx * w.so[row] + xr);
+            }
+            stamp();
+            bar.arrive();
+        }
+
+        // ================= phase 5: RMSNorm + quant -> gate/up rows (64 per workgroup) + SiLU*up =================
+        {
+            i32x4 wr[8][2];
+            const int row0 = wg * 64 + wave * 8;
+#pragma unroll
+            for (int r = 0; r < 8; r++) mega_load_rows<2>(w.wgu, H, row0 + r, lane, wr[r]);
+            bar.wait();
+            stamp();
+            if (t < 8) st_i(&p.o_acc[wg * 8 + t], 0);                // every reader of o_acc has passed the barrier
+            float v[4];
+#pragma unroll
+            for (int i = 0; i < 4; i++) v[i] = ld_f(&p.x2[4 * t + i]);
+            const float sx = norm_quant_2048(v, g1, true, p.eps, L);
+#pragma unroll
+            for (int r = 0; r < 8; r += 2) {
+                const int ag = mega_dot_row<2>(wr[r], L.xq, lane);
+                const int au = mega_dot_row<2>(wr[r + 1], L.xq, lane);
+                if (lane == 0) {
+                    const float gate = (float)ag * sx * w.sgu[row0 + r];
+                    const float up = (float)au * sx * w.sgu[row0 + r + 1];
+                    st_f(&p.h[(row0 + r) >> 1], up * silu_f(gate));
+                }
+            }
+            stamp();
+            bar.arrive();
+        }
+
+        // ================= phase 6: Hadamard R4 + quant -> down rows (8 per workgroup) + residual =================
+        {
+            i32x4 wr[8];
+            const int row = wg * 8 + wave;
+            mega_load_rows<8>(w.wd, I, row, lane, wr);
+            bar.wait();
+            stamp();
+            // 8192-point transform on all 512 threads, stage order bits 1,2,...,12,0 (bit-exact order, see
+            // fht_kernels.h).  A: i = j*2048 + t*4 + e   -> stage 1 in registers, 2..7 across lanes
+            //                  B: i = (t>>8)*4096 + r*256 + (t&255) -> stages 8..11 in registers
+            //                  C: i = r*512 + t          -> stage 12 in registers, stage 0 across lanes
+            float4 a[4];
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                const float* src = p.h + j * 2048 + t * 4;
+                a[j] = make_float4(ld_f(src), ld_f(src + 1), ld_f(src + 2), ld_f(src + 3));
+            }
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                const float u0 = a[j].x, v0 = a[j].z, u1 = a[j].y, v1 = a[j].w;
+                a[j].x = u0 + v0; a[j].z = u0 - v0; a[j].y = u1 + v1; a[j].w = u1 - v1;
+            }
+#define FX_MEGA_STAGE(MASK)                                                                   \
+    {                                                                                         \
+        const bool hi = (lane & MASK) != 0;                                                   \
+        _Pragma("unroll") for (int j = 0; j < 4; j++) {                                       \
+            float px = lane_xor_f<MASK>(a[j].x); a[j].x = hi ? (px - a[j].x) : (a[j].x + px); \
+            float py = lane_xor_f<MASK>(a[j].y); a[j].y = hi ? (py - a[j].y) : (a[j].y + py); \
+            float pz = lane_xor_f<MASK>(a[j].z); a[j].z = hi ? (pz - a[j].z) : (a[j].z + pz); \
+            float pw = lane_xor_f<MASK>(a[j].w); a[j].w = hi ? (pw - a[j].w) : (a[j].w + pw); \
+        }                                                                                     \
+    }
+            FX_MEGA_STAGE(1) FX_MEGA_STAGE(2) FX_MEGA_STAGE(4) FX_MEGA_STAGE(8) FX_MEGA_STAGE(16) FX_MEGA_STAGE(32)
+#undef FX_MEGA_STAGE
+#pragma unroll
+            for (int j = 0; j < 4; j++) reinterpret_cast<float4*>(L.f)[j * 512 + t] = a[j];
+            __syncthreads();
+            float b[16];
+            const int bbase = (t >> 8) * 4096 + (t & 255);
+#pragma unroll
+            for (int r = 0; r < 16; r++) b[r] = L.f[bbase + r * 256];
+#pragma unroll
+            for (int bit = 1; bit < 16; bit <<= 1)
+#pragma unroll
+                for (int r = 0; r < 16; r++)
+                    if ((r & bit) == 0) { const float u = b[r], v = b[r | bit]; b[r] = u + v; b[r | bit] = u - v; }
+            // each thread re-writes exactly the slots it read, so no barrier is needed before this store
+#pragma unroll
+            for (int r = 0; r < 16; r++) L.f[bbase + r * 256] = b[r];
+            __syncthreads();
+#pragma unroll
+            for (int r = 0; r < 16; r++) b[r] = L.f[r * 512 + t];
+#pragma unroll
+            for (int r = 0; r < 8; r++) { const float u = b[r], v = b[r + 8]; b[r] = u + v; b[r + 8] = u - v; }   // bit 12
+            float amax = 0.0f;
+            {
+                const bool hi = (lane & 1) != 0;                                                                      // bit 0
+#pragma unroll
+                for (int r = 0; r < 16; r++) {
+                    const float px = lane_xor_f<1>(b[r]);
+                    b[r] = (hi ? (px - b[r]) : (b[r] + px)) / p.fht_scale;
+                    amax = fmaxf(amax, fabsf(b[r]));
+                }
+            }
+            amax = block_max<kMegaWaves>(amax, L.red);
+            const float sx = sym_scale(amax, 127.0f);
+#pragma unroll
+            for (int r = 0; r < 16; r++) L.xq[r * 512 + t] = (int8_t)quant_round(b[r], sx);
+            __syncthreads();
+            const int a0 = mega_dot_row<8>(wr, L.xq, lane);
+            if (lane == 0) st_f(&p.x[row], (float)a0 * sx * w.sd[row] + ld_f(&p.x2[row]));
+            stamp();
+            bar.arrive();
+        }
+    }
+
+    // ================= head: final RMSNorm -> lm_head rows, per-workgroup argmax candidate =================
+    if (p.want_head) {
+        using h16x8 = _Float16 __attribute__((ext_vector_type(8)));
+        const int rows_per_wg = (p.vocab + kMegaWG - 1) / kMegaWG;
+        const int row_begin = wg * rows_per_wg, row_end = min(p.vocab, row_begin + rows_per_wg);
+        const h16x8* table = reinterpret_cast<const h16x8*>(p.embed);
+        constexpr int U = 4;
+        h16x8 wv[U][4];
+        auto load_group = [&](int r) {
+#pragma unroll
+            for (int u = 0; u < U; u++) {
+                const int row = min(r + u * kMegaWaves, p.vocab - 1);
+#pragma unroll
+                for (int i = 0; i < 4; i++) wv[u][i] = __builtin_nontemporal_load(table + (size_t)row * (H / 8) + lane + 64 * i);
+            }
+        };
+        int r = row_begin + wave;
+        load_group(r);
+        bar.wait();
+        stamp();
+        float v[4];
+#pragma unroll
+        for (int i = 0; i < 4; i++) v[i] = ld_f(&p.x[4 * t + i]);
+        float ss = (v[0] * v[0] + v[1] * v[1]) + (v[2] * v[2] + v[3] * v[3]);
+        ss = block_sum<kMegaWaves>(ss, L.red);
+        const float rms = 1.0f / sqrtf(ss / 2048.0f + p.eps);
+        const float4 g = reinterpret_cast<const float4*>(p.gamma + (size_t)(2 * p.n_layers) * H)[t];
+        reinterpret_cast<float4*>(L.f)[t] = make_float4(v[0] * rms * g.x, v[1] * rms * g.y, v[2] * rms * g.z, v[3] * rms * g.w);
+        __syncthreads();
+        float nv[4][8];
+#pragma unroll
+        for (int i = 0; i < 4; i++)
+#pragma unroll
+            for (int e = 0; e < 8; e++) nv[i][e] = L.f[(lane + 64 * i) * 8 + e];
+        float best = -INFINITY;
+        int bi = 0x7fffffff;
+        for (; r < row_end; r += U * kMegaWaves) {
+            float acc[U];
+#pragma unroll
+            for (int u = 0; u < U; u++) {
+                acc[u] = 0.0f;
+#pragma unroll
+                for (int i = 0; i < 4; i++)
+#pragma unroll
+                    for (int e = 0; e < 8; e++) acc[u] += (float)wv[u][i][e] * nv[i][e];
+            }
+            const int rn = r + U * kMegaWaves;
+            if (rn < row_end) load_group(rn);
+#pragma unroll
+            for (int u = 0; u < U; u++) {
+                const float s = wave_sum(acc[u]);
+                const int row = r + u * kMegaWaves;
+                if (row < row_end) {
+                    if (lane == 0) p.logits[row] = s;
+                    if (s > best || (s == best && row < bi)) { best = s; bi = row; }
+                }
+            }
+        }
+        if (lane == 0) { L.bestv[wave] = best; L.besti[wave] = bi; }
+        __syncthreads();
+        if (t == 0) {
+            for (int i = 1; i < kMegaWaves; i++)
+                if (L.bestv[i] > best || (L.bestv[i] == best && L.besti[i] < bi)) { best = L.bestv[i]; bi = L.besti[i]; }
+            p.am_v[wg] = best;
+            p.am_i[wg] = bi;
+        }
+        stamp();
+    } else {
+        bar.wait();   // keep arrive/wait balanced: the last layer's x is complete when the kernel ends
+    }
+    if (wg == 0 && t == 0) p.state[2] = (int)bar.epoch;
+}
+
+}  // namespace fx

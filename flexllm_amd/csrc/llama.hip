@@ -10,6 +10,7 @@
 #include "fht_kernels.h"
 #include "gemv_i8.h"
 #include "logits_kernels.h"
+#include "decode_mega.h"
 #include "prefill.h"
 #include <vector>
 
@@ -38,6 +39,11 @@ struct flexllm_llama {
     hipStream_t graph_stream = nullptr;
     std::vector<void*> owned;
     fx::PrefillWorkspace pws;
+    fx::LayerW* layers_dev = nullptr;   // device copy of `layers` for the persistent kernel
+    unsigned* bar = nullptr;            // grid-barrier counters of the persistent kernel
+    bool mega_ok = false;               // shapes match the persistent kernel's compile-time constants
+    int decode_mode = 0;                // 0: persistent kernel when possible, 1: one kernel per stage
+    long long* timeline = nullptr;      // stage stamps of the persistent kernel (debug aid)
 };
 
 namespace fx {
@@ -156,9 +162,37 @@ static int decode_head(flexllm_llama* m, float* logits, hipStream_t st) {
     return lm_head_launch(m->embed, m->nrm, logits, c.vocab, c.hidden, st);
 }
 
+static int launch_mega(flexllm_llama* m, const int* token, const float* x_in, float* logits, int want_head, hipStream_t st) {
+    const flexllm_llama_config& c = m->cfg;
+    MegaParams p;
+    p.layers = m->layers_dev;
+    p.gamma = m->gamma; p.q_s = m->q_s; p.k_s = m->k_s; p.v_s = m->v_s; p.a_s = m->a_s;
+    p.rope_sin = m->rope_sin; p.rope_cos = m->rope_cos;
+    p.embed = reinterpret_cast<const __half*>(m->embed);
+    p.k_cache = m->k_cache; p.v_cache = m->v_cache; p.cache_layer_bytes = m->cache_layer_bytes;
+    p.x = m->x; p.x2 = m->x2; p.qkv = m->qkv; p.h = m->h; p.logits = logits ? logits : m->logits;
+    p.stats = m->stats; p.o_acc = m->o_acc; p.state = m->state; p.bar = m->bar;
+    p.token = token; p.x_in = x_in; p.am_v = m->am_v; p.am_i = m->am_i;
+    p.n_layers = c.layers; p.max_pos = c.max_pos; p.vocab = c.vocab; p.want_head = want_head;
+    p.eps = c.eps; p.fht_scale = c.fht_scale;
+    p.timeline = m->timeline;
+    decode_mega_kernel<<<kMegaWG, kMegaT, 0, st>>>(p);
+    FX_LAUNCH_CHECK();
+    return FLEXLLM_OK;
+}
+
+static inline bool use_mega(const flexllm_llama* m) { return m->mega_ok && m->decode_mode == 0; }
+
 // One greedy step: embedding of *token_io -> layers -> head -> argmax -> *token_io, tokens_out[step], pos++.
 static int greedy_step(flexllm_llama* m, int* token_io, int* tokens_out, hipStream_t st) {
     const flexllm_llama_config& c = m->cfg;
+    if (use_mega(m)) {
+        int rc = launch_mega(m, token_io, nullptr, nullptr, 1, st);
+        if (rc) return rc;
+        argmax_final_advance_kernel<<<1, 64, 0, st>>>(m->am_v, m->am_i, kMegaWG, token_io, tokens_out, m->state);
+        FX_LAUNCH_CHECK();
+        return FLEXLLM_OK;
+    }
     embed_kernel<<<(c.hidden + 255) / 256, 256, 0, st>>>(reinterpret_cast<const __half*>(m->embed), token_io, m->x, c.hidden);
     int rc;
     for (int l = 0; l < c.layers; l++)
@@ -265,6 +299,20 @@ int flexllm_llama_create(flexllm_llama** out, const flexllm_llama_config* cfg, c
     FX_TRY(dev_alloc(m, (void**)&m->state, sizeof(int) * 4));
     FX_TRY(dev_alloc(m, (void**)&m->am_v, sizeof(float) * kArgmaxParts));
     FX_TRY(dev_alloc(m, (void**)&m->am_i, sizeof(int) * kArgmaxParts));
+    FX_TRY(dev_alloc(m, (void**)&m->layers_dev, sizeof(LayerW) * L));
+    FX_TRY_HIP(hipMemcpy(m->layers_dev, m->layers.data(), sizeof(LayerW) * L, hipMemcpyHostToDevice));
+    FX_TRY(dev_alloc(m, (void**)&m->bar, sizeof(unsigned) * 64 * (2 + kMegaWG / kMegaGroup)));
+    FX_TRY_HIP(hipMemset(m->bar, 0, sizeof(unsigned) * 64 * (2 + kMegaWG / kMegaGroup)));
+    FX_TRY_HIP(hipMemset(m->state, 0, sizeof(int) * 4));
+    FX_TRY_HIP(hipMemset(m->o_acc, 0, sizeof(int32_t) * H));
+    {
+        int dev = 0, cus = 0;
+        FX_TRY_HIP(hipGetDevice(&dev));
+        FX_TRY_HIP(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev));
+        // the persistent kernel needs all its workgroups resident at once and is compiled for these shapes
+        m->mega_ok = cus >= kMegaWG && c.hidden == 2048 && c.kv_hidden == 512 && c.inter == 8192 && c.q_heads == 32 &&
+                     c.kv_heads == 8 && c.max_pos <= 32 * kChunk && kArgmaxParts >= kMegaWG;
+    }
     FX_TRY_HIP(hipDeviceSynchronize());
 #undef FX_TRY
 #undef FX_TRY_HIP
@@ -282,6 +330,42 @@ int flexllm_llama_destroy(flexllm_llama* m) {
     return FLEXLLM_OK;
 }
 
+int flexllm_llama_set_decode_mode(flexllm_llama* m, int mode) {
+    FX_REQUIRE(m && (mode == 0 || mode == 1), "llama_set_decode_mode: mode=%d (0 persistent kernel, 1 one kernel per stage)", mode);
+    if (m->decode_mode != mode && m->graph_exec) { (void)hipGraphExecDestroy(m->graph_exec); m->graph_exec = nullptr; }
+    m->decode_mode = mode;
+    return FLEXLLM_OK;
+}
+
+int flexllm_llama_stage_timeline(flexllm_llama* m, long long* host_out, int max_entries) {
+    FX_REQUIRE(m && host_out && max_entries > 0, "llama_stage_timeline: bad arguments");
+    const int n = m->cfg.layers * 12 + 2;
+    if (!m->timeline) {
+        int rc = dev_alloc(m, (void**)&m->timeline, sizeof(long long) * n);
+        if (rc) return rc;
+        FX_HIP(hipMemset(m->timeline, 0, sizeof(long long) * n));
+        if (m->graph_exec) { (void)hipGraphExecDestroy(m->graph_exec); m->graph_exec = nullptr; }
+        for (int i = 0; i < max_entries; i++) host_out[i] = 0;
+        return FLEXLLM_OK;
+    }
+    FX_HIP(hipDeviceSynchronize());
+    FX_HIP(hipMemcpy(host_out, m->timeline, sizeof(long long) * (n < max_entries ? n : max_entries), hipMemcpyDeviceToHost));
+    return FLEXLLM_OK;
+}
+
+int flexllm_llama_check(flexllm_llama* m) {
+    FX_REQUIRE(m, "llama_check: null pointer");
+    FX_HIP(hipDeviceSynchronize());
+    int st[4] = {0, 0, 0, 0};
+    FX_HIP(hipMemcpy(st, m->state, sizeof(st), hipMemcpyDeviceToHost));
+    if (st[3] != 0) {
+        (void)hipMemset(&m->state[3], 0, sizeof(int));
+        set_error("persistent decode kernel: a grid barrier timed out (were all %d workgroups resident?)", kMegaWG);
+        return FLEXLLM_EHIP;
+    }
+    return FLEXLLM_OK;
+}
+
 int flexllm_llama_kv_cache(flexllm_llama* m, int8_t** k_cache, int8_t** v_cache) {
     FX_REQUIRE(m && k_cache && v_cache, "llama_kv_cache: null pointer");
     *k_cache = m->k_cache;
@@ -296,6 +380,12 @@ int flexllm_llama_decode_hidden(flexllm_llama* m, const float* x_in, int pos, fl
     hipStream_t st = as_stream(stream);
     const int H = m->cfg.hidden;
     set_state_kernel<<<1, 1, 0, st>>>(m->state, pos, 0);
+    if (use_mega(m)) {
+        int rc = launch_mega(m, nullptr, x_in, logits, logits != nullptr, st);
+        if (rc) return rc;
+        if (hidden_out) FX_HIP(hipMemcpyAsync(hidden_out, m->x, sizeof(float) * H, hipMemcpyDeviceToDevice, st));
+        return FLEXLLM_OK;
+    }
     FX_HIP(hipMemcpyAsync(m->x, x_in, sizeof(float) * H, hipMemcpyDeviceToDevice, st));
     for (int l = 0; l < m->cfg.layers; l++) {
         int rc = decode_layer(m, l, st);

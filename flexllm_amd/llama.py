@@ -97,6 +97,14 @@ class Llama:
         check(lib().flexllm_llama_decode_greedy(self.handle, C.c_void_p(token_io.ptr), int(pos0), int(steps),
                                                 C.c_void_p(tokens_out.ptr), int(use_graph), _s(stream)))
 
+    def set_decode_mode(self, mode):
+        """0: persistent one-kernel-per-token schedule (default), 1: one kernel per stage."""
+        check(lib().flexllm_llama_set_decode_mode(self.handle, int(mode)))
+
+    def check(self):
+        """Synchronise and raise if the persistent decode kernel reported a barrier time-out."""
+        check(lib().flexllm_llama_check(self.handle))
+
     def prefill_hidden(self, x_in, stream=None):
         s = x_in.shape[0]
         hidden = DeviceArray((s, self.cfg["hidden"]), np.float32)

@@ -227,6 +227,16 @@ typedef struct flexllm_llama flexllm_llama;
  * allocates the int8 KV cache [layers][max_pos][kv_hidden] x2 and the activation workspace. */
 int flexllm_llama_create(flexllm_llama** out, const flexllm_llama_config* cfg, const flexllm_llama_weights* w);
 int flexllm_llama_destroy(flexllm_llama* m);
+/* Decode schedule: 0 (default) = one persistent kernel per token (all layers + lm_head, grid barriers between
+ * stages, next stage's weights prefetched across the barrier) when the device has >= 256 CUs and the shapes are
+ * Llama-3.2-1B's with max_pos <= 4096; 1 = one kernel per stage.  Same arithmetic either way. */
+int flexllm_llama_set_decode_mode(flexllm_llama* m, int mode);
+/* Debug aid: the first call switches stage stamping on; later calls copy out workgroup 0's 100 MHz wall-clock
+ * stamps of the last persistent decode step: per layer 6 x (stage start after the barrier, stage end before the
+ * next arrive), then the head's start and end. */
+int flexllm_llama_stage_timeline(flexllm_llama* m, long long* host_out, int max_entries);
+/* Synchronises the device and reports a failed run of the persistent kernel (a grid barrier that timed out). */
+int flexllm_llama_check(flexllm_llama* m);
 /* Device pointers to the int8 caches ([layers][max_pos][kv_hidden]) for inspection / pre-filling. */
 int flexllm_llama_kv_cache(flexllm_llama* m, int8_t** k_cache, int8_t** v_cache);
 /* One decode step at position pos from fp32 embedding x_in (device, [hidden]); writes the residual

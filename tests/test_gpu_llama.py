@@ -6,8 +6,8 @@ import pytest
 pytestmark = pytest.mark.gpu
 
 
-@pytest.fixture(scope="module")
-def small():
+@pytest.fixture(scope="module", params=[0, 1], ids=["persistent", "per_stage"])
+def small(request):
     import flexllm_amd as fx
     from flexllm_amd import llama
     from oracle import oracle
@@ -19,8 +19,10 @@ def small():
     assert np.array_equal(dev_w["sg"][0].numpy(), host_w["sg"][0])
     assert np.array_equal(dev_w["embed"].numpy().view(np.uint16), host_w["embed"])
     model = llama.Llama(cfg, dev_w)
+    model.set_decode_mode(request.param)
     om = oracle.OracleModel(cfg, host_w)
     yield fx, cfg, model, om, host_w
+    model.check()
     model.close()
 
 
@@ -46,6 +48,7 @@ def test_decode_tokens_match_oracle(small):
         assert np.abs(h - hid_ref).max() <= 2e-3 * np.abs(hid_ref).max()
         lg = logits.numpy()
         assert np.abs(lg - logits_ref).max() <= 2e-3 * np.abs(logits_ref).max()
+    model.check()
     k_gpu, v_gpu = model.caches_token_major()
     close_int8(k_gpu[:, :6], kc[:, :6], "k cache")
     close_int8(v_gpu[:, :6], vc[:, :6], "v cache")
@@ -94,4 +97,5 @@ def test_greedy_loop_graph_replay_equals_eager_and_oracle(small):
         _, logits = om.decode_token(x, pos, kc, vc)
         t = int(np.argmax(logits))
         ref.append(t)
+    model.check()
     assert outs[0].tolist() == ref
