@@ -14,7 +14,7 @@ FLAGS = [
     # the reference's arithmetic has no fused multiply-add: keep mul and add separate
     "-ffp-contract=off",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
-    "-Wall", "-Wno-unused-function",
+    "-Wall", "-Wno-unused-function", *os.environ.get("FLEXLLM_EXTRA_FLAGS", "").split(),
 ]
 
 

@@ -157,6 +157,12 @@ __global__ __launch_bounds__(kMegaT, 1) void decode_mega_kernel(MegaParams p) {
     GridBarrier bar{p.bar, (unsigned)p.state[2], &p.state[3]};
     int stamp_i = 0;
     auto stamp = [&]() { if (p.timeline && wg == 0 && t == 0) p.timeline[stamp_i] = wall_clock64(); stamp_i++; };
+#ifdef FX_MEGA_FINE_STAMPS
+    int fine_i = 0;
+    auto fine = [&]() { if (p.timeline && wg == 0 && t == 0 && fine_i < 64) p.timeline[p.n_layers * 12 + 2 + fine_i] = wall_clock64(); fine_i++; };
+#else
+    auto fine = [&]() {};
+#endif
     const int tok = p.x_in ? 0 : p.token[0];
 
     // attention work item of this workgroup
@@ -415,11 +421,14 @@ __global__ __launch_bounds__(kMegaT, 1) void decode_mega_kernel(MegaParams p) {
             float pw = lane_xor_f<MASK>(a[j].w); a[j].w = hi ? (pw - a[j].w) : (a[j].w + pw); \
         }                                                                                     \
     }
+            if (l == 1) fine();
             FX_MEGA_STAGE(1) FX_MEGA_STAGE(2) FX_MEGA_STAGE(4) FX_MEGA_STAGE(8) FX_MEGA_STAGE(16) FX_MEGA_STAGE(32)
 #undef FX_MEGA_STAGE
+            if (l == 1) fine();
 #pragma unroll
             for (int j = 0; j < 4; j++) reinterpret_cast<float4*>(L.f)[j * 512 + t] = a[j];
             __syncthreads();
+            if (l == 1) fine();
             float b[16];
             const int bbase = (t >> 8) * 4096 + (t & 255);
 #pragma unroll
@@ -437,6 +446,7 @@ __global__ __launch_bounds__(kMegaT, 1) void decode_mega_kernel(MegaParams p) {
             for (int r = 0; r < 16; r++) b[r] = L.f[r * 512 + t];
 #pragma unroll
             for (int r = 0; r < 8; r++) { const float u = b[r], v = b[r + 8]; b[r] = u + v; b[r + 8] = u - v; }   // bit 12
+            if (l == 1) fine();
             float amax = 0.0f;
             {
                 const bool hi = (lane & 1) != 0;                                                                      // bit 0
@@ -447,13 +457,18 @@ __global__ __launch_bounds__(kMegaT, 1) void decode_mega_kernel(MegaParams p) {
                     amax = fmaxf(amax, fabsf(b[r]));
                 }
             }
+            if (l == 1) fine();
             amax = block_max<kMegaWaves>(amax, L.red);
             const float sx = sym_scale(amax, 127.0f);
+            if (l == 1) fine();
 #pragma unroll
             for (int r = 0; r < 16; r++) L.xq[r * 512 + t] = (int8_t)quant_round(b[r], sx);
             __syncthreads();
+            if (l == 1) fine();
             const int a0 = mega_dot_row<8>(wr, L.xq, lane);
+            if (l == 1) fine();
             if (lane == 0) st_f(&p.x[row], (float)a0 * sx * w.sd[row] + ld_f(&p.x2[row]));
+            if (l == 1) fine();
             stamp();
             bar.arrive();
         }
