@@ -1,6 +1,7 @@
 // Causal int8 prefill attention (GQA) on MFMA, reading K and V from the layer's int8 cache.
 //
-// One wave owns 32 consecutive queries of one head and walks the key tiles (32 keys) up to its diagonal.
+// A workgroup owns 32 consecutive queries of one head; its four waves split the key tiles (32 keys) up to the
+// diagonal.
 // The score tile is computed TRANSPOSED, S^T = K_tile . Q_tile^T, so that in the 32x32 accumulator layout a
 // lane holds 16 scores of ONE query (column l%32; keys 8a+4g+b for register 4a+b, g = l/32).  That is also
 // the A-operand shape of the second matrix product P.V (row = query l%32, 16 k-values for k-group g), so the
@@ -26,17 +27,21 @@ __device__ __forceinline__ i32x16 zero16() {
     return z;
 }
 
-// grid (ceil(s/128), q_heads), 256 threads: wave w handles queries [(4*blockIdx.x + w)*32, +32)
+// grid (s/32, q_heads), 256 threads: the four waves of a workgroup share one block of 32 queries and split
+// its key tiles round-robin (tile kt goes to wave kt%4).  Row statistics are merged through LDS after pass 1;
+// the int32 P.V partial accumulators of the four waves are added in LDS after pass 2 (integer adds: exact).
+// Long query blocks are scheduled first.
 static __global__ __launch_bounds__(256) void pf_attention_kernel(const int8_t* __restrict__ q8, const int8_t* __restrict__ kc,
                                                                   const int8_t* __restrict__ vc, const float* __restrict__ q_s,
                                                                   const float* __restrict__ k_s, const float* __restrict__ v_s,
                                                                   const float* __restrict__ a_s, float* __restrict__ o,
                                                                   uint8_t* __restrict__ p8_out, int s, int q_heads, int group,
                                                                   int max_pos) {
+    __shared__ float lds_m[4][32], lds_l[4][32];
+    __shared__ int lds_acc[64][35];            // [lane][16 acc0 | 16 acc1 | vsum0 | vsum1], odd pitch against bank conflicts
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int qb = blockIdx.x * 4 + wave;
+    const int qb = (int)gridDim.x - 1 - (int)blockIdx.x;
     const int q0 = qb * kPfTile;
-    if (q0 >= s) return;
     const int h = blockIdx.y, kvh = h / group;
     const int col = lane & 31, g = lane >> 5;
     const int query = q0 + col;
@@ -47,10 +52,12 @@ static __global__ __launch_bounds__(256) void pf_attention_kernel(const int8_t* 
     const i32x4 qf0 = *reinterpret_cast<const i32x4*>(qrow + g * 16);
     const i32x4 qf1 = *reinterpret_cast<const i32x4*>(qrow + 32 + g * 16);
 
-    auto score_tile = [&](int k0, float (&sc)[16]) {
+    auto load_k = [&](int k0, i32x4& kf0, i32x4& kf1) {
         const int8_t* krow = kc + k_index(kvh, k0 + col, max_pos);
-        const i32x4 kf0 = *reinterpret_cast<const i32x4*>(krow + g * 16);
-        const i32x4 kf1 = *reinterpret_cast<const i32x4*>(krow + 32 + g * 16);
+        kf0 = *reinterpret_cast<const i32x4*>(krow + g * 16);
+        kf1 = *reinterpret_cast<const i32x4*>(krow + 32 + g * 16);
+    };
+    auto score_tile = [&](int k0, const i32x4& kf0, const i32x4& kf1, float (&sc)[16]) {
         i32x16 acc = zero16();
         acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(kf0, qf0, acc, 0, 0, 0);
         acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(kf1, qf1, acc, 0, 0, 0);
@@ -63,80 +70,118 @@ static __global__ __launch_bounds__(256) void pf_attention_kernel(const int8_t* 
     };
 
     const int ntiles = qb + 1;
-    // ---- pass 1: row max and row sum of exponentials ----
+    for (int i = threadIdx.x; i < 64 * 35; i += 256) (&lds_acc[0][0])[i] = 0;
+    // ---- pass 1: row max and row sum of exponentials over this wave's tiles ----
     float m_run = -1e32f, l_run = 0.0f;
-    for (int kt = 0; kt < ntiles; kt++) {
-        float sc[16];
-        score_tile(kt * kPfTile, sc);
-        float mt = sc[0];
+    {
+        i32x4 kf0, kf1, nf0, nf1;
+        if (wave < ntiles) load_k(wave * kPfTile, kf0, kf1);
+        for (int kt = wave; kt < ntiles; kt += 4) {
+            if (kt + 4 < ntiles) load_k((kt + 4) * kPfTile, nf0, nf1);
+            float sc[16];
+            score_tile(kt * kPfTile, kf0, kf1, sc);
+            float mt = sc[0];
 #pragma unroll
-        for (int r = 1; r < 16; r++) mt = fmaxf(mt, sc[r]);
-        const float m_new = fmaxf(m_run, mt);
-        float sum = 0.0f;
+            for (int r = 1; r < 16; r++) mt = fmaxf(mt, sc[r]);
+            const float m_new = fmaxf(m_run, mt);
+            float sum = 0.0f;
 #pragma unroll
-        for (int r = 0; r < 16; r++) sum += expf(sc[r] - m_new);
-        l_run = l_run * expf(m_run - m_new) + sum;
-        m_run = m_new;
+            for (int r = 0; r < 16; r++) sum += expf(sc[r] - m_new);
+            l_run = l_run * expf(m_run - m_new) + sum;
+            m_run = m_new;
+            kf0 = nf0; kf1 = nf1;
+        }
     }
-    // merge the two lanes that share a query
-    const float m_o = lane_xor_f<32>(m_run), l_o = lane_xor_f<32>(l_run);
-    const float mx = fmaxf(m_run, m_o);
-    const float total = l_run * expf(m_run - mx) + l_o * expf(m_o - mx);
+    {   // merge the two lanes that share a query, then the four waves
+        const float m_o = lane_xor_f<32>(m_run), l_o = lane_xor_f<32>(l_run);
+        const float mw = fmaxf(m_run, m_o);
+        const float lw = l_run * expf(m_run - mw) + l_o * expf(m_o - mw);
+        if (g == 0) { lds_m[wave][col] = mw; lds_l[wave][col] = lw; }
+    }
+    __syncthreads();
+    float mx = lds_m[0][col];
+#pragma unroll
+    for (int w = 1; w < 4; w++) mx = fmaxf(mx, lds_m[w][col]);
+    float total = 0.0f;
+#pragma unroll
+    for (int w = 0; w < 4; w++) total += lds_l[w][col] * expf(lds_m[w][col] - mx);
     const float cd = 1.0f / total;
 
-    // ---- pass 2: probabilities, P.V ----
+    // ---- pass 2: probabilities, partial P.V over this wave's tiles ----
     i32x16 oacc0 = zero16(), oacc1 = zero16();
     int vsum0 = 0, vsum1 = 0;
-    for (int kt = 0; kt < ntiles; kt++) {
-        const int k0 = kt * kPfTile;
-        float sc[16];
-        score_tile(k0, sc);
-        i32x4 pf;
+    {
+        i32x4 kf0, kf1, nf0, nf1;
+        if (wave < ntiles) load_k(wave * kPfTile, kf0, kf1);
+        for (int kt = wave; kt < ntiles; kt += 4) {
+            const int k0 = kt * kPfTile;
+            if (kt + 4 < ntiles) load_k((kt + 4) * kPfTile, nf0, nf1);
+            // B operand of P.V: V[key][d] for this lane's channel d = col (+32) and the lane's 16 keys, gathered
+            // from the cache's [d][64 pos] blocks; issued before the exponentials so that it is in flight
+            const int8_t* vblk = vc + v_index(kvh, k0, 0, max_pos);
+            i32x4 vf0, vf1;
 #pragma unroll
-        for (int a = 0; a < 4; a++) {
-            uint32_t packed = 0;
-#pragma unroll
-            for (int b = 0; b < 4; b++) {
-                const float p = expf(sc[a * 4 + b] - mx) * cd;
-                int p8 = (int)roundf(p / as);
-                p8 = p8 > 255 ? 255 : p8;
-                if (p8_out) {
-                    const int key = k0 + a * 8 + g * 4 + b;
-                    p8_out[((size_t)h * s + query) * s + key] = (uint8_t)p8;
-                }
-                packed |= (uint32_t)((p8 ^ 0x80) & 0xff) << (8 * b);
+            for (int a = 0; a < 4; a++) {
+                vf0[a] = *reinterpret_cast<const int*>(vblk + (size_t)col * kVBlock + a * 8 + g * 4);
+                vf1[a] = *reinterpret_cast<const int*>(vblk + (size_t)(col + 32) * kVBlock + a * 8 + g * 4);
             }
-            pf[a] = (int)packed;
-        }
-        // B operand: V[key][d] for this lane's channel d = col (+32) and the same 16 keys, from [d][64 pos] blocks
-        const int8_t* vblk = vc + v_index(kvh, k0, 0, max_pos);       // start of (block, d=0) row, at position k0%64
-        i32x4 vf0, vf1;
+            float sc[16];
+            score_tile(k0, kf0, kf1, sc);
+            i32x4 pf;
 #pragma unroll
-        for (int a = 0; a < 4; a++) {
-            vf0[a] = *reinterpret_cast<const int*>(vblk + (size_t)col * kVBlock + a * 8 + g * 4);
-            vf1[a] = *reinterpret_cast<const int*>(vblk + (size_t)(col + 32) * kVBlock + a * 8 + g * 4);
-            vsum0 = __builtin_amdgcn_sdot4(0x01010101, vf0[a], vsum0, false);
-            vsum1 = __builtin_amdgcn_sdot4(0x01010101, vf1[a], vsum1, false);
+            for (int a = 0; a < 4; a++) {
+                uint32_t packed = 0;
+#pragma unroll
+                for (int b = 0; b < 4; b++) {
+                    const float pr = expf(sc[a * 4 + b] - mx) * cd;
+                    int p8 = (int)roundf(pr / as);
+                    p8 = p8 > 255 ? 255 : p8;
+                    if (p8_out) {
+                        const int key = k0 + a * 8 + g * 4 + b;
+                        p8_out[((size_t)h * s + query) * s + key] = (uint8_t)p8;
+                    }
+                    packed |= (uint32_t)((p8 ^ 0x80) & 0xff) << (8 * b);
+                }
+                pf[a] = (int)packed;
+            }
+#pragma unroll
+            for (int a = 0; a < 4; a++) {
+                vsum0 = __builtin_amdgcn_sdot4(0x01010101, vf0[a], vsum0, false);
+                vsum1 = __builtin_amdgcn_sdot4(0x01010101, vf1[a], vsum1, false);
+            }
+            oacc0 = __builtin_amdgcn_mfma_i32_32x32x32_i8(pf, vf0, oacc0, 0, 0, 0);
+            oacc1 = __builtin_amdgcn_mfma_i32_32x32x32_i8(pf, vf1, oacc1, 0, 0, 0);
+            kf0 = nf0; kf1 = nf1;
         }
-        oacc0 = __builtin_amdgcn_mfma_i32_32x32x32_i8(pf, vf0, oacc0, 0, 0, 0);
-        oacc1 = __builtin_amdgcn_mfma_i32_32x32x32_i8(pf, vf1, oacc1, 0, 0, 0);
     }
-    vsum0 += lane_xor_i<32>(vsum0);
-    vsum1 += lane_xor_i<32>(vsum1);
+    // add the four waves' partial accumulators (lds_acc was zeroed before pass 1; two barriers have passed)
+    if (wave < ntiles) {
+#pragma unroll
+        for (int r = 0; r < 16; r++) {
+            atomicAdd(&lds_acc[lane][r], oacc0[r]);
+            atomicAdd(&lds_acc[lane][16 + r], oacc1[r]);
+        }
+        atomicAdd(&lds_acc[lane][32], vsum0);
+        atomicAdd(&lds_acc[lane][33], vsum1);
+    }
+    __syncthreads();
+    const int vs0 = lds_acc[lane][32] + lds_acc[lane ^ 32][32];
+    const int vs1 = lds_acc[lane][33] + lds_acc[lane ^ 32][33];
     const float sv = v_s[kvh], sa = a_s[h];
 #pragma unroll
-    for (int r = 0; r < 16; r++) {
+    for (int rr = 0; rr < 4; rr++) {                          // wave w writes accumulator registers 4w..4w+3
+        const int r = wave * 4 + rr;
         const int row = q0 + (r >> 2) * 8 + g * 4 + (r & 3);
         float* orow = o + ((size_t)row * q_heads + h) * kHd;
-        orow[col] = (float)(oacc0[r] + 128 * vsum0) * sa * sv;
-        orow[col + 32] = (float)(oacc1[r] + 128 * vsum1) * sa * sv;
+        orow[col] = (float)(lds_acc[lane][r] + 128 * vs0) * sa * sv;
+        orow[col + 32] = (float)(lds_acc[lane][16 + r] + 128 * vs1) * sa * sv;
     }
 }
 
 inline int mha_prefill_launch(const int8_t* q8, const int8_t* kc, const int8_t* vc, const float* q_s, const float* k_s,
                               const float* v_s, const float* a_s, float* o, uint8_t* p8_out, int s, int q_heads,
                               int kv_heads, int max_pos, hipStream_t st) {
-    dim3 grid((s + 127) / 128, q_heads);
+    dim3 grid(s / kPfTile, q_heads);
     pf_attention_kernel<<<grid, 256, 0, st>>>(q8, kc, vc, q_s, k_s, v_s, a_s, o, p8_out, s, q_heads, q_heads / kv_heads, max_pos);
     FX_LAUNCH_CHECK();
     return FLEXLLM_OK;
