@@ -54,5 +54,21 @@ def _drain(procs):
             print("\n".join(lines), file=sys.stderr)
 
 
+TB_SRC = os.path.join(HERE, "host", "tb", "modules_tb.cpp")
+TB_BIN = os.path.join(HERE, "host", "tb", "modules_tb")
+
+
+def build_harness():
+    """Compile the C++ testbench-style harness of the host-side module mirror against the built library."""
+    cmd = [HIPCC, "-std=c++17", "-O2", "-x", "c++", TB_SRC, "-o", TB_BIN, "-D__HIP_PLATFORM_AMD__",
+           "-I/opt/rocm/include", "-L" + HERE, "-lflexllm_hip", "-L/opt/rocm/lib", "-lamdhip64",
+           "-Wl,-rpath," + HERE, "-Wl,-rpath,/opt/rocm/lib"]
+    out = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    if out.returncode != 0:
+        raise RuntimeError("harness build failed:\n" + out.stdout)
+    return TB_BIN
+
+
 if __name__ == "__main__":
     print(build(verbose=True))
+    print(build_harness())

@@ -1,0 +1,415 @@
+// Host-side C++ mirror of the reference's Modules/ call surface (same function names, template-parameter order
+// and argument meaning), implemented on top of the C ABI in include/flexllm_hip.h.
+//
+// Each function drains its input stream(s) into a token-major staging buffer (undoing the reference's stream
+// packing: prefill streams carry io_parallel tokens of one feature per vector, Modules/data_io.h:15-19; decode
+// streams carry block_parallel block-partitioned features of one token, Modules/data_io.h:419,437), runs the
+// GPU operator, and writes the result back in the packing the reference's consumer expects.
+//
+// Differences from the reference, all forced by the device boundary:
+//  * Weights do not travel through streams: a linear layer takes a DeviceWeight that was uploaded once from
+//    the row-major int8 [N][K] array (the reference's on-disk format), see DeviceWeight / unpack helpers.
+//  * The int8 instantiation (qint_bit = 8, symmetric) is the W8A8 path; function names keep the reference's
+//    spelling with "i8xi8" where the reference says "i4xi4".
+//  * Errors throw fxhost::Error carrying flexllm_last_error() (the reference prints and returns).
+#pragma once
+#include <hip/hip_runtime_api.h>
+#include <cstdint>
+#include <stdexcept>
+#include <string>
+#include <type_traits>
+#include <vector>
+#include "../../include/flexllm_hip.h"
+#include "stream_types.h"
+
+namespace fxhost {
+
+struct Error : std::runtime_error {
+    using std::runtime_error::runtime_error;
+};
+inline void check(int rc) {
+    if (rc != FLEXLLM_OK) throw Error(std::string("flexllm: ") + flexllm_last_error());
+}
+inline void check_hip(hipError_t e) {
+    if (e != hipSuccess) throw Error(std::string("hip: ") + hipGetErrorString(e));
+}
+
+// RAII device array
+template <class T>
+class DeviceArray {
+public:
+    DeviceArray() = default;
+    explicit DeviceArray(size_t n) { resize(n); }
+    explicit DeviceArray(const std::vector<T>& h) { upload(h); }
+    DeviceArray(const DeviceArray&) = delete;
+    DeviceArray& operator=(const DeviceArray&) = delete;
+    DeviceArray(DeviceArray&& o) noexcept : p_(o.p_), n_(o.n_) { o.p_ = nullptr; o.n_ = 0; }
+    ~DeviceArray() { if (p_) (void)hipFree(p_); }
+    void resize(size_t n) {
+        if (p_) check_hip(hipFree(p_));
+        p_ = nullptr; n_ = n;
+        check_hip(hipMalloc(reinterpret_cast<void**>(&p_), (n ? n : 1) * sizeof(T)));
+    }
+    void upload(const std::vector<T>& h) { upload(h.data(), h.size()); }
+    void upload(const T* h, size_t n) {
+        if (n != n_ || !p_) resize(n);
+        check_hip(hipMemcpy(p_, h, n * sizeof(T), hipMemcpyHostToDevice));
+    }
+    std::vector<T> download() const {
+        std::vector<T> h(n_);
+        check_hip(hipMemcpy(h.data(), p_, n_ * sizeof(T), hipMemcpyDeviceToHost));
+        return h;
+    }
+    T* get() const { return p_; }
+    size_t size() const { return n_; }
+
+private:
+    T* p_ = nullptr;
+    size_t n_ = 0;
+};
+
+// A weight matrix resident in HBM: int8 [out_dim][in_dim] row-major plus optional per-channel scales.
+struct DeviceWeight {
+    DeviceArray<int8_t> w;
+    DeviceArray<float> scale;
+    int out_dim = 0, in_dim = 0;
+    DeviceWeight() = default;
+    DeviceWeight(const int8_t* row_major, int n, int k, const float* s = nullptr) : out_dim(n), in_dim(k) {
+        w.upload(row_major, (size_t)n * k);
+        if (s) scale.upload(s, (size_t)n);
+    }
+};
+
+// ---- stream <-> token-major staging ------------------------------------------------------------------
+template <class T, class IS>
+std::vector<T> drain_pref(IS& in, int seq_len, int dim, int io_parallel) {
+    std::vector<T> x((size_t)seq_len * dim);
+    for (int M = 0; M < seq_len / io_parallel; M++)
+        for (int k = 0; k < dim; k++) {
+            auto pack = in.read();
+            for (int m = 0; m < io_parallel; m++) x[(size_t)(M * io_parallel + m) * dim + k] = (T)pack[m];
+        }
+    return x;
+}
+template <class OS, class T>
+void fill_pref(OS& out, const std::vector<T>& x, int seq_len, int dim, int io_parallel) {
+    using V = typename OS::value_type;
+    using E = typename std::remove_reference<decltype(std::declval<V&>()[0])>::type;
+    for (int M = 0; M < seq_len / io_parallel; M++)
+        for (int k = 0; k < dim; k++) {
+            V pack;
+            for (int m = 0; m < io_parallel; m++) pack[m] = (E)x[(size_t)(M * io_parallel + m) * dim + k];
+            out.write(pack);
+        }
+}
+template <class T, class IS>
+std::vector<T> drain_dec(IS& in, int dim, int block_parallel) {
+    std::vector<T> x(dim);
+    const int per = dim / block_parallel;
+    for (int k = 0; k < per; k++) {
+        auto pack = in.read();
+        for (int i = 0; i < block_parallel; i++) x[(size_t)i * per + k] = (T)pack[i];
+    }
+    return x;
+}
+template <class OS, class T>
+void fill_dec(OS& out, const std::vector<T>& x, int dim, int block_parallel) {
+    using V = typename OS::value_type;
+    using E = typename std::remove_reference<decltype(std::declval<V&>()[0])>::type;
+    const int per = dim / block_parallel;
+    for (int k = 0; k < per; k++) {
+        V pack;
+        for (int i = 0; i < block_parallel; i++) pack[i] = (E)x[(size_t)i * per + k];
+        out.write(pack);
+    }
+}
+
+// ======================================================================================= quant.h
+// Modules/quant.h:6-13
+template <int qint_bit, bool is_act_asym, int io_parallel, int max_input_dim, int max_seq_len = 1024, class IS, class OSB, class OQ>
+void pref_quant_layer_fp32_qint(IS& input_stream, OSB& input_s_b_stream, OQ& output_stream, int seq_len = max_seq_len,
+                                int input_dim = max_input_dim) {
+    static_assert(qint_bit == 8 && !is_act_asym, "the GPU path behind this name is the symmetric int8 instantiation");
+    auto x = drain_pref<float>(input_stream, seq_len, input_dim, io_parallel);
+    DeviceArray<float> dx(x), ds(seq_len);
+    DeviceArray<int8_t> dq((size_t)seq_len * input_dim);
+    check(flexllm_quant_sym_i8(dx.get(), dq.get(), ds.get(), seq_len, input_dim, nullptr));
+    auto s = ds.download();
+    auto q = dq.download();
+    using SV = typename OSB::value_type;
+    for (int t = 0; t < seq_len; t++) { SV p; p[0] = s[t]; input_s_b_stream.write(p); }
+    fill_pref(output_stream, q, seq_len, input_dim, io_parallel);
+}
+// Modules/quant.h:332-338
+template <int qint_bit, bool is_act_asym, int block_parallel, int max_input_dim, class IS, class OSB, class OQ>
+void dec_quant_layer_fp32_qint(IS& input_stream, OSB& input_s_b_stream, OQ& output_stream, int input_dim = max_input_dim) {
+    static_assert(qint_bit == 8 && !is_act_asym, "the GPU path behind this name is the symmetric int8 instantiation");
+    auto x = drain_dec<float>(input_stream, input_dim, block_parallel);
+    DeviceArray<float> dx(x), ds(1);
+    DeviceArray<int8_t> dq(input_dim);
+    check(flexllm_quant_sym_i8(dx.get(), dq.get(), ds.get(), 1, input_dim, nullptr));
+    typename OSB::value_type p;
+    p[0] = ds.download()[0];
+    input_s_b_stream.write(p);
+    fill_dec(output_stream, dq.download(), input_dim, block_parallel);
+}
+// Modules/quant.h:115-123: weight_s_sum_stream carries one {scale} vector per output channel
+template <int qint_bit, bool is_act_asym, int io_parallel, int max_output_dim, int max_seq_len = 1024, class IS, class ISB, class IW, class OS>
+void pref_dequant_layer_qint_fp32(IS& input_stream, ISB& input_s_b_stream, IW& weight_s_sum_stream, OS& output_stream,
+                                  int seq_len = max_seq_len, int output_dim = max_output_dim) {
+    static_assert(!is_act_asym, "symmetric path");
+    // the reference interleaves: per token block, io_parallel scales, then output_dim packs (and the weight
+    // scales once per token block)
+    std::vector<float> s(seq_len), ws(output_dim);
+    std::vector<int32_t> acc((size_t)seq_len * output_dim);
+    for (int M = 0; M < seq_len / io_parallel; M++) {
+        for (int m = 0; m < io_parallel; m++) s[M * io_parallel + m] = input_s_b_stream.read()[0];
+        for (int k = 0; k < output_dim; k++) {
+            auto pack = input_stream.read();
+            ws[k] = weight_s_sum_stream.read()[0];
+            for (int m = 0; m < io_parallel; m++) acc[(size_t)(M * io_parallel + m) * output_dim + k] = (int32_t)pack[m];
+        }
+    }
+    DeviceArray<int32_t> dacc(acc);
+    DeviceArray<float> ds(s), dws(ws), dy((size_t)seq_len * output_dim);
+    check(flexllm_dequant_i32_f32(dacc.get(), ds.get(), nullptr, dws.get(), nullptr, dy.get(), seq_len, output_dim, nullptr));
+    fill_pref(output_stream, dy.download(), seq_len, output_dim, io_parallel);
+}
+// Modules/quant.h:470-477: weight scales arrive in groups of block_parallel*weight_parallel, lane-major
+template <int qint_bit, bool is_act_asym, int block_parallel, int weight_parallel, int max_output_dim, class IS, class ISB, class IW, class OS>
+void dec_dequant_layer_qint_fp32_bandwidth(IS& input_stream, ISB& input_s_b_stream, IW& weight_s_sum_stream, OS& output_stream,
+                                           int output_dim = max_output_dim) {
+    static_assert(!is_act_asym, "symmetric path");
+    const float s = input_s_b_stream.read()[0];
+    const int per = output_dim / block_parallel;
+    std::vector<float> ws(output_dim);
+    std::vector<int32_t> acc(output_dim);
+    for (int k = 0; k < output_dim / (block_parallel * weight_parallel); k++) {
+        // Modules/quant.h:491-501: weight_s[m*weight_parallel+n] belongs to lane m, step n of this group
+        for (int i = 0; i < block_parallel * weight_parallel; i++) {
+            const int lane = i / weight_parallel, n = i % weight_parallel;
+            ws[(size_t)lane * per + k * weight_parallel + n] = weight_s_sum_stream.read()[0];
+        }
+        for (int n = 0; n < weight_parallel; n++) {
+            auto pack = input_stream.read();
+            for (int m = 0; m < block_parallel; m++) acc[(size_t)m * per + k * weight_parallel + n] = (int32_t)pack[m];
+        }
+    }
+    DeviceArray<int32_t> dacc(acc);
+    DeviceArray<float> ds(std::vector<float>{s}), dws(ws), dy(output_dim);
+    check(flexllm_dequant_i32_f32(dacc.get(), ds.get(), nullptr, dws.get(), nullptr, dy.get(), 1, output_dim, nullptr));
+    fill_dec(output_stream, dy.download(), output_dim, block_parallel);
+}
+// Modules/quant.h:252-261 (static per-layer-per-head scale)
+template <int qint_bit, int io_parallel, int max_input_dim, int head_num = 1, int is_signed = true, int max_seq_len = 1024,
+          int decoder_layer_num = 16, class IS, class OS>
+void pref_static_sym_per_tensor_quant_layer_fp32_qint(IS& input_stream, OS& output_stream,
+                                                      const float input_s[decoder_layer_num][head_num], int block_id,
+                                                      int seq_len = max_seq_len, int input_dim = max_input_dim,
+                                                      float mha_scale_factor = 1.0f) {
+    static_assert(qint_bit == 8, "int8 path");
+    auto x = drain_pref<float>(input_stream, seq_len, head_num * input_dim, io_parallel);
+    DeviceArray<float> dx(x), dsc(std::vector<float>(input_s[block_id], input_s[block_id] + head_num));
+    DeviceArray<int8_t> dq(x.size());
+    check(flexllm_static_quant_i8(dx.get(), dq.get(), dsc.get(), mha_scale_factor, is_signed, seq_len, head_num, input_dim, nullptr));
+    auto q = dq.download();
+    if (is_signed) fill_pref(output_stream, q, seq_len, head_num * input_dim, io_parallel);
+    else {
+        std::vector<uint8_t> u(q.begin(), q.end());
+        fill_pref(output_stream, u, seq_len, head_num * input_dim, io_parallel);
+    }
+}
+
+// ======================================================================================= Linear_Layer.h
+// Modules/Linear_Layer.h:293-301 with the weight stream replaced by a resident DeviceWeight
+template <int io_parallel, int weight_parallel, int max_input_dim = 2048, int max_log2_input_dim = 11, int max_output_dim = 2048,
+          int max_seq_len = 1024, bool is_uint_input = false, class IS, class OS>
+void pref_Linear_Layer_i8xi8(IS& input_seq, const DeviceWeight& weight, OS& output_seq, int seq_len = max_seq_len,
+                             int input_dim = max_input_dim, int output_dim = max_output_dim) {
+    static_assert(!is_uint_input, "signed activations");
+    auto a = drain_pref<int8_t>(input_seq, seq_len, input_dim, io_parallel);
+    DeviceArray<int8_t> da(a);
+    DeviceArray<int32_t> dc((size_t)seq_len * output_dim);
+    check(flexllm_linear_i8_gemm(da.get(), weight.w.get(), dc.get(), seq_len, input_dim, output_dim, nullptr));
+    fill_pref(output_seq, dc.download(), seq_len, output_dim, io_parallel);
+}
+// Modules/Linear_Layer.h:862-869; the output is block-partitioned over block_parallel lanes like the input
+template <int block_parallel, int weight_parallel, int max_input_dim = 2048, int max_log2_input_dim = 11, int max_output_dim = 2048,
+          bool is_uint_input = false, class IS, class OS>
+void dec_Linear_Layer_i8xi8(IS& input_seq, const DeviceWeight& weight, OS& output_seq, int input_dim = max_input_dim,
+                            int output_dim = max_output_dim) {
+    static_assert(!is_uint_input, "signed activations");
+    auto x = drain_dec<int8_t>(input_seq, input_dim, block_parallel);
+    DeviceArray<int8_t> dx(x);
+    DeviceArray<int32_t> dc(output_dim);
+    check(flexllm_linear_i8_gemv(dx.get(), weight.w.get(), dc.get(), input_dim, output_dim, nullptr));
+    fill_dec(output_seq, dc.download(), output_dim, block_parallel);
+}
+// Modules/Linear_Layer.h:612-617 / :1103-1108
+template <int io_parallel, int io_hidden_dim, int max_seq_len = 1024, class IA, class IB, class OS>
+void pref_Gate_Layer_fp32xfp32(IA& input_seq, IB& gate_seq, OS& output_seq, int seq_len = max_seq_len) {
+    for (int i = 0; i < seq_len / io_parallel * io_hidden_dim; i++) {
+        auto a = input_seq.read();
+        auto b = gate_seq.read();
+        typename OS::value_type o;
+        for (int m = 0; m < io_parallel; m++) o[m] = a[m] * b[m];
+        output_seq.write(o);
+    }
+}
+template <int block_parallel, int max_hidden_dim = 2048, class IA, class IB, class OS>
+void dec_Gate_Layer_fp32xfp32(IA& input_seq, IB& gate_seq, OS& output_seq, int io_hidden_dim = max_hidden_dim) {
+    for (int i = 0; i < io_hidden_dim / block_parallel; i++) {
+        auto a = input_seq.read();
+        auto b = gate_seq.read();
+        typename OS::value_type o;
+        for (int m = 0; m < block_parallel; m++) o[m] = a[m] * b[m];
+        output_seq.write(o);
+    }
+}
+
+// ======================================================================================= FHT.h
+// Modules/FHT.h:7-13
+template <typename T, int io_parallel, int io_hidden_dim = 2048, int log2_io_hidden_dim = 11, int max_seq_len = 1024, class IS, class OS>
+void pref_FHT(IS& data_in, OS& data_out, int seq_len = max_seq_len, const T scale_factor = 1.0) {
+    static_assert(std::is_same<T, float>::value && (1 << log2_io_hidden_dim) == io_hidden_dim, "fp32, power-of-two length");
+    auto x = drain_pref<float>(data_in, seq_len, io_hidden_dim, io_parallel);
+    DeviceArray<float> dx(x);
+    check(flexllm_fht_f32(dx.get(), dx.get(), seq_len, io_hidden_dim, scale_factor, nullptr));
+    fill_pref(data_out, dx.download(), seq_len, io_hidden_dim, io_parallel);
+}
+// Modules/FHT.h:69-74
+template <typename T, int block_parallel, int io_hidden_dim = 8192, int log2_io_hidden_dim = 13, class IS, class OS>
+void dec_FHT(IS& data_in, OS& data_out, const T scale_factor = 1.0) {
+    static_assert(std::is_same<T, float>::value && (1 << log2_io_hidden_dim) == io_hidden_dim, "fp32, power-of-two length");
+    auto x = drain_dec<float>(data_in, io_hidden_dim, block_parallel);
+    DeviceArray<float> dx(x);
+    check(flexllm_fht_f32(dx.get(), dx.get(), 1, io_hidden_dim, scale_factor, nullptr));
+    fill_dec(data_out, dx.download(), io_hidden_dim, block_parallel);
+}
+
+// ======================================================================================= LayerNorm.h
+// Modules/LayerNorm.h:28-36 (RMSNorm, beta disabled); gamma arrives one value per read
+template <typename T, int io_parallel, int max_hidden_dim = 2048, int max_seq_len = 1024, bool enble_beta = false, bool is_versal = false,
+          class IS, class IG, class OS>
+void pref_Layer_Norm(IS& input_stream, IG& gamma_beta_stream, OS& output_stream, int seq_len = max_seq_len,
+                     int io_hidden_dim = max_hidden_dim, const T eps = 0.00001) {
+    static_assert(!enble_beta, "RMSNorm path");
+    std::vector<float> g(io_hidden_dim);
+    for (int k = 0; k < io_hidden_dim; k++) g[k] = gamma_beta_stream.read();
+    auto x = drain_pref<float>(input_stream, seq_len, io_hidden_dim, io_parallel);
+    DeviceArray<float> dx(x), dg(g), dy(x.size());
+    check(flexllm_rmsnorm_f32(dx.get(), dg.get(), dy.get(), seq_len, io_hidden_dim, eps, nullptr));
+    fill_pref(output_stream, dy.download(), seq_len, io_hidden_dim, io_parallel);
+}
+// Modules/LayerNorm.h:210-217; gamma arrives block-partitioned like the activations
+template <typename T, int block_parallel, int max_hidden_dim = 2048, bool enble_beta = false, bool is_versal = false, class IS, class IG,
+          class OS>
+void dec_Layer_Norm(IS& input_stream, IG& gamma_beta_stream, OS& output_stream, int io_hidden_dim = max_hidden_dim,
+                    const T eps = 0.00001) {
+    static_assert(!enble_beta, "RMSNorm path");
+    auto g = drain_dec<float>(gamma_beta_stream, io_hidden_dim, block_parallel);
+    auto x = drain_dec<float>(input_stream, io_hidden_dim, block_parallel);
+    DeviceArray<float> dx(x), dg(g), dy(x.size());
+    check(flexllm_rmsnorm_f32(dx.get(), dg.get(), dy.get(), 1, io_hidden_dim, eps, nullptr));
+    fill_dec(output_stream, dy.download(), io_hidden_dim, block_parallel);
+}
+
+// ======================================================================================= RoPE.h
+// Modules/RoPE.h:8-15: stream order per token block is head-major, head_dim features per head
+template <typename T, int io_parallel, int io_hidden_dim = 64, int max_head_num = 32, int max_seq_Len = 1024, class IS, class OS>
+void pref_RoPE_layer(IS& input_stream, OS& output_stream, const T PE_sin[max_seq_Len][io_hidden_dim / 2],
+                     const T PE_cos[max_seq_Len][io_hidden_dim / 2], int head_num = max_head_num, int seq_len = max_seq_Len) {
+    auto x = drain_pref<float>(input_stream, seq_len, head_num * io_hidden_dim, io_parallel);
+    DeviceArray<float> dx(x), dy(x.size());
+    DeviceArray<float> ds, dc;
+    ds.upload(&PE_sin[0][0], (size_t)max_seq_Len * (io_hidden_dim / 2));
+    dc.upload(&PE_cos[0][0], (size_t)max_seq_Len * (io_hidden_dim / 2));
+    check(flexllm_rope_f32(dx.get(), dy.get(), ds.get(), dc.get(), seq_len, head_num, io_hidden_dim, 0, nullptr));
+    fill_pref(output_stream, dy.download(), seq_len, head_num * io_hidden_dim, io_parallel);
+}
+
+// ======================================================================================= Swish.h / Residual_Layer.h / Softmax.h
+// Modules/Swish.h:5-10
+template <typename T, int io_parallel, int max_hidden_dim = 8192, int max_seq_len = 1024, class IS, class OS>
+void pref_Swish(IS& input_stream, OS& output_stream, int seq_len = max_seq_len, int io_hidden_dim = max_hidden_dim) {
+    auto x = drain_pref<float>(input_stream, seq_len, io_hidden_dim, io_parallel);
+    DeviceArray<float> dx(x);
+    check(flexllm_swish_f32(dx.get(), dx.get(), x.size(), nullptr));
+    fill_pref(output_stream, dx.download(), seq_len, io_hidden_dim, io_parallel);
+}
+// Modules/Swish.h:26-30
+template <typename T, int block_parallel, int max_hidden_dim = 8192, class IS, class OS>
+void dec_Swish(IS& input_stream, OS& output_stream, int io_hidden_dim = max_hidden_dim) {
+    auto x = drain_dec<float>(input_stream, io_hidden_dim, block_parallel);
+    DeviceArray<float> dx(x);
+    check(flexllm_swish_f32(dx.get(), dx.get(), x.size(), nullptr));
+    fill_dec(output_stream, dx.download(), io_hidden_dim, block_parallel);
+}
+// Modules/Residual_Layer.h:47-53
+template <typename T, int io_parallel, int io_hidden_dim = 2048, int max_seq_len = 1024, class IA, class IB, class OS>
+void pref_Residual_Layer(IA& input_stream, IB& residual_stream, OS& output_stream, int seq_len = max_seq_len) {
+    auto a = drain_pref<float>(input_stream, seq_len, io_hidden_dim, io_parallel);
+    auto b = drain_pref<float>(residual_stream, seq_len, io_hidden_dim, io_parallel);
+    DeviceArray<float> da(a), db(b);
+    check(flexllm_residual_add_f32(da.get(), db.get(), da.get(), a.size(), nullptr));
+    fill_pref(output_stream, da.download(), seq_len, io_hidden_dim, io_parallel);
+}
+// Modules/Residual_Layer.h:69-75
+template <typename T, int block_parallel, int max_hidden_dim = 2048, class IA, class IB, class OS>
+void dec_Residual_Layer(IA& input_stream, IB& residual_stream, OS& output_stream, int io_hidden_dim = max_hidden_dim) {
+    auto a = drain_dec<float>(input_stream, io_hidden_dim, block_parallel);
+    auto b = drain_dec<float>(residual_stream, io_hidden_dim, block_parallel);
+    DeviceArray<float> da(a), db(b);
+    check(flexllm_residual_add_f32(da.get(), db.get(), da.get(), a.size(), nullptr));
+    fill_dec(output_stream, da.download(), io_hidden_dim, block_parallel);
+}
+// Modules/Softmax.h:6-12: per token block, head_num rows of io_hidden_dim scores per token
+template <typename T, int io_parallel, int max_hidden_dim = 2048, int max_seq_len = 1024, int head_num = 1, bool enable_scale = false,
+          bool enable_sub_max = true, bool is_versal = false, class IS, class OS>
+void pref_Softmax(IS& input_stream, OS& output_stream, int seq_len = max_seq_len, int io_hidden_dim = max_hidden_dim,
+                  const T scale_factor = 1.0) {
+    static_assert(!enable_scale && enable_sub_max, "the configuration the shipped graphs use");
+    auto x = drain_pref<float>(input_stream, seq_len, head_num * io_hidden_dim, io_parallel);   // [token][head][dim]
+    DeviceArray<float> dx(x);
+    check(flexllm_softmax_f32(dx.get(), dx.get(), seq_len * head_num, io_hidden_dim, nullptr));
+    fill_pref(output_stream, dx.download(), seq_len, head_num * io_hidden_dim, io_parallel);
+}
+
+// ======================================================================================= MHA_i8xi8.h tops
+// MHA_i8xi8_Prefilling_tb (SpinQuant_Llama_32_1B/MHA_i8xi8.h:369-427) for ONE layer: q_mmap/k_mmap/v_mmap and
+// o_mmap use the prefill packing [(token/TP)*dim + feature][token%TP]; scales are that layer's rows of
+// Q_s/K_s/V_s/A_s.  Returns the kernel time in ns like tapa::invoke.
+template <int TP, int q_heads, int kv_heads, int head_dim, class VF>
+int64_t MHA_i8xi8_Prefilling_layer(const std::vector<VF>& q_mmap, const std::vector<VF>& k_mmap, const std::vector<VF>& v_mmap,
+                                   std::vector<VF>& o_mmap, const float* Q_s, const float* K_s, const float* V_s,
+                                   const float* A_s, int seq_len, float sqrt_head_dim) {
+    const int H = q_heads * head_dim, KV = kv_heads * head_dim;
+    auto unpack = [&](const std::vector<VF>& mm, int dim) {
+        std::vector<float> x((size_t)seq_len * dim);
+        for (int t = 0; t < seq_len; t++)
+            for (int j = 0; j < dim; j++) x[(size_t)t * dim + j] = mm[(size_t)(t / TP) * dim + j][t % TP];
+        return x;
+    };
+    DeviceArray<float> dq(unpack(q_mmap, H)), dk(unpack(k_mmap, KV)), dv(unpack(v_mmap, KV)), dout((size_t)seq_len * H);
+    DeviceArray<float> dqs(std::vector<float>(Q_s, Q_s + q_heads)), dks(std::vector<float>(K_s, K_s + kv_heads)),
+        dvs(std::vector<float>(V_s, V_s + kv_heads)), das(std::vector<float>(A_s, A_s + q_heads));
+    const int max_pos = (seq_len + 63) / 64 * 64;
+    DeviceArray<int8_t> q8((size_t)seq_len * H), kc((size_t)kv_heads * max_pos * head_dim), vc((size_t)kv_heads * max_pos * head_dim);
+    flexllm_mha_scales sc{dqs.get(), dks.get(), dvs.get(), das.get()};
+    hipEvent_t e0, e1;
+    check_hip(hipEventCreate(&e0)); check_hip(hipEventCreate(&e1));
+    check_hip(hipEventRecord(e0, nullptr));
+    check(flexllm_static_quant_i8(dq.get(), q8.get(), dqs.get(), sqrt_head_dim, 1, seq_len, q_heads, head_dim, nullptr));
+    check(flexllm_kv_append_i8(dk.get(), dv.get(), kc.get(), vc.get(), &sc, seq_len, kv_heads, head_dim, max_pos, 0, nullptr));
+    check(flexllm_mha_i8_prefill(q8.get(), kc.get(), vc.get(), &sc, dout.get(), nullptr, seq_len, q_heads, kv_heads, head_dim, max_pos, nullptr));
+    check_hip(hipEventRecord(e1, nullptr)); check_hip(hipEventSynchronize(e1));
+    float ms = 0;
+    check_hip(hipEventElapsedTime(&ms, e0, e1));
+    (void)hipEventDestroy(e0); (void)hipEventDestroy(e1);
+    auto o = dout.download();
+    for (int t = 0; t < seq_len; t++)
+        for (int j = 0; j < H; j++) o_mmap[(size_t)(t / TP) * H + j][t % TP] = o[(size_t)t * H + j];
+    return (int64_t)(ms * 1e6);
+}
+
+}  // namespace fxhost

@@ -1,0 +1,20 @@
+"""Runs the C++ testbench-style harness (flexllm_amd/host/tb/modules_tb.cpp): the reference's module call surface
+(pref_/dec_ quant, Linear_Layer, FHT, Layer_Norm, Swish, Gate, Residual, Softmax, MHA prefill top) driven through
+stream packings exactly as the reference's *_tb.cpp files drive theirs, with in-process goldens."""
+import os
+import subprocess
+
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+BIN = os.path.join(ROOT, "flexllm_amd", "host", "tb", "modules_tb")
+
+
+def test_cpp_module_harness_passes():
+    assert os.path.exists(BIN), "build it with `python -m flexllm_amd.build` (or __graft_entry__.build())"
+    out = subprocess.run([BIN], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=300)
+    print(out.stdout)
+    assert out.returncode == 0, out.stdout
+    assert out.stdout.count("passed correctness check") == 5 and "failed" not in out.stdout
