@@ -375,16 +375,40 @@ __global__ __launch_bounds__(kMegaT, 1) void decode_mega_kernel(MegaParams p) {
 #pragma unroll
             for (int i = 0; i < 4; i++) v[i] = ld_f(&p.x2[4 * t + i]);
             const float sx = norm_quant_2048(v, g1, true, p.eps, L);
+            // eight per-lane partial dot products, folded with a transposing butterfly: each step halves the
+            // number of live values, so 7 + 3 cross-lane exchanges replace 8 x 6.  Afterwards lane L holds the
+            // complete sum of row (L>>2 & 1) + 2*(L>>1 & 1) + 4*(L & 1).
+            int part[8];
 #pragma unroll
-            for (int r = 0; r < 8; r += 2) {
-                const int ag = mega_dot_row<2>(wr[r], L.xq, lane);
-                const int au = mega_dot_row<2>(wr[r + 1], L.xq, lane);
-                if (lane == 0) {
-                    const float gate = (float)ag * sx * w.sgu[row0 + r];
-                    const float up = (float)au * sx * w.sgu[row0 + r + 1];
-                    st_f(&p.h[(row0 + r) >> 1], up * silu_f(gate));
-                }
+            for (int r = 0; r < 8; r++) {
+                int acc = 0;
+#pragma unroll
+                for (int i = 0; i < 2; i++) acc = dot16(wr[r][i], reinterpret_cast<const i32x4*>(L.xq)[lane + 64 * i], acc);
+                part[r] = acc;
             }
+            int q4[4], q2[2];
+            {
+                const bool hi = lane & 1;
+#pragma unroll
+                for (int i = 0; i < 4; i++) q4[i] = (hi ? part[i + 4] : part[i]) + lane_xor_i<1>(hi ? part[i] : part[i + 4]);
+            }
+            {
+                const bool hi = lane & 2;
+#pragma unroll
+                for (int i = 0; i < 2; i++) q2[i] = (hi ? q4[i + 2] : q4[i]) + lane_xor_i<2>(hi ? q4[i] : q4[i + 2]);
+            }
+            int sum;
+            {
+                const bool hi = lane & 4;
+                sum = (hi ? q2[1] : q2[0]) + lane_xor_i<4>(hi ? q2[0] : q2[1]);
+            }
+            sum += lane_xor_i<8>(sum);
+            sum += lane_xor_i<16>(sum);
+            sum += lane_xor_i<32>(sum);
+            const int ridx = ((lane >> 2) & 1) + 2 * ((lane >> 1) & 1) + 4 * (lane & 1);
+            const float mine = (float)sum * sx * w.sgu[row0 + ridx];
+            const float other = lane_xor_f<4>(mine);               // row ridx^1: the other half of the SwiGLU pair
+            if (lane < 4) st_f(&p.h[(row0 + ridx) >> 1], other * silu_f(mine));   // lanes 0..3 hold the gate rows 0,4,2,6
             stamp();
             bar.arrive();
         }
