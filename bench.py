@@ -20,6 +20,11 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0          # MI355X published HBM3E bandwidth
 INT8_PEAK_TOPS = 5000.0        # MI355X published dense int8 MFMA rate
+# HBM traffic of one decode_mega_kernel launch at context ~4092, from two `rocprofv3 --pmc` runs of this file
+# (FETCH_SIZE 777,644 KiB/dispatch, WRITE_SIZE 11,451 KiB/dispatch), each scaled by the same counter's reading
+# for a plain 1 GiB device copy (FETCH_SIZE reads 524,302 KiB for 1,048,576 KiB fetched -> x2.0; WRITE_SIZE
+# reads 1,048,576 KiB -> x1.0).  Only valid for the default 16-layer model at context 4096.
+MEASURED_TRAFFIC_BYTES = int((777644 * 2.0 + 11451 * 1.0) * 1024)
 
 
 def bytes_per_token(cfg, mean_len):
@@ -175,7 +180,7 @@ def main():
         # (the only other kernel in a step is the 1-workgroup argmax/advance kernel).
         "roofline": {"bound": "hbm", "kernel": "decode_mega_kernel (one launch per token)",
                      "achieved": round(bpt / (ev_ms / K * 1e-3) / 1e9, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": round(bpt / (ev_ms / K * 1e-3) / 1e9 / HBM_PEAK_GBS, 4), "traffic": None,
+                     "frac": round(bpt / (ev_ms / K * 1e-3) / 1e9 / HBM_PEAK_GBS, 4), "traffic": MEASURED_TRAFFIC_BYTES if (cfg["layers"] == 16 and pos_end == 4096) else None,
                      "bytes_per_launch": int(bpt), "avg_us": round(ev_ms / K * 1e3, 2)},
         "gemv_gate_up": {"kernel": "gemv_i8_kernel<2,4,swiglu> stand-alone (2048->2x8192), 16 distinct weight buffers",
                          "achieved_GBs": round(kern_gbs, 1), "hbm_frac": round(kern_gbs / HBM_PEAK_GBS, 4),
