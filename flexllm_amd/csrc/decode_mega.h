@@ -15,6 +15,14 @@
 // they are loaded into registers BEFORE waiting on the barrier: HBM keeps streaming while the barrier's
 // round trips are in flight.
 //
+// Wave roles.  Vector-memory results return to a wave in issue order, so a wave with a long weight prefetch in
+// flight cannot see an activation load (or have a store acknowledged) until the prefetch has landed.  The
+// two big matrices are therefore owned by waves 4..7 ("stream waves"): they issue the gate/up rows a full
+// phase ahead (before the o_proj barrier) and the down rows before the gate/up barrier, and while such a
+// prefetch is in flight they touch global memory no further - activations reach them through LDS, and their
+// results leave through LDS.  Waves 0..3 load the activations, own the small q/k/v and o_proj rows and do
+// the global stores of those phases; only they drain their memory counter before arriving at the barrier.
+//
 // Memory-model discipline (no cache flushes inside the kernel): every value that crosses workgroups between
 // barriers (x, x2, qkv, h, chunk statistics, attention accumulators) is written and read with device-scope
 // relaxed atomic stores/loads, which bypass the per-XCD L2 for coherence; each thread drains its outstanding
@@ -61,6 +69,19 @@ __device__ __forceinline__ void st_f(float* p, float v) { __hip_atomic_store(p, 
 __device__ __forceinline__ int ld_i(const int* p) { return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
 __device__ __forceinline__ void st_i(int* p, int v) { __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
 
+// Read-only data at a wave-uniform address (layer table, per-row weight scales): the constant address space
+// makes these scalar loads, off the vector-memory queue.
+__device__ __forceinline__ float ldc_f(const float* p) { return *(const float __attribute__((address_space(4)))*)(uintptr_t)p; }
+
+__device__ __forceinline__ LayerW ldc_layer(const LayerW* p) {
+    static_assert(sizeof(LayerW) == 8 * sizeof(unsigned long long), "LayerW is eight pointers");
+    const unsigned long long __attribute__((address_space(4)))* q = (const unsigned long long __attribute__((address_space(4)))*)(uintptr_t)p;
+    LayerW w;
+    w.wqkv = (int8_t*)q[0]; w.wo = (int8_t*)q[1]; w.wgu = (int8_t*)q[2]; w.wd = (int8_t*)q[3];
+    w.sqkv = (float*)q[4]; w.so = (float*)q[5]; w.sgu = (float*)q[6]; w.sd = (float*)q[7];
+    return w;
+}
+
 // Grid barrier from device-scope relaxed atomics: workgroup w adds 1 to group counter w/32 (8 counters on
 // separate 256-byte lines, so at most 32 atomics serialise on one address); the last arriver of a group adds 1
 // to the top counter, the last of those publishes the epoch in a flag that everybody polls.  (Polling the
@@ -69,8 +90,9 @@ struct GridBarrier {
     unsigned* mem;                              // [0] flag, [64] top counter, [128 + 64*g] group counters
     unsigned epoch;
     int* err;
-    __device__ __forceinline__ void arrive() {
-        __builtin_amdgcn_s_waitcnt(0);          // this thread's stores have been acknowledged
+    // drain == false: the calling wave made no global store in this phase and may keep loads in flight
+    __device__ __forceinline__ void arrive(bool drain = true) {
+        if (drain) __builtin_amdgcn_s_waitcnt(0);          // this thread's stores have been acknowledged
         __syncthreads();
         epoch++;
         if (threadIdx.x == 0) {
@@ -108,6 +130,8 @@ struct MegaLds {
     int osum[4][kHd];
     float bestv[kMegaWaves];
     int besti[kMegaWaves];
+    float hst[32];                                     // SiLU(gate)*up of this workgroup's 32 row pairs, stream waves -> store wave
+    __attribute__((aligned(16))) int8_t wd[8][8192];   // this workgroup's 8 down rows, filled by global->LDS direct loads (64 KiB)
 };
 
 template <int NW>
@@ -115,18 +139,47 @@ __device__ __forceinline__ float mega_block_max(float v, float* red) { return bl
 
 // RMSNorm (optional) + per-token int8 quantisation of a 2048-vector held as 4 values per thread; result in L.xq.
 // Returns the quantisation scale to every thread.
-__device__ __forceinline__ float norm_quant_2048(float (&v)[4], const float* __restrict__ gamma, bool do_norm, float eps,
-                                                 MegaLds& L) {
+// `hook` runs in every thread right after the first workgroup barrier, i.e. once every wave's activation loads
+// have been consumed: the stream waves issue their next slice of weight prefetch there.
+template <class Hook>
+__device__ __forceinline__ float mega_block_sum(float v, float* red, Hook hook) {
+    v = wave_sum(v);
+    __syncthreads();
+    hook();
+    if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = v;
+    __syncthreads();
+    float r = red[0];
+#pragma unroll
+    for (int i = 1; i < kMegaWaves; i++) r += red[i];
+    return r;
+}
+template <class Hook>
+__device__ __forceinline__ float mega_block_max_h(float v, float* red, Hook hook) {
+    v = wave_max(v);
+    __syncthreads();
+    hook();
+    if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = v;
+    __syncthreads();
+    float r = red[0];
+#pragma unroll
+    for (int i = 1; i < kMegaWaves; i++) r = fmaxf(r, red[i]);
+    return r;
+}
+struct NoHook { __device__ __forceinline__ void operator()() const {} };
+
+template <class Hook>
+__device__ __forceinline__ float norm_quant_2048(float (&v)[4], const float4& g, bool do_norm, float eps,
+                                                 MegaLds& L, Hook hook) {
     const int t = threadIdx.x;
     if (do_norm) {
         float ss = (v[0] * v[0] + v[1] * v[1]) + (v[2] * v[2] + v[3] * v[3]);
-        ss = block_sum<kMegaWaves>(ss, L.red);
+        ss = mega_block_sum(ss, L.red, hook);
         const float rms = 1.0f / sqrtf(ss / 2048.0f + eps);
-        const float4 g = reinterpret_cast<const float4*>(gamma)[t];
         v[0] = v[0] * rms * g.x; v[1] = v[1] * rms * g.y; v[2] = v[2] * rms * g.z; v[3] = v[3] * rms * g.w;
     }
     float amax = fmaxf(fmaxf(fabsf(v[0]), fabsf(v[1])), fmaxf(fabsf(v[2]), fabsf(v[3])));
-    amax = block_max<kMegaWaves>(amax, L.red);
+    if (do_norm) amax = mega_block_max_h(amax, L.red, NoHook());
+    else amax = mega_block_max_h(amax, L.red, hook);
     const float sc = sym_scale(amax, 127.0f);
     reinterpret_cast<uint32_t*>(L.xq)[t] = pack4_i8(quant_round(v[0], sc), quant_round(v[1], sc), quant_round(v[2], sc),
                                                     quant_round(v[3], sc));
@@ -134,12 +187,63 @@ __device__ __forceinline__ float norm_quant_2048(float (&v)[4], const float* __r
     return sc;
 }
 
+// Same for 8 values per thread held by the first 256 threads only (thread t < 256 holds elements 8t..8t+7); the
+// other threads pass zeros and take part in the reductions and barriers only.
+template <class Hook>
+__device__ __forceinline__ float norm_quant_2048_half(float (&v)[8], const float4& g0, const float4& g1, bool do_norm, float eps,
+                                                      bool holder, MegaLds& L, Hook hook) {
+    const int t = threadIdx.x;
+    if (do_norm) {
+        float ss = ((v[0] * v[0] + v[1] * v[1]) + (v[2] * v[2] + v[3] * v[3])) + ((v[4] * v[4] + v[5] * v[5]) + (v[6] * v[6] + v[7] * v[7]));
+        ss = mega_block_sum(ss, L.red, hook);
+        const float rms = 1.0f / sqrtf(ss / 2048.0f + eps);
+        if (holder) {
+            v[0] = v[0] * rms * g0.x; v[1] = v[1] * rms * g0.y; v[2] = v[2] * rms * g0.z; v[3] = v[3] * rms * g0.w;
+            v[4] = v[4] * rms * g1.x; v[5] = v[5] * rms * g1.y; v[6] = v[6] * rms * g1.z; v[7] = v[7] * rms * g1.w;
+        }
+    }
+    float amax = fmaxf(fmaxf(fmaxf(fabsf(v[0]), fabsf(v[1])), fmaxf(fabsf(v[2]), fabsf(v[3]))),
+                       fmaxf(fmaxf(fabsf(v[4]), fabsf(v[5])), fmaxf(fabsf(v[6]), fabsf(v[7]))));
+    if (do_norm) amax = mega_block_max_h(amax, L.red, NoHook());
+    else amax = mega_block_max_h(amax, L.red, hook);
+    const float sc = sym_scale(amax, 127.0f);
+    if (holder) {
+        uint2 q;
+        q.x = pack4_i8(quant_round(v[0], sc), quant_round(v[1], sc), quant_round(v[2], sc), quant_round(v[3], sc));
+        q.y = pack4_i8(quant_round(v[4], sc), quant_round(v[5], sc), quant_round(v[6], sc), quant_round(v[7], sc));
+        reinterpret_cast<uint2*>(L.xq)[t] = q;
+    }
+    __syncthreads();
+    return sc;
+}
+
+// Weight rows are read through a pointer that is explicitly in the global address space: a generic pointer
+// would make these FLAT loads, which also count on the LDS/scalar counter, and every LDS wait of the wave
+// would then wait for the weight prefetch as well.
+typedef const i32x4 __attribute__((address_space(1)))* global_i32x4_ptr;
 template <int NCH>
 __device__ __forceinline__ void mega_load_rows(const int8_t* __restrict__ w, int k, int row, int lane, i32x4 (&wr)[NCH]) {
-    const i32x4* p = reinterpret_cast<const i32x4*>(w + (size_t)row * k);
+    const global_i32x4_ptr p = (global_i32x4_ptr)(uintptr_t)(w + (size_t)row * k);
 #pragma unroll
     for (int i = 0; i < NCH; i++) wr[i] = __builtin_nontemporal_load(p + lane + 64 * i);
 }
+// One 8192-byte weight row straight from global memory into LDS (16 bytes per lane, lane i of chunk c lands
+// at byte 1024*c + 16*i): no registers are held while the row is in flight.  Counts on the vector-memory
+// counter like a load; the issuing wave waits for that counter to reach zero before it reads the row.
+__device__ __forceinline__ void mega_row_to_lds(const int8_t* __restrict__ w, int row, int lane, int8_t* lds_row) {
+    const global_i32x4_ptr p = (global_i32x4_ptr)(uintptr_t)(w + (size_t)row * 8192);
+#pragma unroll
+    for (int i = 0; i < 8; i++)
+        __builtin_amdgcn_global_load_lds(p + lane + 64 * i, (__attribute__((address_space(3))) void*)(lds_row + 1024 * i), 16, 0, 0);
+}
+__device__ __forceinline__ int mega_dot_row_lds(const int8_t* w_lds, const int8_t* xq_lds, int lane) {
+    int acc = 0;
+#pragma unroll
+    for (int i = 0; i < 8; i++)
+        acc = dot16(reinterpret_cast<const i32x4*>(w_lds)[lane + 64 * i], reinterpret_cast<const i32x4*>(xq_lds)[lane + 64 * i], acc);
+    return wave_sum_i(acc);
+}
+
 template <int NCH>
 __device__ __forceinline__ int mega_dot_row(const i32x4 (&wr)[NCH], const int8_t* xq_lds, int lane) {
     int acc = 0;
@@ -149,8 +253,12 @@ __device__ __forceinline__ int mega_dot_row(const i32x4 (&wr)[NCH], const int8_t
 }
 
 __global__ __launch_bounds__(kMegaT, 1) void decode_mega_kernel(MegaParams p) {
-    __shared__ MegaLds L;
-    const int t = threadIdx.x, lane = t & 63, wave = t >> 6, wg = blockIdx.x;
+    extern __shared__ __attribute__((aligned(16))) unsigned char mega_smem[];   // sizeof(MegaLds) > the static 64 KiB limit
+    MegaLds& L = *reinterpret_cast<MegaLds*>(mega_smem);
+    const int t = threadIdx.x, lane = t & 63, wg = blockIdx.x;
+    const int wave = __builtin_amdgcn_readfirstlane(t >> 6);
+    const bool is_s = wave >= 4;                        // stream wave (see the file comment)
+    const int sw = wave - 4;
     constexpr int H = 2048, KV = 512, I = 8192, QH = 32, KVH = 8, GROUP = 4;
     const int pos = p.state[0];
     const int len = pos + 1;
@@ -171,7 +279,13 @@ __global__ __launch_bounds__(kMegaT, 1) void decode_mega_kernel(MegaParams p) {
     const bool a_owner = a_active && (pos / kChunk == a_c);       // this chunk holds the new token
 
     for (int l = 0; l < p.n_layers; l++) {
-        const LayerW w = p.layers[l];
+        // An opaque per-layer copy of the thread index: without it the compiler hoists every per-thread address
+        // offset of all phases out of the layer loop, and the ~100 registers they occupy push the prefetched
+        // weights into scratch memory.
+        int t_opaque = threadIdx.x;
+        asm volatile("" : "+v"(t_opaque));
+        const int t = t_opaque, lane = t & 63;
+        const LayerW w = ldc_layer(p.layers + l);
         const float* g0 = p.gamma + (size_t)(2 * l) * H;
         const float* g1 = p.gamma + (size_t)(2 * l + 1) * H;
         const float* q_s = p.q_s + l * QH;
@@ -181,13 +295,34 @@ __global__ __launch_bounds__(kMegaT, 1) void decode_mega_kernel(MegaParams p) {
         int8_t* kc = p.k_cache + (size_t)l * p.cache_layer_bytes;
         int8_t* vc = p.v_cache + (size_t)l * p.cache_layer_bytes;
 
-        // ================= phase 1: RMSNorm + quant -> q/k/v rows (12 rows per workgroup) =================
+        // Stream waves: 16 gate/up rows (interleaved gate, up) and 2 down rows each, fetched in six slices of
+        // 8 KiB per wave, one per phase, each issued once the phase's activation loads have landed.  A slice
+        // (8 MiB over the chip) drains while the phase computes; issuing a whole matrix at once instead fills
+        // the memory queues for microseconds, and the barrier's own round trips then queue behind it.
+        i32x4 gu[16][2];
+        auto gu_slice = [&](int s) {
+            // Every wave first waits for its own older loads (long landed at the points where this is called).
+            // Otherwise the wait inserted for such a load after the branch below has to assume the path without
+            // the slice, and it would make the stream waves sit out their own prefetch.
+            __builtin_amdgcn_s_waitcnt(0x0F70);            // vmcnt(0) only
+            if (is_s) {
+#pragma unroll
+                for (int r = 0; r < 4; r++) mega_load_rows<2>(w.wgu, H, wg * 64 + sw * 16 + 4 * s + r, lane, gu[4 * s + r]);
+            }
+        };
+
+        // ================= phase 1: RMSNorm + quant -> q/k/v rows (12 per workgroup, 3 per wave 0..3) =================
         {
-            i32x4 wr[2][2];
-            const int r0 = wg * 12 + wave, r1 = r0 + 8;
-            const bool has1 = wave < 4;
-            mega_load_rows<2>(w.wqkv, H, r0, lane, wr[0]);
-            if (has1) mega_load_rows<2>(w.wqkv, H, r1, lane, wr[1]);
+            i32x4 wr[3][2];
+            float wsc[3] = {0.0f, 0.0f, 0.0f};
+            if (!is_s) {
+#pragma unroll
+                for (int j = 0; j < 3; j++) {
+                    mega_load_rows<2>(w.wqkv, H, wg * 12 + wave + 4 * j, lane, wr[j]);
+                    wsc[j] = ldc_f(w.sqkv + wg * 12 + wave + 4 * j);
+                }
+            }
+            const float4 gam = reinterpret_cast<const float4*>(g0)[t];
             if (l > 0) bar.wait();                                   // x of the previous layer is complete
             stamp();
             float v[4];
@@ -201,15 +336,17 @@ __global__ __launch_bounds__(kMegaT, 1) void decode_mega_kernel(MegaParams p) {
 #pragma unroll
                 for (int i = 0; i < 4; i++) v[i] = ld_f(&p.x[4 * t + i]);
             }
-            const float sx = norm_quant_2048(v, g0, true, p.eps, L);
-            const int a0 = mega_dot_row<2>(wr[0], L.xq, lane);
-            if (lane == 0) st_f(&p.qkv[r0], (float)a0 * sx * w.sqkv[r0]);
-            if (has1) {
-                const int a1 = mega_dot_row<2>(wr[1], L.xq, lane);
-                if (lane == 0) st_f(&p.qkv[r1], (float)a1 * sx * w.sqkv[r1]);
+            const float sx = norm_quant_2048(v, gam, true, p.eps, L, [&]() { gu_slice(0); });
+            if (!is_s) {
+#pragma unroll
+                for (int j = 0; j < 3; j++) {
+                    const int r = wg * 12 + wave + 4 * j;
+                    const int a = mega_dot_row<2>(wr[j], L.xq, lane);
+                    if (lane == 0) st_f(&p.qkv[r], (float)a * sx * wsc[j]);
+                }
             }
             stamp();
-            bar.arrive();
+            bar.arrive(!is_s);
         }
 
         // ================= phase 2: RoPE/quant/append, scores of this chunk, chunk statistics =================
@@ -218,6 +355,11 @@ __global__ __launch_bounds__(kMegaT, 1) void decode_mega_kernel(MegaParams p) {
             const int key = t >> 2, part = t & 3;
             const int kpos = a_c * kChunk + key;
             if (a_active) kreg = *reinterpret_cast<const i32x4*>(kc + k_index(a_h, min(kpos, p.max_pos - 1), p.max_pos) + part * 16);
+            // static scales of this layer, read ahead of the barrier (and of this phase's prefetch slice)
+            float qs4[GROUP];
+#pragma unroll
+            for (int g = 0; g < GROUP; g++) qs4[g] = ldc_f(q_s + a_h * GROUP + g);
+            const float ks1 = ldc_f(k_s + a_h), vs1 = ldc_f(v_s + a_h);
             bar.wait();
             stamp();
             if (a_active) {
@@ -227,24 +369,25 @@ __global__ __launch_bounds__(kMegaT, 1) void decode_mega_kernel(MegaParams p) {
                     const int g = t >> 5, k = t & 31, qh = a_h * GROUP + g;
                     const float t0 = ld_f(&p.qkv[qh * kHd + k]), t1 = ld_f(&p.qkv[qh * kHd + k + 32]);
                     const float o0 = t0 * cs[k] - t1 * sn[k], o1 = t0 * sn[k] + t1 * cs[k];
-                    const float div = 8.0f * q_s[qh];
+                    const float div = 8.0f * (g == 0 ? qs4[0] : g == 1 ? qs4[1] : g == 2 ? qs4[2] : qs4[3]);
                     L.q8[g][k] = (int8_t)static_q8(o0, div);
                     L.q8[g][k + 32] = (int8_t)static_q8(o1, div);
                 } else if (t < 160) {                                 // k of the new token: 32 pairs
                     const int k = t - 128;
                     const float t0 = ld_f(&p.qkv[H + a_h * kHd + k]), t1 = ld_f(&p.qkv[H + a_h * kHd + k + 32]);
                     const float o0 = t0 * cs[k] - t1 * sn[k], o1 = t0 * sn[k] + t1 * cs[k];
-                    const float div = 1.0f * k_s[a_h];
+                    const float div = 1.0f * ks1;
                     const int8_t b0 = (int8_t)static_q8(o0, div), b1 = (int8_t)static_q8(o1, div);
                     L.knew[k] = b0; L.knew[k + 32] = b1;
                     if (a_owner) { int8_t* dst = kc + k_index(a_h, pos, p.max_pos); dst[k] = b0; dst[k + 32] = b1; }
                 } else if (t < 224) {                                 // v of the new token
                     const int d = t - 160;
-                    const int8_t b = (int8_t)static_q8(ld_f(&p.qkv[H + KV + a_h * kHd + d]), 1.0f * v_s[a_h]);
+                    const int8_t b = (int8_t)static_q8(ld_f(&p.qkv[H + KV + a_h * kHd + d]), 1.0f * vs1);
                     L.vnew[d] = b;
                     if (a_owner) vc[v_index(a_h, pos, d, p.max_pos)] = b;
                 }
                 __syncthreads();
+                gu_slice(1);                                          // the q/k/v loads of this phase have landed
                 if (kpos == pos) kreg = reinterpret_cast<const i32x4*>(L.knew)[part];
                 float s_mine = 0.0f;
 #pragma unroll
@@ -252,7 +395,7 @@ __global__ __launch_bounds__(kMegaT, 1) void decode_mega_kernel(MegaParams p) {
                     int acc = dot16(kreg, reinterpret_cast<const i32x4*>(L.q8[g])[part], 0);
                     acc += lane_xor_i<1>(acc);
                     acc += lane_xor_i<2>(acc);
-                    const float s = (float)acc * q_s[a_h * GROUP + g] * k_s[a_h];
+                    const float s = (float)acc * qs4[g] * ks1;
                     if (part == g) s_mine = s;
                 }
                 L.sc[part][key] = kpos < len ? s_mine : -1e32f;
@@ -267,9 +410,11 @@ __global__ __launch_bounds__(kMegaT, 1) void decode_mega_kernel(MegaParams p) {
                         st_f(&p.stats[(a_h * GROUP + wave) * 32 + a_c].y, sum);
                     }
                 }
+            } else {
+                gu_slice(1);
             }
             stamp();
-            bar.arrive();
+            bar.arrive(!is_s);
         }
 
         // ================= phase 3: row statistics, uint8 probabilities, partial P.V =================
@@ -279,6 +424,7 @@ __global__ __launch_bounds__(kMegaT, 1) void decode_mega_kernel(MegaParams p) {
             const int bpos = a_c * kChunk + blk * kVBlock;
             if (a_active && bpos < p.max_pos)
                 vreg = *reinterpret_cast<const i32x4*>(vc + v_index(a_h, bpos, d, p.max_pos) + part * 16);
+            const float as_g = ldc_f(a_s + a_h * GROUP + (wave >> 1));   // threads 128g..128g+127 (two waves) serve query head g
             bar.wait();
             stamp();
             if (a_active) {
@@ -294,10 +440,11 @@ __global__ __launch_bounds__(kMegaT, 1) void decode_mega_kernel(MegaParams p) {
                     if (lane == 0) { L.rowmax[wave] = mx; L.rowcd[wave] = 1.0f / sum; }
                 }
                 __syncthreads();
+                gu_slice(2);                                          // the chunk statistics have landed
                 {
                     const int g = t >> 7, key = t & 127;
                     const float pr = expf(L.sc[g][key] - L.rowmax[g]) * L.rowcd[g];
-                    int p8 = (int)roundf(pr / (1.0f * a_s[a_h * GROUP + g]));
+                    int p8 = (int)roundf(pr / (1.0f * as_g));
                     p8 = p8 > 255 ? 255 : p8;
                     if (a_c * kChunk + key >= len) p8 = 0;
                     L.pb[g][key] = (uint8_t)(p8 ^ 0x80);
@@ -332,94 +479,124 @@ __global__ __launch_bounds__(kMegaT, 1) void decode_mega_kernel(MegaParams p) {
                         __hip_atomic_fetch_add(&p.o_acc[(a_h * GROUP + g) * kHd + d], tot[g] + L.osum[g][d], __ATOMIC_RELAXED,
                                                __HIP_MEMORY_SCOPE_AGENT);
                 }
+            } else {
+                gu_slice(2);
             }
             stamp();
-            bar.arrive();
+            bar.arrive(!is_s);
         }
 
-        // ================= phase 4: attention dequant + quant -> o_proj rows (8 per workgroup) + residual =================
-        {
-            i32x4 wr[2];
-            const int row = wg * 8 + wave;
-            mega_load_rows<2>(w.wo, H, row, lane, wr);
+        // Phases 4 and 5 are written once per wave role; the two branches execute the same sequence of
+        // workgroup barriers (the branch condition is wave-uniform).
+        if (is_s) {
+            // ---- stream waves, phase 4: last gate/up slice, otherwise only keep step with the barriers ----
             bar.wait();
             stamp();
-            float v[4];
-#pragma unroll
-            for (int i = 0; i < 4; i++) {
-                const int idx = 4 * t + i, qh = idx / kHd;
-                v[i] = (float)ld_i(&p.o_acc[idx]) * a_s[qh] * v_s[qh / GROUP];
-            }
-            const float sx = norm_quant_2048(v, nullptr, false, p.eps, L);
-            const int a0 = mega_dot_row<2>(wr, L.xq, lane);
-            if (lane == 0) {
-                float xr;
-                if (l == 0) xr = p.x_in ? p.x_in[row] : __half2float(p.embed[(size_t)tok * H + row]);
-                else xr = ld_f(&p.x[row]);
-                st_f(&p.x2[row], (float)a0 * sx * w.so[row] + xr);
-            }
+            float z[8] = {0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f};
+            const float4 z4 = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+            (void)norm_quant_2048_half(z, z4, z4, false, p.eps, false, L, [&]() { gu_slice(3); });
             stamp();
-            bar.arrive();
-        }
-
-        // ================= phase 5: RMSNorm + quant -> gate/up rows (64 per workgroup) + SiLU*up =================
-        {
-            i32x4 wr[8][2];
-            const int row0 = wg * 64 + wave * 8;
-#pragma unroll
-            for (int r = 0; r < 8; r++) mega_load_rows<2>(w.wgu, H, row0 + r, lane, wr[r]);
+            bar.arrive(false);
+            // ---- stream waves, phase 5: first down row, gate/up rows + SiLU*up into LDS ----
+            const int ridx = 8 * (lane & 1) + 4 * ((lane >> 1) & 1) + 2 * ((lane >> 2) & 1) + ((lane >> 3) & 1);
+            const float gsc = w.sgu[wg * 64 + sw * 16 + ridx];       // read before this phase's prefetch is issued
             bar.wait();
             stamp();
-            if (t < 8) st_i(&p.o_acc[wg * 8 + t], 0);                // every reader of o_acc has passed the barrier
-            float v[4];
+            const float sx = norm_quant_2048_half(z, z4, z4, true, p.eps, false, L, [&]() { mega_row_to_lds(w.wd, wg * 8 + sw * 2, lane, L.wd[sw * 2]); });
+            // sixteen per-lane partial dot products, folded with a transposing butterfly: each step halves the
+            // number of live values, so 15 + 2 cross-lane exchanges replace 16 x 6.  Afterwards lane L holds
+            // the complete sum of row 8*(L&1) + 4*(L>>1 & 1) + 2*(L>>2 & 1) + (L>>3 & 1).
+            int part[16];
+            {
+                const i32x4 x0 = reinterpret_cast<const i32x4*>(L.xq)[lane], x1 = reinterpret_cast<const i32x4*>(L.xq)[lane + 64];
 #pragma unroll
-            for (int i = 0; i < 4; i++) v[i] = ld_f(&p.x2[4 * t + i]);
-            const float sx = norm_quant_2048(v, g1, true, p.eps, L);
-            // eight per-lane partial dot products, folded with a transposing butterfly: each step halves the
-            // number of live values, so 7 + 3 cross-lane exchanges replace 8 x 6.  Afterwards lane L holds the
-            // complete sum of row (L>>2 & 1) + 2*(L>>1 & 1) + 4*(L & 1).
-            int part[8];
-#pragma unroll
-            for (int r = 0; r < 8; r++) {
-                int acc = 0;
-#pragma unroll
-                for (int i = 0; i < 2; i++) acc = dot16(wr[r][i], reinterpret_cast<const i32x4*>(L.xq)[lane + 64 * i], acc);
-                part[r] = acc;
+                for (int r = 0; r < 16; r++) part[r] = dot16(gu[r][1], x1, dot16(gu[r][0], x0, 0));
             }
-            int q4[4], q2[2];
+            int q8[8], q4[4], q2[2];
             {
                 const bool hi = lane & 1;
 #pragma unroll
-                for (int i = 0; i < 4; i++) q4[i] = (hi ? part[i + 4] : part[i]) + lane_xor_i<1>(hi ? part[i] : part[i + 4]);
+                for (int i = 0; i < 8; i++) q8[i] = (hi ? part[i + 8] : part[i]) + lane_xor_i<1>(hi ? part[i] : part[i + 8]);
             }
             {
                 const bool hi = lane & 2;
 #pragma unroll
-                for (int i = 0; i < 2; i++) q2[i] = (hi ? q4[i + 2] : q4[i]) + lane_xor_i<2>(hi ? q4[i] : q4[i + 2]);
+                for (int i = 0; i < 4; i++) q4[i] = (hi ? q8[i + 4] : q8[i]) + lane_xor_i<2>(hi ? q8[i] : q8[i + 4]);
+            }
+            {
+                const bool hi = lane & 4;
+#pragma unroll
+                for (int i = 0; i < 2; i++) q2[i] = (hi ? q4[i + 2] : q4[i]) + lane_xor_i<4>(hi ? q4[i] : q4[i + 2]);
             }
             int sum;
             {
-                const bool hi = lane & 4;
-                sum = (hi ? q2[1] : q2[0]) + lane_xor_i<4>(hi ? q2[0] : q2[1]);
+                const bool hi = lane & 8;
+                sum = (hi ? q2[1] : q2[0]) + lane_xor_i<8>(hi ? q2[0] : q2[1]);
             }
-            sum += lane_xor_i<8>(sum);
             sum += lane_xor_i<16>(sum);
             sum += lane_xor_i<32>(sum);
-            const int ridx = ((lane >> 2) & 1) + 2 * ((lane >> 1) & 1) + 4 * (lane & 1);
-            const float mine = (float)sum * sx * w.sgu[row0 + ridx];
-            const float other = lane_xor_f<4>(mine);               // row ridx^1: the other half of the SwiGLU pair
-            if (lane < 4) st_f(&p.h[(row0 + ridx) >> 1], other * silu_f(mine));   // lanes 0..3 hold the gate rows 0,4,2,6
+            const float mine = (float)sum * sx * gsc;
+            const float other = lane_xor_f<8>(mine);               // row ridx^1: the other half of the SwiGLU pair
+            if (lane < 8) L.hst[sw * 8 + (ridx >> 1)] = other * silu_f(mine);   // lanes 0..7 hold the (even) gate rows
+            __syncthreads();
             stamp();
-            bar.arrive();
+            bar.arrive(false);
+        } else {
+            // ---- waves 0..3, phase 4: attention dequant + quant -> o_proj rows (8 per workgroup) + residual ----
+            {
+                i32x4 wr[2][2];
+#pragma unroll
+                for (int j = 0; j < 2; j++) mega_load_rows<2>(w.wo, H, wg * 8 + wave + 4 * j, lane, wr[j]);
+                const float wsc0 = ldc_f(w.so + wg * 8 + wave), wsc1 = ldc_f(w.so + wg * 8 + wave + 4);
+                const float osa = a_s[t >> 3], osv = v_s[t >> 5];     // elements 8t..8t+7 lie in query head t/8
+                bar.wait();
+                stamp();
+                float v[8], xr[2] = {0.0f, 0.0f};
+#pragma unroll
+                for (int i = 0; i < 8; i++) v[i] = (float)ld_i(&p.o_acc[8 * t + i]) * osa * osv;
+                if (lane == 0) {                                      // residual inputs, fetched with the activations
+#pragma unroll
+                    for (int j = 0; j < 2; j++) {
+                        const int row = wg * 8 + wave + 4 * j;
+                        if (l == 0) xr[j] = p.x_in ? p.x_in[row] : __half2float(p.embed[(size_t)tok * H + row]);
+                        else xr[j] = ld_f(&p.x[row]);
+                    }
+                }
+                const float4 z4 = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+                const float sx = norm_quant_2048_half(v, z4, z4, false, p.eps, true, L, NoHook());
+#pragma unroll
+                for (int j = 0; j < 2; j++) {
+                    const int row = wg * 8 + wave + 4 * j;
+                    const int a0 = mega_dot_row<2>(wr[j], L.xq, lane);
+                    if (lane == 0) st_f(&p.x2[row], (float)a0 * sx * (j == 0 ? wsc0 : wsc1) + xr[j]);
+                }
+                stamp();
+                bar.arrive(true);
+            }
+            // ---- waves 0..3, phase 5: RMSNorm + quant for the stream waves, then store their SiLU*up results ----
+            {
+                const float4 gam0 = reinterpret_cast<const float4*>(g1)[2 * t], gam1 = reinterpret_cast<const float4*>(g1)[2 * t + 1];
+                bar.wait();
+                stamp();
+                if (t < 8) st_i(&p.o_acc[wg * 8 + t], 0);            // every reader of o_acc has passed the barrier
+                float v[8];
+#pragma unroll
+                for (int i = 0; i < 8; i++) v[i] = ld_f(&p.x2[8 * t + i]);
+                (void)norm_quant_2048_half(v, gam0, gam1, true, p.eps, true, L, NoHook());
+                __syncthreads();
+                if (t < 32) st_f(&p.h[wg * 32 + t], L.hst[t]);
+                stamp();
+                bar.arrive(true);
+            }
         }
 
-        // ================= phase 6: Hadamard R4 + quant -> down rows (8 per workgroup) + residual =================
+        // ================= phase 6: Hadamard R4 + quant -> down rows (8 per workgroup, 2 per stream wave) + residual =================
         {
-            i32x4 wr[8];
-            const int row = wg * 8 + wave;
-            mega_load_rows<8>(w.wd, I, row, lane, wr);
+            float dsc[2] = {0.0f, 0.0f}, xres[2] = {0.0f, 0.0f};
+            if (is_s) { dsc[0] = ldc_f(w.sd + wg * 8 + sw * 2); dsc[1] = ldc_f(w.sd + wg * 8 + sw * 2 + 1); }
             bar.wait();
             stamp();
+            if (is_s && lane == 0) { xres[0] = ld_f(&p.x2[wg * 8 + sw * 2]); xres[1] = ld_f(&p.x2[wg * 8 + sw * 2 + 1]); }
             // 8192-point transform on all 512 threads, stage order bits 1,2,...,12,0 (bit-exact order, see
             // fht_kernels.h).  A: i = j*2048 + t*4 + e   -> stage 1 in registers, 2..7 across lanes
             //                  B: i = (t>>8)*4096 + r*256 + (t&255) -> stages 8..11 in registers
@@ -445,6 +622,7 @@ __global__ __launch_bounds__(kMegaT, 1) void decode_mega_kernel(MegaParams p) {
             float pw = lane_xor_f<MASK>(a[j].w); a[j].w = hi ? (pw - a[j].w) : (a[j].w + pw); \
         }                                                                                     \
     }
+            if (is_s) mega_row_to_lds(w.wd, wg * 8 + sw * 2 + 1, lane, L.wd[sw * 2 + 1]);   // behind the h loads, which stage 1 has consumed
             if (l == 1) fine();
             FX_MEGA_STAGE(1) FX_MEGA_STAGE(2) FX_MEGA_STAGE(4) FX_MEGA_STAGE(8) FX_MEGA_STAGE(16) FX_MEGA_STAGE(32)
 #undef FX_MEGA_STAGE
@@ -489,9 +667,16 @@ __global__ __launch_bounds__(kMegaT, 1) void decode_mega_kernel(MegaParams p) {
             for (int r = 0; r < 16; r++) L.xq[r * 512 + t] = (int8_t)quant_round(b[r], sx);
             __syncthreads();
             if (l == 1) fine();
-            const int a0 = mega_dot_row<8>(wr, L.xq, lane);
+            if (is_s) {
+                __builtin_amdgcn_s_waitcnt(0);        // both down rows of this wave have landed in LDS
+#pragma unroll
+                for (int j = 0; j < 2; j++) {
+                    const int row = wg * 8 + sw * 2 + j;
+                    const int a0 = mega_dot_row_lds(L.wd[sw * 2 + j], L.xq, lane);
+                    if (lane == 0) st_f(&p.x[row], (float)a0 * sx * dsc[j] + xres[j]);
+                }
+            }
             if (l == 1) fine();
-            if (lane == 0) st_f(&p.x[row], (float)a0 * sx * w.sd[row] + ld_f(&p.x2[row]));
             if (l == 1) fine();
             stamp();
             bar.arrive();

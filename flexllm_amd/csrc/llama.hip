@@ -176,7 +176,13 @@ static int launch_mega(flexllm_llama* m, const int* token, const float* x_in, fl
     p.n_layers = c.layers; p.max_pos = c.max_pos; p.vocab = c.vocab; p.want_head = want_head;
     p.eps = c.eps; p.fht_scale = c.fht_scale;
     p.timeline = m->timeline;
-    decode_mega_kernel<<<kMegaWG, kMegaT, 0, st>>>(p);
+    static bool lds_opted_in = false;     // the kernel's LDS block exceeds the default 64 KiB per workgroup
+    if (!lds_opted_in) {
+        FX_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(decode_mega_kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                   (int)sizeof(MegaLds)));
+        lds_opted_in = true;
+    }
+    decode_mega_kernel<<<kMegaWG, kMegaT, sizeof(MegaLds), st>>>(p);
     FX_LAUNCH_CHECK();
     return FLEXLLM_OK;
 }
