@@ -187,36 +187,6 @@ __device__ __forceinline__ float norm_quant_2048(float (&v)[4], const float4& g,
     return sc;
 }
 
-// Same for 8 values per thread held by the first 256 threads only (thread t < 256 holds elements 8t..8t+7); the
-// other threads pass zeros and take part in the reductions and barriers only.
-template <class Hook>
-__device__ __forceinline__ float norm_quant_2048_half(float (&v)[8], const float4& g0, const float4& g1, bool do_norm, float eps,
-                                                      bool holder, MegaLds& L, Hook hook) {
-    const int t = threadIdx.x;
-    if (do_norm) {
-        float ss = ((v[0] * v[0] + v[1] * v[1]) + (v[2] * v[2] + v[3] * v[3])) + ((v[4] * v[4] + v[5] * v[5]) + (v[6] * v[6] + v[7] * v[7]));
-        ss = mega_block_sum(ss, L.red, hook);
-        const float rms = 1.0f / sqrtf(ss / 2048.0f + eps);
-        if (holder) {
-            v[0] = v[0] * rms * g0.x; v[1] = v[1] * rms * g0.y; v[2] = v[2] * rms * g0.z; v[3] = v[3] * rms * g0.w;
-            v[4] = v[4] * rms * g1.x; v[5] = v[5] * rms * g1.y; v[6] = v[6] * rms * g1.z; v[7] = v[7] * rms * g1.w;
-        }
-    }
-    float amax = fmaxf(fmaxf(fmaxf(fabsf(v[0]), fabsf(v[1])), fmaxf(fabsf(v[2]), fabsf(v[3]))),
-                       fmaxf(fmaxf(fabsf(v[4]), fabsf(v[5])), fmaxf(fabsf(v[6]), fabsf(v[7]))));
-    if (do_norm) amax = mega_block_max_h(amax, L.red, NoHook());
-    else amax = mega_block_max_h(amax, L.red, hook);
-    const float sc = sym_scale(amax, 127.0f);
-    if (holder) {
-        uint2 q;
-        q.x = pack4_i8(quant_round(v[0], sc), quant_round(v[1], sc), quant_round(v[2], sc), quant_round(v[3], sc));
-        q.y = pack4_i8(quant_round(v[4], sc), quant_round(v[5], sc), quant_round(v[6], sc), quant_round(v[7], sc));
-        reinterpret_cast<uint2*>(L.xq)[t] = q;
-    }
-    __syncthreads();
-    return sc;
-}
-
 // Weight rows are read through a pointer that is explicitly in the global address space: a generic pointer
 // would make these FLAT loads, which also count on the LDS/scalar counter, and every LDS wait of the wave
 // would then wait for the weight prefetch as well.
@@ -486,108 +456,103 @@ __global__ __launch_bounds__(kMegaT, 1) void decode_mega_kernel(MegaParams p) {
             bar.arrive(!is_s);
         }
 
-        // Phases 4 and 5 are written once per wave role; the two branches execute the same sequence of
-        // workgroup barriers (the branch condition is wave-uniform).
-        if (is_s) {
-            // ---- stream waves, phase 4: last gate/up slice, otherwise only keep step with the barriers ----
-            bar.wait();
-            stamp();
-            float z[8] = {0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f};
-            const float4 z4 = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
-            (void)norm_quant_2048_half(z, z4, z4, false, p.eps, false, L, [&]() { gu_slice(3); });
-            stamp();
-            bar.arrive(false);
-            // ---- stream waves, phase 5: first down row, gate/up rows + SiLU*up into LDS ----
-            const int ridx = 8 * (lane & 1) + 4 * ((lane >> 1) & 1) + 2 * ((lane >> 2) & 1) + ((lane >> 3) & 1);
-            const float gsc = w.sgu[wg * 64 + sw * 16 + ridx];       // read before this phase's prefetch is issued
-            bar.wait();
-            stamp();
-            const float sx = norm_quant_2048_half(z, z4, z4, true, p.eps, false, L, [&]() { mega_row_to_lds(w.wd, wg * 8 + sw * 2, lane, L.wd[sw * 2]); });
-            // sixteen per-lane partial dot products, folded with a transposing butterfly: each step halves the
-            // number of live values, so 15 + 2 cross-lane exchanges replace 16 x 6.  Afterwards lane L holds
-            // the complete sum of row 8*(L&1) + 4*(L>>1 & 1) + 2*(L>>2 & 1) + (L>>3 & 1).
-            int part[16];
-            {
-                const i32x4 x0 = reinterpret_cast<const i32x4*>(L.xq)[lane], x1 = reinterpret_cast<const i32x4*>(L.xq)[lane + 64];
+        // ================= phase 4: attention dequant + quant -> o_proj rows (8 per workgroup, 2 per wave 0..3) + residual =================
+        {
+            i32x4 wr[2][2];
+            float wsc[2] = {0.0f, 0.0f};
+            if (!is_s) {
 #pragma unroll
-                for (int r = 0; r < 16; r++) part[r] = dot16(gu[r][1], x1, dot16(gu[r][0], x0, 0));
-            }
-            int q8[8], q4[4], q2[2];
-            {
-                const bool hi = lane & 1;
-#pragma unroll
-                for (int i = 0; i < 8; i++) q8[i] = (hi ? part[i + 8] : part[i]) + lane_xor_i<1>(hi ? part[i] : part[i + 8]);
-            }
-            {
-                const bool hi = lane & 2;
-#pragma unroll
-                for (int i = 0; i < 4; i++) q4[i] = (hi ? q8[i + 4] : q8[i]) + lane_xor_i<2>(hi ? q8[i] : q8[i + 4]);
-            }
-            {
-                const bool hi = lane & 4;
-#pragma unroll
-                for (int i = 0; i < 2; i++) q2[i] = (hi ? q4[i + 2] : q4[i]) + lane_xor_i<4>(hi ? q4[i] : q4[i + 2]);
-            }
-            int sum;
-            {
-                const bool hi = lane & 8;
-                sum = (hi ? q2[1] : q2[0]) + lane_xor_i<8>(hi ? q2[0] : q2[1]);
-            }
-            sum += lane_xor_i<16>(sum);
-            sum += lane_xor_i<32>(sum);
-            const float mine = (float)sum * sx * gsc;
-            const float other = lane_xor_f<8>(mine);               // row ridx^1: the other half of the SwiGLU pair
-            if (lane < 8) L.hst[sw * 8 + (ridx >> 1)] = other * silu_f(mine);   // lanes 0..7 hold the (even) gate rows
-            __syncthreads();
-            stamp();
-            bar.arrive(false);
-        } else {
-            // ---- waves 0..3, phase 4: attention dequant + quant -> o_proj rows (8 per workgroup) + residual ----
-            {
-                i32x4 wr[2][2];
-#pragma unroll
-                for (int j = 0; j < 2; j++) mega_load_rows<2>(w.wo, H, wg * 8 + wave + 4 * j, lane, wr[j]);
-                const float wsc0 = ldc_f(w.so + wg * 8 + wave), wsc1 = ldc_f(w.so + wg * 8 + wave + 4);
-                const float osa = a_s[t >> 3], osv = v_s[t >> 5];     // elements 8t..8t+7 lie in query head t/8
-                bar.wait();
-                stamp();
-                float v[8], xr[2] = {0.0f, 0.0f};
-#pragma unroll
-                for (int i = 0; i < 8; i++) v[i] = (float)ld_i(&p.o_acc[8 * t + i]) * osa * osv;
-                if (lane == 0) {                                      // residual inputs, fetched with the activations
-#pragma unroll
-                    for (int j = 0; j < 2; j++) {
-                        const int row = wg * 8 + wave + 4 * j;
-                        if (l == 0) xr[j] = p.x_in ? p.x_in[row] : __half2float(p.embed[(size_t)tok * H + row]);
-                        else xr[j] = ld_f(&p.x[row]);
-                    }
+                for (int j = 0; j < 2; j++) {
+                    mega_load_rows<2>(w.wo, H, wg * 8 + wave + 4 * j, lane, wr[j]);
+                    wsc[j] = ldc_f(w.so + wg * 8 + wave + 4 * j);
                 }
-                const float4 z4 = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
-                const float sx = norm_quant_2048_half(v, z4, z4, false, p.eps, true, L, NoHook());
+            }
+            const float osa = a_s[t >> 4], osv = v_s[t >> 6];         // elements 4t..4t+3 lie in query head t/16
+            bar.wait();
+            stamp();
+            // the stream waves' previous slice has landed long ago, so they can share the activation loads
+            float v[4], xr[2] = {0.0f, 0.0f};
+#pragma unroll
+            for (int i = 0; i < 4; i++) v[i] = (float)ld_i(&p.o_acc[4 * t + i]) * osa * osv;
+            if (!is_s && lane == 0) {                                 // residual inputs, fetched with the activations
+#pragma unroll
+                for (int j = 0; j < 2; j++) {
+                    const int row = wg * 8 + wave + 4 * j;
+                    if (l == 0) xr[j] = p.x_in ? p.x_in[row] : __half2float(p.embed[(size_t)tok * H + row]);
+                    else xr[j] = ld_f(&p.x[row]);
+                }
+            }
+            const float4 z4 = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+            const float sx = norm_quant_2048(v, z4, false, p.eps, L, [&]() { gu_slice(3); });
+            if (!is_s) {
 #pragma unroll
                 for (int j = 0; j < 2; j++) {
                     const int row = wg * 8 + wave + 4 * j;
                     const int a0 = mega_dot_row<2>(wr[j], L.xq, lane);
-                    if (lane == 0) st_f(&p.x2[row], (float)a0 * sx * (j == 0 ? wsc0 : wsc1) + xr[j]);
+                    if (lane == 0) st_f(&p.x2[row], (float)a0 * sx * wsc[j] + xr[j]);
                 }
-                stamp();
-                bar.arrive(true);
             }
-            // ---- waves 0..3, phase 5: RMSNorm + quant for the stream waves, then store their SiLU*up results ----
-            {
-                const float4 gam0 = reinterpret_cast<const float4*>(g1)[2 * t], gam1 = reinterpret_cast<const float4*>(g1)[2 * t + 1];
-                bar.wait();
-                stamp();
-                if (t < 8) st_i(&p.o_acc[wg * 8 + t], 0);            // every reader of o_acc has passed the barrier
-                float v[8];
+            stamp();
+            bar.arrive(!is_s);
+        }
+
+        // ================= phase 5: RMSNorm + quant -> gate/up rows (64 per workgroup, 16 per stream wave) + SiLU*up =================
+        {
+            const int ridx = 8 * (lane & 1) + 4 * ((lane >> 1) & 1) + 2 * ((lane >> 2) & 1) + ((lane >> 3) & 1);
+            float gsc = 0.0f;
+            if (is_s) gsc = w.sgu[wg * 64 + sw * 16 + ridx];          // read before this phase's prefetch is issued
+            const float4 gam = reinterpret_cast<const float4*>(g1)[t];
+            bar.wait();
+            stamp();
+            if (t < 8) st_i(&p.o_acc[wg * 8 + t], 0);                // every reader of o_acc has passed the barrier
+            float v[4];
 #pragma unroll
-                for (int i = 0; i < 8; i++) v[i] = ld_f(&p.x2[8 * t + i]);
-                (void)norm_quant_2048_half(v, gam0, gam1, true, p.eps, true, L, NoHook());
-                __syncthreads();
-                if (t < 32) st_f(&p.h[wg * 32 + t], L.hst[t]);
-                stamp();
-                bar.arrive(true);
+            for (int i = 0; i < 4; i++) v[i] = ld_f(&p.x2[4 * t + i]);
+            const float sx = norm_quant_2048(v, gam, true, p.eps, L, [&]() {
+                __builtin_amdgcn_s_waitcnt(0x0F70);                   // vmcnt(0): see gu_slice
+                if (is_s) mega_row_to_lds(w.wd, wg * 8 + sw * 2, lane, L.wd[sw * 2]);
+            });
+            if (is_s) {
+                // sixteen per-lane partial dot products, folded with a transposing butterfly: each step halves
+                // the number of live values, so 15 + 2 cross-lane exchanges replace 16 x 6.  Afterwards lane L
+                // holds the complete sum of row 8*(L&1) + 4*(L>>1 & 1) + 2*(L>>2 & 1) + (L>>3 & 1).
+                int part[16];
+                {
+                    const i32x4 x0 = reinterpret_cast<const i32x4*>(L.xq)[lane], x1 = reinterpret_cast<const i32x4*>(L.xq)[lane + 64];
+#pragma unroll
+                    for (int r = 0; r < 16; r++) part[r] = dot16(gu[r][1], x1, dot16(gu[r][0], x0, 0));
+                }
+                int q8[8], q4[4], q2[2];
+                {
+                    const bool hi = lane & 1;
+#pragma unroll
+                    for (int i = 0; i < 8; i++) q8[i] = (hi ? part[i + 8] : part[i]) + lane_xor_i<1>(hi ? part[i] : part[i + 8]);
+                }
+                {
+                    const bool hi = lane & 2;
+#pragma unroll
+                    for (int i = 0; i < 4; i++) q4[i] = (hi ? q8[i + 4] : q8[i]) + lane_xor_i<2>(hi ? q8[i] : q8[i + 4]);
+                }
+                {
+                    const bool hi = lane & 4;
+#pragma unroll
+                    for (int i = 0; i < 2; i++) q2[i] = (hi ? q4[i + 2] : q4[i]) + lane_xor_i<4>(hi ? q4[i] : q4[i + 2]);
+                }
+                int sum;
+                {
+                    const bool hi = lane & 8;
+                    sum = (hi ? q2[1] : q2[0]) + lane_xor_i<8>(hi ? q2[0] : q2[1]);
+                }
+                sum += lane_xor_i<16>(sum);
+                sum += lane_xor_i<32>(sum);
+                const float mine = (float)sum * sx * gsc;
+                const float other = lane_xor_f<8>(mine);           // row ridx^1: the other half of the SwiGLU pair
+                if (lane < 8) L.hst[sw * 8 + (ridx >> 1)] = other * silu_f(mine);   // lanes 0..7 hold the (even) gate rows
             }
+            __syncthreads();
+            if (t < 32) st_f(&p.h[wg * 32 + t], L.hst[t]);           // stored by a wave with no prefetch in flight
+            stamp();
+            bar.arrive(!is_s);
         }
 
         // ================= phase 6: Hadamard R4 + quant -> down rows (8 per workgroup, 2 per stream wave) + residual =================
