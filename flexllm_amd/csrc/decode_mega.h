@@ -131,7 +131,6 @@ struct MegaLds {
     float bestv[kMegaWaves];
     int besti[kMegaWaves];
     float hst[32];                                     // SiLU(gate)*up of this workgroup's 32 row pairs, stream waves -> store wave
-    __attribute__((aligned(16))) int8_t wd[8][8192];   // this workgroup's 8 down rows, filled by global->LDS direct loads (64 KiB)
 };
 
 template <int NW>
@@ -200,11 +199,17 @@ __device__ __forceinline__ void mega_load_rows(const int8_t* __restrict__ w, int
 // One 8192-byte weight row straight from global memory into LDS (16 bytes per lane, lane i of chunk c lands
 // at byte 1024*c + 16*i): no registers are held while the row is in flight.  Counts on the vector-memory
 // counter like a load; the issuing wave waits for that counter to reach zero before it reads the row.
+// Issued from inline assembly on purpose: for the builtin form the compiler makes every later LDS access that
+// it cannot prove disjoint (all of them here) wait for the transfer, which stalls the issuing wave at once.
+// Loads the compiler does not know of only make its own counter waits stricter, never too lax: results
+// return in issue order.
 __device__ __forceinline__ void mega_row_to_lds(const int8_t* __restrict__ w, int row, int lane, int8_t* lds_row) {
-    const global_i32x4_ptr p = (global_i32x4_ptr)(uintptr_t)(w + (size_t)row * 8192);
+    const int8_t* src = w + (size_t)row * 8192 + lane * 16;
+    const unsigned dst = __builtin_amdgcn_readfirstlane((unsigned)(uintptr_t)(__attribute__((address_space(3))) void*)lds_row);
 #pragma unroll
     for (int i = 0; i < 8; i++)
-        __builtin_amdgcn_global_load_lds(p + lane + 64 * i, (__attribute__((address_space(3))) void*)(lds_row + 1024 * i), 16, 0, 0);
+        asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off"
+                     :: "v"(src + 1024 * i), "s"(dst + 1024u * i) : "memory", "m0");
 }
 __device__ __forceinline__ int mega_dot_row_lds(const int8_t* w_lds, const int8_t* xq_lds, int lane) {
     int acc = 0;
@@ -223,7 +228,11 @@ __device__ __forceinline__ int mega_dot_row(const i32x4 (&wr)[NCH], const int8_t
 }
 
 __global__ __launch_bounds__(kMegaT, 1) void decode_mega_kernel(MegaParams p) {
-    extern __shared__ __attribute__((aligned(16))) unsigned char mega_smem[];   // sizeof(MegaLds) > the static 64 KiB limit
+    // Two LDS objects: the down rows arrive by global->LDS direct loads, and the compiler makes every LDS access
+    // that might alias such a load in flight wait for it.  A variable of its own lets it tell the two apart.
+    // Together they exceed the static 64 KiB limit, so the working set is the dynamic part.
+    __shared__ __attribute__((aligned(16))) int8_t wd_lds[8][8192];             // this workgroup's 8 down rows (64 KiB)
+    extern __shared__ __attribute__((aligned(16))) unsigned char mega_smem[];
     MegaLds& L = *reinterpret_cast<MegaLds*>(mega_smem);
     const int t = threadIdx.x, lane = t & 63, wg = blockIdx.x;
     const int wave = __builtin_amdgcn_readfirstlane(t >> 6);
@@ -510,7 +519,7 @@ __global__ __launch_bounds__(kMegaT, 1) void decode_mega_kernel(MegaParams p) {
             for (int i = 0; i < 4; i++) v[i] = ld_f(&p.x2[4 * t + i]);
             const float sx = norm_quant_2048(v, gam, true, p.eps, L, [&]() {
                 __builtin_amdgcn_s_waitcnt(0x0F70);                   // vmcnt(0): see gu_slice
-                if (is_s) mega_row_to_lds(w.wd, wg * 8 + sw * 2, lane, L.wd[sw * 2]);
+                if (is_s) mega_row_to_lds(w.wd, wg * 8 + sw * 2, lane, wd_lds[sw * 2]);
             });
             if (is_s) {
                 // sixteen per-lane partial dot products, folded with a transposing butterfly: each step halves
@@ -587,7 +596,8 @@ __global__ __launch_bounds__(kMegaT, 1) void decode_mega_kernel(MegaParams p) {
             float pw = lane_xor_f<MASK>(a[j].w); a[j].w = hi ? (pw - a[j].w) : (a[j].w + pw); \
         }                                                                                     \
     }
-            if (is_s) mega_row_to_lds(w.wd, wg * 8 + sw * 2 + 1, lane, L.wd[sw * 2 + 1]);   // behind the h loads, which stage 1 has consumed
+            __builtin_amdgcn_s_waitcnt(0x0F70);               // vmcnt(0): the h loads, which stage 1 has consumed, are complete
+            if (is_s) mega_row_to_lds(w.wd, wg * 8 + sw * 2 + 1, lane, wd_lds[sw * 2 + 1]);
             if (l == 1) fine();
             FX_MEGA_STAGE(1) FX_MEGA_STAGE(2) FX_MEGA_STAGE(4) FX_MEGA_STAGE(8) FX_MEGA_STAGE(16) FX_MEGA_STAGE(32)
 #undef FX_MEGA_STAGE
@@ -637,7 +647,7 @@ __global__ __launch_bounds__(kMegaT, 1) void decode_mega_kernel(MegaParams p) {
 #pragma unroll
                 for (int j = 0; j < 2; j++) {
                     const int row = wg * 8 + sw * 2 + j;
-                    const int a0 = mega_dot_row_lds(L.wd[sw * 2 + j], L.xq, lane);
+                    const int a0 = mega_dot_row_lds(wd_lds[sw * 2 + j], L.xq, lane);
                     if (lane == 0) st_f(&p.x[row], (float)a0 * sx * dsc[j] + xres[j]);
                 }
             }
