@@ -43,6 +43,7 @@ constexpr int kMegaT = 512;        // threads per workgroup
 constexpr int kMegaWaves = kMegaT / 64;
 constexpr int kMegaGroup = 32;     // workgroups per first-level barrier counter
 constexpr int kMegaSpinLimit = 1 << 22;
+constexpr int kMegaMaxSteps = 64;  // tokens per launch in greedy mode (bounds the run time of one launch)
 
 struct MegaParams {
     const LayerW* layers;          // device array [layers]
@@ -55,7 +56,9 @@ struct MegaParams {
     int32_t* o_acc;                // [H]
     int* state;                    // [0] pos, [1] step, [2] barrier epoch base, [3] error flag
     unsigned* bar;                 // [0] flag, [64] top counter, [128+64g] group counters
-    const int* token;              // current token id (device), used when x_in == NULL
+    int* token;                    // current token id (device), used when x_in == NULL; greedy mode leaves the last token here
+    int* tokens_out;               // greedy mode: generated ids are written to tokens_out[state[1] + step]; NULL otherwise
+    int n_steps;                   // tokens per launch (> 1 only in greedy mode)
     const float* x_in;             // optional fp32 input embedding
     float* am_v;                   // [kMegaWG] argmax candidates
     int* am_i;
@@ -131,6 +134,9 @@ struct MegaLds {
     float bestv[kMegaWaves];
     int besti[kMegaWaves];
     float hst[32];                                     // SiLU(gate)*up of this workgroup's 32 row pairs, stream waves -> store wave
+    __attribute__((aligned(16))) int8_t wd[8][8192];   // this workgroup's 8 down rows, filled by global->LDS direct loads (64 KiB);
+                                                       // the odd rows first hold gate/up rows 12..15 of their stream wave
+    __attribute__((aligned(16))) int8_t gu2[4][8192];  // gate/up rows 8..11 of each stream wave (32 KiB)
 };
 
 template <int NW>
@@ -204,12 +210,22 @@ __device__ __forceinline__ void mega_load_rows(const int8_t* __restrict__ w, int
 // Loads the compiler does not know of only make its own counter waits stricter, never too lax: results
 // return in issue order.
 __device__ __forceinline__ void mega_row_to_lds(const int8_t* __restrict__ w, int row, int lane, int8_t* lds_row) {
-    const int8_t* src = w + (size_t)row * 8192 + lane * 16;
+    // scalar base + one 32-bit lane offset; the instruction offset advances the global and the LDS address alike
+    const int8_t* base = w + (size_t)row * 8192;
+    const unsigned voff = lane * 16;
     const unsigned dst = __builtin_amdgcn_readfirstlane((unsigned)(uintptr_t)(__attribute__((address_space(3))) void*)lds_row);
+    unsigned saved_m0;
 #pragma unroll
-    for (int i = 0; i < 8; i++)
-        asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off"
-                     :: "v"(src + 1024 * i), "s"(dst + 1024u * i) : "memory", "m0");
+    for (int half = 0; half < 2; half++)
+        asm volatile("s_mov_b32 %0, m0\n\t"
+                     "s_mov_b32 m0, %3\n\t"
+                     "s_nop 0\n\t"
+                     "global_load_lds_dwordx4 %1, %2\n\t"
+                     "global_load_lds_dwordx4 %1, %2 offset:1024\n\t"
+                     "global_load_lds_dwordx4 %1, %2 offset:2048\n\t"
+                     "global_load_lds_dwordx4 %1, %2 offset:3072\n\t"
+                     "s_mov_b32 m0, %0"
+                     : "=&s"(saved_m0) : "v"(voff), "s"(base + 4096 * half), "s"(dst + 4096u * half) : "memory");
 }
 __device__ __forceinline__ int mega_dot_row_lds(const int8_t* w_lds, const int8_t* xq_lds, int lane) {
     int acc = 0;
@@ -228,29 +244,35 @@ __device__ __forceinline__ int mega_dot_row(const i32x4 (&wr)[NCH], const int8_t
 }
 
 __global__ __launch_bounds__(kMegaT, 1) void decode_mega_kernel(MegaParams p) {
-    // Two LDS objects: the down rows arrive by global->LDS direct loads, and the compiler makes every LDS access
-    // that might alias such a load in flight wait for it.  A variable of its own lets it tell the two apart.
-    // Together they exceed the static 64 KiB limit, so the working set is the dynamic part.
-    __shared__ __attribute__((aligned(16))) int8_t wd_lds[8][8192];             // this workgroup's 8 down rows (64 KiB)
-    extern __shared__ __attribute__((aligned(16))) unsigned char mega_smem[];
+    extern __shared__ __attribute__((aligned(16))) unsigned char mega_smem[];   // sizeof(MegaLds) > the static 64 KiB limit
     MegaLds& L = *reinterpret_cast<MegaLds*>(mega_smem);
     const int t = threadIdx.x, lane = t & 63, wg = blockIdx.x;
     const int wave = __builtin_amdgcn_readfirstlane(t >> 6);
     const bool is_s = wave >= 4;                        // stream wave (see the file comment)
     const int sw = wave - 4;
     constexpr int H = 2048, KV = 512, I = 8192, QH = 32, KVH = 8, GROUP = 4;
-    const int pos = p.state[0];
-    const int len = pos + 1;
+    const int pos0 = p.state[0];
     GridBarrier bar{p.bar, (unsigned)p.state[2], &p.state[3]};
     int stamp_i = 0;
-    auto stamp = [&]() { if (p.timeline && wg == 0 && t == 0) p.timeline[stamp_i] = wall_clock64(); stamp_i++; };
+    // 'thread 0 of workgroup 0' from scalars and the hardware lane id: no per-thread value has to stay live for it
+    auto is_t0 = [&]() { return wave == 0 && __builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u)) == 0; };
+    auto stamp = [&]() { if (p.timeline && wg == 0 && is_t0()) p.timeline[stamp_i] = wall_clock64(); stamp_i++; };
 #ifdef FX_MEGA_FINE_STAMPS
     int fine_i = 0;
-    auto fine = [&]() { if (p.timeline && wg == 0 && t == 0 && fine_i < 64) p.timeline[p.n_layers * 12 + 2 + fine_i] = wall_clock64(); fine_i++; };
+    auto fine = [&]() { if (p.timeline && wg == 0 && is_t0() && fine_i < 64) p.timeline[p.n_layers * 12 + 2 + fine_i] = wall_clock64(); fine_i++; };
+    if (p.timeline && is_t0()) p.timeline[p.n_layers * 12 + 2 + 64 + wg] = wall_clock64();               // workgroup entry
 #else
     auto fine = [&]() {};
 #endif
-    const int tok = p.x_in ? 0 : p.token[0];
+    int tok = p.x_in ? 0 : p.token[0];
+    const bool greedy = p.tokens_out != nullptr;
+
+    // Greedy mode runs several tokens in one launch: after the lm_head every workgroup reduces the per-workgroup
+    // candidates itself, so all of them know the next token and position without a further exchange.
+    for (int step = 0; step < p.n_steps; step++) {
+    const int pos = pos0 + step;
+    const int len = pos + 1;
+    stamp_i = 0;                                                  // a timeline holds the stamps of the last step
 
     // attention work item of this workgroup
     const int a_h = wg / 32, a_c = wg % 32;
@@ -278,15 +300,25 @@ __global__ __launch_bounds__(kMegaT, 1) void decode_mega_kernel(MegaParams p) {
         // 8 KiB per wave, one per phase, each issued once the phase's activation loads have landed.  A slice
         // (8 MiB over the chip) drains while the phase computes; issuing a whole matrix at once instead fills
         // the memory queues for microseconds, and the barrier's own round trips then queue behind it.
-        i32x4 gu[16][2];
+        // Slices 0 and 1 (rows 0..7) wait in registers, slices 2 and 3 and the down rows in LDS.
+        i32x4 gu[8][2];
+        // Only the stream waves ever define these registers.  An empty asm "defines" them for every wave here,
+        // or the compiler would carry the stale values of the other waves around the layer and token loops.
+#pragma unroll
+        for (int r = 0; r < 8; r++) asm volatile("" : "=v"(gu[r][0]), "=v"(gu[r][1]));
         auto gu_slice = [&](int s) {
             // Every wave first waits for its own older loads (long landed at the points where this is called).
             // Otherwise the wait inserted for such a load after the branch below has to assume the path without
             // the slice, and it would make the stream waves sit out their own prefetch.
             __builtin_amdgcn_s_waitcnt(0x0F70);            // vmcnt(0) only
             if (is_s) {
+                if (s < 2) {
 #pragma unroll
-                for (int r = 0; r < 4; r++) mega_load_rows<2>(w.wgu, H, wg * 64 + sw * 16 + 4 * s + r, lane, gu[4 * s + r]);
+                    for (int r = 0; r < 4; r++) mega_load_rows<2>(w.wgu, H, wg * 64 + sw * 16 + 4 * s + r, lane, gu[(4 * s + r) & 7]);
+                } else {
+                    // four consecutive 2048-byte rows are one 8192-byte run
+                    mega_row_to_lds(w.wgu, wg * 16 + sw * 4 + s, lane, s == 2 ? L.gu2[sw] : L.wd[sw * 2 + 1]);
+                }
             }
         };
 
@@ -519,7 +551,7 @@ __global__ __launch_bounds__(kMegaT, 1) void decode_mega_kernel(MegaParams p) {
             for (int i = 0; i < 4; i++) v[i] = ld_f(&p.x2[4 * t + i]);
             const float sx = norm_quant_2048(v, gam, true, p.eps, L, [&]() {
                 __builtin_amdgcn_s_waitcnt(0x0F70);                   // vmcnt(0): see gu_slice
-                if (is_s) mega_row_to_lds(w.wd, wg * 8 + sw * 2, lane, wd_lds[sw * 2]);
+                if (is_s) mega_row_to_lds(w.wd, wg * 8 + sw * 2, lane, L.wd[sw * 2]);
             });
             if (is_s) {
                 // sixteen per-lane partial dot products, folded with a transposing butterfly: each step halves
@@ -529,7 +561,15 @@ __global__ __launch_bounds__(kMegaT, 1) void decode_mega_kernel(MegaParams p) {
                 {
                     const i32x4 x0 = reinterpret_cast<const i32x4*>(L.xq)[lane], x1 = reinterpret_cast<const i32x4*>(L.xq)[lane + 64];
 #pragma unroll
-                    for (int r = 0; r < 16; r++) part[r] = dot16(gu[r][1], x1, dot16(gu[r][0], x0, 0));
+                    for (int r = 0; r < 8; r++) part[r] = dot16(gu[r][1], x1, dot16(gu[r][0], x0, 0));
+                    // rows 8..15 from LDS (complete: the wait at the head of this phase's prefetch hook covered them)
+                    const i32x4* g2 = reinterpret_cast<const i32x4*>(L.gu2[sw]);
+                    const i32x4* g3 = reinterpret_cast<const i32x4*>(L.wd[sw * 2 + 1]);
+#pragma unroll
+                    for (int r = 0; r < 4; r++) {
+                        part[8 + r] = dot16(g2[lane + 64 * (2 * r + 1)], x1, dot16(g2[lane + 64 * (2 * r)], x0, 0));
+                        part[12 + r] = dot16(g3[lane + 64 * (2 * r + 1)], x1, dot16(g3[lane + 64 * (2 * r)], x0, 0));
+                    }
                 }
                 int q8[8], q4[4], q2[2];
                 {
@@ -597,7 +637,7 @@ __global__ __launch_bounds__(kMegaT, 1) void decode_mega_kernel(MegaParams p) {
         }                                                                                     \
     }
             __builtin_amdgcn_s_waitcnt(0x0F70);               // vmcnt(0): the h loads, which stage 1 has consumed, are complete
-            if (is_s) mega_row_to_lds(w.wd, wg * 8 + sw * 2 + 1, lane, wd_lds[sw * 2 + 1]);
+            if (is_s) mega_row_to_lds(w.wd, wg * 8 + sw * 2 + 1, lane, L.wd[sw * 2 + 1]);
             if (l == 1) fine();
             FX_MEGA_STAGE(1) FX_MEGA_STAGE(2) FX_MEGA_STAGE(4) FX_MEGA_STAGE(8) FX_MEGA_STAGE(16) FX_MEGA_STAGE(32)
 #undef FX_MEGA_STAGE
@@ -647,7 +687,7 @@ __global__ __launch_bounds__(kMegaT, 1) void decode_mega_kernel(MegaParams p) {
 #pragma unroll
                 for (int j = 0; j < 2; j++) {
                     const int row = wg * 8 + sw * 2 + j;
-                    const int a0 = mega_dot_row_lds(wd_lds[sw * 2 + j], L.xq, lane);
+                    const int a0 = mega_dot_row_lds(L.wd[sw * 2 + j], L.xq, lane);
                     if (lane == 0) st_f(&p.x[row], (float)a0 * sx * dsc[j] + xres[j]);
                 }
             }
@@ -660,6 +700,9 @@ __global__ __launch_bounds__(kMegaT, 1) void decode_mega_kernel(MegaParams p) {
 
     // ================= head: final RMSNorm -> lm_head rows, per-workgroup argmax candidate =================
     if (p.want_head) {
+        int t_head = threadIdx.x;                 // opaque copy, as in the layer loop: nothing per-thread stays live across it
+        asm volatile("" : "+v"(t_head));
+        const int t = t_head, lane = t & 63;
         using h16x8 = _Float16 __attribute__((ext_vector_type(8)));
         const int rows_per_wg = (p.vocab + kMegaWG - 1) / kMegaWG;
         const int row_begin = wg * rows_per_wg, row_end = min(p.vocab, row_begin + rows_per_wg);
@@ -721,14 +764,44 @@ __global__ __launch_bounds__(kMegaT, 1) void decode_mega_kernel(MegaParams p) {
         if (t == 0) {
             for (int i = 1; i < kMegaWaves; i++)
                 if (L.bestv[i] > best || (L.bestv[i] == best && L.besti[i] < bi)) { best = L.bestv[i]; bi = L.besti[i]; }
-            p.am_v[wg] = best;
-            p.am_i[wg] = bi;
+            st_f(&p.am_v[wg], best);
+            st_i(&p.am_i[wg], bi);
         }
         stamp();
+        if (greedy) {
+            // every workgroup picks the winner among the kMegaWG candidates (largest value, then smallest index)
+            bar.arrive();
+            bar.wait();
+            float cv = -INFINITY;
+            int ci = 0x7fffffff;
+            if (t < kMegaWG) { cv = ld_f(&p.am_v[t]); ci = ld_i(&p.am_i[t]); }
+#pragma unroll
+            for (int m = 1; m < 64; m <<= 1) {
+                const float ov = __shfl_xor(cv, m);
+                const int oi = __shfl_xor(ci, m);
+                if (ov > cv || (ov == cv && oi < ci)) { cv = ov; ci = oi; }
+            }
+            if (lane == 0) { L.bestv[t >> 6] = cv; L.besti[t >> 6] = ci; }
+            __syncthreads();
+            cv = L.bestv[0]; ci = L.besti[0];
+#pragma unroll
+            for (int i = 1; i < kMegaWG / 64; i++)
+                if (L.bestv[i] > cv || (L.bestv[i] == cv && L.besti[i] < ci)) { cv = L.bestv[i]; ci = L.besti[i]; }
+            tok = __builtin_amdgcn_readfirstlane(ci == 0x7fffffff ? 0 : ci);
+            if (wg == 0 && t == 0) p.tokens_out[p.state[1] + step] = tok;
+            __syncthreads();                                        // L.bestv/besti are reused by the next step
+        }
     } else {
         bar.wait();   // keep arrive/wait balanced: the last layer's x is complete when the kernel ends
     }
-    if (wg == 0 && t == 0) p.state[2] = (int)bar.epoch;
+    }   // step loop
+    if (wg == 0 && is_t0()) {
+        p.state[2] = (int)bar.epoch;
+        if (greedy) { p.token[0] = tok; p.state[0] = pos0 + p.n_steps; p.state[1] += p.n_steps; }
+    }
+#ifdef FX_MEGA_FINE_STAMPS
+    if (p.timeline && is_t0()) p.timeline[p.n_layers * 12 + 2 + 64 + kMegaWG + wg] = wall_clock64();     // workgroup exit
+#endif
 }
 
 }  // namespace fx

@@ -162,7 +162,9 @@ static int decode_head(flexllm_llama* m, float* logits, hipStream_t st) {
     return lm_head_launch(m->embed, m->nrm, logits, c.vocab, c.hidden, st);
 }
 
-static int launch_mega(flexllm_llama* m, const int* token, const float* x_in, float* logits, int want_head, hipStream_t st) {
+// tokens_out != NULL: greedy mode, `steps` tokens in this launch (argmax, token hand-over and position advance inside the kernel)
+static int launch_mega(flexllm_llama* m, int* token, const float* x_in, float* logits, int want_head, hipStream_t st,
+                       int* tokens_out = nullptr, int steps = 1) {
     const flexllm_llama_config& c = m->cfg;
     MegaParams p;
     p.layers = m->layers_dev;
@@ -172,7 +174,7 @@ static int launch_mega(flexllm_llama* m, const int* token, const float* x_in, fl
     p.k_cache = m->k_cache; p.v_cache = m->v_cache; p.cache_layer_bytes = m->cache_layer_bytes;
     p.x = m->x; p.x2 = m->x2; p.qkv = m->qkv; p.h = m->h; p.logits = logits ? logits : m->logits;
     p.stats = m->stats; p.o_acc = m->o_acc; p.state = m->state; p.bar = m->bar;
-    p.token = token; p.x_in = x_in; p.am_v = m->am_v; p.am_i = m->am_i;
+    p.token = token; p.tokens_out = tokens_out; p.n_steps = steps; p.x_in = x_in; p.am_v = m->am_v; p.am_i = m->am_i;
     p.n_layers = c.layers; p.max_pos = c.max_pos; p.vocab = c.vocab; p.want_head = want_head;
     p.eps = c.eps; p.fht_scale = c.fht_scale;
     p.timeline = m->timeline;
@@ -192,13 +194,6 @@ static inline bool use_mega(const flexllm_llama* m) { return m->mega_ok && m->de
 // One greedy step: embedding of *token_io -> layers -> head -> argmax -> *token_io, tokens_out[step], pos++.
 static int greedy_step(flexllm_llama* m, int* token_io, int* tokens_out, hipStream_t st) {
     const flexllm_llama_config& c = m->cfg;
-    if (use_mega(m)) {
-        int rc = launch_mega(m, token_io, nullptr, nullptr, 1, st);
-        if (rc) return rc;
-        argmax_final_advance_kernel<<<1, 64, 0, st>>>(m->am_v, m->am_i, kMegaWG, token_io, tokens_out, m->state);
-        FX_LAUNCH_CHECK();
-        return FLEXLLM_OK;
-    }
     embed_kernel<<<(c.hidden + 255) / 256, 256, 0, st>>>(reinterpret_cast<const __half*>(m->embed), token_io, m->x, c.hidden);
     int rc;
     for (int l = 0; l < c.layers; l++)
@@ -345,7 +340,7 @@ int flexllm_llama_set_decode_mode(flexllm_llama* m, int mode) {
 
 int flexllm_llama_stage_timeline(flexllm_llama* m, long long* host_out, int max_entries) {
     FX_REQUIRE(m && host_out && max_entries > 0, "llama_stage_timeline: bad arguments");
-    const int n = m->cfg.layers * 12 + 2 + 64;
+    const int n = m->cfg.layers * 12 + 2 + 64 + 2 * fx::kMegaWG;    // stage stamps, fine stamps, per-workgroup entry and exit
     if (!m->timeline) {
         int rc = dev_alloc(m, (void**)&m->timeline, sizeof(long long) * n);
         if (rc) return rc;
@@ -413,6 +408,14 @@ int flexllm_llama_decode_greedy(flexllm_llama* m, int* token_io, int pos0, int s
     hipStream_t st = as_stream(stream);
     set_state_kernel<<<1, 1, 0, st>>>(m->state, pos0, 0);
     FX_LAUNCH_CHECK();
+    if (use_mega(m)) {
+        // the persistent kernel generates up to kMegaMaxSteps tokens per launch; a graph would have nothing to add
+        for (int s = 0; s < steps; s += kMegaMaxSteps) {
+            int rc = launch_mega(m, token_io, nullptr, nullptr, 1, st, tokens_out, steps - s < kMegaMaxSteps ? steps - s : kMegaMaxSteps);
+            if (rc) return rc;
+        }
+        return FLEXLLM_OK;
+    }
     if (!use_graph) {
         for (int s = 0; s < steps; s++) {
             int rc = greedy_step(m, token_io, tokens_out, st);
