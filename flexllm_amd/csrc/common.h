@@ -63,6 +63,8 @@ template <int MASK>
 __device__ __forceinline__ float lane_xor_f(float v) {
     return __int_as_float(lane_xor_i<MASK>(__float_as_int(v)));
 }
+// SiLU as the reference evaluates it: x / (1 + exp(-x)), one IEEE division.
+__device__ __forceinline__ float silu_f(float v) { return v / (1.0f + expf(-v)); }
 
 __device__ __forceinline__ float wave_max(float v) {
     v = fmaxf(v, lane_xor_f<1>(v));

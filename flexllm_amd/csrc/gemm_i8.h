@@ -154,16 +154,252 @@ __global__ __launch_bounds__(256) void gemm_i8_kernel(const int8_t* __restrict__
         }
 }
 
+// ---------------------------------------------------------------------------------------------------------
+// Second kernel: tiles go global -> LDS by direct loads (global_load_lds_dwordx4), bypassing registers, three
+// stages deep.  Tile BM x BN x 64, 4 waves (2x2), wave tile (BM/2)x(BN/2); at 256x256 every fragment read from
+// LDS feeds four MFMAs, which halves the LDS traffic per operation of the 128x128 tile.
+//
+// LDS stage layout: row-major, 64 bytes (= four 16-byte k-chunks) per tile row.  A direct load writes lane i
+// at base + 16*i, i.e. four lanes per row, which is also the coalesced order in global memory.  To keep the
+// MFMA fragment reads (32 rows x one chunk) free of bank conflicts the chunks of a row are stored rotated:
+// slot s of row r holds k-chunk s ^ ((r >> 2) & 3).  The rotation is applied on the global side of the
+// direct load (the LDS side is fixed by the hardware).
+//
+// The loads are issued from inline assembly: the compiler does not track them, so the k-loop waits for them
+// with explicit counters (results return in issue order).
+__host__ __device__ constexpr int gemm_dma_lds_bytes(int bm, int bn, int stages) {
+    return stages * (bm + bn) * 64 > 4 * 32 * 36 * 4 ? stages * (bm + bn) * 64 : 4 * 32 * 36 * 4;   // stages, or the four epilogue patches
+}
+
+enum GemmDmaEpi { kDmaRaw = 0, kDmaDequant = 1, kDmaSwiglu = 2 };
+
+__device__ __forceinline__ void gemm_dma_issue(const int8_t* base, unsigned voff, unsigned lds_dst) {
+    unsigned saved_m0;
+    asm volatile("s_mov_b32 %0, m0\n\t"
+                 "s_mov_b32 m0, %3\n\t"
+                 "s_nop 0\n\t"
+                 "global_load_lds_dwordx4 %1, %2\n\t"
+                 "s_mov_b32 m0, %0"
+                 : "=&s"(saved_m0) : "v"(voff), "s"(base), "s"(lds_dst) : "memory");
+}
+
+template <int N>
+__device__ __forceinline__ void gemm_wait_vmcnt() {            // s_waitcnt vmcnt(N) only; the count is a 6-bit split immediate
+    static_assert(N >= 0 && N < 64, "vmcnt range");
+    __builtin_amdgcn_s_waitcnt(0x0F70 | (N & 15) | ((N >> 4) << 14));
+}
+
+// kDmaStages LDS stages; WPE = waves per SIMD the register allocation has to leave room for
+template <int BM, int BN, int EPI, int kDmaStages, int WPE>
+__global__ __launch_bounds__(256, WPE) void gemm_i8_dma_kernel(const int8_t* __restrict__ a, const int8_t* __restrict__ w,
+                                                          int32_t* __restrict__ c_out, const float* __restrict__ s_x,
+                                                          const float* __restrict__ w_s, const float* __restrict__ residual,
+                                                          float* __restrict__ y, int m, int k, int n, int tiles_m, int tiles_n) {
+    constexpr int WM = BM / 2, WN = BN / 2, TM = WM / 32, TN = WN / 32;
+    constexpr int A_INSTR = BM / 64, B_INSTR = BN / 64;       // direct loads per wave per stage (16 rows each)
+    constexpr int STAGE = (BM + BN) * 64;
+    extern __shared__ __attribute__((aligned(16))) int8_t gemm_smem[];
+
+    int tm, tn;
+    if ((tiles_n & 7) == 0) {                                  // see gemm_i8_kernel: one range of weight columns per XCD
+        const int xcd = blockIdx.x & 7, idx = blockIdx.x >> 3;
+        tn = xcd * (tiles_n >> 3) + idx / tiles_m;
+        tm = idx % tiles_m;
+    } else {
+        tm = blockIdx.x / tiles_n;
+        tn = blockIdx.x % tiles_n;
+    }
+    int row0 = tm * BM, col0 = tn * BN;
+    const int t = threadIdx.x, lane = t & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(t >> 6);
+    const int wm = (wave >> 1) * WM, wn = (wave & 1) * WN;
+
+    // per-lane global offsets of this wave's direct loads (without the k offset, which is uniform)
+    unsigned offa[A_INSTR], offb[B_INSTR];
+#pragma unroll
+    for (int j = 0; j < A_INSTR; j++) {
+        const int r = (wave * A_INSTR + j) * 16 + (lane >> 2);
+        offa[j] = (unsigned)min(row0 + r, m - 1) * (unsigned)k + (unsigned)(((lane & 3) ^ ((r >> 2) & 3)) * 16);
+    }
+#pragma unroll
+    for (int j = 0; j < B_INSTR; j++) {
+        const int r = (wave * B_INSTR + j) * 16 + (lane >> 2);
+        offb[j] = (unsigned)min(col0 + r, n - 1) * (unsigned)k + (unsigned)(((lane & 3) ^ ((r >> 2) & 3)) * 16);
+    }
+    const unsigned lds0 = (unsigned)(uintptr_t)(__attribute__((address_space(3))) void*)gemm_smem;
+    auto issue_stage = [&](int kt) {
+        const unsigned sb = lds0 + (unsigned)(kt % kDmaStages) * STAGE;
+#pragma unroll
+        for (int j = 0; j < A_INSTR; j++) gemm_dma_issue(a + (size_t)kt * kGemmBK, offa[j], sb + (wave * A_INSTR + j) * 1024);
+#pragma unroll
+        for (int j = 0; j < B_INSTR; j++) gemm_dma_issue(w + (size_t)kt * kGemmBK, offb[j], sb + BM * 64 + (wave * B_INSTR + j) * 1024);
+    };
+
+    i32x16 acc[TM][TN];
+#pragma unroll
+    for (int i = 0; i < TM; i++)
+#pragma unroll
+        for (int j = 0; j < TN; j++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) acc[i][j][r] = 0;
+
+    const int nk = k / kGemmBK;
+    constexpr int PER = A_INSTR + B_INSTR;                     // direct loads per wave per stage
+#pragma unroll
+    for (int s0 = 0; s0 < kDmaStages - 1; s0++)
+        if (s0 < nk) issue_stage(s0);
+    // fragment addressing: lane l reads row (l % 32) of a 32-row tile, k-chunk 2*ks + l/32, from its rotated slot
+    const int fr = lane & 31, fg = lane >> 5;
+    auto read_frags = [&](int kt, int ks, i32x4 (&fa)[TM], i32x4 (&fb)[TN]) {
+        const int8_t* sa = gemm_smem + (kt % kDmaStages) * STAGE;
+        const int8_t* sb = sa + BM * 64;
+#pragma unroll
+        for (int i = 0; i < TM; i++) {
+            const int r = wm + i * 32 + fr;
+            fa[i] = *reinterpret_cast<const i32x4*>(sa + r * 64 + (((ks * 2 + fg) ^ ((r >> 2) & 3)) * 16));
+        }
+#pragma unroll
+        for (int j = 0; j < TN; j++) {
+            const int r = wn + j * 32 + fr;
+            fb[j] = *reinterpret_cast<const i32x4*>(sb + r * 64 + (((ks * 2 + fg) ^ ((r >> 2) & 3)) * 16));
+        }
+    };
+    auto mma = [&](const i32x4 (&fa)[TM], const i32x4 (&fb)[TN]) {
+#pragma unroll
+        for (int i = 0; i < TM; i++)
+#pragma unroll
+            for (int j = 0; j < TN; j++)
+                acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[i], fb[j], acc[i][j], 0, 0, 0);
+    };
+    // stage kt has landed once only the younger stages in flight remain outstanding
+    auto wait_stage = [&](int kt) {
+        const int younger = min(kDmaStages - 2, nk - 1 - kt);
+        if (younger >= 3) gemm_wait_vmcnt<3 * PER>();
+        else if (younger == 2) gemm_wait_vmcnt<2 * PER>();
+        else if (younger == 1) gemm_wait_vmcnt<PER>();
+        else gemm_wait_vmcnt<0>();
+    };
+
+    // Software pipeline over half-stages (32 k-bytes): the fragments of the next half-stage are read from LDS
+    // before the MFMAs of the current one are issued, so the LDS latency runs under matrix work.  The
+    // workgroup barrier sits in the middle of an iteration: after it stage kt+1 is complete in LDS and every
+    // wave has finished reading stage kt, whose buffer the direct loads of the iteration after next overwrite.
+    i32x4 fa0[TM], fb0[TN], fa1[TM], fb1[TN];
+    wait_stage(0);
+    __syncthreads();
+    read_frags(0, 0, fa0, fb0);
+    for (int kt = 0; kt < nk; kt++) {
+        read_frags(kt, 1, fa1, fb1);
+        if (kt + kDmaStages - 1 < nk) issue_stage(kt + kDmaStages - 1);   // into the buffer that held stage kt-1
+        __builtin_amdgcn_sched_barrier(0);
+        mma(fa0, fb0);
+        __builtin_amdgcn_sched_barrier(0);
+        if (kt + 1 < nk) {
+            wait_stage(kt + 1);
+            __syncthreads();
+            read_frags(kt + 1, 0, fa0, fb0);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        mma(fa1, fb1);
+        __builtin_amdgcn_sched_barrier(0);
+    }
+
+    // Epilogue.  In the accumulator layout a lane holds ONE column (l%32) and 16 rows of a 32x32 tile, so direct
+    // stores would be 4 bytes per lane.  Each wave instead turns its tiles through a private LDS patch
+    // (32 x 36 words) and then owns 4 consecutive columns of a row: 16-byte loads of the residual, 16-byte stores
+    // (8 bytes for the SiLU*up pairs), 128 contiguous bytes per row.
+    __syncthreads();                                           // all waves are done with the stage buffers
+    constexpr int EP = 36;                                     // patch pitch in words (rows stay 16-byte aligned)
+    int* patch = reinterpret_cast<int*>(gemm_smem) + wave * (32 * EP);
+    const int pr = lane >> 3, pc = (lane & 7) * 4;             // row within a group of 8, first of this lane's 4 columns
+#pragma unroll
+    for (int j = 0; j < TN; j++) {
+        const int col = col0 + wn + j * 32 + pc;               // n is a multiple of 4 (checked by the launcher)
+        const bool col_ok = col < n;
+        float4 ws = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+        if constexpr (EPI != kDmaRaw) { if (col_ok) ws = *reinterpret_cast<const float4*>(w_s + col); }
+#pragma unroll
+        for (int i = 0; i < TM; i++) {
+#pragma unroll
+            for (int r = 0; r < 16; r++)
+                patch[((r >> 2) * 8 + (lane >> 5) * 4 + (r & 3)) * EP + (lane & 31)] = acc[i][j][r];
+            // the patch is private to the wave: the LDS operations of a wave complete in order, the compiler is kept from
+            // moving them across this point
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+#pragma unroll
+            for (int p = 0; p < 4; p++) {
+                const int lr = p * 8 + pr;
+                const int row = row0 + wm + i * 32 + lr;
+                const i32x4 v = *reinterpret_cast<const i32x4*>(patch + lr * EP + pc);
+                if (!(col_ok && row < m)) continue;
+                if constexpr (EPI == kDmaRaw) {
+                    *reinterpret_cast<i32x4*>(c_out + (size_t)row * n + col) = v;
+                } else {
+                    const float sx = s_x[row];
+                    float4 o;
+                    o.x = (float)v[0] * sx * ws.x; o.y = (float)v[1] * sx * ws.y;
+                    o.z = (float)v[2] * sx * ws.z; o.w = (float)v[3] * sx * ws.w;
+                    if constexpr (EPI == kDmaDequant) {
+                        if (residual) {
+                            const float4 rs = *reinterpret_cast<const float4*>(residual + (size_t)row * n + col);
+                            o.x = o.x + rs.x; o.y = o.y + rs.y; o.z = o.z + rs.z; o.w = o.w + rs.w;
+                        }
+                        *reinterpret_cast<float4*>(y + (size_t)row * n + col) = o;
+                    } else {
+                        // weight rows are interleaved (2c gate, 2c+1 up): columns (col, col+1) and (col+2, col+3) are pairs
+                        float2 h;
+                        h.x = o.y * silu_f(o.x);
+                        h.y = o.w * silu_f(o.z);
+                        *reinterpret_cast<float2*>(y + (size_t)row * (n >> 1) + (col >> 1)) = h;
+                    }
+                }
+            }
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            __builtin_amdgcn_wave_barrier();               // reads of this tile before the next tile's writes
+            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        }
+    }
+}
+
+template <int BM, int BN, int EPI, int STAGES = 3, int WPE = 1>
+inline int launch_gemm_dma(const int8_t* a, const int8_t* w, int32_t* c, const float* s_x, const float* w_s,
+                           const float* residual, float* y, int m, int k, int n, hipStream_t st) {
+    static bool opted_in = false;             // more than the default 64 KiB of LDS per workgroup
+    if (!opted_in) {
+        FX_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_i8_dma_kernel<BM, BN, EPI, STAGES, WPE>),
+                                   hipFuncAttributeMaxDynamicSharedMemorySize, gemm_dma_lds_bytes(BM, BN, STAGES)));
+        opted_in = true;
+    }
+    const int tm = (m + BM - 1) / BM, tn = (n + BN - 1) / BN;
+    gemm_i8_dma_kernel<BM, BN, EPI, STAGES, WPE><<<tm * tn, 256, gemm_dma_lds_bytes(BM, BN, STAGES), st>>>(a, w, c, s_x, w_s, residual, y, m, k, n, tm, tn);
+    FX_LAUNCH_CHECK();
+    return FLEXLLM_OK;
+}
+
 template <int EPI>
 inline int launch_gemm(const int8_t* a, const int8_t* w, int32_t* c, const float* s_x, const float* w_s,
                        const float* residual, float* y, int m, int k, int n, hipStream_t st) {
-    // Measured on MI355X at M=1024: 128x128 tiles win once there are >= 4 workgroups per CU (gate/up), 64x64
-    // tiles win for the narrow projections (more workgroups hide the per-k-step barrier better).
+    // Measured on MI355X at M=1024: the direct-load kernel wins wherever it applies; 128x128 tiles once they fill
+    // the chip about three times over (gate/up), 64x64 tiles for the narrow projections.  FLEXLLM_GEMM_TILE
+    // forces a variant (0..2: register-staged 128x128 / 64x128 / 64x64, 10..13: direct-load 256x256 / 128x128 /
+    // 128x256 / 64x64).
     auto tiles = [&](int bm, int bn) { return ((m + bm - 1) / bm) * ((n + bn - 1) / bn); };
     static const char* force = getenv("FLEXLLM_GEMM_TILE");
-    int mode = tiles(128, 128) >= 1024 ? 0 : 2;
+    // the direct-load kernel needs 32-bit element offsets into both operands and 16-byte aligned output rows
+    const bool dma_ok = (size_t)m * k < (1ull << 31) && (size_t)n * k < (1ull << 31) && n % 4 == 0;
+    int mode = dma_ok ? (tiles(128, 128) >= 768 ? 11 : 13) : (tiles(128, 128) >= 1024 ? 0 : 2);
     if (force) mode = atoi(force);
+    if (mode >= 10 && !dma_ok) mode = 2;
     const int nk = k / kGemmBK;
+    if (mode >= 10) {
+        constexpr int DE = EPI == kGemmDequant ? kDmaDequant : kDmaRaw;
+        if (mode == 10) return launch_gemm_dma<256, 256, DE>(a, w, c, s_x, w_s, residual, y, m, k, n, st);
+        if (mode == 11) return launch_gemm_dma<128, 128, DE>(a, w, c, s_x, w_s, residual, y, m, k, n, st);
+        if (mode == 12) return launch_gemm_dma<128, 256, DE>(a, w, c, s_x, w_s, residual, y, m, k, n, st);
+        return launch_gemm_dma<64, 64, DE>(a, w, c, s_x, w_s, residual, y, m, k, n, st);
+    }
 #define FX_GEMM_LAUNCH(BM, BN, DD)                                                                                \
     do {                                                                                                          \
         const int tm = (m + BM - 1) / BM, tn = (n + BN - 1) / BN;                                                 \
@@ -176,6 +412,23 @@ inline int launch_gemm(const int8_t* a, const int8_t* w, int32_t* c, const float
 #undef FX_GEMM_LAUNCH
     FX_LAUNCH_CHECK();
     return FLEXLLM_OK;
+}
+
+// Gate/up projection with the SiLU(gate)*up product in the epilogue; n2 = 2 * intermediate size (interleaved rows).
+inline int launch_gemm_swiglu(const int8_t* a, const int8_t* w_gu, const float* s_x, const float* w_s_gu, float* h, int m,
+                              int k, int n2, hipStream_t st) {
+    FX_REQUIRE((size_t)m * k < (1ull << 31) && (size_t)n2 * k < (1ull << 31) && n2 % 4 == 0,
+               "linear_i8_gemm_swiglu: m=%d k=%d n=%d outside the direct-load kernel's range", m, k, n2 / 2);
+    // Measured at M=1024, 2048 -> 2x8192: 128x256 tiles, two stages, two workgroups per CU (one round of 512
+    // workgroups) beat 128x128 tiles (1024 workgroups in three slots per CU: a second, mostly empty round).
+    static const char* force = getenv("FLEXLLM_GEMM_TILE");
+    const int tiles_big = ((m + 127) / 128) * ((n2 + 255) / 256);
+    int mode = tiles_big >= 384 ? 16 : 13;
+    if (force) mode = atoi(force);
+    if (mode == 10) return launch_gemm_dma<256, 256, kDmaSwiglu>(a, w_gu, nullptr, s_x, w_s_gu, nullptr, h, m, k, n2, st);
+    if (mode == 11) return launch_gemm_dma<128, 128, kDmaSwiglu, 3, 3>(a, w_gu, nullptr, s_x, w_s_gu, nullptr, h, m, k, n2, st);
+    if (mode == 12 || mode == 16) return launch_gemm_dma<128, 256, kDmaSwiglu, 2, 2>(a, w_gu, nullptr, s_x, w_s_gu, nullptr, h, m, k, n2, st);
+    return launch_gemm_dma<64, 64, kDmaSwiglu>(a, w_gu, nullptr, s_x, w_s_gu, nullptr, h, m, k, n2, st);
 }
 
 }  // namespace fx

@@ -72,7 +72,6 @@ constexpr int kGemvWaves = kGemvBlock / kWave;
 
 enum GemvEpi { kEpiRaw = 0, kEpiDequant = 1, kEpiSwiglu = 2 };
 
-__device__ __forceinline__ float silu_f(float v) { return v / (1.0f + expf(-v)); }
 
 // rows_per_wave consecutive rows per wave; grid covers ceil(n / (4*rows_per_wave)) blocks.
 //   kEpiRaw:     acc_out[row] = sum

@@ -70,8 +70,8 @@ int llama_prefill_run(const flexllm_llama_config& c, const LayerW* layers, const
         if ((rc = launch_gemm<kGemmDequant>(b.xq, w.wo, nullptr, b.xs, w.so, b.x, b.x2, s, H, H, st))) return rc;
         // feed-forward block
         rmsnorm_kernel<2, true><<<s, kBlock, 0, st>>>(b.x2, g1, nullptr, b.xq, b.xs, H, c.eps);
-        if ((rc = launch_gemm<kGemmDequant>(b.xq, w.wgu, nullptr, b.xs, w.sgu, nullptr, b.gu, s, H, 2 * I, st))) return rc;
-        fht_kernel<13, true, true><<<s, kFhtBlock, 0, st>>>(b.gu, nullptr, b.xq, b.xs, c.fht_scale);
+        if ((rc = launch_gemm_swiglu(b.xq, w.wgu, b.xs, w.sgu, b.gu, s, H, 2 * I, st))) return rc;     // b.gu = SiLU(gate)*up [s][I]
+        fht_kernel<13, true, false><<<s, kFhtBlock, 0, st>>>(b.gu, nullptr, b.xq, b.xs, c.fht_scale);
         if ((rc = launch_gemm<kGemmDequant>(b.xq, w.wd, nullptr, b.xs, w.sd, b.x2, b.x, s, I, H, st))) return rc;
     }
     FX_LAUNCH_CHECK();

@@ -78,6 +78,15 @@ def linear_i8_gemv_dequant(x, s_x, w, w_s, residual=None, stream=None, out=None)
     return y
 
 
+def linear_i8_gemv_swiglu(x, s_x, w_gu, w_s_gu, stream=None, out=None):
+    """x int8 [k], w_gu int8 [2n][k] (rows interleaved gate, up) -> y fp32 [n] = up * silu(gate)."""
+    k = x.shape[-1]
+    n = w_gu.shape[0] // 2
+    y = out if out is not None else DeviceArray((n,), np.float32)
+    check(lib().flexllm_linear_i8_gemv_swiglu(_p(x), _p(s_x), _p(w_gu), _p(w_s_gu), _p(y), k, n, _s(stream)))
+    return y
+
+
 def linear_i8_gemm(a, w, stream=None, out=None):
     m, k = a.shape
     n = w.shape[0]
@@ -92,6 +101,15 @@ def linear_i8_gemm_dequant(a, s_x, w, w_s, residual=None, stream=None, out=None)
     y = out if out is not None else DeviceArray((m, n), np.float32)
     check(lib().flexllm_linear_i8_gemm_dequant(_p(a), _p(s_x), _p(w), _p(w_s), _p(residual), _p(y), m, k, n, _s(stream)))
     return y
+
+
+def linear_i8_gemm_swiglu(a, s_x, w_gu, w_s_gu, stream=None, out=None):
+    """a int8 [m][k], w_gu int8 [2n][k] (rows interleaved gate, up) -> h fp32 [m][n] = up * silu(gate)."""
+    m, k = a.shape
+    n = w_gu.shape[0] // 2
+    h = out if out is not None else DeviceArray((m, n), np.float32)
+    check(lib().flexllm_linear_i8_gemm_swiglu(_p(a), _p(s_x), _p(w_gu), _p(w_s_gu), _p(h), m, k, n, _s(stream)))
+    return h
 
 
 # ---------------------------------------------------------------- FHT.h

@@ -111,6 +111,14 @@ int flexllm_linear_i8_gemm(const int8_t* a, const int8_t* w, int32_t* acc, int m
  * = GEMM + pref_dequant_layer_qint_fp32 (Modules/quant.h:115-164) (+ pref_Residual_Layer). */
 int flexllm_linear_i8_gemm_dequant(const int8_t* a, const float* s_x, const int8_t* w, const float* w_s,
                                    const float* residual, float* y, int m, int k, int n, void* stream);
+/* Fused prefill gate/up projection + SwiGLU, the GEMM counterpart of flexllm_linear_i8_gemv_swiglu: w_gu is int8
+ * [2n][k] with rows interleaved (row 2i = gate_i, row 2i+1 = up_i), w_s_gu the matching 2n scales;
+ * h[m][i] = up_i * (gate_i/(1+exp(-gate_i))) with gate/up = (float(acc)*s_x[m])*w_s_gu[.].  Row m of h equals
+ * the GEMV entry point's result for token m bit for bit.  = two pref_Linear_Layer + pref_dequant
+ * (Modules/quant.h:115-164) + pref_Swish (Modules/Swish.h:7-24) + pref_Gate_Layer_fp32xfp32
+ * (Modules/Linear_Layer.h:1083-1101).  k % 64 == 0, n even. */
+int flexllm_linear_i8_gemm_swiglu(const int8_t* a, const float* s_x, const int8_t* w_gu, const float* w_s_gu, float* h,
+                                  int m, int k, int n, void* stream);
 
 /* ---- FHT.h ---------------------------------------------------------------------------- */
 /* y = H_n x / scale (Sylvester order, butterfly stage order of the reference's omega network, so

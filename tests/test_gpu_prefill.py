@@ -53,6 +53,28 @@ def test_gemm_dequant_residual_bit_exact(fx, oracle):
     assert np.array_equal(yv, y[5])
 
 
+@pytest.mark.parametrize("m,k,n", [(160, 2048, 384), (64, 128, 32), (1024, 2048, 8192), (33, 64, 6)])
+def test_gemm_swiglu(fx, oracle, m, k, n):
+    """Gate/up GEMM with SiLU(gate)*up in the epilogue: == dequant GEMM + gate layer on the device bit for bit, == the
+    decode GEMV entry point row by row, and == the oracle up to the device's expf (<= 2 ulp -> 2e-6 relative)."""
+    x = rng.standard_normal((m, k)).astype(np.float32)
+    w = rng.integers(-127, 128, (2 * n, k)).astype(np.int8)           # rows interleaved: 2i gate, 2i+1 up
+    w_s = rng.uniform(1e-3, 1e-2, 2 * n).astype(np.float32)
+    q, s = fx.ops.quant_sym_i8(fx.to_device(x))
+    dw, dws = fx.to_device(w), fx.to_device(w_s)
+    h = fx.ops.linear_i8_gemm_swiglu(q, s, dw, dws).numpy()
+    assert h.shape == (m, n)
+    gu = fx.ops.linear_i8_gemm_dequant(q, s, dw, dws).numpy()
+    gate, up = np.ascontiguousarray(gu[:, 0::2]), np.ascontiguousarray(gu[:, 1::2])
+    assert np.array_equal(h, fx.ops.swiglu_f32(fx.to_device(gate), fx.to_device(up)).numpy())
+    q_ref, s_ref = oracle.quant_sym(x)
+    gu_ref = oracle.dequant(oracle.linear_i8(q_ref, w), s_ref, w_s)
+    np.testing.assert_allclose(h, oracle.gate(gu_ref[:, 1::2], oracle.swish(gu_ref[:, 0::2])), rtol=2e-6, atol=1e-30)
+    for row in (0, m - 1):
+        hv = fx.ops.linear_i8_gemv_swiglu(fx.to_device(q_ref[row]), fx.to_device(s_ref[row:row + 1]), dw, dws).numpy()
+        assert np.array_equal(hv, h[row])
+
+
 def mha_scales(qh=32, kvh=8, seed=3):
     r = np.random.default_rng(seed)
     return (r.uniform(0.003, 0.005, qh).astype(np.float32), r.uniform(0.02, 0.04, kvh).astype(np.float32),
