@@ -190,7 +190,7 @@ __device__ __forceinline__ void gemm_wait_vmcnt() {            // s_waitcnt vmcn
 }
 
 // kDmaStages LDS stages; WPE = waves per SIMD the register allocation has to leave room for
-template <int BM, int BN, int EPI, int kDmaStages, int WPE>
+template <int BM, int BN, int EPI, int kDmaStages, int WPE>   // at most 7 stages (the wait below distinguishes up to 5 younger ones)
 __global__ __launch_bounds__(256, WPE) void gemm_i8_dma_kernel(const int8_t* __restrict__ a, const int8_t* __restrict__ w,
                                                           int32_t* __restrict__ c_out, const float* __restrict__ s_x,
                                                           const float* __restrict__ w_s, const float* __restrict__ residual,
@@ -274,7 +274,9 @@ __global__ __launch_bounds__(256, WPE) void gemm_i8_dma_kernel(const int8_t* __r
     // stage kt has landed once only the younger stages in flight remain outstanding
     auto wait_stage = [&](int kt) {
         const int younger = min(kDmaStages - 2, nk - 1 - kt);
-        if (younger >= 3) gemm_wait_vmcnt<3 * PER>();
+        if (younger >= 5) gemm_wait_vmcnt<(5 * PER < 64 ? 5 * PER : 63)>();
+        else if (younger == 4) gemm_wait_vmcnt<(4 * PER < 64 ? 4 * PER : 63)>();
+        else if (younger == 3) gemm_wait_vmcnt<3 * PER>();
         else if (younger == 2) gemm_wait_vmcnt<2 * PER>();
         else if (younger == 1) gemm_wait_vmcnt<PER>();
         else gemm_wait_vmcnt<0>();
@@ -384,12 +386,13 @@ inline int launch_gemm(const int8_t* a, const int8_t* w, int32_t* c, const float
     // Measured on MI355X at M=1024: the direct-load kernel wins wherever it applies; 128x128 tiles once they fill
     // the chip about three times over (gate/up), 64x64 tiles for the narrow projections.  FLEXLLM_GEMM_TILE
     // forces a variant (0..2: register-staged 128x128 / 64x128 / 64x64, 10..13: direct-load 256x256 / 128x128 /
-    // 128x256 / 64x64).
+    // 128x256 / 64x64, 17..20: deeper pipelines 64x64 S4 / 64x64 S6 / 64x128 S4 / 128x128 S4).  Long-K narrow outputs
+    // (down projection) stream cold weights: 64x128 tiles four stages deep keep more bytes in flight.
     auto tiles = [&](int bm, int bn) { return ((m + bm - 1) / bm) * ((n + bn - 1) / bn); };
     static const char* force = getenv("FLEXLLM_GEMM_TILE");
     // the direct-load kernel needs 32-bit element offsets into both operands and 16-byte aligned output rows
     const bool dma_ok = (size_t)m * k < (1ull << 31) && (size_t)n * k < (1ull << 31) && n % 4 == 0;
-    int mode = dma_ok ? (tiles(128, 128) >= 768 ? 11 : 13) : (tiles(128, 128) >= 1024 ? 0 : 2);
+    int mode = dma_ok ? (tiles(128, 128) >= 768 ? 11 : (k >= 4096 && tiles(64, 128) >= 256) ? 19 : 13) : (tiles(128, 128) >= 1024 ? 0 : 2);
     if (force) mode = atoi(force);
     if (mode >= 10 && !dma_ok) mode = 2;
     const int nk = k / kGemmBK;
@@ -398,6 +401,10 @@ inline int launch_gemm(const int8_t* a, const int8_t* w, int32_t* c, const float
         if (mode == 10) return launch_gemm_dma<256, 256, DE>(a, w, c, s_x, w_s, residual, y, m, k, n, st);
         if (mode == 11) return launch_gemm_dma<128, 128, DE>(a, w, c, s_x, w_s, residual, y, m, k, n, st);
         if (mode == 12) return launch_gemm_dma<128, 256, DE>(a, w, c, s_x, w_s, residual, y, m, k, n, st);
+        if (mode == 17) return launch_gemm_dma<64, 64, DE, 4, 2>(a, w, c, s_x, w_s, residual, y, m, k, n, st);
+        if (mode == 18) return launch_gemm_dma<64, 64, DE, 6, 2>(a, w, c, s_x, w_s, residual, y, m, k, n, st);
+        if (mode == 19) return launch_gemm_dma<64, 128, DE, 4, 2>(a, w, c, s_x, w_s, residual, y, m, k, n, st);
+        if (mode == 20) return launch_gemm_dma<128, 128, DE, 4, 2>(a, w, c, s_x, w_s, residual, y, m, k, n, st);
         return launch_gemm_dma<64, 64, DE>(a, w, c, s_x, w_s, residual, y, m, k, n, st);
     }
 #define FX_GEMM_LAUNCH(BM, BN, DD)                                                                                \

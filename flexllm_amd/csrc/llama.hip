@@ -325,7 +325,7 @@ int flexllm_llama_destroy(flexllm_llama* m) {
     if (!m) return FLEXLLM_OK;
     (void)hipDeviceSynchronize();
     if (m->graph_exec) (void)hipGraphExecDestroy(m->graph_exec);
-    prefill_workspace_free(&m->pws);
+    prefill_workspace_destroy(&m->pws);
     for (void* p : m->owned) (void)hipFree(p);
     delete m;
     return FLEXLLM_OK;
