@@ -27,22 +27,29 @@ __device__ __forceinline__ i32x16 zero16() {
     return z;
 }
 
-// grid (s/32, q_heads), 256 threads: the four waves of a workgroup share one block of 32 queries and split
+// grid (s/32 * q_heads), 256 threads: the four waves of a workgroup share one block of 32 queries and split
 // its key tiles round-robin (tile kt goes to wave kt%4).  Row statistics are merged through LDS after pass 1;
 // the int32 P.V partial accumulators of the four waves are added in LDS after pass 2 (integer adds: exact).
-// Long query blocks are scheduled first.
+//
+// Work per query block grows linearly with its index (causal), and workgroups b, b+P, b+2P, ... (P = number of
+// CUs) end up resident on the same CU.  The (block, head) items are therefore taken in order of decreasing
+// length and dealt out in snake order (round 0 forwards, round 1 backwards, ...): every CU gets the same total.
 static __global__ __launch_bounds__(256) void pf_attention_kernel(const int8_t* __restrict__ q8, const int8_t* __restrict__ kc,
                                                                   const int8_t* __restrict__ vc, const float* __restrict__ q_s,
                                                                   const float* __restrict__ k_s, const float* __restrict__ v_s,
                                                                   const float* __restrict__ a_s, float* __restrict__ o,
                                                                   uint8_t* __restrict__ p8_out, int s, int q_heads, int group,
-                                                                  int max_pos) {
+                                                                  int max_pos, int period) {
     __shared__ float lds_m[4][32], lds_l[4][32];
     __shared__ int lds_acc[64][35];            // [lane][16 acc0 | 16 acc1 | vsum0 | vsum1], odd pitch against bank conflicts
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int qb = (int)gridDim.x - 1 - (int)blockIdx.x;
+    const int n_items = (int)gridDim.x, nqb = s / kPfTile;
+    const int round = (int)blockIdx.x / period, c = (int)blockIdx.x % period;
+    const int in_round = min(period, n_items - round * period);
+    const int item = round * period + ((round & 1) ? in_round - 1 - c : c);   // index into the items sorted by decreasing length
+    const int qb = nqb - 1 - item / q_heads;
     const int q0 = qb * kPfTile;
-    const int h = blockIdx.y, kvh = h / group;
+    const int h = item % q_heads, kvh = h / group;
     const int col = lane & 31, g = lane >> 5;
     const int query = q0 + col;
     const float sq = q_s[h], sk = k_s[kvh], as = 1.0f * a_s[h];
@@ -181,8 +188,15 @@ static __global__ __launch_bounds__(256) void pf_attention_kernel(const int8_t* 
 inline int mha_prefill_launch(const int8_t* q8, const int8_t* kc, const int8_t* vc, const float* q_s, const float* k_s,
                               const float* v_s, const float* a_s, float* o, uint8_t* p8_out, int s, int q_heads,
                               int kv_heads, int max_pos, hipStream_t st) {
-    dim3 grid(s / kPfTile, q_heads);
-    pf_attention_kernel<<<grid, 256, 0, st>>>(q8, kc, vc, q_s, k_s, v_s, a_s, o, p8_out, s, q_heads, q_heads / kv_heads, max_pos);
+    static int n_cu = 0;
+    if (!n_cu) {
+        int dev = 0;
+        FX_HIP(hipGetDevice(&dev));
+        FX_HIP(hipDeviceGetAttribute(&n_cu, hipDeviceAttributeMultiprocessorCount, dev));
+        if (n_cu <= 0) n_cu = 256;
+    }
+    pf_attention_kernel<<<(s / kPfTile) * q_heads, 256, 0, st>>>(q8, kc, vc, q_s, k_s, v_s, a_s, o, p8_out, s, q_heads,
+                                                               q_heads / kv_heads, max_pos, n_cu);
     FX_LAUNCH_CHECK();
     return FLEXLLM_OK;
 }
