@@ -1,6 +1,6 @@
 // Causal int8 prefill attention (GQA) on MFMA, reading K and V from the layer's int8 cache.
 //
-// A workgroup owns 32 consecutive queries of one head; its four waves split the key tiles (32 keys) up to the
+// A workgroup owns 32 consecutive queries of one head; its waves split the key tiles (32 keys) up to the
 // diagonal.
 // The score tile is computed TRANSPOSED, S^T = K_tile . Q_tile^T, so that in the 32x32 accumulator layout a
 // lane holds 16 scores of ONE query (column l%32; keys 8a+4g+b for register 4a+b, g = l/32).  That is also
@@ -27,20 +27,21 @@ __device__ __forceinline__ i32x16 zero16() {
     return z;
 }
 
-// grid (s/32 * q_heads), 256 threads: the four waves of a workgroup share one block of 32 queries and split
-// its key tiles round-robin (tile kt goes to wave kt%4).  Row statistics are merged through LDS after pass 1;
-// the int32 P.V partial accumulators of the four waves are added in LDS after pass 2 (integer adds: exact).
+// grid (s/32 * q_heads), 64 * kPfWaves threads: the waves of a workgroup share one block of 32 queries and split
+// its key tiles round-robin (tile kt goes to wave kt % kPfWaves).  Row statistics are merged through LDS after pass 1;
+// the int32 P.V partial accumulators of the waves are added in LDS after pass 2 (integer adds: exact).
 //
 // Work per query block grows linearly with its index (causal), and workgroups b, b+P, b+2P, ... (P = number of
 // CUs) end up resident on the same CU.  The (block, head) items are therefore taken in order of decreasing
 // length and dealt out in snake order (round 0 forwards, round 1 backwards, ...): every CU gets the same total.
-static __global__ __launch_bounds__(256) void pf_attention_kernel(const int8_t* __restrict__ q8, const int8_t* __restrict__ kc,
+constexpr int kPfWaves = 4;        // waves per workgroup (8 measured slower: the kernel is bound by VALU throughput, not by the longest block)
+static __global__ __launch_bounds__(64 * kPfWaves) void pf_attention_kernel(const int8_t* __restrict__ q8, const int8_t* __restrict__ kc,
                                                                   const int8_t* __restrict__ vc, const float* __restrict__ q_s,
                                                                   const float* __restrict__ k_s, const float* __restrict__ v_s,
                                                                   const float* __restrict__ a_s, float* __restrict__ o,
                                                                   uint8_t* __restrict__ p8_out, int s, int q_heads, int group,
                                                                   int max_pos, int period) {
-    __shared__ float lds_m[4][32], lds_l[4][32];
+    __shared__ float lds_m[kPfWaves][32], lds_l[kPfWaves][32];
     __shared__ int lds_acc[64][35];            // [lane][16 acc0 | 16 acc1 | vsum0 | vsum1], odd pitch against bank conflicts
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int n_items = (int)gridDim.x, nqb = s / kPfTile;
@@ -77,14 +78,14 @@ static __global__ __launch_bounds__(256) void pf_attention_kernel(const int8_t* 
     };
 
     const int ntiles = qb + 1;
-    for (int i = threadIdx.x; i < 64 * 35; i += 256) (&lds_acc[0][0])[i] = 0;
+    for (int i = threadIdx.x; i < 64 * 35; i += 64 * kPfWaves) (&lds_acc[0][0])[i] = 0;
     // ---- pass 1: row max and row sum of exponentials over this wave's tiles ----
     float m_run = -1e32f, l_run = 0.0f;
     {
         i32x4 kf0, kf1, nf0, nf1;
         if (wave < ntiles) load_k(wave * kPfTile, kf0, kf1);
-        for (int kt = wave; kt < ntiles; kt += 4) {
-            if (kt + 4 < ntiles) load_k((kt + 4) * kPfTile, nf0, nf1);
+        for (int kt = wave; kt < ntiles; kt += kPfWaves) {
+            if (kt + kPfWaves < ntiles) load_k((kt + kPfWaves) * kPfTile, nf0, nf1);
             float sc[16];
             score_tile(kt * kPfTile, kf0, kf1, sc);
             float mt = sc[0];
@@ -99,7 +100,7 @@ static __global__ __launch_bounds__(256) void pf_attention_kernel(const int8_t* 
             kf0 = nf0; kf1 = nf1;
         }
     }
-    {   // merge the two lanes that share a query, then the four waves
+    {   // merge the two lanes that share a query, then the waves
         const float m_o = lane_xor_f<32>(m_run), l_o = lane_xor_f<32>(l_run);
         const float mw = fmaxf(m_run, m_o);
         const float lw = l_run * expf(m_run - mw) + l_o * expf(m_o - mw);
@@ -108,10 +109,10 @@ static __global__ __launch_bounds__(256) void pf_attention_kernel(const int8_t* 
     __syncthreads();
     float mx = lds_m[0][col];
 #pragma unroll
-    for (int w = 1; w < 4; w++) mx = fmaxf(mx, lds_m[w][col]);
+    for (int w = 1; w < kPfWaves; w++) mx = fmaxf(mx, lds_m[w][col]);
     float total = 0.0f;
 #pragma unroll
-    for (int w = 0; w < 4; w++) total += lds_l[w][col] * expf(lds_m[w][col] - mx);
+    for (int w = 0; w < kPfWaves; w++) total += lds_l[w][col] * expf(lds_m[w][col] - mx);
     const float cd = 1.0f / total;
 
     // ---- pass 2: probabilities, partial P.V over this wave's tiles ----
@@ -120,9 +121,9 @@ static __global__ __launch_bounds__(256) void pf_attention_kernel(const int8_t* 
     {
         i32x4 kf0, kf1, nf0, nf1;
         if (wave < ntiles) load_k(wave * kPfTile, kf0, kf1);
-        for (int kt = wave; kt < ntiles; kt += 4) {
+        for (int kt = wave; kt < ntiles; kt += kPfWaves) {
             const int k0 = kt * kPfTile;
-            if (kt + 4 < ntiles) load_k((kt + 4) * kPfTile, nf0, nf1);
+            if (kt + kPfWaves < ntiles) load_k((kt + kPfWaves) * kPfTile, nf0, nf1);
             // B operand of P.V: V[key][d] for this lane's channel d = col (+32) and the lane's 16 keys, gathered
             // from the cache's [d][64 pos] blocks; issued before the exponentials so that it is in flight
             const int8_t* vblk = vc + v_index(kvh, k0, 0, max_pos);
@@ -161,7 +162,7 @@ static __global__ __launch_bounds__(256) void pf_attention_kernel(const int8_t* 
             kf0 = nf0; kf1 = nf1;
         }
     }
-    // add the four waves' partial accumulators (lds_acc was zeroed before pass 1; two barriers have passed)
+    // add the waves' partial accumulators (lds_acc was zeroed before pass 1; two barriers have passed)
     if (wave < ntiles) {
 #pragma unroll
         for (int r = 0; r < 16; r++) {
@@ -176,8 +177,8 @@ static __global__ __launch_bounds__(256) void pf_attention_kernel(const int8_t* 
     const int vs1 = lds_acc[lane][33] + lds_acc[lane ^ 32][33];
     const float sv = v_s[kvh], sa = a_s[h];
 #pragma unroll
-    for (int rr = 0; rr < 4; rr++) {                          // wave w writes accumulator registers 4w..4w+3
-        const int r = wave * 4 + rr;
+    for (int rr = 0; rr < 16 / kPfWaves; rr++) {              // each wave writes its share of the 16 accumulator registers
+        const int r = wave * (16 / kPfWaves) + rr;
         const int row = q0 + (r >> 2) * 8 + g * 4 + (r & 3);
         float* orow = o + ((size_t)row * q_heads + h) * kHd;
         orow[col] = (float)(lds_acc[lane][r] + 128 * vs0) * sa * sv;
@@ -195,7 +196,7 @@ inline int mha_prefill_launch(const int8_t* q8, const int8_t* kc, const int8_t* 
         FX_HIP(hipDeviceGetAttribute(&n_cu, hipDeviceAttributeMultiprocessorCount, dev));
         if (n_cu <= 0) n_cu = 256;
     }
-    pf_attention_kernel<<<(s / kPfTile) * q_heads, 256, 0, st>>>(q8, kc, vc, q_s, k_s, v_s, a_s, o, p8_out, s, q_heads,
+    pf_attention_kernel<<<(s / kPfTile) * q_heads, 64 * kPfWaves, 0, st>>>(q8, kc, vc, q_s, k_s, v_s, a_s, o, p8_out, s, q_heads,
                                                                q_heads / kv_heads, max_pos, n_cu);
     FX_LAUNCH_CHECK();
     return FLEXLLM_OK;
