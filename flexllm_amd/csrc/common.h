@@ -148,6 +148,30 @@ __device__ __forceinline__ float block_sum(float v, float* red) {
 // round half away from zero of x/s with IEEE division, wrapped to 8 bits like (ap_int<8>)round(x/s).
 __device__ __forceinline__ int quant_round(float x, float s) { return (int)roundf(x / s); }
 
+// round(x / s) for a whole vector that shares s, without a division per element.  q~ = x * (1/s) is within
+// 3 * 2^-24 * |q| <= 2.3e-5 of the correctly rounded quotient (|q| <= 127.5), so both round to the same integer
+// unless q~ lies within 1e-4 of a tie (k + 0.5); `near_tie` collects those cases and the caller redoes them
+// with the exact expression.  Valid while 1/s is a normal number (`quant_fast_ok`).
+__device__ __forceinline__ bool quant_fast_ok(float s) { return s >= 0x1p-100f && s <= 0x1p100f; }
+__device__ __forceinline__ int quant_round_fast(float x, float rs, bool& near_tie) {
+    const float q = x * rs;
+    near_tie |= fabsf(__builtin_amdgcn_fractf(fabsf(q)) - 0.5f) < 1e-4f;
+    return (int)(q + copysignf(0.5f, q));            // conversion truncates toward zero: round half away from zero
+}
+template <int N>
+__device__ __forceinline__ void quant_vector(const float (&v)[N], float s, int (&n)[N]) {
+    bool redo = !quant_fast_ok(s);
+    if (!redo) {
+        const float rs = 1.0f / s;
+#pragma unroll
+        for (int i = 0; i < N; i++) n[i] = quant_round_fast(v[i], rs, redo);
+    }
+    if (redo) {                                      // rare (about 1e-4 per element): exact path for this lane
+#pragma unroll
+        for (int i = 0; i < N; i++) n[i] = quant_round(v[i], s);
+    }
+}
+
 __device__ __forceinline__ uint32_t pack4_i8(int a, int b, int c, int d) {
     return (uint32_t)(a & 0xff) | ((uint32_t)(b & 0xff) << 8) | ((uint32_t)(c & 0xff) << 16) | ((uint32_t)(d & 0xff) << 24);
 }

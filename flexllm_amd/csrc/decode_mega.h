@@ -123,7 +123,8 @@ struct GridBarrier {
 struct MegaLds {
     __attribute__((aligned(16))) float f[8192];        // FHT buffer / fp32 staging (32 KiB)
     __attribute__((aligned(16))) int8_t xq[8192];      // quantised activation vector of the current GEMV
-    float red[kMegaWaves];
+    float red[kMegaWaves];                             // two-barrier reductions of the lm_head section
+    float red_sum[kMegaWaves], red_max[kMegaWaves];    // one-barrier reductions (a slot is rewritten only several barriers after its last read)
     float sc[4][kChunk];                               // scores of this chunk, 4 query heads
     __attribute__((aligned(16))) int8_t q8[4][kHd];
     __attribute__((aligned(16))) int8_t knew[kHd];
@@ -142,52 +143,51 @@ struct MegaLds {
 template <int NW>
 __device__ __forceinline__ float mega_block_max(float v, float* red) { return block_max<NW>(v, red); }
 
-// RMSNorm (optional) + per-token int8 quantisation of a 2048-vector held as 4 values per thread; result in L.xq.
-// Returns the quantisation scale to every thread.
-// `hook` runs in every thread right after the first workgroup barrier, i.e. once every wave's activation loads
-// have been consumed: the stream waves issue their next slice of weight prefetch there.
 template <class Hook>
-__device__ __forceinline__ float mega_block_sum(float v, float* red, Hook hook) {
+__device__ __forceinline__ float mega_block_sum(float v, float* slot, Hook hook) {
     v = wave_sum(v);
+    if ((threadIdx.x & 63) == 0) slot[threadIdx.x >> 6] = v;
     __syncthreads();
     hook();
-    if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = v;
-    __syncthreads();
-    float r = red[0];
+    float r = slot[0];
 #pragma unroll
-    for (int i = 1; i < kMegaWaves; i++) r += red[i];
+    for (int i = 1; i < kMegaWaves; i++) r += slot[i];
     return r;
 }
 template <class Hook>
-__device__ __forceinline__ float mega_block_max_h(float v, float* red, Hook hook) {
+__device__ __forceinline__ float mega_block_max_h(float v, float* slot, Hook hook) {
     v = wave_max(v);
+    if ((threadIdx.x & 63) == 0) slot[threadIdx.x >> 6] = v;
     __syncthreads();
     hook();
-    if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = v;
-    __syncthreads();
-    float r = red[0];
+    float r = slot[0];
 #pragma unroll
-    for (int i = 1; i < kMegaWaves; i++) r = fmaxf(r, red[i]);
+    for (int i = 1; i < kMegaWaves; i++) r = fmaxf(r, slot[i]);
     return r;
 }
 struct NoHook { __device__ __forceinline__ void operator()() const {} };
 
+// RMSNorm (optional) + per-token int8 quantisation of a 2048-vector held as 4 values per thread; result in L.xq.
+// Returns the quantisation scale to every thread.
+// `hook` runs in every thread right after the first workgroup barrier, i.e. once every wave's activation loads
+// have been consumed: the stream waves issue their next slice of weight prefetch there.
 template <class Hook>
 __device__ __forceinline__ float norm_quant_2048(float (&v)[4], const float4& g, bool do_norm, float eps,
                                                  MegaLds& L, Hook hook) {
     const int t = threadIdx.x;
     if (do_norm) {
         float ss = (v[0] * v[0] + v[1] * v[1]) + (v[2] * v[2] + v[3] * v[3]);
-        ss = mega_block_sum(ss, L.red, hook);
+        ss = mega_block_sum(ss, L.red_sum, hook);
         const float rms = 1.0f / sqrtf(ss / 2048.0f + eps);
         v[0] = v[0] * rms * g.x; v[1] = v[1] * rms * g.y; v[2] = v[2] * rms * g.z; v[3] = v[3] * rms * g.w;
     }
     float amax = fmaxf(fmaxf(fabsf(v[0]), fabsf(v[1])), fmaxf(fabsf(v[2]), fabsf(v[3])));
-    if (do_norm) amax = mega_block_max_h(amax, L.red, NoHook());
-    else amax = mega_block_max_h(amax, L.red, hook);
+    if (do_norm) amax = mega_block_max_h(amax, L.red_max, NoHook());
+    else amax = mega_block_max_h(amax, L.red_max, hook);
     const float sc = sym_scale(amax, 127.0f);
-    reinterpret_cast<uint32_t*>(L.xq)[t] = pack4_i8(quant_round(v[0], sc), quant_round(v[1], sc), quant_round(v[2], sc),
-                                                    quant_round(v[3], sc));
+    int n[4];
+    quant_vector(v, sc, n);
+    reinterpret_cast<uint32_t*>(L.xq)[t] = pack4_i8(n[0], n[1], n[2], n[3]);
     __syncthreads();
     return sc;
 }
@@ -659,27 +659,40 @@ __global__ __launch_bounds__(kMegaT, 1) void decode_mega_kernel(MegaParams p) {
 #pragma unroll
             for (int r = 0; r < 16; r++) L.f[bbase + r * 256] = b[r];
             __syncthreads();
+            // last pass in the layout of the first one (i = q*2048 + 4t + e): bit 12 pairs q with q^2, bit 0 pairs e with
+            // e^1, both inside the thread, and the quantised bytes of a thread are four consecutive ones per q
+            float4 c4[4];
 #pragma unroll
-            for (int r = 0; r < 16; r++) b[r] = L.f[r * 512 + t];
+            for (int q = 0; q < 4; q++) c4[q] = reinterpret_cast<const float4*>(L.f)[q * 512 + t];
 #pragma unroll
-            for (int r = 0; r < 8; r++) { const float u = b[r], v = b[r + 8]; b[r] = u + v; b[r + 8] = u - v; }   // bit 12
-            if (l == 1) fine();
-            float amax = 0.0f;
-            {
-                const bool hi = (lane & 1) != 0;                                                                      // bit 0
-#pragma unroll
-                for (int r = 0; r < 16; r++) {
-                    const float px = lane_xor_f<1>(b[r]);
-                    b[r] = (hi ? (px - b[r]) : (b[r] + px)) / p.fht_scale;
-                    amax = fmaxf(amax, fabsf(b[r]));
-                }
+            for (int q = 0; q < 2; q++) {                                                                             // bit 12
+                const float4 u = c4[q], v = c4[q + 2];
+                c4[q] = make_float4(u.x + v.x, u.y + v.y, u.z + v.z, u.w + v.w);
+                c4[q + 2] = make_float4(u.x - v.x, u.y - v.y, u.z - v.z, u.w - v.w);
             }
             if (l == 1) fine();
-            amax = block_max<kMegaWaves>(amax, L.red);
+            float amax = 0.0f;
+            float b2[16];
+#pragma unroll
+            for (int q = 0; q < 4; q++) {                                                                             // bit 0
+                b2[4 * q + 0] = (c4[q].x + c4[q].y) / p.fht_scale;
+                b2[4 * q + 1] = (c4[q].x - c4[q].y) / p.fht_scale;
+                b2[4 * q + 2] = (c4[q].z + c4[q].w) / p.fht_scale;
+                b2[4 * q + 3] = (c4[q].z - c4[q].w) / p.fht_scale;
+            }
+#pragma unroll
+            for (int r = 0; r < 16; r++) amax = fmaxf(amax, fabsf(b2[r]));
+            if (l == 1) fine();
+            amax = mega_block_max_h(amax, L.red_max, NoHook());
             const float sx = sym_scale(amax, 127.0f);
             if (l == 1) fine();
+            {
+                int n16[16];
+                quant_vector(b2, sx, n16);
 #pragma unroll
-            for (int r = 0; r < 16; r++) L.xq[r * 512 + t] = (int8_t)quant_round(b[r], sx);
+                for (int q = 0; q < 4; q++)
+                    reinterpret_cast<uint32_t*>(L.xq)[q * 512 + t] = pack4_i8(n16[4 * q], n16[4 * q + 1], n16[4 * q + 2], n16[4 * q + 3]);
+            }
             __syncthreads();
             if (l == 1) fine();
             if (is_s) {

@@ -37,9 +37,12 @@ __global__ __launch_bounds__(kBlock) void quant_sym_kernel(const float* __restri
 #pragma unroll
     for (int i = 0; i < VPT; i++) {
         const int idx = threadIdx.x + i * kBlock;
-        if (idx < nvec)
-            qr[idx] = pack4_i8(quant_round(v[i].x, sc), quant_round(v[i].y, sc), quant_round(v[i].z, sc),
-                               quant_round(v[i].w, sc));
+        if (idx < nvec) {
+            const float f[4] = {v[i].x, v[i].y, v[i].z, v[i].w};
+            int n[4];
+            quant_vector(f, sc, n);
+            qr[idx] = pack4_i8(n[0], n[1], n[2], n[3]);
+        }
     }
 }
 

@@ -49,6 +49,39 @@ def test_quant_sym_bit_exact(fx, oracle, rows, dim):
     assert np.array_equal(q.numpy(), q_ref)
 
 
+def test_quant_sym_ties_and_near_ties(fx, oracle):
+    """The kernels quantise with x * (1/s) and fall back to the exact x / s near a tie: rows built so that most
+    values sit on, or a few ulps beside, a rounding tie (k + 0.5) * s, for power-of-two and arbitrary scales."""
+    r = np.random.default_rng(123)
+    rows = []
+    for s in [1.0, 0.5, 3.0 / 127, 1e-3, 7.77e-2, 123.456, float(np.float32(1.0) / np.float32(255.0))] + list(r.uniform(1e-4, 10, 9)):
+        s = np.float32(s)
+        k = np.arange(-126, 127, dtype=np.float32)
+        base = ((k + np.float32(0.5)) * s).astype(np.float32)
+        vals = [base]
+        for step in (1, 2, 3, 8, 40):
+            up, dn = base.copy(), base.copy()
+            for _ in range(step):
+                up = np.nextafter(up, np.float32(np.inf)); dn = np.nextafter(dn, np.float32(-np.inf))
+            vals += [up, dn]
+        row = np.concatenate(vals + [r.uniform(-126, 126, 2048).astype(np.float32) * s])
+        row = np.concatenate([row, [np.float32(127.0) * s]])            # pins absmax, hence the scale, to 127*s/127
+        rows.append(row.astype(np.float32))
+    dim = max(len(x) for x in rows)
+    dim += (-dim) % 4
+    x = np.zeros((len(rows), dim), np.float32)
+    for i, row in enumerate(rows):
+        x[i, :len(row)] = row
+    q, s_out = fx.ops.quant_sym_i8(fx.to_device(x))
+    q_ref, s_ref = oracle.quant_sym(x)
+    assert np.array_equal(s_out.numpy().reshape(-1), s_ref.reshape(-1))
+    assert np.array_equal(q.numpy(), q_ref)
+    # and a bulk check: 4M values over 256 scales
+    xb = (r.standard_normal((256, 16384)) * r.uniform(1e-3, 50, (256, 1))).astype(np.float32)
+    qb, _ = fx.ops.quant_sym_i8(fx.to_device(xb))
+    assert np.array_equal(qb.numpy(), oracle.quant_sym(xb)[0])
+
+
 @pytest.mark.parametrize("bits", [4, 8])
 def test_quant_asym_bit_exact(fx, oracle, bits):
     x = rng.uniform(-1, 1, (17, 2048)).astype(np.float32)
