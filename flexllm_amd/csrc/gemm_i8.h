@@ -8,6 +8,7 @@
 // Workgroup tile BM x BN x 64, 256 threads = 4 waves in a 2x2 grid, each wave (BM/2)x(BN/2) as 32x32 MFMA
 // tiles, double-buffered LDS, four k-steps of global loads in flight in registers.
 #pragma once
+#include "attn_decode_kernels.h"
 #include "common.h"
 #include <stdlib.h>
 
@@ -171,7 +172,16 @@ __host__ __device__ constexpr int gemm_dma_lds_bytes(int bm, int bn, int stages)
     return stages * (bm + bn) * 64 > 4 * 32 * 36 * 4 ? stages * (bm + bn) * 64 : 4 * 32 * 36 * 4;   // stages, or the four epilogue patches
 }
 
-enum GemmDmaEpi { kDmaRaw = 0, kDmaDequant = 1, kDmaSwiglu = 2 };
+enum GemmDmaEpi { kDmaRaw = 0, kDmaDequant = 1, kDmaSwiglu = 2, kDmaQkv = 3 };
+
+// Arguments of the q/k/v epilogue: the 64-column tile of the fused [q | k | v] projection is one attention head,
+// so RoPE (pairs k, k+32), the static int8 quantisation and the store into q8 / the K cache / the transposed V
+// cache blocks all happen on the tile (64 tokens x 64 channels; a V cache block is 64 positions x 64 channels).
+struct QkvEpiArgs {
+    const float *sin_t, *cos_t, *q_s, *k_s, *v_s;
+    int8_t *q8, *kc, *vc;
+    int pos0, q_heads, kv_heads, max_pos;
+};
 
 __device__ __forceinline__ void gemm_dma_issue(const int8_t* base, unsigned voff, unsigned lds_dst) {
     unsigned saved_m0;
@@ -194,7 +204,8 @@ template <int BM, int BN, int EPI, int kDmaStages, int WPE>   // at most 7 stage
 __global__ __launch_bounds__(256, WPE) void gemm_i8_dma_kernel(const int8_t* __restrict__ a, const int8_t* __restrict__ w,
                                                           int32_t* __restrict__ c_out, const float* __restrict__ s_x,
                                                           const float* __restrict__ w_s, const float* __restrict__ residual,
-                                                          float* __restrict__ y, int m, int k, int n, int tiles_m, int tiles_n) {
+                                                          float* __restrict__ y, int m, int k, int n, int tiles_m, int tiles_n,
+                                                          QkvEpiArgs qa) {
     constexpr int WM = BM / 2, WN = BN / 2, TM = WM / 32, TN = WN / 32;
     constexpr int A_INSTR = BM / 64, B_INSTR = BN / 64;       // direct loads per wave per stage (16 rows each)
     constexpr int STAGE = (BM + BN) * 64;
@@ -311,6 +322,59 @@ __global__ __launch_bounds__(256, WPE) void gemm_i8_dma_kernel(const int8_t* __r
     // (32 x 36 words) and then owns 4 consecutive columns of a row: 16-byte loads of the residual, 16-byte stores
     // (8 bytes for the SiLU*up pairs), 128 contiguous bytes per row.
     __syncthreads();                                           // all waves are done with the stage buffers
+    if constexpr (EPI == kDmaQkv) {
+        static_assert(EPI != kDmaQkv || (BM == 64 && BN == 64), "the q/k/v epilogue works on 64x64 tiles");
+        constexpr int TP = 65;                                 // odd pitch: a column walk hits every bank once
+        float* tile = reinterpret_cast<float*>(gemm_smem);     // dequantised tile [64 tokens][64 channels]
+        {
+            const int col = col0 + wn + (lane & 31);
+            const float ws = w_s[col];
+#pragma unroll
+            for (int r = 0; r < 16; r++) {
+                const int lr = wm + (r >> 2) * 8 + (lane >> 5) * 4 + (r & 3);
+                tile[lr * TP + wn + (lane & 31)] = (float)acc[0][0][r] * s_x[min(row0 + lr, m - 1)] * ws;
+            }
+        }
+        __syncthreads();
+        const int head = col0 / kHd;                           // uniform: 0..q_heads-1 q, then k heads, then v heads
+        const int sel = t & 63, part = t >> 6;
+        if (head < qa.q_heads + qa.kv_heads) {
+            // RoPE + static quantisation: thread = (token sel, pairs 8*part .. 8*part+7)
+            const int row = row0 + sel, pos = qa.pos0 + row;
+            if (row < m) {
+                const bool is_q = head < qa.q_heads;
+                const int hk = is_q ? head : head - qa.q_heads;
+                const float div = is_q ? 8.0f * qa.q_s[hk] : 1.0f * qa.k_s[hk];     // sqrt(head_dim) folded into the Q scale
+                const float* sn = qa.sin_t + (size_t)pos * 32 + part * 8;
+                const float* cs = qa.cos_t + (size_t)pos * 32 + part * 8;
+                uint32_t lo[2] = {0, 0}, hi[2] = {0, 0};
+#pragma unroll
+                for (int j = 0; j < 8; j++) {
+                    const float t0 = tile[sel * TP + part * 8 + j], t1 = tile[sel * TP + part * 8 + j + 32];
+                    const float o0 = t0 * cs[j] - t1 * sn[j];
+                    const float o1 = t0 * sn[j] + t1 * cs[j];
+                    lo[j >> 2] |= (uint32_t)(static_q8(o0, div) & 0xff) << (8 * (j & 3));
+                    hi[j >> 2] |= (uint32_t)(static_q8(o1, div) & 0xff) << (8 * (j & 3));
+                }
+                int8_t* dst = is_q ? qa.q8 + ((size_t)row * qa.q_heads + hk) * kHd : qa.kc + k_index(hk, pos, qa.max_pos);
+                *reinterpret_cast<uint2*>(dst + part * 8) = make_uint2(lo[0], lo[1]);
+                *reinterpret_cast<uint2*>(dst + part * 8 + 32) = make_uint2(hi[0], hi[1]);
+            }
+        } else {
+            // V: thread = (channel sel, 16 consecutive positions 16*part ..): one 16-byte run of the transposed cache block
+            const int hv = head - qa.q_heads - qa.kv_heads;
+            const int rbase = row0 + part * 16;
+            if (rbase < m) {                                   // m is a multiple of 32 (checked by the launcher)
+                const float div = 1.0f * qa.v_s[hv];
+                uint32_t wv4[4] = {0, 0, 0, 0};
+#pragma unroll
+                for (int i = 0; i < 16; i++)
+                    wv4[i >> 2] |= (uint32_t)(static_q8(tile[(part * 16 + i) * TP + sel], div) & 0xff) << (8 * (i & 3));
+                *reinterpret_cast<uint4*>(qa.vc + v_index(hv, qa.pos0 + rbase, sel, qa.max_pos)) = make_uint4(wv4[0], wv4[1], wv4[2], wv4[3]);
+            }
+        }
+        return;
+    }
     constexpr int EP = 36;                                     // patch pitch in words (rows stay 16-byte aligned)
     int* patch = reinterpret_cast<int*>(gemm_smem) + wave * (32 * EP);
     const int pr = lane >> 3, pc = (lane & 7) * 4;             // row within a group of 8, first of this lane's 4 columns
@@ -367,7 +431,7 @@ __global__ __launch_bounds__(256, WPE) void gemm_i8_dma_kernel(const int8_t* __r
 
 template <int BM, int BN, int EPI, int STAGES = 3, int WPE = 1>
 inline int launch_gemm_dma(const int8_t* a, const int8_t* w, int32_t* c, const float* s_x, const float* w_s,
-                           const float* residual, float* y, int m, int k, int n, hipStream_t st) {
+                           const float* residual, float* y, int m, int k, int n, hipStream_t st, QkvEpiArgs qa = QkvEpiArgs()) {
     static bool opted_in = false;             // more than the default 64 KiB of LDS per workgroup
     if (!opted_in) {
         FX_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_i8_dma_kernel<BM, BN, EPI, STAGES, WPE>),
@@ -375,7 +439,7 @@ inline int launch_gemm_dma(const int8_t* a, const int8_t* w, int32_t* c, const f
         opted_in = true;
     }
     const int tm = (m + BM - 1) / BM, tn = (n + BN - 1) / BN;
-    gemm_i8_dma_kernel<BM, BN, EPI, STAGES, WPE><<<tm * tn, 256, gemm_dma_lds_bytes(BM, BN, STAGES), st>>>(a, w, c, s_x, w_s, residual, y, m, k, n, tm, tn);
+    gemm_i8_dma_kernel<BM, BN, EPI, STAGES, WPE><<<tm * tn, 256, gemm_dma_lds_bytes(BM, BN, STAGES), st>>>(a, w, c, s_x, w_s, residual, y, m, k, n, tm, tn, qa);
     FX_LAUNCH_CHECK();
     return FLEXLLM_OK;
 }
@@ -436,6 +500,17 @@ inline int launch_gemm_swiglu(const int8_t* a, const int8_t* w_gu, const float* 
     if (mode == 11) return launch_gemm_dma<128, 128, kDmaSwiglu, 3, 3>(a, w_gu, nullptr, s_x, w_s_gu, nullptr, h, m, k, n2, st);
     if (mode == 12 || mode == 16) return launch_gemm_dma<128, 256, kDmaSwiglu, 2, 2>(a, w_gu, nullptr, s_x, w_s_gu, nullptr, h, m, k, n2, st);
     return launch_gemm_dma<64, 64, kDmaSwiglu>(a, w_gu, nullptr, s_x, w_s_gu, nullptr, h, m, k, n2, st);
+}
+
+// Fused q/k/v projection: GEMM over the concatenated [q | k | v] weight rows with RoPE, static int8 quantisation and
+// the stores into q8 [tokens][q_heads][64], the K cache and the V cache in the epilogue.  Token i sits at position
+// pos0 + i; pos0 % 64 == 0 and m % 32 == 0 so that a tile of 64 tokens is one block of the transposed V cache.
+inline int launch_gemm_qkv(const int8_t* a, const int8_t* w_qkv, const float* s_x, const float* w_s, int m, int k,
+                           const QkvEpiArgs& qa, hipStream_t st) {
+    const int n = (qa.q_heads + 2 * qa.kv_heads) * kHd;
+    FX_REQUIRE(m % 32 == 0 && qa.pos0 % 64 == 0 && qa.pos0 + m <= qa.max_pos, "gemm_qkv: m=%d pos0=%d max_pos=%d", m, qa.pos0, qa.max_pos);
+    FX_REQUIRE((size_t)m * k < (1ull << 31) && (size_t)n * k < (1ull << 31), "gemm_qkv: m=%d k=%d outside the direct-load kernel's range", m, k);
+    return launch_gemm_dma<64, 64, kDmaQkv>(a, w_qkv, nullptr, s_x, w_s, nullptr, nullptr, m, k, n, st, qa);
 }
 
 }  // namespace fx

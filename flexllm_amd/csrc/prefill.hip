@@ -86,9 +86,13 @@ int llama_prefill_run(const flexllm_llama_config& c, const LayerW* layers, const
         int8_t* vc = v_cache + (size_t)l * cache_layer_bytes;
         // attention block
         rmsnorm_kernel<2, true><<<s, kBlock, 0, st>>>(b.x, g0, nullptr, b.xq, b.xs, H, c.eps);
-        if ((rc = launch_gemm<kGemmDequant>(b.xq, w.wqkv, nullptr, b.xs, w.sqkv, nullptr, b.qkv, s, H, H + 2 * KV, st))) return rc;
-        qkv_post_kernel<<<s, 256, 0, st>>>(b.qkv, rope_sin, rope_cos, q_s, k_s, v_s, b.q8, kc, vc, nullptr, 0, c.q_heads,
-                                           c.kv_heads, c.max_pos);
+        {   // q/k/v projection with RoPE, static quantisation and the cache stores in the GEMM epilogue
+            QkvEpiArgs qa;
+            qa.sin_t = rope_sin; qa.cos_t = rope_cos; qa.q_s = q_s; qa.k_s = k_s; qa.v_s = v_s;
+            qa.q8 = b.q8; qa.kc = kc; qa.vc = vc;
+            qa.pos0 = 0; qa.q_heads = c.q_heads; qa.kv_heads = c.kv_heads; qa.max_pos = c.max_pos;
+            if ((rc = launch_gemm_qkv(b.xq, w.wqkv, b.xs, w.sqkv, s, H, qa, st))) return rc;
+        }
         if (!no_touch) {                                   // fork: weights of o, gate/up, down and the next layer's q/k/v
             TouchRanges tr;
             tr.p[0] = w.wo; tr.bytes[0] = (size_t)H * H;

@@ -207,6 +207,17 @@ def kv_append_i8(k, v, k_cache, v_cache, scales, pos0, stream=None):
                                      _s(stream)))
 
 
+def linear_i8_gemm_qkv_rope_cache(a, s_x, w_qkv, w_s, sin_t, cos_t, scales, k_cache, v_cache, q_heads, pos0=0, stream=None):
+    """Fused q/k/v projection + RoPE + static quantisation + cache stores; returns q8 [m][q_heads][64]."""
+    m, k = a.shape
+    kv_heads, max_pos = k_cache.shape[0], k_cache.shape[1]
+    q8 = DeviceArray((m, q_heads, 64), np.int8)
+    check(lib().flexllm_linear_i8_gemm_qkv_rope_cache(_p(a), _p(s_x), _p(w_qkv), _p(w_s), _p(sin_t), _p(cos_t), scales.ref(),
+                                                      _p(q8), _p(k_cache), _p(v_cache), m, k, q_heads, kv_heads, max_pos,
+                                                      pos0, _s(stream)))
+    return q8
+
+
 def kv_store_i8(k8, v8, k_cache, v_cache, pos0, stream=None):
     tokens, kvh, hd = k8.shape
     max_pos = k_cache.shape[1]

@@ -179,6 +179,18 @@ typedef struct {
 int flexllm_kv_append_i8(const float* k, const float* v, int8_t* k_cache, int8_t* v_cache,
                          const flexllm_mha_scales* sc, int tokens, int kv_heads, int head_dim, int max_pos,
                          int pos0, void* stream);
+/* Fused prefill q/k/v projection: one GEMM over w_qkv int8 [(q_heads + 2 kv_heads)*64][k] = [Wq | Wk | Wv] rows with
+ * everything between the projection and attention in its epilogue: dequant, RoPE on q and k (token i at position
+ * pos0+i), static int8 quantisation (q by 8*Q_s[h], k by K_s[h], v by V_s[h]) and the stores into q8
+ * [m][q_heads][64], the K cache and the transposed V cache blocks.  Bit-identical to
+ * flexllm_linear_i8_gemm_dequant -> flexllm_rope_f32 -> flexllm_static_quant_i8 / flexllm_kv_append_i8.
+ * = pref_Linear_Layer x3 + pref_dequant (Modules/quant.h:115-164) + pref_RoPE_layer (Modules/RoPE.h:8-94) +
+ * pref_static_sym_per_tensor_quant_layer_fp32_qint (Modules/quant.h:252-293) + the K/V cache writers
+ * (Modules/MHA.h:74-109, :299-336).  head_dim 64, k % 64 == 0, m % 32 == 0, pos0 % 64 == 0. */
+int flexllm_linear_i8_gemm_qkv_rope_cache(const int8_t* a, const float* s_x, const int8_t* w_qkv, const float* w_s,
+                                          const float* sin_t, const float* cos_t, const flexllm_mha_scales* sc,
+                                          int8_t* q8, int8_t* k_cache, int8_t* v_cache, int m, int k, int q_heads,
+                                          int kv_heads, int max_pos, int pos0, void* stream);
 /* Same for already-quantised int8 k8/v8 [tokens][kv_heads][head_dim] (pure relayout). */
 int flexllm_kv_store_i8(const int8_t* k8, const int8_t* v8, int8_t* k_cache, int8_t* v_cache, int tokens,
                         int kv_heads, int head_dim, int max_pos, int pos0, void* stream);

@@ -75,6 +75,47 @@ def test_gemm_swiglu(fx, oracle, m, k, n):
         assert np.array_equal(hv, h[row])
 
 
+@pytest.mark.parametrize("m,qh,kvh,pos0", [(128, 32, 8, 0), (96, 8, 2, 64), (32, 4, 4, 0), (1024, 32, 8, 0)])
+def test_gemm_qkv_rope_cache_fused(fx, oracle, m, qh, kvh, pos0):
+    """q/k/v GEMM with RoPE + static quantisation + cache stores in the epilogue: int8 outputs bit-exact against the
+    oracle's chain (linear -> dequant -> RoPE -> static quant) and against the unfused device entry points."""
+    k, max_pos = 2048, 1280
+    n = (qh + 2 * kvh) * 64
+    x = rng.standard_normal((m, k)).astype(np.float32)
+    w = rng.integers(-127, 128, (n, k)).astype(np.int8)
+    w_s = rng.uniform(1e-3, 3e-3, n).astype(np.float32)
+    r = np.random.default_rng(11)
+    q_s = r.uniform(0.02, 0.05, qh).astype(np.float32); k_s = r.uniform(0.1, 0.3, kvh).astype(np.float32)
+    v_s = r.uniform(0.05, 0.2, kvh).astype(np.float32); a_s = np.full(qh, 1.0 / 255, np.float32)
+    sin_t, cos_t = oracle.rope_table(max_pos)
+    sc = fx.ops.Scales(q_s, k_s, v_s, a_s)
+    q, s = fx.ops.quant_sym_i8(fx.to_device(x))
+    dw, dws, dsin, dcos = fx.to_device(w), fx.to_device(w_s), fx.to_device(sin_t), fx.to_device(cos_t)
+    kc, vc = fx.ops.kv_cache(kvh, max_pos)
+    q8 = fx.ops.linear_i8_gemm_qkv_rope_cache(q, s, dw, dws, dsin, dcos, sc, kc, vc, qh, pos0=pos0).numpy()
+    # oracle chain
+    q_ref, s_ref = oracle.quant_sym(x)
+    y = oracle.dequant(oracle.linear_i8(q_ref, w), s_ref, w_s)
+    qf = oracle.rope(y[:, :qh * 64].reshape(m, qh, 64), sin_t, cos_t, pos0)
+    kf = oracle.rope(y[:, qh * 64:(qh + kvh) * 64].reshape(m, kvh, 64), sin_t, cos_t, pos0)
+    vf = np.ascontiguousarray(y[:, (qh + kvh) * 64:].reshape(m, kvh, 64))
+    assert np.array_equal(q8, oracle.static_quant(qf, q_s, 8.0))
+    k8_ref, v8_ref = oracle.static_quant(kf, k_s, 1.0), oracle.static_quant(vf, v_s, 1.0)
+    kc_h, vc_h = kc.numpy(), vc.numpy()                       # [kvh][pos][64], [kvh][pos/64][64 ch][64 pos]
+    assert np.array_equal(kc_h[:, pos0:pos0 + m, :], k8_ref.transpose(1, 0, 2))
+    v_lin = vc_h.transpose(0, 1, 3, 2).reshape(kvh, max_pos, 64)
+    assert np.array_equal(v_lin[:, pos0:pos0 + m, :], v8_ref.transpose(1, 0, 2))
+    assert not kc_h[:, pos0 + m:, :].any() and not v_lin[:, pos0 + m:, :].any() and not kc_h[:, :pos0, :].any()
+    # unfused device path
+    yd = fx.ops.linear_i8_gemm_dequant(q, s, dw, dws).numpy()
+    qd = fx.ops.rope_f32(fx.to_device(np.ascontiguousarray(yd[:, :qh * 64]).reshape(m, qh, 64)), dsin, dcos, pos0=pos0)
+    assert np.array_equal(q8, fx.ops.static_quant_i8(qd, fx.to_device(q_s), 8.0).numpy())
+    kd = fx.ops.rope_f32(fx.to_device(np.ascontiguousarray(yd[:, qh * 64:(qh + kvh) * 64]).reshape(m, kvh, 64)), dsin, dcos, pos0=pos0)
+    kc2, vc2 = fx.ops.kv_cache(kvh, max_pos)
+    fx.ops.kv_append_i8(kd, fx.to_device(np.ascontiguousarray(yd[:, (qh + kvh) * 64:]).reshape(m, kvh, 64)), kc2, vc2, sc, pos0)
+    assert np.array_equal(kc_h, kc2.numpy()) and np.array_equal(vc_h, vc2.numpy())
+
+
 def mha_scales(qh=32, kvh=8, seed=3):
     r = np.random.default_rng(seed)
     return (r.uniform(0.003, 0.005, qh).astype(np.float32), r.uniform(0.02, 0.04, kvh).astype(np.float32),
