@@ -444,6 +444,35 @@ int flexllm_llama_decode_greedy(flexllm_llama* m, int* token_io, int pos0, int s
     return FLEXLLM_OK;
 }
 
+int flexllm_llama_decode_sample(flexllm_llama* m, int* token_io, int pos0, int steps, const float* rands, int top_k,
+                                int* tokens_out, void* stream) {
+    FX_REQUIRE(m && token_io && tokens_out && rands, "llama_decode_sample: null pointer");
+    FX_REQUIRE(steps >= 0 && pos0 >= 0 && pos0 + steps <= m->cfg.max_pos,
+               "llama_decode_sample: pos0=%d steps=%d exceed max_pos=%d", pos0, steps, m->cfg.max_pos);
+    FX_REQUIRE(top_k >= 1 && top_k <= kTopKMax && top_k <= m->cfg.vocab, "llama_decode_sample: top_k=%d (1..%d)", top_k, kTopKMax);
+    hipStream_t st = as_stream(stream);
+    const flexllm_llama_config& c = m->cfg;
+    set_state_kernel<<<1, 1, 0, st>>>(m->state, pos0, 0);
+    FX_LAUNCH_CHECK();
+    // per token: layers + lm_head into m->logits, then the sampler picks the token (rands[step]), hands it over
+    // through token_io and advances position and step in device memory
+    TopKOut out = {nullptr, nullptr, nullptr, nullptr, token_io, tokens_out, m->state};
+    for (int s = 0; s < steps; s++) {
+        int rc;
+        if (use_mega(m)) {
+            if ((rc = launch_mega(m, token_io, nullptr, m->logits, 1, st))) return rc;
+        } else {
+            embed_kernel<<<(c.hidden + 255) / 256, 256, 0, st>>>(reinterpret_cast<const __half*>(m->embed), token_io, m->x, c.hidden);
+            for (int l = 0; l < c.layers; l++)
+                if ((rc = decode_layer(m, l, st))) return rc;
+            if ((rc = decode_head(m, m->logits, st))) return rc;
+        }
+        topk_sample_kernel<<<1, kTopKThreads, 0, st>>>(m->logits, c.vocab, top_k, rands, 1, 1, out);
+        FX_LAUNCH_CHECK();
+    }
+    return FLEXLLM_OK;
+}
+
 int flexllm_llama_prefill_hidden(flexllm_llama* m, const float* x_in, int s, float* hidden_out, void* stream) {
     FX_REQUIRE(m && x_in, "llama_prefill_hidden: null pointer");
     return llama_prefill_run(m->cfg, m->layers.data(), m->gamma, m->q_s, m->k_s, m->v_s, m->a_s, m->rope_sin, m->rope_cos,

@@ -28,4 +28,14 @@ int flexllm_argmax_f32(const float* x, int n, int* result, void* stream) {
     return argmax_launch(x, n, result, g_pv, g_pi, as_stream(stream));
 }
 
+int flexllm_sample_topk_f32(const float* logits, int n, int top_k, const float* rand, int enable_sub_max, int* token,
+                            int* top_idx, float* top_val, float* top_prob, void* stream) {
+    FX_REQUIRE(logits && rand && token, "sample_topk: null pointer");
+    FX_REQUIRE(n > 0 && top_k >= 1 && top_k <= kTopKMax && top_k <= n, "sample_topk: n=%d top_k=%d (1..%d)", n, top_k, kTopKMax);
+    TopKOut out = {token, top_idx, top_val, top_prob, nullptr, nullptr, nullptr};
+    topk_sample_kernel<<<1, kTopKThreads, 0, as_stream(stream)>>>(logits, n, top_k, rand, 0, enable_sub_max, out);
+    FX_LAUNCH_CHECK();
+    return FLEXLLM_OK;
+}
+
 }  // extern "C"

@@ -92,6 +92,99 @@ static __global__ __launch_bounds__(64) void argmax_final_kernel(const float* __
     if (threadIdx.x == 0) result[0] = bi == 0x7fffffff ? 0 : bi;
 }
 
+// ---- top-k sampling (Modules/Logits.h:145-279) ------------------------------------------------------------
+// One workgroup of 1024 threads.  Each thread keeps the k best (value, index) of its strided share, ordered by
+// value descending then index ascending; k rounds of a block-wide arg-max over the threads' current heads pop the
+// global top-k in that order.  Thread 0 then does what the reference does with the k candidates: softmax with
+// two partial sums (exp(v_k - v_0)), cumulative distribution, first k with rand < cdf[k] (else the last one).
+// The reference orders EQUAL logits by its lane scan order instead of by index; the candidates' values, hence the
+// probabilities, are the same either way, only which of two equal logits is reported can differ.
+constexpr int kTopKMax = 16;
+constexpr int kTopKThreads = 1024;
+struct TopKOut { int* token; int* top_idx; float* top_val; float* top_prob; int* token_io; int* tokens_out; int* state; };
+
+__device__ __forceinline__ bool topk_better(float v, int i, float bv, int bi) { return v > bv || (v == bv && i < bi); }
+
+static __global__ __launch_bounds__(kTopKThreads) void topk_sample_kernel(const float* __restrict__ logits, int n, int top_k,
+                                                                         const float* __restrict__ rand_ptr, int rand_index_from_state,
+                                                                         int enable_sub_max, TopKOut out) {
+    __shared__ float s_val[kTopKThreads / 64];
+    __shared__ int s_idx[kTopKThreads / 64], s_own[kTopKThreads / 64];
+    __shared__ float f_val[kTopKMax];
+    __shared__ int f_idx[kTopKMax];
+    __shared__ int s_winner;
+    const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
+    float val[kTopKMax];
+    int idx[kTopKMax];
+#pragma unroll
+    for (int k = 0; k < kTopKMax; k++) { val[k] = -1e32f; idx[k] = 0x7fffffff; }
+    for (int i = t; i < n; i += kTopKThreads) {
+        // insertion into the sorted list (k is small; statically indexed so that the lists stay in registers)
+        float cv = logits[i];
+        int ci = i;
+#pragma unroll
+        for (int k = 0; k < kTopKMax; k++) {
+            if (k < top_k && topk_better(cv, ci, val[k], idx[k])) {
+                const float tv = val[k]; const int ti = idx[k];
+                val[k] = cv; idx[k] = ci; cv = tv; ci = ti;
+            }
+        }
+    }
+    int head = 0;                                   // this thread's best not yet taken
+    for (int r = 0; r < top_k; r++) {
+        float bv = -1e32f; int bi = 0x7fffffff, bo = t;
+#pragma unroll
+        for (int k = 0; k < kTopKMax; k++) if (k == head) { bv = val[k]; bi = idx[k]; }
+        if (head >= top_k) { bv = -1e32f; bi = 0x7fffffff; }
+#pragma unroll
+        for (int m = 1; m < 64; m <<= 1) {
+            const float ov = __shfl_xor(bv, m); const int oi = __shfl_xor(bi, m); const int oo = __shfl_xor(bo, m);
+            if (topk_better(ov, oi, bv, bi) || (ov == bv && oi == bi && oo < bo)) { bv = ov; bi = oi; bo = oo; }
+        }
+        if (lane == 0) { s_val[wave] = bv; s_idx[wave] = bi; s_own[wave] = bo; }
+        __syncthreads();
+        if (t == 0) {
+            float wv = s_val[0]; int wi = s_idx[0], wo = s_own[0];
+            for (int w = 1; w < kTopKThreads / 64; w++)
+                if (topk_better(s_val[w], s_idx[w], wv, wi) || (s_val[w] == wv && s_idx[w] == wi && s_own[w] < wo)) { wv = s_val[w]; wi = s_idx[w]; wo = s_own[w]; }
+            f_val[r] = wv; f_idx[r] = wi == 0x7fffffff ? -1 : wi; s_winner = wo;
+        }
+        __syncthreads();
+        if (t == s_winner) head++;
+        __syncthreads();
+    }
+    if (t == 0) {
+        float prob[kTopKMax], cdf[kTopKMax];
+        float sum_partial[2] = {0.0f, 0.0f};
+        for (int k = 0; k < top_k; k++) {
+            const float e = enable_sub_max ? expf(f_val[k] - f_val[0]) : expf(f_val[k]);
+            prob[k] = e;
+            sum_partial[k % 2] += e;
+        }
+        const float sum = sum_partial[0] + sum_partial[1];
+        for (int k = 0; k < top_k; k++) prob[k] = prob[k] / sum;
+        cdf[0] = prob[0];
+        for (int k = 1; k < top_k; k++) cdf[k] = prob[k] + cdf[k - 1];
+        const float rnd = rand_ptr[rand_index_from_state && out.state ? out.state[1] : 0];
+        int selected = top_k - 1;
+        for (int k = 0; k < top_k; k++)
+            if (rnd < cdf[k] && selected == top_k - 1) selected = k;
+        const int tok = f_idx[selected];
+        if (out.token) out.token[0] = tok;
+        for (int k = 0; k < top_k; k++) {
+            if (out.top_idx) out.top_idx[k] = f_idx[k];
+            if (out.top_val) out.top_val[k] = f_val[k];
+            if (out.top_prob) out.top_prob[k] = prob[k];
+        }
+        if (out.state) {                            // generation loop: hand the token over and advance position / step
+            out.token_io[0] = tok;
+            out.tokens_out[out.state[1]] = tok;
+            out.state[0] += 1;
+            out.state[1] += 1;
+        }
+    }
+}
+
 constexpr int kArgmaxParts = 256;
 inline float* g_pv = nullptr;
 inline int* g_pi = nullptr;

@@ -97,6 +97,11 @@ class Llama:
         check(lib().flexllm_llama_decode_greedy(self.handle, C.c_void_p(token_io.ptr), int(pos0), int(steps),
                                                 C.c_void_p(tokens_out.ptr), int(use_graph), _s(stream)))
 
+    def decode_sample(self, token_io, pos0, steps, rands, top_k, tokens_out, stream=None):
+        """Top-k sampling loop; rands: device float32 [steps] in [0,1)."""
+        check(lib().flexllm_llama_decode_sample(self.handle, C.c_void_p(token_io.ptr), int(pos0), int(steps),
+                                                C.c_void_p(rands.ptr), int(top_k), C.c_void_p(tokens_out.ptr), _s(stream)))
+
     def set_decode_mode(self, mode):
         """0: persistent one-kernel-per-token schedule (default), 1: one kernel per stage."""
         check(lib().flexllm_llama_set_decode_mode(self.handle, int(mode)))

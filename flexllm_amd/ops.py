@@ -262,3 +262,14 @@ def argmax_f32(x, stream=None):
     r = DeviceArray((1,), np.int32)
     check(lib().flexllm_argmax_f32(_p(x), x.size, _p(r), _s(stream)))
     return r
+
+
+def sample_topk_f32(logits, top_k=5, rand=0.5, enable_sub_max=True, stream=None):
+    """Top-k sampling (Logits.h): returns (token, top_idx, top_val, top_prob) as host values."""
+    n = logits.size
+    r = to_device(np.array([rand], np.float32))
+    tok = DeviceArray((1,), np.int32)
+    idx = DeviceArray((top_k,), np.int32); val = DeviceArray((top_k,), np.float32); prob = DeviceArray((top_k,), np.float32)
+    check(lib().flexllm_sample_topk_f32(_p(logits), n, top_k, _p(r), int(enable_sub_max), _p(tok), _p(idx), _p(val), _p(prob),
+                                        _s(stream)))
+    return int(tok.numpy()[0]), idx.numpy(), val.numpy(), prob.numpy()

@@ -213,11 +213,20 @@ int flexllm_mha_i8_prefill(const int8_t* q8, const int8_t* k_cache, const int8_t
                            const flexllm_mha_scales* sc, float* o, uint8_t* p8_out, int s, int q_heads,
                            int kv_heads, int head_dim, int max_pos, void* stream);
 
-/* ---- Logits.h (greedy) ---------------------------------------------------------------- */
+/* ---- Logits.h (greedy and top-k sampling) ---------------------------------------------- */
 /* logits[v] = sum_k fp16(E[v][k]) * n[k] (fp32 accumulate): tied fp16 lm_head GEMV. */
 int flexllm_lm_head_f16(const uint16_t* embed, const float* n, float* logits, int vocab, int hidden, void* stream);
 /* Index of the maximum (lowest index on ties); result is a device int. */
 int flexllm_argmax_f32(const float* x, int n, int* result, void* stream);
+/* Top-k sampling of the next token: the k largest logits, softmax over them (exp(v_k - v_0) when enable_sub_max,
+ * two partial sums), cumulative distribution, the first k with rand < cdf[k] (the last candidate otherwise).
+ * Replaces the selection/sampling part of dec_Sampling_Embedding_Layer (Modules/Logits.h:145-279, insertion
+ * routine :5-31); the embedding look-up that follows there is flexllm_embed_f16.  rand: device pointer to one
+ * float in [0,1) (the reference's host-supplied rand_seed); token: device int.  top_idx/top_val/top_prob
+ * (optional, device, [top_k]) return the candidates in rank order.  Equal logits are ranked by index (the
+ * reference ranks them by its lane scan order; values and probabilities are the same).  1 <= top_k <= 16. */
+int flexllm_sample_topk_f32(const float* logits, int n, int top_k, const float* rand, int enable_sub_max, int* token,
+                            int* top_idx, float* top_val, float* top_prob, void* stream);
 /* y = fp32(E[token]) with the token id read from device memory. */
 int flexllm_embed_f16(const uint16_t* embed, const int* token, float* y, int hidden, void* stream);
 
@@ -270,6 +279,13 @@ int flexllm_llama_decode_hidden(flexllm_llama* m, const float* x_in, int pos, fl
  * and replayed. */
 int flexllm_llama_decode_greedy(flexllm_llama* m, int* token_io, int pos0, int steps, int* tokens_out,
                                 int use_graph, void* stream);
+/* Generation with top-k sampling, the reference's own loop (SpinQuant_Decoding_mem_opt.h:924-940 with
+ * dec_Sampling_Embedding_Layer, Modules/Logits.h:145-279; host random numbers as in
+ * SpinQuant_Prefilling_Decoding_mem_opt_tb.cpp:827-830): for step s the token is drawn from the top_k logits
+ * with rands[s] (device array of `steps` floats in [0,1)), written to tokens_out[s] (device) and fed back through
+ * token_io (device int, holds the first input token on entry). */
+int flexllm_llama_decode_sample(flexllm_llama* m, int* token_io, int pos0, int steps, const float* rands, int top_k,
+                                int* tokens_out, void* stream);
 /* Prefill s tokens at positions 0..s-1 from fp32 embeddings x_in (device [s][hidden]); fills the KV cache,
  * writes the residual stream to hidden_out (device [s][hidden], may be NULL). */
 int flexllm_llama_prefill_hidden(flexllm_llama* m, const float* x_in, int s, float* hidden_out, void* stream);

@@ -378,6 +378,59 @@ int fxo_argmax(const float* x, int n) {
     return best;
 }
 
+/* Top-k sampling of the next token, Modules/Logits.h:145-279 (dec_Sampling_Embedding_Layer), with the insertion
+ * routine of Modules/Logits.h:5-31 (sort_top_k: strict '>', so of two equal logits the one inserted first keeps
+ * the higher rank).  `lanes` = block_parallel_samp: lane i scans the contiguous index range
+ * [i*n/lanes, (i+1)*n/lanes) in order (Logits.h:216, inner_block_parallel = 1), the per-lane lists are merged
+ * rank-major (Logits.h:224-232); softmax over the k candidates with two partial sums (Logits.h:239-254); CDF
+ * and "first k with rand < cdf[k]" (Logits.h:258-275).  n % lanes == 0, top_k <= 16.
+ * Outputs (each optional): the k candidates, their probabilities; returns the sampled token id. */
+static void fxo_sort_top_k(int* idx, float* val, int top_k, int v_idx, float v) {
+    int insert_pos = top_k;
+    for (int k = 0; k < top_k; k++)
+        if (v > val[k] && insert_pos == top_k) insert_pos = k;
+    for (int k = top_k - 1; k >= 0; k--) {
+        if (k > insert_pos) { idx[k] = idx[k - 1]; val[k] = val[k - 1]; }
+        else if (k == insert_pos) { idx[k] = v_idx; val[k] = v; }
+    }
+}
+
+int fxo_sample_topk(const float* logits, int n, int top_k, int lanes, float rand_seed, int enable_sub_max,
+                    int* top_idx, float* top_val, float* top_prob) {
+    int* lidx = (int*)malloc(sizeof(int) * (size_t)lanes * top_k);
+    float* lval = (float*)malloc(sizeof(float) * (size_t)lanes * top_k);
+    int fidx[16]; float fval[16], prob[16], cdf[16];
+    for (int i = 0; i < lanes * top_k; i++) { lidx[i] = -1; lval[i] = -1e32f; }
+    for (int k = 0; k < top_k; k++) { fidx[k] = -1; fval[k] = -1e32f; }
+    const int per = n / lanes;
+    for (int m = 0; m < per; m++)
+        for (int i = 0; i < lanes; i++)
+            fxo_sort_top_k(lidx + (size_t)i * top_k, lval + (size_t)i * top_k, top_k, i * per + m, logits[i * per + m]);
+    for (int K = 0; K < top_k; K++)
+        for (int i = 0; i < lanes; i++)
+            fxo_sort_top_k(fidx, fval, top_k, lidx[(size_t)i * top_k + K], lval[(size_t)i * top_k + K]);
+    float sum_partial[2] = {0.0f, 0.0f};
+    for (int k = 0; k < top_k; k++) {
+        const float t = enable_sub_max ? expf(fval[k] - fval[0]) : expf(fval[k]);
+        prob[k] = t;
+        sum_partial[k % 2] += t;
+    }
+    const float sum = sum_partial[0] + sum_partial[1];
+    for (int k = 0; k < top_k; k++) prob[k] /= sum;
+    cdf[0] = prob[0];
+    for (int k = 1; k < top_k; k++) cdf[k] = prob[k] + cdf[k - 1];
+    int selected_k = top_k - 1;
+    for (int k = 0; k < top_k; k++)
+        if (rand_seed < cdf[k] && selected_k == top_k - 1) selected_k = k;
+    for (int k = 0; k < top_k; k++) {
+        if (top_idx) top_idx[k] = fidx[k];
+        if (top_val) top_val[k] = fval[k];
+        if (top_prob) top_prob[k] = prob[k];
+    }
+    free(lidx); free(lval);
+    return fidx[selected_k];
+}
+
 /* ------------------------------------------------------ layer / model graphs */
 
 static void linear_w8a8(const float* x, int rows, int k, int n, const int8_t* w, const float* ws, float* y) {

@@ -129,6 +129,9 @@ void fxo_llama_prefill(const fxo_model* m, const float* x_in, int s, int8_t* k_c
 float fxo_half_to_float(uint16_t h);
 void fxo_embed(const uint16_t* table, int hidden, int token, float* y);
 void fxo_lm_head(const uint16_t* table, int vocab, int hidden, const float* n, float* logits);
+/* Logits.h:145-279 top-k sampling (see the .c file for the exact correspondence); returns the sampled token id */
+int fxo_sample_topk(const float* logits, int n, int top_k, int lanes, float rand_seed, int enable_sub_max,
+                    int* top_idx, float* top_val, float* top_prob);
 int fxo_argmax(const float* x, int n);
 
 /* ---- data_io.h layouts ----------------------------------------------------- */

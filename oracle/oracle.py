@@ -243,6 +243,18 @@ def lm_head(table_u16, n):
     return logits
 
 
+def sample_topk(logits, top_k=5, rand=0.5, lanes=8, enable_sub_max=True):
+    """Logits.h:145-279.  Returns (token, top_idx[k], top_val[k], top_prob[k])."""
+    logits = _f32(logits).reshape(-1)
+    n = logits.shape[0]
+    assert n % lanes == 0 and top_k <= 16
+    idx = np.empty(top_k, np.int32); val = np.empty(top_k, np.float32); prob = np.empty(top_k, np.float32)
+    f = lib().fxo_sample_topk
+    f.restype = C.c_int
+    tok = f(_p(logits), n, top_k, lanes, _f(rand), int(enable_sub_max), _p(idx), _p(val), _p(prob))
+    return int(tok), idx, val, prob
+
+
 def pack_pref(x, tp):
     x = _f32(x); tokens, dim = x.shape
     out = np.empty((tokens // tp, dim, tp), np.float32)

@@ -99,3 +99,30 @@ def test_greedy_loop_graph_replay_equals_eager_and_oracle(small):
         ref.append(t)
     model.check()
     assert outs[0].tolist() == ref
+
+
+def test_topk_sampling_loop_matches_oracle(small):
+    """The reference's generation loop: top-5 sampling with host-supplied uniform numbers, token fed back."""
+    fx, cfg, model, om, host_w = small
+    from oracle import oracle
+    steps, tok0, k = 6, 29, 5
+    rands = np.random.default_rng(8).uniform(0, 1, steps).astype(np.float32)
+    stream = fx.Stream()
+    model.k_cache.zero_(); model.v_cache.zero_()
+    tok = fx.to_device(np.array([tok0], np.int32))
+    out = fx.zeros((steps,), np.int32)
+    model.decode_sample(tok, 0, steps, fx.to_device(rands), k, out, stream=stream)
+    stream.sync()
+    model.check()
+    kc, vc = om.new_caches()
+    t = tok0
+    ref = []
+    for pos in range(steps):
+        x = oracle.embed(host_w["embed"], t)
+        _, logits = om.decode_token(x, pos, kc, vc)
+        t, idx, val, prob = oracle.sample_topk(logits, k, float(rands[pos]), 8)
+        # the draw must not sit on a boundary of the cumulative distribution for the comparison to be meaningful
+        assert np.abs(np.cumsum(prob.astype(np.float64)) - rands[pos]).min() > 1e-4
+        ref.append(t)
+    assert out.numpy().tolist() == ref
+    assert int(tok.numpy()[0]) == ref[-1]

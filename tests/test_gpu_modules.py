@@ -338,3 +338,23 @@ def test_bad_arguments_are_rejected_with_a_message(fx):
         fx.ops.fht_f32(fx.to_device(np.zeros((1, 3000), np.float32)))
     with pytest.raises(FlexLLMError, match="multiple of 16"):
         fx.ops.linear_i8_gemv(fx.to_device(np.zeros(8, np.int8)), fx.to_device(np.zeros((4, 8), np.int8)))
+
+
+# ------------------------------------------------------------------ Logits.h top-k sampling
+@pytest.mark.parametrize("n,k", [(128256, 5), (131072, 5), (4096, 1), (1000, 8), (64, 16)])
+def test_sample_topk(fx, oracle, n, k):
+    r = np.random.default_rng(n + k)
+    x = (r.standard_normal(n) * 4).astype(np.float32)
+    dx = fx.to_device(x)
+    lanes = 8 if n % 8 == 0 else 1
+    for rand in (0.0, 0.07, 0.31, 0.5, 0.83, 0.9999):
+        tok, idx, val, prob = fx.ops.sample_topk_f32(dx, k, rand)
+        tok_r, idx_r, val_r, prob_r = oracle.sample_topk(x, k, rand, lanes)
+        assert np.array_equal(idx, idx_r) and np.array_equal(val, val_r)           # candidates: exact
+        np.testing.assert_allclose(prob, prob_r, rtol=2e-6)                        # device expf vs glibc expf
+        if np.abs(np.cumsum(prob_r.astype(np.float64)) - rand).min() > 1e-5:
+            assert tok == tok_r
+    # equal logits: same values and probabilities as the reference order, candidates ranked by index
+    y = np.full(n, -3.0, np.float32); y[[n - 1, 5, n // 2]] = 9.0
+    tok, idx, val, prob = fx.ops.sample_topk_f32(fx.to_device(y), min(k, 3) if k >= 3 else 1, 0.0)
+    assert list(idx) == sorted([n - 1, 5, n // 2])[:len(idx)] and np.all(val == 9.0) and tok == 5

@@ -284,3 +284,43 @@ def test_half_to_float_and_lm_head(oracle):
     E = rng.standard_normal((50, 128)).astype(np.float16)
     n = rng.standard_normal(128).astype(np.float32)
     np.testing.assert_allclose(oracle.lm_head(E.view(np.uint16), n), E.astype(np.float64) @ n, rtol=1e-4, atol=1e-4)
+
+
+# ------------------------------------------------------------------ Logits.h top-k sampling
+def test_sample_topk_against_sorting_and_closed_forms(oracle):
+    """Pins fxo_sample_topk (Logits.h:145-279) with facts outside its own loops: the candidates are the k largest
+    logits (numpy sort, no ties in random data) for any lane count; the probabilities are the softmax of the k values
+    (float64); the token is the first candidate whose cumulative probability exceeds rand, the last one otherwise."""
+    r = np.random.default_rng(5)
+    for n, k, lanes in [(128256, 5, 8), (4096, 1, 4), (1024, 8, 16), (64, 16, 1), (131072, 5, 32)]:
+        x = (r.standard_normal(n) * 4).astype(np.float32)
+        order = np.argsort(-x.astype(np.float64), kind="stable")[:k]
+        p64 = np.exp(x[order].astype(np.float64) - float(x[order][0])); p64 /= p64.sum()
+        cdf32 = np.cumsum(p64)
+        for rand in (0.0, 0.13, 0.5, 0.77, 0.999999):
+            tok, idx, val, prob = oracle.sample_topk(x, k, rand, lanes)
+            assert np.array_equal(idx, order) and np.array_equal(val, x[order])
+            np.testing.assert_allclose(prob, p64, rtol=2e-6)
+            margins = np.abs(cdf32 - rand)
+            if margins.min() > 1e-5:                       # away from a boundary the choice is unambiguous
+                sel = int(np.argmax(cdf32 > rand)) if (cdf32 > rand).any() else k - 1
+                assert tok == order[sel]
+    # rand beyond the last cumulative value (rounding): the last candidate
+    x = np.zeros(64, np.float32); x[[3, 9, 20]] = [2.0, 1.0, 0.5]
+    assert oracle.sample_topk(x, 3, 1.5, 8)[0] == 20
+    # enable_sub_max=False: plain exp of the logits, same normalised probabilities here
+    a = oracle.sample_topk(x, 3, 0.2, 8, enable_sub_max=False)[3]
+    b = oracle.sample_topk(x, 3, 0.2, 8, enable_sub_max=True)[3]
+    np.testing.assert_allclose(a, b, rtol=1e-6)
+
+
+def test_sample_topk_tie_order_is_the_insertion_order(oracle):
+    """sort_top_k inserts with a strict '>' (Logits.h:15): of equal logits the one inserted first ranks higher.
+    Within a lane that is the smaller index; across lanes the merge is rank-major (Logits.h:224-232), so a lane's
+    second equal value ranks behind another lane's first one even if its index is smaller."""
+    x = np.full(32, -5.0, np.float32)
+    x[[1, 2]] = 7.0          # lane 0 (indices 0..7) holds two equal maxima
+    x[9] = 7.0               # lane 1 holds one
+    tok, idx, val, prob = oracle.sample_topk(x, 3, 0.0, 4)
+    assert list(idx) == [1, 9, 2] and np.all(val == 7.0)
+    np.testing.assert_allclose(prob, [1 / 3] * 3, rtol=1e-6)
