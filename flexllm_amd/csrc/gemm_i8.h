@@ -20,13 +20,35 @@ constexpr int kGemmBK = 64;        // k-bytes per stage
 // spreads the four chunks of one row, written by four neighbouring lanes, over all banks.
 __host__ __device__ constexpr int gemm_plane(int rows) { return rows * 16 + 32; }
 
-enum GemmEpi { kGemmRaw = 0, kGemmDequant = 1 };
+enum GemmEpi { kGemmRaw = 0, kGemmDequant = 1, kGemmDequantAsym = 2 };
 
-template <int BM, int BN, int EPI, int D>
+// 16 nibbles (8 bytes, low nibble = even index) -> 16 bytes in index order; SIGNED: two's-complement nibbles
+// are sign-extended (the weights), otherwise they stay 0..15 (the activations).
+template <bool SIGNED>
+__device__ __forceinline__ i32x4 unpack16_nibbles(uint2 p) {
+    i32x4 r;
+    const uint32_t src[2] = {p.x, p.y};
+#pragma unroll
+    for (int h = 0; h < 2; h++) {
+        uint32_t lo = src[h] & 0x0F0F0F0Fu, hi = (src[h] >> 4) & 0x0F0F0F0Fu;       // elements 0,2,4,6 and 1,3,5,7
+        if constexpr (SIGNED) {
+            lo |= (lo & 0x08080808u) * 30u;                                          // 0x08 -> 0xF8: sign bits of the byte
+            hi |= (hi & 0x08080808u) * 30u;
+        }
+        r[2 * h] = (int)__builtin_amdgcn_perm(hi, lo, 0x05010400u);                 // bytes lo0, hi0, lo1, hi1
+        r[2 * h + 1] = (int)__builtin_amdgcn_perm(hi, lo, 0x07030602u);             // bytes lo2, hi2, lo3, hi3
+    }
+    return r;
+}
+
+// PACKED: both operands hold two 4-bit values per byte (rows of k/2 bytes; activations unsigned, weights signed);
+// they are widened to int8 between the global load and the LDS store, the MFMA path is the same.
+template <int BM, int BN, int EPI, int D, bool PACKED = false>
 __global__ __launch_bounds__(256) void gemm_i8_kernel(const int8_t* __restrict__ a, const int8_t* __restrict__ w,
                                                       int32_t* __restrict__ c_out, const float* __restrict__ s_x,
                                                       const float* __restrict__ w_s, const float* __restrict__ residual,
-                                                      float* __restrict__ y, int m, int k, int n, int tiles_m, int tiles_n) {
+                                                      float* __restrict__ y, int m, int k, int n, int tiles_m, int tiles_n,
+                                                      const float* __restrict__ b_x = nullptr, const float* __restrict__ w_sum = nullptr) {
     constexpr int WM = BM / 2, WN = BN / 2;          // wave tile
     constexpr int TM = WM / 32, TN = WN / 32;        // 32x32 MFMA tiles per wave
     constexpr int A_CHUNKS = BM * 4 / 256;           // 16-byte chunks per thread per stage
@@ -61,18 +83,26 @@ __global__ __launch_bounds__(256) void gemm_i8_kernel(const int8_t* __restrict__
 #pragma unroll
     for (int i = 0; i < A_CHUNKS; i++) {
         const int c = t + 256 * i;
-        a_ptr[i] = a + (size_t)min(row0 + (c >> 2), m - 1) * k + (c & 3) * 16;
+        a_ptr[i] = PACKED ? a + (size_t)min(row0 + (c >> 2), m - 1) * (k >> 1) + (c & 3) * 8
+                          : a + (size_t)min(row0 + (c >> 2), m - 1) * k + (c & 3) * 16;
     }
 #pragma unroll
     for (int i = 0; i < B_CHUNKS; i++) {
         const int c = t + 256 * i;
-        b_ptr[i] = w + (size_t)min(col0 + (c >> 2), n - 1) * k + (c & 3) * 16;
+        b_ptr[i] = PACKED ? w + (size_t)min(col0 + (c >> 2), n - 1) * (k >> 1) + (c & 3) * 8
+                          : w + (size_t)min(col0 + (c >> 2), n - 1) * k + (c & 3) * 16;
     }
     auto load_global = [&](int k0, i32x4 (&xa)[A_CHUNKS], i32x4 (&xb)[B_CHUNKS]) {
 #pragma unroll
-        for (int i = 0; i < A_CHUNKS; i++) xa[i] = *reinterpret_cast<const i32x4*>(a_ptr[i] + k0);
+        for (int i = 0; i < A_CHUNKS; i++) {
+            if constexpr (PACKED) xa[i] = unpack16_nibbles<false>(*reinterpret_cast<const uint2*>(a_ptr[i] + (k0 >> 1)));
+            else xa[i] = *reinterpret_cast<const i32x4*>(a_ptr[i] + k0);
+        }
 #pragma unroll
-        for (int i = 0; i < B_CHUNKS; i++) xb[i] = *reinterpret_cast<const i32x4*>(b_ptr[i] + k0);
+        for (int i = 0; i < B_CHUNKS; i++) {
+            if constexpr (PACKED) xb[i] = unpack16_nibbles<true>(*reinterpret_cast<const uint2*>(b_ptr[i] + (k0 >> 1)));
+            else xb[i] = *reinterpret_cast<const i32x4*>(b_ptr[i] + k0);
+        }
     };
     auto store_lds = [&](int buf, const i32x4 (&xa)[A_CHUNKS], const i32x4 (&xb)[B_CHUNKS]) {
 #pragma unroll
@@ -138,14 +168,16 @@ __global__ __launch_bounds__(256) void gemm_i8_kernel(const int8_t* __restrict__
         for (int j = 0; j < TN; j++) {
             const int col = col0 + wn + j * 32 + (lane & 31);
             if (col >= n) continue;
-            float ws = 0.0f;
-            if constexpr (EPI == kGemmDequant) ws = w_s[col];
+            float ws = 0.0f, wsm = 0.0f;
+            if constexpr (EPI != kGemmRaw) ws = w_s[col];
+            if constexpr (EPI == kGemmDequantAsym) wsm = w_sum[col];
 #pragma unroll
             for (int r = 0; r < 16; r++) {
                 const int row = row0 + wm + i * 32 + (r >> 2) * 8 + (lane >> 5) * 4 + (r & 3);
                 if (row >= m) continue;
-                if constexpr (EPI == kGemmDequant) {
+                if constexpr (EPI != kGemmRaw) {
                     float v = (float)acc[i][j][r] * s_x[row] * ws;
+                    if constexpr (EPI == kGemmDequantAsym) v = v + b_x[row] * wsm;      // zero point times the row sum of W
                     if (residual) v = v + residual[(size_t)row * n + col];
                     y[(size_t)row * n + col] = v;
                 } else {
@@ -481,6 +513,24 @@ inline int launch_gemm(const int8_t* a, const int8_t* w, int32_t* c, const float
     else if (mode == 1) { if (deep) FX_GEMM_LAUNCH(64, 128, 4); else FX_GEMM_LAUNCH(64, 128, 1); }
     else { if (deep) FX_GEMM_LAUNCH(64, 64, 4); else FX_GEMM_LAUNCH(64, 64, 1); }
 #undef FX_GEMM_LAUNCH
+    FX_LAUNCH_CHECK();
+    return FLEXLLM_OK;
+}
+
+// W4A4 prefill GEMM on nibble-packed operands (register-staged kernel, nibbles widened on the way to LDS).
+template <int EPI>
+inline int launch_gemm_u4i4(const uint8_t* a4, const uint8_t* w4, int32_t* c, const float* s_x, const float* b_x,
+                            const float* w_s, const float* w_sum, const float* residual, float* y, int m, int k, int n, hipStream_t st) {
+    const int8_t* a = reinterpret_cast<const int8_t*>(a4);
+    const int8_t* w = reinterpret_cast<const int8_t*>(w4);
+    const bool big = ((m + 127) / 128) * ((n + 127) / 128) >= 768;
+    if (big) {
+        const int tm = (m + 127) / 128, tn = (n + 127) / 128;
+        gemm_i8_kernel<128, 128, EPI, 1, true><<<tm * tn, 256, 0, st>>>(a, w, c, s_x, w_s, residual, y, m, k, n, tm, tn, b_x, w_sum);
+    } else {
+        const int tm = (m + 63) / 64, tn = (n + 63) / 64;
+        gemm_i8_kernel<64, 64, EPI, 1, true><<<tm * tn, 256, 0, st>>>(a, w, c, s_x, w_s, residual, y, m, k, n, tm, tn, b_x, w_sum);
+    }
     FX_LAUNCH_CHECK();
     return FLEXLLM_OK;
 }

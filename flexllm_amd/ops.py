@@ -112,6 +112,44 @@ def linear_i8_gemm_swiglu(a, s_x, w_gu, w_s_gu, stream=None, out=None):
     return h
 
 
+# ---------------------------------------------------------------- W4A4 (Linear_Layer.h i4 PEs)
+def pack_nibbles(values, stream=None):
+    """uint8/int8 [..., k] one value per byte -> uint8 [..., k/2], low nibble = even index."""
+    out = DeviceArray(values.shape[:-1] + (values.shape[-1] // 2,), np.uint8)
+    check(lib().flexllm_pack_nibbles(_p(values), _p(out), C.c_size_t(values.size), _s(stream)))
+    return out
+
+
+def linear_u4i4_gemv(x4, w4, stream=None):
+    n, k = w4.shape[0], w4.shape[1] * 2
+    acc = DeviceArray((n,), np.int32)
+    check(lib().flexllm_linear_u4i4_gemv(_p(x4), _p(w4), _p(acc), k, n, _s(stream)))
+    return acc
+
+
+def linear_u4i4_gemv_dequant(x4, s_x, b_x, w4, w_s, w_sum, residual=None, stream=None):
+    n, k = w4.shape[0], w4.shape[1] * 2
+    y = DeviceArray((n,), np.float32)
+    check(lib().flexllm_linear_u4i4_gemv_dequant(_p(x4), _p(s_x), _p(b_x), _p(w4), _p(w_s), _p(w_sum), _p(residual), _p(y),
+                                                 k, n, _s(stream)))
+    return y
+
+
+def linear_u4i4_gemm(a4, w4, stream=None):
+    m, n, k = a4.shape[0], w4.shape[0], w4.shape[1] * 2
+    acc = DeviceArray((m, n), np.int32)
+    check(lib().flexllm_linear_u4i4_gemm(_p(a4), _p(w4), _p(acc), m, k, n, _s(stream)))
+    return acc
+
+
+def linear_u4i4_gemm_dequant(a4, s_x, b_x, w4, w_s, w_sum, residual=None, stream=None):
+    m, n, k = a4.shape[0], w4.shape[0], w4.shape[1] * 2
+    y = DeviceArray((m, n), np.float32)
+    check(lib().flexllm_linear_u4i4_gemm_dequant(_p(a4), _p(s_x), _p(b_x), _p(w4), _p(w_s), _p(w_sum), _p(residual), _p(y),
+                                                 m, k, n, _s(stream)))
+    return y
+
+
 # ---------------------------------------------------------------- FHT.h
 def fht_f32(x, scale=1.0, stream=None, out=None):
     y = out if out is not None else DeviceArray(x.shape, np.float32)

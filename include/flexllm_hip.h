@@ -120,6 +120,28 @@ int flexllm_linear_i8_gemm_dequant(const int8_t* a, const float* s_x, const int8
 int flexllm_linear_i8_gemm_swiglu(const int8_t* a, const float* s_x, const int8_t* w_gu, const float* w_s_gu, float* h,
                                   int m, int k, int n, void* stream);
 
+/* ---- W4A4 linear layers (the reference's shipped configuration) ------------------------------ */
+/* Activations asymmetric uint4 (flexllm_quant_asym_u8 with bits=4: value 0..15, scale s_x, zero point b_x = row
+ * minimum), weights symmetric int4 (-8..7), both packed two per byte along K: byte j of a row holds element 2j in
+ * its low nibble, element 2j+1 in its high nibble (the reference packs two output channels per byte in a
+ * port-specific order, SpinQuant_Llama_32_1B/Linear_Layer_Decoding_tb.cpp:176-186; the host adapter repacks).
+ * y[n] = (float(acc[n]) * s_x) * w_s[n] + b_x * w_sum[n] (+ residual[n]) with acc = sum_k a[k]*w[n][k] and
+ * w_sum[n] = sum_k w[n][k]*w_s[n] supplied by the caller, as the testbench computes it (…_tb.cpp:187-190).
+ * Replaces pref_/dec_Linear_Layer_i4xi4 (Modules/Linear_Layer.h:293-341, 862-923) + the asymmetric dequant
+ * (Modules/quant.h:146-149). */
+/* Packs values held one per byte (low 4 bits used) two per byte; n_values even. */
+int flexllm_pack_nibbles(const uint8_t* values, uint8_t* packed, size_t n_values, void* stream);
+/* Decode: x4 [k/2], w4 [n][k/2]; k % 32 == 0, k <= 16384. */
+int flexllm_linear_u4i4_gemv(const uint8_t* x4, const uint8_t* w4, int32_t* acc, int k, int n, void* stream);
+int flexllm_linear_u4i4_gemv_dequant(const uint8_t* x4, const float* s_x, const float* b_x, const uint8_t* w4,
+                                     const float* w_s, const float* w_sum, const float* residual, float* y, int k, int n,
+                                     void* stream);
+/* Prefill: a4 [m][k/2], s_x/b_x [m], w4 [n][k/2]; k % 64 == 0. */
+int flexllm_linear_u4i4_gemm(const uint8_t* a4, const uint8_t* w4, int32_t* acc, int m, int k, int n, void* stream);
+int flexllm_linear_u4i4_gemm_dequant(const uint8_t* a4, const float* s_x, const float* b_x, const uint8_t* w4,
+                                     const float* w_s, const float* w_sum, const float* residual, float* y, int m, int k,
+                                     int n, void* stream);
+
 /* ---- FHT.h ---------------------------------------------------------------------------- */
 /* y = H_n x / scale (Sylvester order, butterfly stage order of the reference's omega network, so
  * the fp32 result is bit-identical).  Replaces pref_FHT (Modules/FHT.h:7-67) and dec_FHT

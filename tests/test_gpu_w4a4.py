@@ -1,0 +1,95 @@
+"""W4A4 linear layers (asymmetric uint4 activations x symmetric int4 weights, two values per byte): the decode GEMV
+and the prefill GEMM against the oracle, built the way the reference's Linear_Layer_*_tb.cpp builds its inputs."""
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+rng = np.random.default_rng(404)
+
+
+@pytest.fixture(scope="module")
+def fx():
+    import flexllm_amd as fx
+    fx.lib()
+    return fx
+
+
+def pack(values):
+    v = np.asarray(values).astype(np.uint8) & 0xF
+    return (v[..., 0::2] | (v[..., 1::2] << 4)).astype(np.uint8)
+
+
+def quantise_weights_int4(w):
+    """As Linear_Layer_Decoding_tb.cpp:160-190: per output channel scale = max|w|/7 (0 -> 1), q = clamp(round(w/s)),
+    w_sum = running float32 sum of the dequantised weights."""
+    scale = (np.abs(w).max(axis=1) / np.float32(7.0)).astype(np.float32)
+    scale[scale == 0] = 1.0
+    q = np.clip(np.round(w / scale[:, None]), -8, 7).astype(np.int8)
+    deq = (q.astype(np.float32) * scale[:, None]).astype(np.float32)
+    w_sum = np.zeros(w.shape[0], np.float32)
+    for j in range(w.shape[1]):
+        w_sum = (w_sum + deq[:, j]).astype(np.float32)
+    return q, scale, w_sum, deq
+
+
+def test_pack_nibbles(fx):
+    v = rng.integers(-8, 8, (7, 64)).astype(np.int8)
+    assert np.array_equal(fx.ops.pack_nibbles(fx.to_device(v)).numpy(), pack(v))
+    u = rng.integers(0, 16, (3, 4096)).astype(np.uint8)
+    assert np.array_equal(fx.ops.pack_nibbles(fx.to_device(u)).numpy(), pack(u))
+
+
+@pytest.mark.parametrize("k,n", [(2048, 2048), (8192, 2048), (2048, 16384), (32, 1), (64, 33), (4096, 500)])
+def test_gemv_u4i4_exact(fx, k, n):
+    x = rng.integers(0, 16, k).astype(np.uint8)
+    w = rng.integers(-8, 8, (n, k)).astype(np.int8)
+    acc = fx.ops.linear_u4i4_gemv(fx.to_device(pack(x)), fx.to_device(pack(w))).numpy()
+    assert np.array_equal(acc, w.astype(np.int32) @ x.astype(np.int32))
+    # extremes: all 15 x all -8
+    xe = np.full(k, 15, np.uint8); we = np.full((n, k), -8, np.int8)
+    assert np.all(fx.ops.linear_u4i4_gemv(fx.to_device(pack(xe)), fx.to_device(pack(we))).numpy() == -120 * k)
+
+
+@pytest.mark.parametrize("m,k,n", [(128, 64, 128), (160, 2048, 384), (1024, 2048, 2048), (33, 128, 257), (1, 64, 1)])
+def test_gemm_u4i4_exact(fx, m, k, n):
+    a = rng.integers(0, 16, (m, k)).astype(np.uint8)
+    w = rng.integers(-8, 8, (n, k)).astype(np.int8)
+    acc = fx.ops.linear_u4i4_gemm(fx.to_device(pack(a)), fx.to_device(pack(w))).numpy()
+    assert np.array_equal(acc, a.astype(np.int32) @ w.astype(np.int32).T)
+
+
+def test_w4a4_layer_like_the_reference_testbench(fx, oracle):
+    """quant (asym uint4) -> linear -> dequant with zero point, decode and prefill shapes: bit-exact against the oracle
+    chain, and within the testbench's own 1e-2 criterion of the fake-quant golden (…_tb.cpp:215-236)."""
+    m, k, n = 96, 2048, 2048
+    x = rng.standard_normal((m, k)).astype(np.float32)
+    wf = rng.standard_normal((n, k)).astype(np.float32)
+    q_w, w_s, w_sum, w_deq = quantise_weights_int4(wf)
+    res = rng.standard_normal((m, n)).astype(np.float32)
+    # device: quantise, pack, multiply
+    dq, ds, db = fx.ops.quant_asym_u8(fx.to_device(x), bits=4)
+    a4 = fx.ops.pack_nibbles(dq)
+    w4 = fx.to_device(pack(q_w))
+    dws, dwsum = fx.to_device(w_s), fx.to_device(w_sum)
+    y = fx.ops.linear_u4i4_gemm_dequant(a4, ds, db, w4, dws, dwsum).numpy()
+    y_res = fx.ops.linear_u4i4_gemm_dequant(a4, ds, db, w4, dws, dwsum, residual=fx.to_device(res)).numpy()
+    # oracle chain
+    q_ref, s_ref, b_ref = oracle.quant_asym(x, bits=4)
+    assert np.array_equal(dq.numpy(), q_ref)
+    acc_ref = q_ref.astype(np.int32) @ q_w.astype(np.int32).T
+    ref = oracle.dequant(acc_ref, s_ref, w_s, b_x=b_ref, w_sum=w_sum)
+    assert np.array_equal(y, ref)
+    assert np.array_equal(y_res, oracle.residual(ref, res))
+    # decode path row by row
+    a4_h, s_h, b_h = a4.numpy(), ds.numpy().reshape(-1), db.numpy().reshape(-1)
+    for row in (0, 17, m - 1):
+        yv = fx.ops.linear_u4i4_gemv_dequant(fx.to_device(a4_h[row]), fx.to_device(s_h[row:row + 1]), fx.to_device(b_h[row:row + 1]),
+                                             w4, dws, dwsum).numpy()
+        assert np.array_equal(yv, ref[row])
+    # the testbench's criterion against the fake-quant golden (float matmul of the dequantised operands).  The
+    # golden needs the fake-quantised input: x_fq = q*s + b
+    x_fq = (q_ref.astype(np.float32) * s_ref[:, None] + b_ref[:, None]).astype(np.float32)
+    gold = x_fq.astype(np.float64) @ w_deq.astype(np.float64).T
+    big = np.abs(gold) > 1.0
+    assert np.max(np.abs(y[big] - gold[big]) / np.abs(gold[big])) < 1e-2
