@@ -41,6 +41,97 @@ def bytes_per_token(cfg, mean_len):
     return w + scales + gamma + lm_head + kv_read + kv_write
 
 
+def _time(stream, Event, fn, reps):
+    fn(0)
+    stream.sync()
+    e0, e1 = Event(), Event()
+    e0.record(stream)
+    for i in range(reps):
+        fn(i)
+    e1.record(stream)
+    e1.sync()
+    return e0.elapsed_ms(e1) * 1e3 / reps          # microseconds per call
+
+
+def module_legs(fx, lib, synth, ops, stream, Event):
+    """Single-module timings on seeded synthetic inputs, weights cycled through rings larger than the 256 MB
+    memory-side cache: (1) decode linear 2048x2048, (2) Hadamard + per-token quantisation of 1024 tokens,
+    (3) the prefill linear stack of one layer at M=1024, (4) prefill attention at S=1024."""
+    P = lambda a: C.c_void_p(a.ptr) if a is not None else None
+    out = {}
+    # (1) quantise -> GEMV -> dequant, 1 x 2048 against 2048 x 2048
+    K = N = 2048
+    ring = [synth.device_i8((N, K), 9000 + i) for i in range(80)]                       # 336 MB
+    x = synth.device_uniform_f32((1, K), 9100, -3, 3)
+    w_s = synth.device_uniform_f32((N,), 9101, 1e-3, 1e-2)
+    xq = fx.empty((1, K), np.int8); xs = fx.empty((1,), np.float32); y = fx.empty((N,), np.float32)
+    def leg1(i):
+        lib.flexllm_quant_sym_i8(P(x), P(xq), P(xs), 1, K, stream.handle)
+        lib.flexllm_linear_i8_gemv_dequant(P(xq), P(xs), P(ring[i % len(ring)]), P(w_s), None, P(y), K, N, stream.handle)
+    us = _time(stream, Event, leg1, 160)
+    def leg1b(i):
+        lib.flexllm_linear_i8_gemv_dequant(P(xq), P(xs), P(ring[i % len(ring)]), P(w_s), None, P(y), K, N, stream.handle)
+    us_b = _time(stream, Event, leg1b, 160)
+    b1 = N * K + 4 * N + 4 * K + 4 * N
+    out["linear_decode_2048x2048"] = {"bytes": b1, "us_quant_gemv_dequant": round(us, 2), "us_gemv_dequant": round(us_b, 2),
+                                      "GBs_gemv": round(b1 / us_b / 1e3, 1), "hbm_frac_gemv": round(b1 / us_b / 1e3 / HBM_PEAK_GBS, 4)}
+    del ring
+    # (2) FHT / sqrt(n) -> per-token int8, 1024 tokens
+    for n in (2048, 8192):
+        xf = synth.device_normal_f32((1024, n), 9200 + n) if hasattr(synth, "device_normal_f32") else synth.device_uniform_f32((1024, n), 9200 + n, -2, 2)
+        q = fx.empty((1024, n), np.int8); sc = fx.empty((1024,), np.float32)
+        def leg2(i):
+            lib.flexllm_fht_quant_i8(P(xf), P(q), P(sc), 1024, n, C.c_float(float(np.sqrt(n))), stream.handle)
+        us = _time(stream, Event, leg2, 20)
+        b2 = 1024 * (4 * n + n + 4)
+        out["fht_quant_1024x%d" % n] = {"bytes": b2, "us": round(us, 2), "GBs": round(b2 / us / 1e3, 1),
+                                        "hbm_frac": round(b2 / us / 1e3 / HBM_PEAK_GBS, 4)}
+    # (3) prefill linear stack of one layer, M = 1024
+    M, H, KV, I = 1024, 2048, 512, 8192
+    a = synth.device_i8((M, H), 9300); a8 = synth.device_i8((M, I), 9301)
+    s_x = synth.device_uniform_f32((M,), 9302, 0.01, 0.02)
+    res = synth.device_uniform_f32((M, H), 9303, -1, 1)
+    nl = 6                                                                               # 6 x 60.8 MB = 365 MB of weights
+    wq = [synth.device_i8((H + 2 * KV, H), 9310 + i) for i in range(nl)]
+    wo = [synth.device_i8((H, H), 9320 + i) for i in range(nl)]
+    wg = [synth.device_i8((2 * I, H), 9330 + i) for i in range(nl)]
+    wd = [synth.device_i8((H, I), 9340 + i) for i in range(nl)]
+    sc_n = synth.device_uniform_f32((2 * I,), 9350, 1e-4, 2e-4)
+    yq = fx.empty((M, H + 2 * KV), np.float32); yo = fx.empty((M, H), np.float32); yh = fx.empty((M, I), np.float32)
+    legs = {
+        "qkv": (lambda i: lib.flexllm_linear_i8_gemm_dequant(P(a), P(s_x), P(wq[i % nl]), P(sc_n), None, P(yq), M, H, H + 2 * KV, stream.handle), 2 * M * H * (H + 2 * KV)),
+        "o+res": (lambda i: lib.flexllm_linear_i8_gemm_dequant(P(a), P(s_x), P(wo[i % nl]), P(sc_n), P(res), P(yo), M, H, H, stream.handle), 2 * M * H * H),
+        "gate_up+swiglu": (lambda i: lib.flexllm_linear_i8_gemm_swiglu(P(a), P(s_x), P(wg[i % nl]), P(sc_n), P(yh), M, H, I, stream.handle), 2 * M * H * 2 * I),
+        "down+res": (lambda i: lib.flexllm_linear_i8_gemm_dequant(P(a8), P(s_x), P(wd[i % nl]), P(sc_n), P(res), P(yo), M, I, H, stream.handle), 2 * M * I * H),
+    }
+    stack = {}
+    tot_us, tot_ops = 0.0, 0
+    for name, (fn, opsn) in legs.items():
+        us = _time(stream, Event, fn, 4 * nl)
+        stack[name] = {"us": round(us, 2), "TOPs": round(opsn / us / 1e6, 1), "mfma_frac": round(opsn / us / 1e6 / INT8_PEAK_TOPS, 4)}
+        tot_us += us; tot_ops += opsn
+    stack["total"] = {"us": round(tot_us, 2), "GOP": round(tot_ops / 1e9, 2), "TOPs": round(tot_ops / tot_us / 1e6, 1),
+                      "mfma_frac": round(tot_ops / tot_us / 1e6 / INT8_PEAK_TOPS, 4)}
+    out["prefill_linear_stack_M1024"] = stack
+    del wq, wo, wg, wd
+    # (4) prefill attention, S = 1024, 32/8 heads, reading the int8 cache
+    S, QH, KVH = 1024, 32, 8
+    q8 = synth.device_i8((S, QH, 64), 9400)
+    kc, vc = ops.kv_cache(KVH, S)
+    lib.flexllm_rt_fill_i8(P(kc), C.c_size_t(kc.size), C.c_uint64(9401), -100, 100, stream.handle)
+    lib.flexllm_rt_fill_i8(P(vc), C.c_size_t(vc.size), C.c_uint64(9402), -100, 100, stream.handle)
+    scl = ops.Scales(np.full(QH, 4e-3, np.float32), np.full(KVH, 0.03, np.float32), np.full(KVH, 0.03, np.float32), np.full(QH, 1.0 / 255, np.float32))
+    o = fx.empty((S, QH, 64), np.float32)
+    def leg4(i):
+        lib.flexllm_mha_i8_prefill(P(q8), P(kc), P(vc), scl.ref(), P(o), None, S, QH, KVH, 64, S, stream.handle)
+    us = _time(stream, Event, leg4, 20)
+    ops4 = 2 * 2 * QH * S * S * 64
+    out["attention_prefill_S1024"] = {"us": round(us, 2), "GOP_full_S2": round(ops4 / 1e9, 2), "TOPs_full_S2": round(ops4 / us / 1e6, 1),
+                                      "mfma_frac_full_S2": round(ops4 / us / 1e6 / INT8_PEAK_TOPS, 4),
+                                      "note": "causal half computed, scores twice (two-pass softmax); bound by exp/division per probability"}
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -48,6 +139,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=8)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-prefill", action="store_true", help="skip the prefill timing")
+    ap.add_argument("--no-modules", action="store_true", help="skip the module-level legs")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on one GPU only (no collectives, no sharding); use --gpus 1", file=sys.stderr)
@@ -138,6 +230,11 @@ def main():
         except Exception as e:  # prefill path not available in this build
             print("prefill leg skipped: %s" % e, file=sys.stderr)
 
+    # ---- module-level legs: the other configurations the metric's source names, each against its roofline ----
+    modules = None
+    if not args.no_modules:
+        modules = module_legs(fx, lib, synth, ops, stream, Event)
+
     # ---- CPU baseline: the oracle (scalar C port of the reference modules), bounded sample --------------
     cpu = None
     if not args.no_cpu:
@@ -190,6 +287,7 @@ def main():
         "gemv_gate_up": {"kernel": "gemv_i8_kernel<2,4,swiglu> stand-alone (2048->2x8192), 16 distinct weight buffers",
                          "achieved_GBs": round(kern_gbs, 1), "hbm_frac": round(kern_gbs / HBM_PEAK_GBS, 4),
                          "bytes_per_launch": int(kern_bytes), "avg_us": round(kern_ms * 1e3, 3)},
+        "modules": modules,
         "cpu_baseline": cpu,
     }
     print(json.dumps(result))
