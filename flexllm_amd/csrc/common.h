@@ -160,15 +160,22 @@ __device__ __forceinline__ int quant_round_fast(float x, float rs, bool& near_ti
 }
 template <int N>
 __device__ __forceinline__ void quant_vector(const float (&v)[N], float s, int (&n)[N]) {
-    bool redo = !quant_fast_ok(s);
-    if (!redo) {
-        const float rs = 1.0f / s;
-#pragma unroll
-        for (int i = 0; i < N; i++) n[i] = quant_round_fast(v[i], rs, redo);
-    }
-    if (redo) {                                      // rare (about 1e-4 per element): exact path for this lane
+    if (!quant_fast_ok(s)) {
 #pragma unroll
         for (int i = 0; i < N; i++) n[i] = quant_round(v[i], s);
+        return;
+    }
+    const float rs = 1.0f / s;
+    constexpr int G = N % 4 == 0 ? 4 : N;            // the exact path is taken per group: rare (about 2e-4 per element)
+#pragma unroll
+    for (int g = 0; g < N / G; g++) {
+        bool redo = false;
+#pragma unroll
+        for (int i = 0; i < G; i++) n[g * G + i] = quant_round_fast(v[g * G + i], rs, redo);
+        if (redo) {
+#pragma unroll
+            for (int i = 0; i < G; i++) n[g * G + i] = quant_round(v[g * G + i], s);
+        }
     }
 }
 

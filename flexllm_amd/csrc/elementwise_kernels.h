@@ -126,9 +126,12 @@ __global__ __launch_bounds__(kBlock) void rmsnorm_kernel(const float* __restrict
 #pragma unroll
         for (int i = 0; i < VPT; i++) {
             const int idx = threadIdx.x + i * kBlock;
-            if (idx < nvec)
-                qr[idx] = pack4_i8(quant_round(v[i].x, sc), quant_round(v[i].y, sc), quant_round(v[i].z, sc),
-                                   quant_round(v[i].w, sc));
+            if (idx < nvec) {
+                const float f[4] = {v[i].x, v[i].y, v[i].z, v[i].w};
+                int nq[4];
+                quant_vector(f, sc, nq);
+                qr[idx] = pack4_i8(nq[0], nq[1], nq[2], nq[3]);
+            }
         }
     }
 }

@@ -124,8 +124,12 @@ __global__ __launch_bounds__(kFhtBlock) void fht_kernel(const float* __restrict_
         const float sc = sym_scale(amax, 127.0f);
         if (t == 0) s[row] = sc;
         int8_t* lds_q = reinterpret_cast<int8_t*>(lds);
+        {
+            int nq[NR];
+            quant_vector(b, sc, nq);          // x * (1/s) with the exact x / s near rounding ties: same integers
 #pragma unroll
-        for (int r = 0; r < NR; r++) lds_q[r * 256 + t] = (int8_t)quant_round(b[r], sc);
+            for (int r = 0; r < NR; r++) lds_q[r * 256 + t] = (int8_t)nq[r];
+        }
         __syncthreads();
         i32x4* qr = reinterpret_cast<i32x4*>(q + row * N);
         for (int c = t; c < N / 16; c += kFhtBlock) qr[c] = reinterpret_cast<const i32x4*>(lds_q)[c];
