@@ -143,8 +143,19 @@ void pref_quant_layer_fp32_qint(IS& input_stream, OSB& input_s_b_stream, OQ& out
 // Modules/quant.h:332-338
 template <int qint_bit, bool is_act_asym, int block_parallel, int max_input_dim, class IS, class OSB, class OQ>
 void dec_quant_layer_fp32_qint(IS& input_stream, OSB& input_s_b_stream, OQ& output_stream, int input_dim = max_input_dim) {
-    static_assert(qint_bit == 8 && !is_act_asym, "the GPU path behind this name is the symmetric int8 instantiation");
+    static_assert((qint_bit == 8 && !is_act_asym) || is_act_asym, "symmetric int8, or asymmetric unsigned with 2..8 bits");
     auto x = drain_dec<float>(input_stream, input_dim, block_parallel);
+    if constexpr (is_act_asym) {             // Modules/quant.h:382-405: scale (max-min)/(2^bits-1), zero point = min
+        DeviceArray<float> dxa(x), dsa(1), dba(1);
+        DeviceArray<uint8_t> dqa(input_dim);
+        check(flexllm_quant_asym_u8(dxa.get(), dqa.get(), dsa.get(), dba.get(), qint_bit, 1, input_dim, nullptr));
+        typename OSB::value_type pa;
+        pa[0] = dsa.download()[0];
+        pa[1] = dba.download()[0];
+        input_s_b_stream.write(pa);
+        fill_dec(output_stream, dqa.download(), input_dim, block_parallel);
+        return;
+    }
     DeviceArray<float> dx(x), ds(1);
     DeviceArray<int8_t> dq(input_dim);
     check(flexllm_quant_sym_i8(dx.get(), dq.get(), ds.get(), 1, input_dim, nullptr));
@@ -179,16 +190,19 @@ void pref_dequant_layer_qint_fp32(IS& input_stream, ISB& input_s_b_stream, IW& w
 template <int qint_bit, bool is_act_asym, int block_parallel, int weight_parallel, int max_output_dim, class IS, class ISB, class IW, class OS>
 void dec_dequant_layer_qint_fp32_bandwidth(IS& input_stream, ISB& input_s_b_stream, IW& weight_s_sum_stream, OS& output_stream,
                                            int output_dim = max_output_dim) {
-    static_assert(!is_act_asym, "symmetric path");
-    const float s = input_s_b_stream.read()[0];
+    const auto s_b_pack = input_s_b_stream.read();
+    const float s = s_b_pack[0];
+    const float b = is_act_asym ? s_b_pack[is_act_asym ? 1 : 0] : 0.0f;
     const int per = output_dim / block_parallel;
-    std::vector<float> ws(output_dim);
+    std::vector<float> ws(output_dim), wsum(output_dim);
     std::vector<int32_t> acc(output_dim);
     for (int k = 0; k < output_dim / (block_parallel * weight_parallel); k++) {
         // Modules/quant.h:491-501: weight_s[m*weight_parallel+n] belongs to lane m, step n of this group
         for (int i = 0; i < block_parallel * weight_parallel; i++) {
             const int lane = i / weight_parallel, n = i % weight_parallel;
-            ws[(size_t)lane * per + k * weight_parallel + n] = weight_s_sum_stream.read()[0];
+            const auto wp = weight_s_sum_stream.read();
+            ws[(size_t)lane * per + k * weight_parallel + n] = wp[0];
+            if (is_act_asym) wsum[(size_t)lane * per + k * weight_parallel + n] = wp[is_act_asym ? 1 : 0];
         }
         for (int n = 0; n < weight_parallel; n++) {
             auto pack = input_stream.read();
@@ -196,8 +210,9 @@ void dec_dequant_layer_qint_fp32_bandwidth(IS& input_stream, ISB& input_s_b_stre
         }
     }
     DeviceArray<int32_t> dacc(acc);
-    DeviceArray<float> ds(std::vector<float>{s}), dws(ws), dy(output_dim);
-    check(flexllm_dequant_i32_f32(dacc.get(), ds.get(), nullptr, dws.get(), nullptr, dy.get(), 1, output_dim, nullptr));
+    DeviceArray<float> ds(std::vector<float>{s}), db(std::vector<float>{b}), dws(ws), dwsum(wsum), dy(output_dim);
+    check(flexllm_dequant_i32_f32(dacc.get(), ds.get(), is_act_asym ? db.get() : nullptr, dws.get(),
+                                  is_act_asym ? dwsum.get() : nullptr, dy.get(), 1, output_dim, nullptr));
     fill_dec(output_stream, dy.download(), output_dim, block_parallel);
 }
 // Modules/quant.h:252-261 (static per-layer-per-head scale)
@@ -243,6 +258,33 @@ void dec_Linear_Layer_i8xi8(IS& input_seq, const DeviceWeight& weight, OS& outpu
     DeviceArray<int8_t> dx(x);
     DeviceArray<int32_t> dc(output_dim);
     check(flexllm_linear_i8_gemv(dx.get(), weight.w.get(), dc.get(), input_dim, output_dim, nullptr));
+    fill_dec(output_seq, dc.download(), output_dim, block_parallel);
+}
+// A 4-bit weight matrix resident in HBM: values -8..7, two per byte along the input dimension (low nibble = even
+// index), from the row-major one-value-per-byte form the testbenches build (q_weight_val, …_tb.cpp:184).
+struct DeviceWeight4 {
+    DeviceArray<uint8_t> w4;
+    int out_dim = 0, in_dim = 0;
+    DeviceWeight4() = default;
+    DeviceWeight4(const int8_t* row_major, int n, int k) : out_dim(n), in_dim(k) {
+        std::vector<uint8_t> p((size_t)n * k / 2);
+        for (size_t i = 0; i < p.size(); i++) p[i] = (uint8_t)((row_major[2 * i] & 0xF) | ((row_major[2 * i + 1] & 0xF) << 4));
+        w4.upload(p);
+    }
+};
+// Modules/Linear_Layer.h:862-869 (is_uint_input = true: unsigned 4-bit activations), weight streams replaced by
+// a resident DeviceWeight4
+template <int block_parallel, int weight_parallel, int max_input_dim = 2048, int max_log2_input_dim = 11, int max_output_dim = 2048,
+          bool is_uint_input = false, class IS, class OS>
+void dec_Linear_Layer_i4xi4(IS& input_seq, const DeviceWeight4& weight, OS& output_seq, int input_dim = max_input_dim,
+                            int output_dim = max_output_dim) {
+    static_assert(is_uint_input, "the W4A4 path has unsigned (asymmetric) activations");
+    auto x = drain_dec<uint8_t>(input_seq, input_dim, block_parallel);
+    std::vector<uint8_t> x4(input_dim / 2);
+    for (int i = 0; i < input_dim / 2; i++) x4[i] = (uint8_t)((x[2 * i] & 0xF) | ((x[2 * i + 1] & 0xF) << 4));
+    DeviceArray<uint8_t> dx(x4);
+    DeviceArray<int32_t> dc(output_dim);
+    check(flexllm_linear_u4i4_gemv(dx.get(), weight.w4.get(), dc.get(), input_dim, output_dim, nullptr));
     fill_dec(output_seq, dc.download(), output_dim, block_parallel);
 }
 // Modules/Linear_Layer.h:612-617 / :1103-1108

@@ -95,6 +95,76 @@ static void QuantWrapper_Linear_Layer_q_decoding_test() {
     verdict("QuantWrapper Linear Layer (decode, W8A8)", correct);
 }
 
+// The reference's own configuration of this testbench (Linear_Layer_Decoding_tb.cpp:93-251): asymmetric uint4
+// activations, symmetric int4 weights, dequant with zero point times the row sum of the dequantised weights.
+static void QuantWrapper_Linear_Layer_q_decoding_w4a4_test() {
+    const int T = 8, K = HIDDEN_DIM, N = HIDDEN_DIM, BP = T_BLOCK_PARALLEL, per = K / BP;
+    std::default_random_engine gen(42);
+    std::uniform_real_distribution<float> dist(-1.0, 1.0);
+    std::vector<float> input_gold((size_t)T * K), weight_gold((size_t)N * K), weight_s(N), weight_sum(N);
+    std::vector<int8_t> q_weight((size_t)N * K);
+    std::vector<vec<float, BP>> input_mmap((size_t)T * per);
+    for (int i = 0; i < T; i++) {
+        float vmax = -1e30f, vmin = 1e30f;
+        for (int j = 0; j < K; j++) {
+            float val = dist(gen);
+            input_gold[(size_t)i * K + j] = val;
+            vmax = std::max(vmax, val); vmin = std::min(vmin, val);
+            input_mmap[(size_t)i * per + j % per][j / per] = val;
+        }
+        float scale = (vmax - vmin) / 15.0f;
+        if (scale == 0) scale = 1.0f;
+        for (int j = 0; j < K; j++) {          // fake quant, …_tb.cpp:137-147
+            float& v = input_gold[(size_t)i * K + j];
+            v = std::round((v - vmin) / scale) * scale + vmin;
+        }
+    }
+    for (int i = 0; i < N; i++) {              // …_tb.cpp:160-190
+        float w_max = 0;
+        for (int j = 0; j < K; j++) { weight_gold[(size_t)i * K + j] = dist(gen); w_max = std::max(w_max, std::abs(weight_gold[(size_t)i * K + j])); }
+        float scale = w_max / 7.0f;
+        if (scale == 0) scale = 1.0f;
+        weight_s[i] = scale; weight_sum[i] = 0;
+        for (int j = 0; j < K; j++) {
+            int qval = (int)std::round(weight_gold[(size_t)i * K + j] / scale);
+            qval = std::max(-8, std::min(7, qval));
+            weight_gold[(size_t)i * K + j] = qval * scale;
+            q_weight[(size_t)i * K + j] = (int8_t)qval;
+            weight_sum[i] += weight_gold[(size_t)i * K + j];
+        }
+    }
+    DeviceWeight4 weight(q_weight.data(), N, K);
+    std::vector<vec<float, BP>> output_mmap((size_t)T * N / BP);
+    for (int t = 0; t < T; t++) {
+        stream<vec<float, BP>> x_s, y_s;
+        stream<vec<float, 2>> s_b, w_s;
+        stream<vec<uint8_t, BP>> q_s;
+        stream<vec<int32_t, BP>> acc_s;
+        for (int k = 0; k < per; k++) x_s.write(input_mmap[(size_t)t * per + k]);
+        dec_quant_layer_fp32_qint<4, true, BP, HIDDEN_DIM>(x_s, s_b, q_s, K);
+        dec_Linear_Layer_i4xi4<BP, DEC_W_PARALLEL, HIDDEN_DIM, 11, HIDDEN_DIM, true>(q_s, weight, acc_s, K, N);
+        for (int kk = 0; kk < N / (BP * DEC_W_PARALLEL); kk++)
+            for (int m = 0; m < BP; m++)
+                for (int n = 0; n < DEC_W_PARALLEL; n++) {
+                    vec<float, 2> p;
+                    p[0] = weight_s[(size_t)m * (N / BP) + kk * DEC_W_PARALLEL + n];
+                    p[1] = weight_sum[(size_t)m * (N / BP) + kk * DEC_W_PARALLEL + n];
+                    w_s.write(p);
+                }
+        dec_dequant_layer_qint_fp32_bandwidth<4, true, BP, DEC_W_PARALLEL, HIDDEN_DIM>(acc_s, s_b, w_s, y_s, N);
+        for (int k = 0; k < N / BP; k++) output_mmap[(size_t)t * (N / BP) + k] = y_s.read();
+    }
+    bool correct = true;
+    for (int i = 0; i < T && correct; i++)
+        for (int j = 0; j < N; j++) {
+            double gold = 0;
+            for (int k = 0; k < K; k++) gold += (double)input_gold[(size_t)i * K + k] * weight_gold[(size_t)j * K + k];
+            const float my = output_mmap[(size_t)i * (N / BP) + j % (N / BP)][j / (N / BP)];
+            if (std::abs(my - gold) > 1e-2 * std::abs(gold) + 1e-3) { correct = false; std::cout << "Mismatch at (" << i << ", " << j << "): My: " << my << ", Ref_fq: " << gold << std::endl; break; }
+        }
+    verdict("QuantWrapper Linear Layer (decode, W4A4 asymmetric: the reference's shipped configuration)", correct);
+}
+
 static void QuantWrapper_Linear_Layer_q_prefilling_test() {
     const int S = 64, K = HIDDEN_DIM, N = KV_HIDDEN_DIM, TP = TOKEN_PARALLEL;
     std::default_random_engine gen(42);
@@ -297,6 +367,7 @@ static void pref_MHA_test() {
 int main() {
     try {
         QuantWrapper_Linear_Layer_q_decoding_test();
+        QuantWrapper_Linear_Layer_q_decoding_w4a4_test();
         QuantWrapper_Linear_Layer_q_prefilling_test();
         FHT_test();
         Elementwise_test();

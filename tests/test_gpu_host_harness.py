@@ -17,4 +17,4 @@ def test_cpp_module_harness_passes():
     out = subprocess.run([BIN], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=300)
     print(out.stdout)
     assert out.returncode == 0, out.stdout
-    assert out.stdout.count("passed correctness check") == 5 and "failed" not in out.stdout
+    assert out.stdout.count("passed correctness check") == 6 and "failed" not in out.stdout
