@@ -140,6 +140,9 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-prefill", action="store_true", help="skip the prefill timing")
     ap.add_argument("--no-modules", action="store_true", help="skip the module-level legs")
+    ap.add_argument("--copy-probe", action="store_true",
+                    help="only run three 1 GiB device-to-device copies and exit: the transfer of known size that scales "
+                         "the FETCH_SIZE / WRITE_SIZE counters")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on one GPU only (no collectives, no sharding); use --gpus 1", file=sys.stderr)
@@ -150,6 +153,16 @@ def main():
     from flexllm_amd.device import Event, device_sync
 
     lib = fx.lib()
+    if args.copy_probe:
+        n = 1 << 30
+        src = synth.device_i8((n,), 1)
+        dst = fx.empty((n,), np.int8)
+        device_sync()
+        for _ in range(3):
+            fx.check(lib.flexllm_rt_memcpy_d2d(C.c_void_p(dst.ptr), C.c_void_p(src.ptr), C.c_size_t(n), None))
+        device_sync()
+        print(json.dumps({"copy_probe_bytes": n, "copies": 3}))
+        return
     cfg = llama.make_config()
     K, W = args.steps, args.warmup
     assert K + W < cfg["max_pos"]
