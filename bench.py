@@ -140,6 +140,8 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-prefill", action="store_true", help="skip the prefill timing")
     ap.add_argument("--no-modules", action="store_true", help="skip the module-level legs")
+    ap.add_argument("--decode-mode", type=int, default=0, choices=[0, 1],
+                    help="0: persistent decode kernel (default), 1: one kernel per stage replayed as a HIP graph")
     ap.add_argument("--copy-probe", action="store_true",
                     help="only run three 1 GiB device-to-device copies and exit: the transfer of known size that scales "
                          "the FETCH_SIZE / WRITE_SIZE counters")
@@ -168,6 +170,7 @@ def main():
     assert K + W < cfg["max_pos"]
     dev_w = llama.synth_weights(cfg, seed=1, device=True)
     model = llama.Llama(cfg, dev_w)
+    model.set_decode_mode(args.decode_mode)
     # cache pre-filled with seeded int8 values directly in cache layout, as the reference's decode harness does
     C_fill = lib.flexllm_rt_fill_i8
     fx.check(C_fill(C.c_void_p(model.k_cache.ptr), C.c_size_t(model.k_cache.size), C.c_uint64(901), -100, 100, None))
@@ -282,7 +285,8 @@ def main():
         "ms_per_step": round(ms_per_step, 5), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "int8", "data": "synthetic",
         "config": {"workload": "Llama-3.2-1B W8A8 SpinQuant greedy decode, batch 1, int8 KV cache, context %d..%d, "
-                               "fp16 tied lm_head, one persistent-kernel launch per %d tokens" % (pos_timed + 1, pos_end, TOKENS_PER_LAUNCH),
+                               "fp16 tied lm_head, %s" % (pos_timed + 1, pos_end, ("one persistent-kernel launch per %d tokens" % TOKENS_PER_LAUNCH)
+                                                         if args.decode_mode == 0 else "one kernel per stage, HIP graph replay"),
                    "layers": cfg["layers"], "context": pos_end, "device": fx.device.device_name()},
         "decode": {"bytes_per_token": int(bpt), "achieved_GBs": round(token_gbs, 1),
                    "hbm_frac": round(token_gbs / HBM_PEAK_GBS, 4), "event_ms_per_step": round(ev_ms / K, 5),
