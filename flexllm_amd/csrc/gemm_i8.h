@@ -200,8 +200,8 @@ __global__ __launch_bounds__(256) void gemm_i8_kernel(const int8_t* __restrict__
 //
 // The loads are issued from inline assembly: the compiler does not track them, so the k-loop waits for them
 // with explicit counters (results return in issue order).
-__host__ __device__ constexpr int gemm_dma_lds_bytes(int bm, int bn, int stages) {
-    return stages * (bm + bn) * 64 > 4 * 32 * 36 * 4 ? stages * (bm + bn) * 64 : 4 * 32 * 36 * 4;   // stages, or the four epilogue patches
+__host__ __device__ constexpr int gemm_dma_lds_bytes(int bm, int bn, int stages, int bkb = 64) {
+    return stages * (bm + bn) * bkb > 4 * 32 * 36 * 4 ? stages * (bm + bn) * bkb : 4 * 32 * 36 * 4;   // stages, or the four epilogue patches
 }
 
 enum GemmDmaEpi { kDmaRaw = 0, kDmaDequant = 1, kDmaSwiglu = 2, kDmaQkv = 3 };
@@ -231,16 +231,23 @@ __device__ __forceinline__ void gemm_wait_vmcnt() {            // s_waitcnt vmcn
     __builtin_amdgcn_s_waitcnt(0x0F70 | (N & 15) | ((N >> 4) << 14));
 }
 
-// kDmaStages LDS stages; WPE = waves per SIMD the register allocation has to leave room for
-template <int BM, int BN, int EPI, int kDmaStages, int WPE>   // at most 7 stages (the wait below distinguishes up to 5 younger ones)
+// kDmaStages LDS stages; WPE = waves per SIMD the register allocation has to leave room for.
+// BKB = k-bytes of a row per stage, 64 or 128.  A 64-byte segment is half a cache line, and the other half is asked
+// for again one stage later: measured with the loads alone (no math, 128 x 256 tiles at K = 2048), the chip moves
+// 23 TB/s into LDS in whole 128-byte lines and 14.5 TB/s in halves.  With 128-byte rows the slot rotation is
+// s ^ ((r >> 1) & 7): two rows span the 64 banks, so 16 consecutive rows of one chunk fall on 16 different bank groups.
+template <int BM, int BN, int EPI, int kDmaStages, int WPE, int BKB>   // at most 7 stages (the wait below distinguishes up to 5 younger ones)
 __global__ __launch_bounds__(256, WPE) void gemm_i8_dma_kernel(const int8_t* __restrict__ a, const int8_t* __restrict__ w,
                                                           int32_t* __restrict__ c_out, const float* __restrict__ s_x,
                                                           const float* __restrict__ w_s, const float* __restrict__ residual,
                                                           float* __restrict__ y, int m, int k, int n, int tiles_m, int tiles_n,
                                                           QkvEpiArgs qa) {
     constexpr int WM = BM / 2, WN = BN / 2, TM = WM / 32, TN = WN / 32;
-    constexpr int A_INSTR = BM / 64, B_INSTR = BN / 64;       // direct loads per wave per stage (16 rows each)
-    constexpr int STAGE = (BM + BN) * 64;
+    static_assert(BKB == 64 || BKB == 128, "64 or 128 k-bytes per row and stage");
+    constexpr int CPR = BKB / 16, RPI = 64 / CPR;             // 16-byte chunks per row; rows per direct load (1 KiB)
+    constexpr int A_INSTR = BM / (4 * RPI), B_INSTR = BN / (4 * RPI);   // direct loads per wave per stage
+    constexpr int STAGE = (BM + BN) * BKB, KS = BKB / 32;     // KS MFMA k-steps per stage
+    auto rot = [](int r) { return BKB == 64 ? (r >> 2) & 3 : (r >> 1) & 7; };
     extern __shared__ __attribute__((aligned(16))) int8_t gemm_smem[];
 
     int tm, tn;
@@ -261,21 +268,21 @@ __global__ __launch_bounds__(256, WPE) void gemm_i8_dma_kernel(const int8_t* __r
     unsigned offa[A_INSTR], offb[B_INSTR];
 #pragma unroll
     for (int j = 0; j < A_INSTR; j++) {
-        const int r = (wave * A_INSTR + j) * 16 + (lane >> 2);
-        offa[j] = (unsigned)min(row0 + r, m - 1) * (unsigned)k + (unsigned)(((lane & 3) ^ ((r >> 2) & 3)) * 16);
+        const int r = (wave * A_INSTR + j) * RPI + lane / CPR;
+        offa[j] = (unsigned)min(row0 + r, m - 1) * (unsigned)k + (unsigned)(((lane % CPR) ^ rot(r)) * 16);
     }
 #pragma unroll
     for (int j = 0; j < B_INSTR; j++) {
-        const int r = (wave * B_INSTR + j) * 16 + (lane >> 2);
-        offb[j] = (unsigned)min(col0 + r, n - 1) * (unsigned)k + (unsigned)(((lane & 3) ^ ((r >> 2) & 3)) * 16);
+        const int r = (wave * B_INSTR + j) * RPI + lane / CPR;
+        offb[j] = (unsigned)min(col0 + r, n - 1) * (unsigned)k + (unsigned)(((lane % CPR) ^ rot(r)) * 16);
     }
     const unsigned lds0 = (unsigned)(uintptr_t)(__attribute__((address_space(3))) void*)gemm_smem;
     auto issue_stage = [&](int kt) {
         const unsigned sb = lds0 + (unsigned)(kt % kDmaStages) * STAGE;
 #pragma unroll
-        for (int j = 0; j < A_INSTR; j++) gemm_dma_issue(a + (size_t)kt * kGemmBK, offa[j], sb + (wave * A_INSTR + j) * 1024);
+        for (int j = 0; j < A_INSTR; j++) gemm_dma_issue(a + (size_t)kt * BKB, offa[j], sb + (wave * A_INSTR + j) * 1024);
 #pragma unroll
-        for (int j = 0; j < B_INSTR; j++) gemm_dma_issue(w + (size_t)kt * kGemmBK, offb[j], sb + BM * 64 + (wave * B_INSTR + j) * 1024);
+        for (int j = 0; j < B_INSTR; j++) gemm_dma_issue(w + (size_t)kt * BKB, offb[j], sb + BM * BKB + (wave * B_INSTR + j) * 1024);
     };
 
     i32x16 acc[TM][TN];
@@ -286,7 +293,7 @@ __global__ __launch_bounds__(256, WPE) void gemm_i8_dma_kernel(const int8_t* __r
 #pragma unroll
             for (int r = 0; r < 16; r++) acc[i][j][r] = 0;
 
-    const int nk = k / kGemmBK;
+    const int nk = k / BKB;
     constexpr int PER = A_INSTR + B_INSTR;                     // direct loads per wave per stage
 #pragma unroll
     for (int s0 = 0; s0 < kDmaStages - 1; s0++)
@@ -295,16 +302,16 @@ __global__ __launch_bounds__(256, WPE) void gemm_i8_dma_kernel(const int8_t* __r
     const int fr = lane & 31, fg = lane >> 5;
     auto read_frags = [&](int kt, int ks, i32x4 (&fa)[TM], i32x4 (&fb)[TN]) {
         const int8_t* sa = gemm_smem + (kt % kDmaStages) * STAGE;
-        const int8_t* sb = sa + BM * 64;
+        const int8_t* sb = sa + BM * BKB;
 #pragma unroll
         for (int i = 0; i < TM; i++) {
             const int r = wm + i * 32 + fr;
-            fa[i] = *reinterpret_cast<const i32x4*>(sa + r * 64 + (((ks * 2 + fg) ^ ((r >> 2) & 3)) * 16));
+            fa[i] = *reinterpret_cast<const i32x4*>(sa + r * BKB + (((ks * 2 + fg) ^ rot(r)) * 16));
         }
 #pragma unroll
         for (int j = 0; j < TN; j++) {
             const int r = wn + j * 32 + fr;
-            fb[j] = *reinterpret_cast<const i32x4*>(sb + r * 64 + (((ks * 2 + fg) ^ ((r >> 2) & 3)) * 16));
+            fb[j] = *reinterpret_cast<const i32x4*>(sb + r * BKB + (((ks * 2 + fg) ^ rot(r)) * 16));
         }
     };
     auto mma = [&](const i32x4 (&fa)[TM], const i32x4 (&fb)[TN]) {
@@ -325,28 +332,33 @@ __global__ __launch_bounds__(256, WPE) void gemm_i8_dma_kernel(const int8_t* __r
         else gemm_wait_vmcnt<0>();
     };
 
-    // Software pipeline over half-stages (32 k-bytes): the fragments of the next half-stage are read from LDS
-    // before the MFMAs of the current one are issued, so the LDS latency runs under matrix work.  The
-    // workgroup barrier sits in the middle of an iteration: after it stage kt+1 is complete in LDS and every
-    // wave has finished reading stage kt, whose buffer the direct loads of the iteration after next overwrite.
+    // Software pipeline over k-steps of 32 bytes: the fragments of the next k-step are read from LDS before the
+    // MFMAs of the current one are issued, so the LDS latency runs under matrix work.  The workgroup barrier
+    // sits before the last k-step of a stage: after it stage kt+1 is complete in LDS and every wave has finished
+    // reading stage kt, whose buffer the direct loads of the iteration after next overwrite.
     i32x4 fa0[TM], fb0[TN], fa1[TM], fb1[TN];
     wait_stage(0);
     __syncthreads();
     read_frags(0, 0, fa0, fb0);
     for (int kt = 0; kt < nk; kt++) {
-        read_frags(kt, 1, fa1, fb1);
-        if (kt + kDmaStages - 1 < nk) issue_stage(kt + kDmaStages - 1);   // into the buffer that held stage kt-1
-        __builtin_amdgcn_sched_barrier(0);
-        mma(fa0, fb0);
-        __builtin_amdgcn_sched_barrier(0);
-        if (kt + 1 < nk) {
-            wait_stage(kt + 1);
-            __syncthreads();
-            read_frags(kt + 1, 0, fa0, fb0);
+#pragma unroll
+        for (int ks = 0; ks < KS; ks += 2) {
+            read_frags(kt, ks + 1, fa1, fb1);
+            if (ks == 0 && kt + kDmaStages - 1 < nk) issue_stage(kt + kDmaStages - 1);   // into the buffer that held stage kt-1
+            __builtin_amdgcn_sched_barrier(0);
+            mma(fa0, fb0);
+            __builtin_amdgcn_sched_barrier(0);
+            if (ks + 2 < KS) {
+                read_frags(kt, ks + 2, fa0, fb0);
+            } else if (kt + 1 < nk) {
+                wait_stage(kt + 1);
+                __syncthreads();
+                read_frags(kt + 1, 0, fa0, fb0);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+            mma(fa1, fb1);
+            __builtin_amdgcn_sched_barrier(0);
         }
-        __builtin_amdgcn_sched_barrier(0);
-        mma(fa1, fb1);
-        __builtin_amdgcn_sched_barrier(0);
     }
 
     // Epilogue.  In the accumulator layout a lane holds ONE column (l%32) and 16 rows of a 32x32 tile, so direct
@@ -461,17 +473,17 @@ __global__ __launch_bounds__(256, WPE) void gemm_i8_dma_kernel(const int8_t* __r
     }
 }
 
-template <int BM, int BN, int EPI, int STAGES = 3, int WPE = 1>
+template <int BM, int BN, int EPI, int STAGES = 3, int WPE = 1, int BKB = 64>
 inline int launch_gemm_dma(const int8_t* a, const int8_t* w, int32_t* c, const float* s_x, const float* w_s,
                            const float* residual, float* y, int m, int k, int n, hipStream_t st, QkvEpiArgs qa = QkvEpiArgs()) {
     static bool opted_in = false;             // more than the default 64 KiB of LDS per workgroup
     if (!opted_in) {
-        FX_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_i8_dma_kernel<BM, BN, EPI, STAGES, WPE>),
-                                   hipFuncAttributeMaxDynamicSharedMemorySize, gemm_dma_lds_bytes(BM, BN, STAGES)));
+        FX_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_i8_dma_kernel<BM, BN, EPI, STAGES, WPE, BKB>),
+                                   hipFuncAttributeMaxDynamicSharedMemorySize, gemm_dma_lds_bytes(BM, BN, STAGES, BKB)));
         opted_in = true;
     }
     const int tm = (m + BM - 1) / BM, tn = (n + BN - 1) / BN;
-    gemm_i8_dma_kernel<BM, BN, EPI, STAGES, WPE><<<tm * tn, 256, gemm_dma_lds_bytes(BM, BN, STAGES), st>>>(a, w, c, s_x, w_s, residual, y, m, k, n, tm, tn, qa);
+    gemm_i8_dma_kernel<BM, BN, EPI, STAGES, WPE, BKB><<<tm * tn, 256, gemm_dma_lds_bytes(BM, BN, STAGES, BKB), st>>>(a, w, c, s_x, w_s, residual, y, m, k, n, tm, tn, qa);
     FX_LAUNCH_CHECK();
     return FLEXLLM_OK;
 }
@@ -489,6 +501,9 @@ inline int launch_gemm(const int8_t* a, const int8_t* w, int32_t* c, const float
     // the direct-load kernel needs 32-bit element offsets into both operands and 16-byte aligned output rows
     const bool dma_ok = (size_t)m * k < (1ull << 31) && (size_t)n * k < (1ull << 31) && n % 4 == 0;
     int mode = dma_ok ? (tiles(128, 128) >= 768 ? 11 : (k >= 4096 && tiles(64, 128) >= 256) ? 19 : 13) : (tiles(128, 128) >= 1024 ? 0 : 2);
+    // whole 128-byte lines per row and stage where K allows: three workgroups of 48 KiB per CU when the grid has
+    // that many, else two of 64 KiB with a fourth stage (the narrow projections stream their weights cold)
+    if ((mode == 13 || mode == 19) && k % 128 == 0) mode = tiles(64, 64) >= 768 ? 38 : 36;
     if (force) mode = atoi(force);
     if (mode >= 10 && !dma_ok) mode = 2;
     const int nk = k / kGemmBK;
@@ -501,6 +516,15 @@ inline int launch_gemm(const int8_t* a, const int8_t* w, int32_t* c, const float
         if (mode == 18) return launch_gemm_dma<64, 64, DE, 6, 2>(a, w, c, s_x, w_s, residual, y, m, k, n, st);
         if (mode == 19) return launch_gemm_dma<64, 128, DE, 4, 2>(a, w, c, s_x, w_s, residual, y, m, k, n, st);
         if (mode == 20) return launch_gemm_dma<128, 128, DE, 4, 2>(a, w, c, s_x, w_s, residual, y, m, k, n, st);
+        if (k % 128 == 0) {
+            if (mode == 31) return launch_gemm_dma<128, 128, DE, 2, 2, 128>(a, w, c, s_x, w_s, residual, y, m, k, n, st);
+            if (mode == 33) return launch_gemm_dma<64, 128, DE, 2, 3, 128>(a, w, c, s_x, w_s, residual, y, m, k, n, st);
+            if (mode == 35) return launch_gemm_dma<64, 64, DE, 2, 4, 128>(a, w, c, s_x, w_s, residual, y, m, k, n, st);
+            if (mode == 36) return launch_gemm_dma<64, 64, DE, 4, 2, 128>(a, w, c, s_x, w_s, residual, y, m, k, n, st);
+            if (mode == 37) return launch_gemm_dma<64, 128, DE, 3, 2, 128>(a, w, c, s_x, w_s, residual, y, m, k, n, st);
+            if (mode == 38) return launch_gemm_dma<64, 64, DE, 3, 3, 128>(a, w, c, s_x, w_s, residual, y, m, k, n, st);
+            if (mode == 39) return launch_gemm_dma<64, 64, DE, 5, 2, 128>(a, w, c, s_x, w_s, residual, y, m, k, n, st);
+        }
         return launch_gemm_dma<64, 64, DE>(a, w, c, s_x, w_s, residual, y, m, k, n, st);
     }
 #define FX_GEMM_LAUNCH(BM, BN, DD)                                                                                \
@@ -549,6 +573,13 @@ inline int launch_gemm_swiglu(const int8_t* a, const int8_t* w_gu, const float* 
     if (mode == 10) return launch_gemm_dma<256, 256, kDmaSwiglu>(a, w_gu, nullptr, s_x, w_s_gu, nullptr, h, m, k, n2, st);
     if (mode == 11) return launch_gemm_dma<128, 128, kDmaSwiglu, 3, 3>(a, w_gu, nullptr, s_x, w_s_gu, nullptr, h, m, k, n2, st);
     if (mode == 12 || mode == 16) return launch_gemm_dma<128, 256, kDmaSwiglu, 2, 2>(a, w_gu, nullptr, s_x, w_s_gu, nullptr, h, m, k, n2, st);
+    if (k % 128 == 0) {
+        if (mode == 30) return launch_gemm_dma<128, 256, kDmaSwiglu, 2, 1, 128>(a, w_gu, nullptr, s_x, w_s_gu, nullptr, h, m, k, n2, st);
+        if (mode == 31) return launch_gemm_dma<128, 128, kDmaSwiglu, 2, 2, 128>(a, w_gu, nullptr, s_x, w_s_gu, nullptr, h, m, k, n2, st);
+        if (mode == 32) return launch_gemm_dma<128, 256, kDmaSwiglu, 3, 1, 128>(a, w_gu, nullptr, s_x, w_s_gu, nullptr, h, m, k, n2, st);
+        if (mode == 33) return launch_gemm_dma<64, 128, kDmaSwiglu, 2, 3, 128>(a, w_gu, nullptr, s_x, w_s_gu, nullptr, h, m, k, n2, st);
+        if (mode == 34) return launch_gemm_dma<128, 128, kDmaSwiglu, 3, 1, 128>(a, w_gu, nullptr, s_x, w_s_gu, nullptr, h, m, k, n2, st);
+    }
     return launch_gemm_dma<64, 64, kDmaSwiglu>(a, w_gu, nullptr, s_x, w_s_gu, nullptr, h, m, k, n2, st);
 }
 
@@ -560,6 +591,14 @@ inline int launch_gemm_qkv(const int8_t* a, const int8_t* w_qkv, const float* s_
     const int n = (qa.q_heads + 2 * qa.kv_heads) * kHd;
     FX_REQUIRE(m % 32 == 0 && qa.pos0 % 64 == 0 && qa.pos0 + m <= qa.max_pos, "gemm_qkv: m=%d pos0=%d max_pos=%d", m, qa.pos0, qa.max_pos);
     FX_REQUIRE((size_t)m * k < (1ull << 31) && (size_t)n * k < (1ull << 31), "gemm_qkv: m=%d k=%d outside the direct-load kernel's range", m, k);
+    static const char* force = getenv("FLEXLLM_GEMM_TILE");
+    const int mode = force ? atoi(force) : (((m + 63) / 64) * (n / 64) >= 768 ? 38 : 36);
+    if (k % 128 == 0) {
+        if (mode == 36) return launch_gemm_dma<64, 64, kDmaQkv, 4, 2, 128>(a, w_qkv, nullptr, s_x, w_s, nullptr, nullptr, m, k, n, st, qa);
+        if (mode == 38) return launch_gemm_dma<64, 64, kDmaQkv, 3, 3, 128>(a, w_qkv, nullptr, s_x, w_s, nullptr, nullptr, m, k, n, st, qa);
+        if (mode == 39) return launch_gemm_dma<64, 64, kDmaQkv, 5, 2, 128>(a, w_qkv, nullptr, s_x, w_s, nullptr, nullptr, m, k, n, st, qa);
+        if (mode == 35) return launch_gemm_dma<64, 64, kDmaQkv, 2, 4, 128>(a, w_qkv, nullptr, s_x, w_s, nullptr, nullptr, m, k, n, st, qa);
+    }
     return launch_gemm_dma<64, 64, kDmaQkv>(a, w_qkv, nullptr, s_x, w_s, nullptr, nullptr, m, k, n, st, qa);
 }
 
