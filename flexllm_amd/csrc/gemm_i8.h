@@ -422,14 +422,40 @@ __global__ __launch_bounds__(256, WPE) void gemm_i8_dma_kernel(const int8_t* __r
     constexpr int EP = 36;                                     // patch pitch in words (rows stay 16-byte aligned)
     int* patch = reinterpret_cast<int*>(gemm_smem) + wave * (32 * EP);
     const int pr = lane >> 3, pc = (lane & 7) * 4;             // row within a group of 8, first of this lane's 4 columns
+    // Every scale this lane needs is loaded before the first tile: a load inside the tile loop would be waited for
+    // together with the stores issued before it (one counter covers both), once per group of rows.
+    float sxv[TM][4];
+    float4 wsv[TN];
+    if constexpr (EPI != kDmaRaw) {
+#pragma unroll
+        for (int i = 0; i < TM; i++)
+#pragma unroll
+            for (int p = 0; p < 4; p++) sxv[i][p] = s_x[min(row0 + wm + i * 32 + p * 8 + pr, m - 1)];
+#pragma unroll
+        for (int j = 0; j < TN; j++) {
+            const int col = col0 + wn + j * 32 + pc;
+            wsv[j] = col < n ? *reinterpret_cast<const float4*>(w_s + col) : make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+        }
+    }
 #pragma unroll
     for (int j = 0; j < TN; j++) {
         const int col = col0 + wn + j * 32 + pc;               // n is a multiple of 4 (checked by the launcher)
         const bool col_ok = col < n;
-        float4 ws = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
-        if constexpr (EPI != kDmaRaw) { if (col_ok) ws = *reinterpret_cast<const float4*>(w_s + col); }
 #pragma unroll
         for (int i = 0; i < TM; i++) {
+            float4 rs[4];                                      // the tile's residual rows, in flight during the turn through LDS
+            bool has_res = false;
+            if constexpr (EPI == kDmaDequant) {
+                has_res = residual != nullptr;
+                if (has_res) {
+#pragma unroll
+                    for (int p = 0; p < 4; p++) {
+                        const int row = row0 + wm + i * 32 + p * 8 + pr;
+                        rs[p] = col_ok && row < m ? *reinterpret_cast<const float4*>(residual + (size_t)row * n + col)
+                                                  : make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+                    }
+                }
+            }
 #pragma unroll
             for (int r = 0; r < 16; r++)
                 patch[((r >> 2) * 8 + (lane >> 5) * 4 + (r & 3)) * EP + (lane & 31)] = acc[i][j][r];
@@ -438,31 +464,35 @@ __global__ __launch_bounds__(256, WPE) void gemm_i8_dma_kernel(const int8_t* __r
             __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
             __builtin_amdgcn_wave_barrier();
             __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+            // One explicit wait per tile, outside the guarded stores: the scales (first tile) and this tile's residual
+            // rows have landed.  Left to the compiler the wait sits behind the store guards, is repeated for every group
+            // of rows, and then also waits for the store issued just before it.
+            if constexpr (EPI != kDmaRaw) { if ((i == 0 && j == 0) || has_res) gemm_wait_vmcnt<0>(); }
 #pragma unroll
             for (int p = 0; p < 4; p++) {
                 const int lr = p * 8 + pr;
                 const int row = row0 + wm + i * 32 + lr;
                 const i32x4 v = *reinterpret_cast<const i32x4*>(patch + lr * EP + pc);
-                if (!(col_ok && row < m)) continue;
+                // the arithmetic runs for every lane and only the store is guarded: a wait placed behind a branch
+                // would be repeated at every later use, and there it would also wait for the stores in between
+                const bool ok = col_ok && row < m;
                 if constexpr (EPI == kDmaRaw) {
-                    *reinterpret_cast<i32x4*>(c_out + (size_t)row * n + col) = v;
+                    if (ok) *reinterpret_cast<i32x4*>(c_out + (size_t)row * n + col) = v;
                 } else {
-                    const float sx = s_x[row];
+                    const float sx = sxv[i][p];
+                    const float4 ws = wsv[j];
                     float4 o;
                     o.x = (float)v[0] * sx * ws.x; o.y = (float)v[1] * sx * ws.y;
                     o.z = (float)v[2] * sx * ws.z; o.w = (float)v[3] * sx * ws.w;
                     if constexpr (EPI == kDmaDequant) {
-                        if (residual) {
-                            const float4 rs = *reinterpret_cast<const float4*>(residual + (size_t)row * n + col);
-                            o.x = o.x + rs.x; o.y = o.y + rs.y; o.z = o.z + rs.z; o.w = o.w + rs.w;
-                        }
-                        *reinterpret_cast<float4*>(y + (size_t)row * n + col) = o;
+                        if (has_res) { o.x = o.x + rs[p].x; o.y = o.y + rs[p].y; o.z = o.z + rs[p].z; o.w = o.w + rs[p].w; }
+                        if (ok) *reinterpret_cast<float4*>(y + (size_t)row * n + col) = o;
                     } else {
                         // weight rows are interleaved (2c gate, 2c+1 up): columns (col, col+1) and (col+2, col+3) are pairs
                         float2 h;
                         h.x = o.y * silu_f(o.x);
                         h.y = o.w * silu_f(o.z);
-                        *reinterpret_cast<float2*>(y + (size_t)row * (n >> 1) + (col >> 1)) = h;
+                        if (ok) *reinterpret_cast<float2*>(y + (size_t)row * (n >> 1) + (col >> 1)) = h;
                     }
                 }
             }
