@@ -246,11 +246,11 @@ __device__ __forceinline__ int mega_dot_row(const i32x4 (&wr)[NCH], const int8_t
 __global__ __launch_bounds__(kMegaT, 1) void decode_mega_kernel(MegaParams p) {
     extern __shared__ __attribute__((aligned(16))) unsigned char mega_smem[];   // sizeof(MegaLds) > the static 64 KiB limit
     MegaLds& L = *reinterpret_cast<MegaLds*>(mega_smem);
-    const int t = threadIdx.x, lane = t & 63, wg = blockIdx.x;
+    const int t = threadIdx.x, wg = blockIdx.x;
     const int wave = __builtin_amdgcn_readfirstlane(t >> 6);
     const bool is_s = wave >= 4;                        // stream wave (see the file comment)
     const int sw = wave - 4;
-    constexpr int H = 2048, KV = 512, I = 8192, QH = 32, KVH = 8, GROUP = 4;
+    constexpr int H = 2048, KV = 512, QH = 32, KVH = 8, GROUP = 4;
     const int pos0 = p.state[0];
     GridBarrier bar{p.bar, (unsigned)p.state[2], &p.state[3]};
     int stamp_i = 0;

@@ -609,6 +609,9 @@ inline int launch_gemm_swiglu(const int8_t* a, const int8_t* w_gu, const float* 
         if (mode == 32) return launch_gemm_dma<128, 256, kDmaSwiglu, 3, 1, 128>(a, w_gu, nullptr, s_x, w_s_gu, nullptr, h, m, k, n2, st);
         if (mode == 33) return launch_gemm_dma<64, 128, kDmaSwiglu, 2, 3, 128>(a, w_gu, nullptr, s_x, w_s_gu, nullptr, h, m, k, n2, st);
         if (mode == 34) return launch_gemm_dma<128, 128, kDmaSwiglu, 3, 1, 128>(a, w_gu, nullptr, s_x, w_s_gu, nullptr, h, m, k, n2, st);
+        if (mode == 40) return launch_gemm_dma<256, 256, kDmaSwiglu, 2, 1, 128>(a, w_gu, nullptr, s_x, w_s_gu, nullptr, h, m, k, n2, st);
+        if (mode == 41) return launch_gemm_dma<256, 256, kDmaSwiglu, 4, 1, 64>(a, w_gu, nullptr, s_x, w_s_gu, nullptr, h, m, k, n2, st);
+        if (mode == 42) return launch_gemm_dma<256, 128, kDmaSwiglu, 2, 1, 128>(a, w_gu, nullptr, s_x, w_s_gu, nullptr, h, m, k, n2, st);
     }
     return launch_gemm_dma<64, 64, kDmaSwiglu>(a, w_gu, nullptr, s_x, w_s_gu, nullptr, h, m, k, n2, st);
 }

@@ -12,10 +12,6 @@ struct LayerW {
 struct PrefillWorkspace {
     int tokens = 0;
     void* base = nullptr;
-    // side stream that pulls the coming GEMMs' weights into the memory-side cache while attention computes
-    hipStream_t side = nullptr;
-    hipEvent_t ev_fork = nullptr, ev_join = nullptr;
-    int* sink = nullptr;
 };
 
 inline void prefill_workspace_free(PrefillWorkspace* ws) {
@@ -25,11 +21,6 @@ inline void prefill_workspace_free(PrefillWorkspace* ws) {
 }
 inline void prefill_workspace_destroy(PrefillWorkspace* ws) {
     prefill_workspace_free(ws);
-    if (ws->side) (void)hipStreamDestroy(ws->side);
-    if (ws->ev_fork) (void)hipEventDestroy(ws->ev_fork);
-    if (ws->ev_join) (void)hipEventDestroy(ws->ev_join);
-    if (ws->sink) (void)hipFree(ws->sink);
-    ws->side = nullptr; ws->ev_fork = ws->ev_join = nullptr; ws->sink = nullptr;
 }
 
 int llama_prefill_run(const flexllm_llama_config& cfg, const LayerW* layers, const float* gamma, const float* q_s,

@@ -40,30 +40,6 @@ static int prefill_workspace_get(PrefillWorkspace* ws, const flexllm_llama_confi
     return FLEXLLM_OK;
 }
 
-// Reads up to four weight ranges once and throws the data away: the memory-side cache (256 MiB) keeps them, so
-// the GEMMs that follow find their weights there instead of in HBM.  Runs on a side stream under the attention
-// kernel, which is bound by exp/division and leaves the memory system idle.
-struct TouchRanges { const void* p[4]; size_t bytes[4]; };
-static __global__ __launch_bounds__(256) void touch_kernel(TouchRanges r, int* sink) {
-    int acc = 0;
-    for (int i = 0; i < 4; i++) {
-        const i32x4* q = reinterpret_cast<const i32x4*>(r.p[i]);
-        const size_t n = r.bytes[i] / 16;
-        const size_t stride = (size_t)gridDim.x * 256;
-        size_t j = (size_t)blockIdx.x * 256 + threadIdx.x;
-        for (; j + 3 * stride < n; j += 4 * stride) {              // four loads in flight per thread
-            const i32x4 v0 = q[j], v1 = q[j + stride], v2 = q[j + 2 * stride], v3 = q[j + 3 * stride];
-            acc ^= (v0[0] ^ v0[1] ^ v0[2] ^ v0[3]) ^ (v1[0] ^ v1[1] ^ v1[2] ^ v1[3]) ^ (v2[0] ^ v2[1] ^ v2[2] ^ v2[3]) ^
-                   (v3[0] ^ v3[1] ^ v3[2] ^ v3[3]);
-        }
-        for (; j < n; j += stride) {
-            const i32x4 v = q[j];
-            acc ^= v[0] ^ v[1] ^ v[2] ^ v[3];
-        }
-    }
-    if (acc == 0x5a5a1234 && sink) sink[threadIdx.x & 63] = acc;    // practically never: keeps the loads alive
-}
-
 int llama_prefill_run(const flexllm_llama_config& c, const LayerW* layers, const float* gamma, const float* q_s_all,
                       const float* k_s_all, const float* v_s_all, const float* a_s_all, const float* rope_sin,
                       const float* rope_cos, int8_t* k_cache, int8_t* v_cache, size_t cache_layer_bytes,
@@ -72,14 +48,7 @@ int llama_prefill_run(const flexllm_llama_config& c, const LayerW* layers, const
     PrefillBuffers b;
     int rc = prefill_workspace_get(ws, c, s, &b);
     if (rc) return rc;
-    const int H = c.hidden, KV = c.kv_hidden, I = c.inter;
-    if (!ws->side) {
-        FX_HIP(hipStreamCreateWithFlags(&ws->side, hipStreamNonBlocking));
-        FX_HIP(hipEventCreateWithFlags(&ws->ev_fork, hipEventDisableTiming));
-        FX_HIP(hipEventCreateWithFlags(&ws->ev_join, hipEventDisableTiming));
-        FX_HIP(hipMalloc(&ws->sink, 64 * sizeof(int)));
-    }
-    static const bool no_touch = getenv("FLEXLLM_NO_WEIGHT_TOUCH") != nullptr;
+    const int H = c.hidden, I = c.inter;
     FX_HIP(hipMemcpyAsync(b.x, x_in, sizeof(float) * (size_t)s * H, hipMemcpyDeviceToDevice, st));
     for (int l = 0; l < c.layers; l++) {
         const LayerW& w = layers[l];
@@ -100,17 +69,6 @@ int llama_prefill_run(const flexllm_llama_config& c, const LayerW* layers, const
             qa.pos0 = 0; qa.q_heads = c.q_heads; qa.kv_heads = c.kv_heads; qa.max_pos = c.max_pos;
             if ((rc = launch_gemm_qkv(b.xq, w.wqkv, b.xs, w.sqkv, s, H, qa, st))) return rc;
         }
-        if (!no_touch) {                                   // fork: weights of o, gate/up, down and the next layer's q/k/v
-            TouchRanges tr;
-            tr.p[0] = w.wo; tr.bytes[0] = (size_t)H * H;
-            tr.p[1] = w.wgu; tr.bytes[1] = (size_t)2 * I * H;
-            tr.p[2] = w.wd; tr.bytes[2] = (size_t)H * I;
-            tr.p[3] = l + 1 < c.layers ? layers[l + 1].wqkv : nullptr; tr.bytes[3] = l + 1 < c.layers ? (size_t)(H + 2 * KV) * H : 0;
-            FX_HIP(hipEventRecord(ws->ev_fork, st));
-            FX_HIP(hipStreamWaitEvent(ws->side, ws->ev_fork, 0));
-            touch_kernel<<<256, 256, 0, ws->side>>>(tr, ws->sink);
-            FX_HIP(hipEventRecord(ws->ev_join, ws->side));
-        }
         if ((rc = mha_prefill_launch(b.q8, kc, vc, q_s, k_s, v_s, a_s, b.att, nullptr, s, c.q_heads, c.kv_heads, c.max_pos, st))) return rc;
         quant_sym_kernel<2><<<s, kBlock, 0, st>>>(b.att, b.xq, b.xs, H);
         if ((rc = launch_gemm<kGemmDequant>(b.xq, w.wo, nullptr, b.xs, w.so, b.x, b.x2, s, H, H, st))) return rc;
@@ -119,7 +77,6 @@ int llama_prefill_run(const flexllm_llama_config& c, const LayerW* layers, const
         if ((rc = launch_gemm_swiglu(b.xq, w.wgu, b.xs, w.sgu, b.gu, s, H, 2 * I, st))) return rc;     // b.gu = SiLU(gate)*up [s][I]
         fht_kernel<13, true, false><<<s, kFhtBlock, 0, st>>>(b.gu, nullptr, b.xq, b.xs, c.fht_scale);
         if ((rc = launch_gemm<kGemmDequant>(b.xq, w.wd, nullptr, b.xs, w.sd, b.x2, b.x, s, I, H, st))) return rc;
-        if (!no_touch) FX_HIP(hipStreamWaitEvent(st, ws->ev_join, 0));     // join: the side stream never runs ahead by more than a layer
     }
     FX_LAUNCH_CHECK();
     if (hidden_out) FX_HIP(hipMemcpyAsync(hidden_out, b.x, sizeof(float) * (size_t)s * H, hipMemcpyDeviceToDevice, st));
