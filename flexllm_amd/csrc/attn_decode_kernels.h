@@ -153,7 +153,7 @@ static __global__ __launch_bounds__(256) void dec_scores_kernel(const int8_t* __
     float sum = 0.0f;
 #pragma unroll
     for (int j = 0; j < kChunk / 64; j++)
-        if (chunk * kChunk + j * 64 + lane < len) sum += expf(sc[j] - mx);
+        if (chunk * kChunk + j * 64 + lane < len) sum += exp_f(sc[j] - mx);
     sum = wave_sum(sum);
     if (lane == 0) stats[qh * kMaxChunks + chunk] = make_float2(mx, sum);
 }
@@ -175,7 +175,7 @@ static __global__ __launch_bounds__(256) void dec_pv_kernel(const float* __restr
     float m_c = -1e32f, l_c = 0.0f;
     if (lane < nchunks) { const float2 st = stats[qh * kMaxChunks + lane]; m_c = st.x; l_c = st.y; }
     const float mx = wave_max(m_c);
-    const float sum = wave_sum(lane < nchunks ? l_c * expf(m_c - mx) : 0.0f);
+    const float sum = wave_sum(lane < nchunks ? l_c * exp_f(m_c - mx) : 0.0f);
     const float cd = 1.0f / sum;
     const float as = 1.0f * a_s[qh];
     uint8_t* pb = reinterpret_cast<uint8_t*>(p_lds[g]);
@@ -184,7 +184,7 @@ static __global__ __launch_bounds__(256) void dec_pv_kernel(const float* __restr
         const int pos = chunk * kChunk + j * 64 + lane;
         int p8 = 0;
         if (pos < len) {
-            const float p = expf(scores[(size_t)qh * ld + pos] - mx) * cd;
+            const float p = exp_f(scores[(size_t)qh * ld + pos] - mx) * cd;
             p8 = (int)roundf(p / as);
             p8 = p8 > 255 ? 255 : p8;
             if (p8_out) p8_out[(size_t)qh * len + pos] = (uint8_t)p8;

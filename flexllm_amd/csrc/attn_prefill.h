@@ -94,8 +94,8 @@ static __global__ __launch_bounds__(64 * kPfWaves) void pf_attention_kernel(cons
             const float m_new = fmaxf(m_run, mt);
             float sum = 0.0f;
 #pragma unroll
-            for (int r = 0; r < 16; r++) sum += expf(sc[r] - m_new);
-            l_run = l_run * expf(m_run - m_new) + sum;
+            for (int r = 0; r < 16; r++) sum += exp_f(sc[r] - m_new);
+            l_run = l_run * exp_f(m_run - m_new) + sum;
             m_run = m_new;
             kf0 = nf0; kf1 = nf1;
         }
@@ -103,7 +103,7 @@ static __global__ __launch_bounds__(64 * kPfWaves) void pf_attention_kernel(cons
     {   // merge the two lanes that share a query, then the waves
         const float m_o = lane_xor_f<32>(m_run), l_o = lane_xor_f<32>(l_run);
         const float mw = fmaxf(m_run, m_o);
-        const float lw = l_run * expf(m_run - mw) + l_o * expf(m_o - mw);
+        const float lw = l_run * exp_f(m_run - mw) + l_o * exp_f(m_o - mw);
         if (g == 0) { lds_m[wave][col] = mw; lds_l[wave][col] = lw; }
     }
     __syncthreads();
@@ -112,8 +112,10 @@ static __global__ __launch_bounds__(64 * kPfWaves) void pf_attention_kernel(cons
     for (int w = 1; w < kPfWaves; w++) mx = fmaxf(mx, lds_m[w][col]);
     float total = 0.0f;
 #pragma unroll
-    for (int w = 0; w < kPfWaves; w++) total += lds_l[w][col] * expf(lds_m[w][col] - mx);
+    for (int w = 0; w < kPfWaves; w++) total += lds_l[w][col] * exp_f(lds_m[w][col] - mx);
     const float cd = 1.0f / total;
+    const bool fast_q = quant_fast_ok(as);
+    const float ras = 1.0f / as;
 
     // ---- pass 2: probabilities, partial P.V over this wave's tiles ----
     i32x16 oacc0 = zero16(), oacc1 = zero16();
@@ -138,17 +140,29 @@ static __global__ __launch_bounds__(64 * kPfWaves) void pf_attention_kernel(cons
             i32x4 pf;
 #pragma unroll
             for (int a = 0; a < 4; a++) {
+                // four probabilities -> four bytes; round(pr / as) through the reciprocal, redone with the division
+                // for the whole group when one of them comes near a rounding tie
+                float pr[4];
+                int p8[4];
+                bool redo = !fast_q;
+#pragma unroll
+                for (int b = 0; b < 4; b++) {
+                    pr[b] = exp_f(sc[a * 4 + b] - mx) * cd;
+                    p8[b] = quant_round_fast(pr[b], ras, redo);
+                }
+                if (redo) {
+#pragma unroll
+                    for (int b = 0; b < 4; b++) p8[b] = (int)roundf(pr[b] / as);
+                }
                 uint32_t packed = 0;
 #pragma unroll
                 for (int b = 0; b < 4; b++) {
-                    const float pr = expf(sc[a * 4 + b] - mx) * cd;
-                    int p8 = (int)roundf(pr / as);
-                    p8 = p8 > 255 ? 255 : p8;
+                    const int pq = p8[b] > 255 ? 255 : p8[b];
                     if (p8_out) {
                         const int key = k0 + a * 8 + g * 4 + b;
-                        p8_out[((size_t)h * s + query) * s + key] = (uint8_t)p8;
+                        p8_out[((size_t)h * s + query) * s + key] = (uint8_t)pq;
                     }
-                    packed |= (uint32_t)((p8 ^ 0x80) & 0xff) << (8 * b);
+                    packed |= (uint32_t)((pq ^ 0x80) & 0xff) << (8 * b);
                 }
                 pf[a] = (int)packed;
             }

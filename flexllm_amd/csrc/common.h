@@ -63,8 +63,19 @@ template <int MASK>
 __device__ __forceinline__ float lane_xor_f(float v) {
     return __int_as_float(lane_xor_i<MASK>(__float_as_int(v)));
 }
-// SiLU as the reference evaluates it: x / (1 + exp(-x)), one IEEE division.
-__device__ __forceinline__ float silu_f(float v) { return v / (1.0f + expf(-v)); }
+// e^x on the hardware's 2^x unit (1 ulp).  The exponent x*log2(e) is formed in two parts: t is the rounded
+// product, lo its rounding error plus the low part of log2(e), folded back as e*(1 + lo*ln2).  Result within about
+// 2 ulp of the correctly rounded value for any x whose result is a normal number; t is capped so that 2^t stays
+// finite (callers pass x <= 0 or take 1/(1+e^x), where a cap at 2^126 changes nothing representable).
+__device__ __forceinline__ float exp_f(float x) {
+    const float t = x * 1.44269502162933349609375f;
+    const float lo = __builtin_fmaf(x, 1.92596299e-8f, __builtin_fmaf(x, 1.44269502162933349609375f, -t));
+    const float e = __builtin_amdgcn_exp2f(fminf(t, 126.0f));
+    return __builtin_fmaf(e, lo * 0.693147182464599609375f, e);
+}
+// SiLU x / (1 + exp(-x)) with the hardware reciprocal (1 ulp) in place of the division: within 4 ulp of the
+// reference's value.  Every kernel that applies SiLU calls this one function, so they agree bit for bit.
+__device__ __forceinline__ float silu_f(float v) { return v * __builtin_amdgcn_rcpf(1.0f + exp_f(-v)); }
 
 __device__ __forceinline__ float wave_max(float v) {
     v = fmaxf(v, lane_xor_f<1>(v));

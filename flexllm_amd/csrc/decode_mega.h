@@ -414,7 +414,7 @@ __global__ __launch_bounds__(kMegaT, 1) void decode_mega_kernel(MegaParams p) {
                 if (wave < GROUP) {
                     const float s0 = L.sc[wave][lane], s1 = L.sc[wave][lane + 64];
                     const float m = wave_max(fmaxf(s0, s1));
-                    float sum = (a_c * kChunk + lane < len ? expf(s0 - m) : 0.0f) + (a_c * kChunk + lane + 64 < len ? expf(s1 - m) : 0.0f);
+                    float sum = (a_c * kChunk + lane < len ? exp_f(s0 - m) : 0.0f) + (a_c * kChunk + lane + 64 < len ? exp_f(s1 - m) : 0.0f);
                     sum = wave_sum(sum);
                     if (lane == 0) {
                         st_f(&p.stats[(a_h * GROUP + wave) * 32 + a_c].x, m);
@@ -447,14 +447,14 @@ __global__ __launch_bounds__(kMegaT, 1) void decode_mega_kernel(MegaParams p) {
                         l_c = ld_f(&p.stats[(a_h * GROUP + wave) * 32 + lane].y);
                     }
                     const float mx = wave_max(m_c);
-                    const float sum = wave_sum(lane < nchunks ? l_c * expf(m_c - mx) : 0.0f);
+                    const float sum = wave_sum(lane < nchunks ? l_c * exp_f(m_c - mx) : 0.0f);
                     if (lane == 0) { L.rowmax[wave] = mx; L.rowcd[wave] = 1.0f / sum; }
                 }
                 __syncthreads();
                 gu_slice(2);                                          // the chunk statistics have landed
                 {
                     const int g = t >> 7, key = t & 127;
-                    const float pr = expf(L.sc[g][key] - L.rowmax[g]) * L.rowcd[g];
+                    const float pr = exp_f(L.sc[g][key] - L.rowmax[g]) * L.rowcd[g];
                     int p8 = (int)roundf(pr / (1.0f * as_g));
                     p8 = p8 > 255 ? 255 : p8;
                     if (a_c * kChunk + key >= len) p8 = 0;

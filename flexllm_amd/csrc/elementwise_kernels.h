@@ -235,7 +235,7 @@ static __global__ __launch_bounds__(kBlock) void rope_kernel(const float* __rest
     }
 }
 
-__device__ __forceinline__ float silu(float v) { return v / (1.0f + expf(-v)); }
+__device__ __forceinline__ float silu(float v) { return silu_f(v); }
 
 static __global__ __launch_bounds__(kBlock) void swish_kernel(const float* __restrict__ x, float* __restrict__ y, size_t n) {
     for (size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += (size_t)gridDim.x * kBlock) y[i] = silu(x[i]);

@@ -45,10 +45,10 @@ __global__ __launch_bounds__(kFhtBlock) void fht_kernel(const float* __restrict_
 #pragma unroll
         for (int j = 0; j < NJ; j++) {
             const float4 p0 = xr[(j * 256 + t) * 2], p1 = xr[(j * 256 + t) * 2 + 1];
-            a[j].x = p0.y * (p0.x / (1.0f + expf(-p0.x)));
-            a[j].y = p0.w * (p0.z / (1.0f + expf(-p0.z)));
-            a[j].z = p1.y * (p1.x / (1.0f + expf(-p1.x)));
-            a[j].w = p1.w * (p1.z / (1.0f + expf(-p1.z)));
+            a[j].x = p0.y * silu_f(p0.x);
+            a[j].y = p0.w * silu_f(p0.z);
+            a[j].z = p1.y * silu_f(p1.x);
+            a[j].w = p1.w * silu_f(p1.z);
         }
     } else {
         const float4* xr = reinterpret_cast<const float4*>(x + row * N);
