@@ -44,15 +44,21 @@ void set_error(const char* fmt, ...);
 inline hipStream_t as_stream(void* s) { return reinterpret_cast<hipStream_t>(s); }
 
 // ---------------------------------------------------------------- cross-lane exchange
-// Value held by lane (lane ^ MASK).  1,2: DPP quad_perm; 4,8,16: ds_swizzle bit mode (no LDS
-// traffic, crossbar only); 32: bpermute.
+// Value held by lane (lane ^ MASK).  1,2: DPP quad_perm; 8: DPP row rotate by 8; 4: two DPP row shifts, each
+// writing the banks (groups of four lanes) it is right for; 16: ds_swizzle bit mode (no LDS traffic, crossbar
+// only); 32: bpermute.  The DPP forms are plain VALU moves which the compiler folds into the consuming add.
 template <int MASK>
 __device__ __forceinline__ int lane_xor_i(int v) {
     if constexpr (MASK == 1) {
         return __builtin_amdgcn_mov_dpp(v, 0xB1, 0xF, 0xF, true);   // quad_perm [1,0,3,2]
     } else if constexpr (MASK == 2) {
         return __builtin_amdgcn_mov_dpp(v, 0x4E, 0xF, 0xF, true);   // quad_perm [2,3,0,1]
-    } else if constexpr (MASK == 4 || MASK == 8 || MASK == 16) {
+    } else if constexpr (MASK == 4) {
+        const int lo = __builtin_amdgcn_update_dpp(v, v, 0x104, 0xF, 0x5, false);   // row_shl:4 into banks 0,2: lane i <- i+4
+        return __builtin_amdgcn_update_dpp(lo, v, 0x114, 0xF, 0xA, false);          // row_shr:4 into banks 1,3: lane i <- i-4
+    } else if constexpr (MASK == 8) {
+        return __builtin_amdgcn_mov_dpp(v, 0x128, 0xF, 0xF, true);  // row_ror:8
+    } else if constexpr (MASK == 16) {
         return __builtin_amdgcn_ds_swizzle(v, (MASK << 10) | 0x1F); // and=0x1f or=0 xor=MASK
     } else {
         static_assert(MASK == 32, "lane_xor mask");
@@ -63,6 +69,27 @@ template <int MASK>
 __device__ __forceinline__ float lane_xor_f(float v) {
     return __int_as_float(lane_xor_i<MASK>(__float_as_int(v)));
 }
+// Butterfly across lanes: the lane whose MASK bit is clear gets a + p, the other p - a, with p the partner's value.
+// `sign` is 0 or 0x80000000 by that bit: p + (+-a) is the same IEEE sum or difference, in one add.
+template <int MASK>
+__device__ __forceinline__ unsigned lane_sign(int lane) { return (lane & MASK) ? 0x80000000u : 0u; }
+template <int MASK>
+__device__ __forceinline__ float lane_butterfly_s(float a, unsigned sign) {
+    return lane_xor_f<MASK>(a) + __int_as_float(__float_as_int(a) ^ (int)sign);
+}
+
+// x / d for a divisor used many times, r = 1.0f / d: the product x*r is within an ulp of the quotient, its exact
+// residual (one fma) corrects it, and the corrected value is the correctly rounded quotient whenever r is the
+// correctly rounded reciprocal and nothing under- or overflows (Markstein).  Callers keep |x| within
+// [2^-60, 2^100] or fall back to the division (`div_fast_ok` on the largest magnitude they divide).
+__device__ __forceinline__ float div_fast(float x, float d, float r) {
+    const float q = x * r;
+    return __builtin_fmaf(__builtin_fmaf(-q, d, x), r, q);
+}
+__device__ __forceinline__ bool div_fast_ok(float amax, float d) {
+    return amax >= 0x1p-60f && amax <= 0x1p100f && d >= 0x1p-20f && d <= 0x1p20f;
+}
+
 // e^x on the hardware's 2^x unit (1 ulp).  The exponent x*log2(e) is formed in two parts: t is the rounded
 // product, lo its rounding error plus the low part of log2(e), folded back as e*(1 + lo*ln2).  Result within about
 // 2 ulp of the correctly rounded value for any x whose result is a normal number; t is capped so that 2^t stays

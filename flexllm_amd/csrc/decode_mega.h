@@ -628,12 +628,12 @@ __global__ __launch_bounds__(kMegaT, 1) void decode_mega_kernel(MegaParams p) {
             }
 #define FX_MEGA_STAGE(MASK)                                                                   \
     {                                                                                         \
-        const bool hi = (lane & MASK) != 0;                                                   \
+        const unsigned sg = lane_sign<MASK>(lane);                                            \
         _Pragma("unroll") for (int j = 0; j < 4; j++) {                                       \
-            float px = lane_xor_f<MASK>(a[j].x); a[j].x = hi ? (px - a[j].x) : (a[j].x + px); \
-            float py = lane_xor_f<MASK>(a[j].y); a[j].y = hi ? (py - a[j].y) : (a[j].y + py); \
-            float pz = lane_xor_f<MASK>(a[j].z); a[j].z = hi ? (pz - a[j].z) : (a[j].z + pz); \
-            float pw = lane_xor_f<MASK>(a[j].w); a[j].w = hi ? (pw - a[j].w) : (a[j].w + pw); \
+            a[j].x = lane_butterfly_s<MASK>(a[j].x, sg);                                      \
+            a[j].y = lane_butterfly_s<MASK>(a[j].y, sg);                                      \
+            a[j].z = lane_butterfly_s<MASK>(a[j].z, sg);                                      \
+            a[j].w = lane_butterfly_s<MASK>(a[j].w, sg);                                      \
         }                                                                                     \
     }
             __builtin_amdgcn_s_waitcnt(0x0F70);               // vmcnt(0): the h loads, which stage 1 has consumed, are complete
@@ -675,13 +675,24 @@ __global__ __launch_bounds__(kMegaT, 1) void decode_mega_kernel(MegaParams p) {
             float b2[16];
 #pragma unroll
             for (int q = 0; q < 4; q++) {                                                                             // bit 0
-                b2[4 * q + 0] = (c4[q].x + c4[q].y) / p.fht_scale;
-                b2[4 * q + 1] = (c4[q].x - c4[q].y) / p.fht_scale;
-                b2[4 * q + 2] = (c4[q].z + c4[q].w) / p.fht_scale;
-                b2[4 * q + 3] = (c4[q].z - c4[q].w) / p.fht_scale;
+                b2[4 * q + 0] = c4[q].x + c4[q].y;
+                b2[4 * q + 1] = c4[q].x - c4[q].y;
+                b2[4 * q + 2] = c4[q].z + c4[q].w;
+                b2[4 * q + 3] = c4[q].z - c4[q].w;
             }
 #pragma unroll
             for (int r = 0; r < 16; r++) amax = fmaxf(amax, fabsf(b2[r]));
+            // division by the transform's scale as in fht_kernels.h: reciprocal + exact residual step, plain division
+            // outside the safe range; the largest quotient is the quotient of the largest magnitude
+            if (div_fast_ok(amax, p.fht_scale)) {
+                const float rs = 1.0f / p.fht_scale;
+#pragma unroll
+                for (int r = 0; r < 16; r++) b2[r] = div_fast(b2[r], p.fht_scale, rs);
+            } else {
+#pragma unroll
+                for (int r = 0; r < 16; r++) b2[r] = b2[r] / p.fht_scale;
+            }
+            amax = amax / p.fht_scale;
             if (l == 1) fine();
             amax = mega_block_max_h(amax, L.red_max, NoHook());
             const float sx = sym_scale(amax, 127.0f);

@@ -21,12 +21,6 @@ namespace fx {
 
 constexpr int kFhtBlock = 256;
 
-template <int MASK>
-__device__ __forceinline__ float lane_butterfly(float a, bool bit_set) {
-    const float p = lane_xor_f<MASK>(a);
-    return bit_set ? (p - a) : (a + p);
-}
-
 template <int LOG2N, bool QUANT, bool SWIGLU = false>
 __global__ __launch_bounds__(kFhtBlock) void fht_kernel(const float* __restrict__ x, float* __restrict__ y,
                                                         int8_t* __restrict__ q, float* __restrict__ s, float scale) {
@@ -66,12 +60,12 @@ __global__ __launch_bounds__(kFhtBlock) void fht_kernel(const float* __restrict_
     // stages: bits 2..7 = lane bits 0..5
 #define FX_LANE_STAGE(MASK)                                             \
     {                                                                   \
-        const bool hi = (lane & MASK) != 0;                             \
+        const unsigned sg = lane_sign<MASK>(lane);                      \
         _Pragma("unroll") for (int j = 0; j < NJ; j++) {                \
-            a[j].x = lane_butterfly<MASK>(a[j].x, hi);                  \
-            a[j].y = lane_butterfly<MASK>(a[j].y, hi);                  \
-            a[j].z = lane_butterfly<MASK>(a[j].z, hi);                  \
-            a[j].w = lane_butterfly<MASK>(a[j].w, hi);                  \
+            a[j].x = lane_butterfly_s<MASK>(a[j].x, sg);                \
+            a[j].y = lane_butterfly_s<MASK>(a[j].y, sg);                \
+            a[j].z = lane_butterfly_s<MASK>(a[j].z, sg);                \
+            a[j].w = lane_butterfly_s<MASK>(a[j].w, sg);                \
         }                                                               \
     }
     FX_LANE_STAGE(1)
@@ -104,16 +98,31 @@ __global__ __launch_bounds__(kFhtBlock) void fht_kernel(const float* __restrict_
     }
     // last stage: bit 0 = lane bit 0
     {
-        const bool hi = (lane & 1) != 0;
+        const unsigned sg = lane_sign<1>(lane);
 #pragma unroll
-        for (int r = 0; r < NR; r++) b[r] = lane_butterfly<1>(b[r], hi);
+        for (int r = 0; r < NR; r++) b[r] = lane_butterfly_s<1>(b[r], sg);
     }
 
     float amax = 0.0f;
+    if constexpr (!QUANT) {
 #pragma unroll
-    for (int r = 0; r < NR; r++) {
-        b[r] = b[r] / scale;
-        if constexpr (QUANT) amax = fmaxf(amax, fabsf(b[r]));
+        for (int r = 0; r < NR; r++) b[r] = b[r] / scale;
+    } else {
+        // b / scale through the reciprocal with an exact residual step: the correctly rounded quotient for every
+        // magnitude this thread holds, or the plain division when its largest one is outside the safe range
+        // (smaller elements of a thread that passes quantise to zero under either form).  Division by a
+        // positive constant is monotonic, so the largest quotient is the quotient of the largest magnitude.
+#pragma unroll
+        for (int r = 0; r < NR; r++) amax = fmaxf(amax, fabsf(b[r]));
+        if (div_fast_ok(amax, scale)) {
+            const float rs = 1.0f / scale;
+#pragma unroll
+            for (int r = 0; r < NR; r++) b[r] = div_fast(b[r], scale, rs);
+        } else {
+#pragma unroll
+            for (int r = 0; r < NR; r++) b[r] = b[r] / scale;
+        }
+        amax = amax / scale;
     }
     if constexpr (!QUANT) {
         float* yr = y + row * N;
