@@ -176,6 +176,23 @@ def test_fht_bit_exact(fx, oracle, n):
     assert np.array_equal(s.numpy(), s_ref) and np.array_equal(q.numpy(), q_ref)
 
 
+@pytest.mark.parametrize("n", [2048, 8192])
+def test_fht_quant_division_paths(fx, oracle, n):
+    """The fused transform + quantisation divides by the scale through a reciprocal with an exact residual step and
+    falls back to the plain division outside the safe magnitude range: rows of ordinary, huge, tiny and mixed
+    magnitude (and a zero row) must all give the oracle's bytes and scales."""
+    base = rng.standard_normal((12, n)).astype(np.float32)
+    mags = np.array([1.0, 1e-3, 1e3, 1e28, 3e32, 1e-15, 1e-22, 1e-30, 1.0, 1.0, 0.0, 1e10], np.float32)
+    x = base * mags[:, None]
+    x[8, ::3] *= np.float32(1e-26)            # a normal row with elements far below the safe range
+    x[9, : n // 2] = 0.0
+    scale = np.float32(90.50966799) if n == 8192 else np.float32(np.sqrt(n))
+    q, s = fx.ops.fht_quant_i8(fx.to_device(x), scale)
+    q_ref, s_ref = oracle.quant_sym(oracle.fht(x, scale))
+    assert np.array_equal(s.numpy(), s_ref)
+    assert np.array_equal(q.numpy(), q_ref)
+
+
 def test_fht_config2_full_size_properties(fx, oracle):
     """1024 x 2048 and 1024 x 8192 with 1% outlier channels x20: spot rows against the oracle, all rows
     through size-independent properties (involution H(Hx)/n = x, Parseval, dequantised error bound)."""
