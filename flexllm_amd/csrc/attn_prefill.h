@@ -69,11 +69,16 @@ static __global__ __launch_bounds__(64 * kPfWaves) void pf_attention_kernel(cons
         i32x16 acc = zero16();
         acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(kf0, qf0, acc, 0, 0, 0);
         acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(kf1, qf1, acc, 0, 0, 0);
+        if (k0 == q0) {                                   // only the diagonal tile has keys beyond the query (uniform branch)
 #pragma unroll
-        for (int r = 0; r < 16; r++) {
-            const int key = k0 + (r >> 2) * 8 + g * 4 + (r & 3);
-            const float v = (float)acc[r] * sq * sk;
-            sc[r] = key <= query ? v : -1e32f;
+            for (int r = 0; r < 16; r++) {
+                const int key = k0 + (r >> 2) * 8 + g * 4 + (r & 3);
+                const float v = (float)acc[r] * sq * sk;
+                sc[r] = key <= query ? v : -1e32f;
+            }
+        } else {
+#pragma unroll
+            for (int r = 0; r < 16; r++) sc[r] = (float)acc[r] * sq * sk;
         }
     };
 
@@ -94,8 +99,8 @@ static __global__ __launch_bounds__(64 * kPfWaves) void pf_attention_kernel(cons
             const float m_new = fmaxf(m_run, mt);
             float sum = 0.0f;
 #pragma unroll
-            for (int r = 0; r < 16; r++) sum += exp_f(sc[r] - m_new);
-            l_run = l_run * exp_f(m_run - m_new) + sum;
+            for (int r = 0; r < 16; r++) sum += exp_f<false>(sc[r] - m_new);
+            l_run = l_run * exp_f<false>(m_run - m_new) + sum;
             m_run = m_new;
             kf0 = nf0; kf1 = nf1;
         }
@@ -147,8 +152,10 @@ static __global__ __launch_bounds__(64 * kPfWaves) void pf_attention_kernel(cons
                 bool redo = !fast_q;
 #pragma unroll
                 for (int b = 0; b < 4; b++) {
-                    pr[b] = exp_f(sc[a * 4 + b] - mx) * cd;
-                    p8[b] = quant_round_fast(pr[b], ras, redo);
+                    pr[b] = exp_f<false>(sc[a * 4 + b] - mx) * cd;
+                    const float qv = pr[b] * ras;               // >= 0: round half up = truncate(qv + 0.5)
+                    redo |= fabsf(__builtin_amdgcn_fractf(qv) - 0.5f) < 1e-4f;
+                    p8[b] = (int)(qv + 0.5f);
                 }
                 if (redo) {
 #pragma unroll

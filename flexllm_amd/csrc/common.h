@@ -94,10 +94,11 @@ __device__ __forceinline__ bool div_fast_ok(float amax, float d) {
 // product, lo its rounding error plus the low part of log2(e), folded back as e*(1 + lo*ln2).  Result within about
 // 2 ulp of the correctly rounded value for any x whose result is a normal number; t is capped so that 2^t stays
 // finite (callers pass x <= 0 or take 1/(1+e^x), where a cap at 2^126 changes nothing representable).
+template <bool CLAMP = true>                     // CLAMP = false for callers that guarantee x <= 0
 __device__ __forceinline__ float exp_f(float x) {
     const float t = x * 1.44269502162933349609375f;
     const float lo = __builtin_fmaf(x, 1.92596299e-8f, __builtin_fmaf(x, 1.44269502162933349609375f, -t));
-    const float e = __builtin_amdgcn_exp2f(fminf(t, 126.0f));
+    const float e = __builtin_amdgcn_exp2f(CLAMP ? fminf(t, 126.0f) : t);
     return __builtin_fmaf(e, lo * 0.693147182464599609375f, e);
 }
 // SiLU x / (1 + exp(-x)) with the hardware reciprocal (1 ulp) in place of the division: within 4 ulp of the
