@@ -522,10 +522,9 @@ template <int EPI>
 inline int launch_gemm(const int8_t* a, const int8_t* w, int32_t* c, const float* s_x, const float* w_s,
                        const float* residual, float* y, int m, int k, int n, hipStream_t st) {
     // Measured on MI355X at M=1024: the direct-load kernel wins wherever it applies; 128x128 tiles once they fill
-    // the chip about three times over (gate/up), 64x64 tiles for the narrow projections.  FLEXLLM_GEMM_TILE
-    // forces a variant (0..2: register-staged 128x128 / 64x128 / 64x64, 10..13: direct-load 256x256 / 128x128 /
-    // 128x256 / 64x64, 17..20: deeper pipelines 64x64 S4 / 64x64 S6 / 64x128 S4 / 128x128 S4).  Long-K narrow outputs
-    // (down projection) stream cold weights: 64x128 tiles four stages deep keep more bytes in flight.
+    // the chip about three times over, 64x64 tiles for the narrow projections.  FLEXLLM_GEMM_TILE forces a variant
+    // (0..2: register-staged 128x128 / 64x128 / 64x64; direct-load: 11 = 128x128, 13 = 64x64, 19 = 64x128 four
+    // stages, all with 64-byte rows; 36 = 64x64 four stages and 38 = 64x64 three stages with 128-byte rows).
     auto tiles = [&](int bm, int bn) { return ((m + bm - 1) / bm) * ((n + bn - 1) / bn); };
     static const char* force = getenv("FLEXLLM_GEMM_TILE");
     // the direct-load kernel needs 32-bit element offsets into both operands and 16-byte aligned output rows
@@ -539,21 +538,11 @@ inline int launch_gemm(const int8_t* a, const int8_t* w, int32_t* c, const float
     const int nk = k / kGemmBK;
     if (mode >= 10) {
         constexpr int DE = EPI == kGemmDequant ? kDmaDequant : kDmaRaw;
-        if (mode == 10) return launch_gemm_dma<256, 256, DE>(a, w, c, s_x, w_s, residual, y, m, k, n, st);
         if (mode == 11) return launch_gemm_dma<128, 128, DE>(a, w, c, s_x, w_s, residual, y, m, k, n, st);
-        if (mode == 12) return launch_gemm_dma<128, 256, DE>(a, w, c, s_x, w_s, residual, y, m, k, n, st);
-        if (mode == 17) return launch_gemm_dma<64, 64, DE, 4, 2>(a, w, c, s_x, w_s, residual, y, m, k, n, st);
-        if (mode == 18) return launch_gemm_dma<64, 64, DE, 6, 2>(a, w, c, s_x, w_s, residual, y, m, k, n, st);
         if (mode == 19) return launch_gemm_dma<64, 128, DE, 4, 2>(a, w, c, s_x, w_s, residual, y, m, k, n, st);
-        if (mode == 20) return launch_gemm_dma<128, 128, DE, 4, 2>(a, w, c, s_x, w_s, residual, y, m, k, n, st);
         if (k % 128 == 0) {
-            if (mode == 31) return launch_gemm_dma<128, 128, DE, 2, 2, 128>(a, w, c, s_x, w_s, residual, y, m, k, n, st);
-            if (mode == 33) return launch_gemm_dma<64, 128, DE, 2, 3, 128>(a, w, c, s_x, w_s, residual, y, m, k, n, st);
-            if (mode == 35) return launch_gemm_dma<64, 64, DE, 2, 4, 128>(a, w, c, s_x, w_s, residual, y, m, k, n, st);
             if (mode == 36) return launch_gemm_dma<64, 64, DE, 4, 2, 128>(a, w, c, s_x, w_s, residual, y, m, k, n, st);
-            if (mode == 37) return launch_gemm_dma<64, 128, DE, 3, 2, 128>(a, w, c, s_x, w_s, residual, y, m, k, n, st);
             if (mode == 38) return launch_gemm_dma<64, 64, DE, 3, 3, 128>(a, w, c, s_x, w_s, residual, y, m, k, n, st);
-            if (mode == 39) return launch_gemm_dma<64, 64, DE, 5, 2, 128>(a, w, c, s_x, w_s, residual, y, m, k, n, st);
         }
         return launch_gemm_dma<64, 64, DE>(a, w, c, s_x, w_s, residual, y, m, k, n, st);
     }
@@ -594,25 +583,14 @@ inline int launch_gemm_swiglu(const int8_t* a, const int8_t* w_gu, const float* 
                               int k, int n2, hipStream_t st) {
     FX_REQUIRE((size_t)m * k < (1ull << 31) && (size_t)n2 * k < (1ull << 31) && n2 % 4 == 0,
                "linear_i8_gemm_swiglu: m=%d k=%d n=%d outside the direct-load kernel's range", m, k, n2 / 2);
-    // Measured at M=1024, 2048 -> 2x8192: 128x256 tiles, two stages, two workgroups per CU (one round of 512
-    // workgroups) beat 128x128 tiles (1024 workgroups in three slots per CU: a second, mostly empty round).
+    // Measured at M=1024, 2048 -> 2x8192: 128x256 tiles, two stages of 64-byte rows, two workgroups per CU (one
+    // round of 512 workgroups): 48-49 us.  128x128 tiles (two or three per CU, 64- or 128-byte rows) and 256x256
+    // tiles (one per CU) came out at 48-58 us; FLEXLLM_GEMM_TILE=13 forces the 64x64 fallback.
     static const char* force = getenv("FLEXLLM_GEMM_TILE");
     const int tiles_big = ((m + 127) / 128) * ((n2 + 255) / 256);
     int mode = tiles_big >= 384 ? 16 : 13;
     if (force) mode = atoi(force);
-    if (mode == 10) return launch_gemm_dma<256, 256, kDmaSwiglu>(a, w_gu, nullptr, s_x, w_s_gu, nullptr, h, m, k, n2, st);
-    if (mode == 11) return launch_gemm_dma<128, 128, kDmaSwiglu, 3, 3>(a, w_gu, nullptr, s_x, w_s_gu, nullptr, h, m, k, n2, st);
-    if (mode == 12 || mode == 16) return launch_gemm_dma<128, 256, kDmaSwiglu, 2, 2>(a, w_gu, nullptr, s_x, w_s_gu, nullptr, h, m, k, n2, st);
-    if (k % 128 == 0) {
-        if (mode == 30) return launch_gemm_dma<128, 256, kDmaSwiglu, 2, 1, 128>(a, w_gu, nullptr, s_x, w_s_gu, nullptr, h, m, k, n2, st);
-        if (mode == 31) return launch_gemm_dma<128, 128, kDmaSwiglu, 2, 2, 128>(a, w_gu, nullptr, s_x, w_s_gu, nullptr, h, m, k, n2, st);
-        if (mode == 32) return launch_gemm_dma<128, 256, kDmaSwiglu, 3, 1, 128>(a, w_gu, nullptr, s_x, w_s_gu, nullptr, h, m, k, n2, st);
-        if (mode == 33) return launch_gemm_dma<64, 128, kDmaSwiglu, 2, 3, 128>(a, w_gu, nullptr, s_x, w_s_gu, nullptr, h, m, k, n2, st);
-        if (mode == 34) return launch_gemm_dma<128, 128, kDmaSwiglu, 3, 1, 128>(a, w_gu, nullptr, s_x, w_s_gu, nullptr, h, m, k, n2, st);
-        if (mode == 40) return launch_gemm_dma<256, 256, kDmaSwiglu, 2, 1, 128>(a, w_gu, nullptr, s_x, w_s_gu, nullptr, h, m, k, n2, st);
-        if (mode == 41) return launch_gemm_dma<256, 256, kDmaSwiglu, 4, 1, 64>(a, w_gu, nullptr, s_x, w_s_gu, nullptr, h, m, k, n2, st);
-        if (mode == 42) return launch_gemm_dma<256, 128, kDmaSwiglu, 2, 1, 128>(a, w_gu, nullptr, s_x, w_s_gu, nullptr, h, m, k, n2, st);
-    }
+    if (mode == 16) return launch_gemm_dma<128, 256, kDmaSwiglu, 2, 2>(a, w_gu, nullptr, s_x, w_s_gu, nullptr, h, m, k, n2, st);
     return launch_gemm_dma<64, 64, kDmaSwiglu>(a, w_gu, nullptr, s_x, w_s_gu, nullptr, h, m, k, n2, st);
 }
 
@@ -629,8 +607,6 @@ inline int launch_gemm_qkv(const int8_t* a, const int8_t* w_qkv, const float* s_
     if (k % 128 == 0) {
         if (mode == 36) return launch_gemm_dma<64, 64, kDmaQkv, 4, 2, 128>(a, w_qkv, nullptr, s_x, w_s, nullptr, nullptr, m, k, n, st, qa);
         if (mode == 38) return launch_gemm_dma<64, 64, kDmaQkv, 3, 3, 128>(a, w_qkv, nullptr, s_x, w_s, nullptr, nullptr, m, k, n, st, qa);
-        if (mode == 39) return launch_gemm_dma<64, 64, kDmaQkv, 5, 2, 128>(a, w_qkv, nullptr, s_x, w_s, nullptr, nullptr, m, k, n, st, qa);
-        if (mode == 35) return launch_gemm_dma<64, 64, kDmaQkv, 2, 4, 128>(a, w_qkv, nullptr, s_x, w_s, nullptr, nullptr, m, k, n, st, qa);
     }
     return launch_gemm_dma<64, 64, kDmaQkv>(a, w_qkv, nullptr, s_x, w_s, nullptr, nullptr, m, k, n, st, qa);
 }
