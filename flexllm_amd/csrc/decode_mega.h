@@ -52,7 +52,8 @@ struct MegaParams {
     int8_t *k_cache, *v_cache;
     size_t cache_layer_bytes;
     float *x, *x2, *qkv, *h, *logits;
-    float2* stats;                 // [q_heads][32]
+    float2* stats;                 // [q_heads][32] (one-kernel-per-stage path)
+    unsigned long long* stats_tag; // [q_heads][32][2]: chunk max and chunk sum of exponentials, each with the epoch in its high word
     int32_t* o_acc;                // [H]
     int* state;                    // [0] pos, [1] step, [2] barrier epoch base, [3] error flag
     unsigned* bar;                 // [0] flag, [64] top counter, [128+64g] group counters
@@ -71,6 +72,13 @@ __device__ __forceinline__ float ld_f(const float* p) { return __hip_atomic_load
 __device__ __forceinline__ void st_f(float* p, float v) { __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
 __device__ __forceinline__ int ld_i(const int* p) { return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
 __device__ __forceinline__ void st_i(int* p, int v) { __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
+// A float that carries the epoch it was written in: one 64-bit store, so a reader that sees the tag sees the value.
+__device__ __forceinline__ void st_tagged(unsigned long long* p, float v, unsigned tag) {
+    __hip_atomic_store(p, ((unsigned long long)tag << 32) | (unsigned)__float_as_int(v), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ unsigned long long ld_u64(const unsigned long long* p) {
+    return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
 
 // Read-only data at a wave-uniform address (layer table, per-row weight scales): the constant address space
 // makes these scalar loads, off the vector-memory queue.
@@ -366,6 +374,13 @@ __global__ __launch_bounds__(kMegaT, 1) void decode_mega_kernel(MegaParams p) {
             const int key = t >> 2, part = t & 3;
             const int kpos = a_c * kChunk + key;
             if (a_active) kreg = *reinterpret_cast<const i32x4*>(kc + k_index(a_h, min(kpos, p.max_pos - 1), p.max_pos) + part * 16);
+            // this chunk's V block for the second half of the phase (d = channel, 16 positions per thread)
+            i32x4 vreg = {0, 0, 0, 0};
+            const int blk = t >> 8, d = (t >> 2) & 63;
+            const int bpos = a_c * kChunk + blk * kVBlock;
+            if (a_active && bpos < p.max_pos)
+                vreg = *reinterpret_cast<const i32x4*>(vc + v_index(a_h, bpos, d, p.max_pos) + part * 16);
+            const float as_g = ldc_f(a_s + a_h * GROUP + (wave >> 1));   // threads 128g..128g+127 (two waves) serve query head g
             // static scales of this layer, read ahead of the barrier (and of this phase's prefetch slice)
             float qs4[GROUP];
 #pragma unroll
@@ -417,39 +432,42 @@ __global__ __launch_bounds__(kMegaT, 1) void decode_mega_kernel(MegaParams p) {
                     float sum = (a_c * kChunk + lane < len ? exp_f(s0 - m) : 0.0f) + (a_c * kChunk + lane + 64 < len ? exp_f(s1 - m) : 0.0f);
                     sum = wave_sum(sum);
                     if (lane == 0) {
-                        st_f(&p.stats[(a_h * GROUP + wave) * 32 + a_c].x, m);
-                        st_f(&p.stats[(a_h * GROUP + wave) * 32 + a_c].y, sum);
+                        unsigned long long* slot = p.stats_tag + (size_t)((a_h * GROUP + wave) * 32 + a_c) * 2;
+                        st_tagged(slot, m, bar.epoch);
+                        st_tagged(slot + 1, sum, bar.epoch);
                     }
                 }
             } else {
                 gu_slice(1);
             }
             stamp();
-            bar.arrive(!is_s);
-        }
-
-        // ================= phase 3: row statistics, uint8 probabilities, partial P.V =================
-        {
-            i32x4 vreg = {0, 0, 0, 0};
-            const int blk = t >> 8, d = (t >> 2) & 63, part = t & 3;
-            const int bpos = a_c * kChunk + blk * kVBlock;
-            if (a_active && bpos < p.max_pos)
-                vreg = *reinterpret_cast<const i32x4*>(vc + v_index(a_h, bpos, d, p.max_pos) + part * 16);
-            const float as_g = ldc_f(a_s + a_h * GROUP + (wave >> 1));   // threads 128g..128g+127 (two waves) serve query head g
-            bar.wait();
-            stamp();
+            // ---- second half: row statistics, uint8 probabilities, partial P.V ----
+            // The only thing that crosses workgroups between the halves is the pair (max, sum) of every chunk of the
+            // same head.  Each value carries the barrier epoch of this phase in its high word, so the 32 workgroups of
+            // a KV head poll those words directly instead of going through a grid barrier and a load after it; the
+            // slot is next written a layer later, three grid barriers after every reader has finished with it.
             if (a_active) {
                 const int nchunks = (len + kChunk - 1) / kChunk;
                 if (wave < GROUP) {
                     float m_c = -1e32f, l_c = 0.0f;
-                    if (lane < nchunks) {
-                        m_c = ld_f(&p.stats[(a_h * GROUP + wave) * 32 + lane].x);
-                        l_c = ld_f(&p.stats[(a_h * GROUP + wave) * 32 + lane].y);
+                    {
+                        const unsigned long long* slot = p.stats_tag + (size_t)((a_h * GROUP + wave) * 32 + min(lane, nchunks - 1)) * 2;
+                        unsigned long long w0 = 0, w1 = 0;
+                        int it = 0;
+                        for (;;) {
+                            w0 = ld_u64(slot);
+                            w1 = ld_u64(slot + 1);
+                            const bool ok = (unsigned)(w0 >> 32) == bar.epoch && (unsigned)(w1 >> 32) == bar.epoch;
+                            if (__builtin_amdgcn_ballot_w64(!ok) == 0) break;
+                            if (++it > kMegaSpinLimit) { if (lane == 0) st_i(bar.err, 1); break; }
+                        }
+                        if (lane < nchunks) { m_c = __int_as_float((int)(unsigned)w0); l_c = __int_as_float((int)(unsigned)w1); }
                     }
                     const float mx = wave_max(m_c);
                     const float sum = wave_sum(lane < nchunks ? l_c * exp_f(m_c - mx) : 0.0f);
                     if (lane == 0) { L.rowmax[wave] = mx; L.rowcd[wave] = 1.0f / sum; }
                 }
+                stamp();                                              // workgroup 0 is always active: its timeline keeps 12 stamps per layer
                 __syncthreads();
                 gu_slice(2);                                          // the chunk statistics have landed
                 {
