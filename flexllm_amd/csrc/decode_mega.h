@@ -53,6 +53,7 @@ struct MegaParams {
     size_t cache_layer_bytes;
     float *x, *x2, *qkv, *h, *logits;
     float2* stats;                 // [q_heads][32] (one-kernel-per-stage path)
+    unsigned long long* qkv_tag;   // [H + 2*KV]: q/k/v projection outputs, each with the epoch in its high word
     unsigned long long* stats_tag; // [q_heads][32][2]: chunk max and chunk sum of exponentials, each with the epoch in its high word
     int32_t* o_acc;                // [H]
     int* state;                    // [0] pos, [1] step, [2] barrier epoch base, [3] error flag
@@ -78,6 +79,21 @@ __device__ __forceinline__ void st_tagged(unsigned long long* p, float v, unsign
 }
 __device__ __forceinline__ unsigned long long ld_u64(const unsigned long long* p) {
     return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+// Polls two tagged words until both carry `tag` in every active lane of the wave (bounded: raises the error flag).
+__device__ __forceinline__ void poll_tagged2(const unsigned long long* a, const unsigned long long* b, unsigned tag,
+                                             int* err, float& fa, float& fb) {
+    unsigned long long w0 = 0, w1 = 0;
+    int it = 0;
+    for (;;) {
+        w0 = ld_u64(a);
+        w1 = ld_u64(b);
+        const bool ok = (unsigned)(w0 >> 32) == tag && (unsigned)(w1 >> 32) == tag;
+        if (__builtin_amdgcn_ballot_w64(!ok) == 0) break;
+        if (++it > kMegaSpinLimit) { st_i(err, 1); break; }
+    }
+    fa = __int_as_float((int)(unsigned)w0);
+    fb = __int_as_float((int)(unsigned)w1);
 }
 
 // Read-only data at a wave-uniform address (layer table, per-row weight scales): the constant address space
@@ -361,11 +377,11 @@ __global__ __launch_bounds__(kMegaT, 1) void decode_mega_kernel(MegaParams p) {
                 for (int j = 0; j < 3; j++) {
                     const int r = wg * 12 + wave + 4 * j;
                     const int a = mega_dot_row<2>(wr[j], L.xq, lane);
-                    if (lane == 0) st_f(&p.qkv[r], (float)a * sx * wsc[j]);
+                    if (lane == 0) st_tagged(&p.qkv_tag[r], (float)a * sx * wsc[j], bar.epoch);
                 }
             }
             stamp();
-            bar.arrive(!is_s);
+            // no grid barrier here: a KV head's 32 workgroups need 384 of the 3072 outputs and poll their tagged words
         }
 
         // ================= phase 2: RoPE/quant/append, scores of this chunk, chunk statistics =================
@@ -386,21 +402,21 @@ __global__ __launch_bounds__(kMegaT, 1) void decode_mega_kernel(MegaParams p) {
 #pragma unroll
             for (int g = 0; g < GROUP; g++) qs4[g] = ldc_f(q_s + a_h * GROUP + g);
             const float ks1 = ldc_f(k_s + a_h), vs1 = ldc_f(v_s + a_h);
-            bar.wait();
-            stamp();
             if (a_active) {
                 const float* sn = p.rope_sin + (size_t)pos * 32;
                 const float* cs = p.rope_cos + (size_t)pos * 32;
                 if (t < 128) {                                        // q: 4 heads x 32 pairs
                     const int g = t >> 5, k = t & 31, qh = a_h * GROUP + g;
-                    const float t0 = ld_f(&p.qkv[qh * kHd + k]), t1 = ld_f(&p.qkv[qh * kHd + k + 32]);
+                    float t0, t1;
+                    poll_tagged2(&p.qkv_tag[qh * kHd + k], &p.qkv_tag[qh * kHd + k + 32], bar.epoch, bar.err, t0, t1);
                     const float o0 = t0 * cs[k] - t1 * sn[k], o1 = t0 * sn[k] + t1 * cs[k];
                     const float div = 8.0f * (g == 0 ? qs4[0] : g == 1 ? qs4[1] : g == 2 ? qs4[2] : qs4[3]);
                     L.q8[g][k] = (int8_t)static_q8(o0, div);
                     L.q8[g][k + 32] = (int8_t)static_q8(o1, div);
                 } else if (t < 160) {                                 // k of the new token: 32 pairs
                     const int k = t - 128;
-                    const float t0 = ld_f(&p.qkv[H + a_h * kHd + k]), t1 = ld_f(&p.qkv[H + a_h * kHd + k + 32]);
+                    float t0, t1;
+                    poll_tagged2(&p.qkv_tag[H + a_h * kHd + k], &p.qkv_tag[H + a_h * kHd + k + 32], bar.epoch, bar.err, t0, t1);
                     const float o0 = t0 * cs[k] - t1 * sn[k], o1 = t0 * sn[k] + t1 * cs[k];
                     const float div = 1.0f * ks1;
                     const int8_t b0 = (int8_t)static_q8(o0, div), b1 = (int8_t)static_q8(o1, div);
@@ -408,10 +424,13 @@ __global__ __launch_bounds__(kMegaT, 1) void decode_mega_kernel(MegaParams p) {
                     if (a_owner) { int8_t* dst = kc + k_index(a_h, pos, p.max_pos); dst[k] = b0; dst[k + 32] = b1; }
                 } else if (t < 224) {                                 // v of the new token
                     const int d = t - 160;
-                    const int8_t b = (int8_t)static_q8(ld_f(&p.qkv[H + KV + a_h * kHd + d]), 1.0f * vs1);
+                    float tv, tv_again;
+                    poll_tagged2(&p.qkv_tag[H + KV + a_h * kHd + d], &p.qkv_tag[H + KV + a_h * kHd + d], bar.epoch, bar.err, tv, tv_again);
+                    const int8_t b = (int8_t)static_q8(tv, 1.0f * vs1);
                     L.vnew[d] = b;
                     if (a_owner) vc[v_index(a_h, pos, d, p.max_pos)] = b;
                 }
+                stamp();
                 __syncthreads();
                 gu_slice(1);                                          // the q/k/v loads of this phase have landed
                 if (kpos == pos) kreg = reinterpret_cast<const i32x4*>(L.knew)[part];

@@ -29,6 +29,7 @@ struct flexllm_llama {
     float* xs = nullptr;
     float* scores = nullptr;
     float2* stats = nullptr;
+    unsigned long long* qkv_tag = nullptr;     // persistent kernel: q/k/v outputs tagged with the barrier epoch
     unsigned long long* stats_tag = nullptr;   // persistent kernel: chunk statistics tagged with the barrier epoch
     int32_t* o_acc = nullptr;
     int* state = nullptr;           // [0] position of the token being processed, [1] step index
@@ -174,7 +175,7 @@ static int launch_mega(flexllm_llama* m, int* token, const float* x_in, float* l
     p.embed = reinterpret_cast<const __half*>(m->embed);
     p.k_cache = m->k_cache; p.v_cache = m->v_cache; p.cache_layer_bytes = m->cache_layer_bytes;
     p.x = m->x; p.x2 = m->x2; p.qkv = m->qkv; p.h = m->h; p.logits = logits ? logits : m->logits;
-    p.stats = m->stats; p.stats_tag = m->stats_tag; p.o_acc = m->o_acc; p.state = m->state; p.bar = m->bar;
+    p.stats = m->stats; p.stats_tag = m->stats_tag; p.qkv_tag = m->qkv_tag; p.o_acc = m->o_acc; p.state = m->state; p.bar = m->bar;
     p.token = token; p.tokens_out = tokens_out; p.n_steps = steps; p.x_in = x_in; p.am_v = m->am_v; p.am_i = m->am_i;
     p.n_layers = c.layers; p.max_pos = c.max_pos; p.vocab = c.vocab; p.want_head = want_head;
     p.eps = c.eps; p.fht_scale = c.fht_scale;
@@ -298,8 +299,10 @@ int flexllm_llama_create(flexllm_llama** out, const flexllm_llama_config* cfg, c
     FX_TRY(dev_alloc(m, (void**)&m->scores, sizeof(float) * (size_t)c.q_heads * c.max_pos));
     FX_TRY(dev_alloc(m, (void**)&m->stats, sizeof(float2) * (size_t)c.q_heads * kMaxChunks));
     FX_TRY(dev_alloc(m, (void**)&m->o_acc, sizeof(int32_t) * H));
+    FX_TRY(dev_alloc(m, (void**)&m->qkv_tag, sizeof(unsigned long long) * (size_t)(H + 2 * KV)));
+    FX_TRY_HIP(hipMemset(m->qkv_tag, 0xFF, sizeof(unsigned long long) * (size_t)(H + 2 * KV)));   // tag 0xFFFFFFFF: never a live epoch (the first is 0)
     FX_TRY(dev_alloc(m, (void**)&m->stats_tag, sizeof(unsigned long long) * 2 * (size_t)c.q_heads * kMaxChunks));
-    FX_TRY_HIP(hipMemset(m->stats_tag, 0, sizeof(unsigned long long) * 2 * (size_t)c.q_heads * kMaxChunks));
+    FX_TRY_HIP(hipMemset(m->stats_tag, 0xFF, sizeof(unsigned long long) * 2 * (size_t)c.q_heads * kMaxChunks));
     FX_TRY(dev_alloc(m, (void**)&m->state, sizeof(int) * 4));
     FX_TRY(dev_alloc(m, (void**)&m->am_v, sizeof(float) * kArgmaxParts));
     FX_TRY(dev_alloc(m, (void**)&m->am_i, sizeof(int) * kArgmaxParts));
