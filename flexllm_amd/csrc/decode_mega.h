@@ -10,10 +10,14 @@
 //              5 RMSNorm+quant (redundant) -> gate/up rows + SiLU*up
 //              6 Hadamard R4 + quant (redundant) -> down rows + residual
 //   then       final RMSNorm (redundant) -> lm_head rows, per-workgroup argmax candidates.
-// Phases are separated by a grid barrier built from device-scope relaxed atomics (two-level arrive, one
-// broadcast flag).  The weights a workgroup needs in the NEXT phase do not depend on the activations, so
-// they are loaded into registers BEFORE waiting on the barrier: HBM keeps streaming while the barrier's
-// round trips are in flight.
+// Where every workgroup needs what every other one produced (3->4, 4->5, 5->6, 6->1) the phases are separated
+// by a grid barrier built from device-scope relaxed atomics (two-level arrive, one broadcast flag).  Where the
+// consumers are few (1->2: a KV head's 32 workgroups need 384 of the 3072 q/k/v outputs; 2->3: the same 32
+// workgroups need each other's chunk statistics) there is no barrier: each value is stored as one 64-bit word
+// with the barrier epoch of its phase in the high half, and the consumers poll the words they need.  A slot is
+// rewritten a layer later, at least three grid barriers after its last reader.  The weights a workgroup needs
+// in the NEXT phase do not depend on the activations, so they are loaded into registers BEFORE waiting on
+// the barrier: HBM keeps streaming while the barrier's round trips are in flight.
 //
 // Wave roles.  Vector-memory results return to a wave in issue order, so a wave with a long weight prefetch in
 // flight cannot see an activation load (or have a store acknowledged) until the prefetch has landed.  The
