@@ -200,8 +200,8 @@ __global__ __launch_bounds__(256) void gemm_i8_kernel(const int8_t* __restrict__
 //
 // The loads are issued from inline assembly: the compiler does not track them, so the k-loop waits for them
 // with explicit counters (results return in issue order).
-__host__ __device__ constexpr int gemm_dma_lds_bytes(int bm, int bn, int stages, int bkb = 64) {
-    return stages * (bm + bn) * bkb > 4 * 32 * 36 * 4 ? stages * (bm + bn) * bkb : 4 * 32 * 36 * 4;   // stages, or the four epilogue patches
+__host__ __device__ constexpr int gemm_dma_lds_bytes(int bm, int bn, int stages, int bkb = 64, int nw = 4) {
+    return stages * (bm + bn) * bkb > nw * 32 * 36 * 4 ? stages * (bm + bn) * bkb : nw * 32 * 36 * 4;   // stages, or one epilogue patch per wave
 }
 
 enum GemmDmaEpi { kDmaRaw = 0, kDmaDequant = 1, kDmaSwiglu = 2, kDmaQkv = 3 };
@@ -236,16 +236,20 @@ __device__ __forceinline__ void gemm_wait_vmcnt() {            // s_waitcnt vmcn
 // for again one stage later: measured with the loads alone (no math, 128 x 256 tiles at K = 2048), the chip moves
 // 23 TB/s into LDS in whole 128-byte lines and 14.5 TB/s in halves.  With 128-byte rows the slot rotation is
 // s ^ ((r >> 1) & 7): two rows span the 64 banks, so 16 consecutive rows of one chunk fall on 16 different bank groups.
-template <int BM, int BN, int EPI, int kDmaStages, int WPE, int BKB>   // at most 7 stages (the wait below distinguishes up to 5 younger ones)
-__global__ __launch_bounds__(256, WPE) void gemm_i8_dma_kernel(const int8_t* __restrict__ a, const int8_t* __restrict__ w,
+// NW = waves per workgroup, 4 (2x2 wave grid) or 8 (2x4): eight waves let a 256x256 tile keep two waves per SIMD.
+template <int BM, int BN, int EPI, int kDmaStages, int WPE, int BKB, int NW>   // at most 7 stages (the wait below distinguishes up to 5 younger ones)
+__global__ __launch_bounds__(NW * 64, WPE) void gemm_i8_dma_kernel(const int8_t* __restrict__ a, const int8_t* __restrict__ w,
                                                           int32_t* __restrict__ c_out, const float* __restrict__ s_x,
                                                           const float* __restrict__ w_s, const float* __restrict__ residual,
                                                           float* __restrict__ y, int m, int k, int n, int tiles_m, int tiles_n,
                                                           QkvEpiArgs qa) {
-    constexpr int WM = BM / 2, WN = BN / 2, TM = WM / 32, TN = WN / 32;
+    static_assert(NW == 4 || NW == 8, "four or eight waves");
+    constexpr int WGN = NW / 2;                               // waves along N
+    constexpr int WM = BM / 2, WN = BN / WGN, TM = WM / 32, TN = WN / 32;
     static_assert(BKB == 64 || BKB == 128, "64 or 128 k-bytes per row and stage");
     constexpr int CPR = BKB / 16, RPI = 64 / CPR;             // 16-byte chunks per row; rows per direct load (1 KiB)
-    constexpr int A_INSTR = BM / (4 * RPI), B_INSTR = BN / (4 * RPI);   // direct loads per wave per stage
+    constexpr int A_INSTR = BM / (NW * RPI), B_INSTR = BN / (NW * RPI);   // direct loads per wave per stage
+    static_assert(A_INSTR >= 1 && B_INSTR >= 1 && TM >= 1 && TN >= 1, "tile too small for this wave count");
     constexpr int STAGE = (BM + BN) * BKB, KS = BKB / 32;     // KS MFMA k-steps per stage
     auto rot = [](int r) { return BKB == 64 ? (r >> 2) & 3 : (r >> 1) & 7; };
     extern __shared__ __attribute__((aligned(16))) int8_t gemm_smem[];
@@ -262,7 +266,7 @@ __global__ __launch_bounds__(256, WPE) void gemm_i8_dma_kernel(const int8_t* __r
     int row0 = tm * BM, col0 = tn * BN;
     const int t = threadIdx.x, lane = t & 63;
     const int wave = __builtin_amdgcn_readfirstlane(t >> 6);
-    const int wm = (wave >> 1) * WM, wn = (wave & 1) * WN;
+    const int wm = (wave / WGN) * WM, wn = (wave % WGN) * WN;
 
     // per-lane global offsets of this wave's direct loads (without the k offset, which is uniform)
     unsigned offa[A_INSTR], offb[B_INSTR];
@@ -367,7 +371,7 @@ __global__ __launch_bounds__(256, WPE) void gemm_i8_dma_kernel(const int8_t* __r
     // (8 bytes for the SiLU*up pairs), 128 contiguous bytes per row.
     __syncthreads();                                           // all waves are done with the stage buffers
     if constexpr (EPI == kDmaQkv) {
-        static_assert(EPI != kDmaQkv || (BM == 64 && BN == 64), "the q/k/v epilogue works on 64x64 tiles");
+        static_assert(EPI != kDmaQkv || (BM == 64 && BN == 64 && NW == 4), "the q/k/v epilogue works on 64x64 tiles with four waves");
         constexpr int TP = 65;                                 // odd pitch: a column walk hits every bank once
         float* tile = reinterpret_cast<float*>(gemm_smem);     // dequantised tile [64 tokens][64 channels]
         {
@@ -503,17 +507,17 @@ __global__ __launch_bounds__(256, WPE) void gemm_i8_dma_kernel(const int8_t* __r
     }
 }
 
-template <int BM, int BN, int EPI, int STAGES = 3, int WPE = 1, int BKB = 64>
+template <int BM, int BN, int EPI, int STAGES = 3, int WPE = 1, int BKB = 64, int NW = 4>
 inline int launch_gemm_dma(const int8_t* a, const int8_t* w, int32_t* c, const float* s_x, const float* w_s,
                            const float* residual, float* y, int m, int k, int n, hipStream_t st, QkvEpiArgs qa = QkvEpiArgs()) {
     static bool opted_in = false;             // more than the default 64 KiB of LDS per workgroup
     if (!opted_in) {
-        FX_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_i8_dma_kernel<BM, BN, EPI, STAGES, WPE, BKB>),
-                                   hipFuncAttributeMaxDynamicSharedMemorySize, gemm_dma_lds_bytes(BM, BN, STAGES, BKB)));
+        FX_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_i8_dma_kernel<BM, BN, EPI, STAGES, WPE, BKB, NW>),
+                                   hipFuncAttributeMaxDynamicSharedMemorySize, gemm_dma_lds_bytes(BM, BN, STAGES, BKB, NW)));
         opted_in = true;
     }
     const int tm = (m + BM - 1) / BM, tn = (n + BN - 1) / BN;
-    gemm_i8_dma_kernel<BM, BN, EPI, STAGES, WPE, BKB><<<tm * tn, 256, gemm_dma_lds_bytes(BM, BN, STAGES, BKB), st>>>(a, w, c, s_x, w_s, residual, y, m, k, n, tm, tn, qa);
+    gemm_i8_dma_kernel<BM, BN, EPI, STAGES, WPE, BKB, NW><<<tm * tn, NW * 64, gemm_dma_lds_bytes(BM, BN, STAGES, BKB, NW), st>>>(a, w, c, s_x, w_s, residual, y, m, k, n, tm, tn, qa);
     FX_LAUNCH_CHECK();
     return FLEXLLM_OK;
 }
@@ -583,13 +587,18 @@ inline int launch_gemm_swiglu(const int8_t* a, const int8_t* w_gu, const float* 
                               int k, int n2, hipStream_t st) {
     FX_REQUIRE((size_t)m * k < (1ull << 31) && (size_t)n2 * k < (1ull << 31) && n2 % 4 == 0,
                "linear_i8_gemm_swiglu: m=%d k=%d n=%d outside the direct-load kernel's range", m, k, n2 / 2);
-    // Measured at M=1024, 2048 -> 2x8192: 128x256 tiles, two stages of 64-byte rows, two workgroups per CU (one
-    // round of 512 workgroups): 48-49 us.  128x128 tiles (two or three per CU, 64- or 128-byte rows) and 256x256
-    // tiles (one per CU) came out at 48-58 us; FLEXLLM_GEMM_TILE=13 forces the 64x64 fallback.
+    // Measured at M=1024, 2048 -> 2x8192 (us): 256x256 tiles on eight waves, two stages of 128-byte rows, one
+    // workgroup per CU: 42.0; the same with four stages of 64-byte rows: 43.6; 128x256 tiles on four waves, two
+    // stages of 64-byte rows, two workgroups per CU: 49.3; 128x256 on eight waves: 48-57; 128x128 tiles (two or
+    // three per CU) and 256x256 on four waves: 48-58.  The big tile is taken when its grid fills the 256 CUs in
+    // whole rounds (or many of them); FLEXLLM_GEMM_TILE forces 50 / 16 / 13 (the 64x64 fallback).
     static const char* force = getenv("FLEXLLM_GEMM_TILE");
+    const int tiles_256 = ((m + 255) / 256) * ((n2 + 255) / 256);
     const int tiles_big = ((m + 127) / 128) * ((n2 + 255) / 256);
-    int mode = tiles_big >= 384 ? 16 : 13;
+    int mode = (k % 128 == 0 && tiles_256 >= 256 && (tiles_256 % 256 == 0 || tiles_256 >= 1024)) ? 50 : tiles_big >= 384 ? 16 : 13;
     if (force) mode = atoi(force);
+    if (mode == 50 && k % 128 == 0)
+        return launch_gemm_dma<256, 256, kDmaSwiglu, 2, 2, 128, 8>(a, w_gu, nullptr, s_x, w_s_gu, nullptr, h, m, k, n2, st);
     if (mode == 16) return launch_gemm_dma<128, 256, kDmaSwiglu, 2, 2>(a, w_gu, nullptr, s_x, w_s_gu, nullptr, h, m, k, n2, st);
     return launch_gemm_dma<64, 64, kDmaSwiglu>(a, w_gu, nullptr, s_x, w_s_gu, nullptr, h, m, k, n2, st);
 }
