@@ -200,8 +200,12 @@ __global__ __launch_bounds__(256) void gemm_i8_kernel(const int8_t* __restrict__
 //
 // The loads are issued from inline assembly: the compiler does not track them, so the k-loop waits for them
 // with explicit counters (results return in issue order).
-__host__ __device__ constexpr int gemm_dma_lds_bytes(int bm, int bn, int stages, int bkb = 64, int nw = 4) {
-    return stages * (bm + bn) * bkb > nw * 32 * 36 * 4 ? stages * (bm + bn) * bkb : nw * 32 * 36 * 4;   // stages, or one epilogue patch per wave
+__host__ __device__ constexpr int gemm_dma_lds_bytes(int bm, int bn, int stages, int bkb = 64, int nw = 4, int ksplit = 1) {
+    // the stage rings (one per k-group), or the epilogue: one patch per wave plus, with two k-groups, the second
+    // group's accumulators
+    const int rings = ksplit * stages * (bm + bn) * bkb;
+    const int epi = nw * 32 * 36 * 4 + (ksplit > 1 ? bm * bn * 4 : 0);
+    return rings > epi ? rings : epi;
 }
 
 enum GemmDmaEpi { kDmaRaw = 0, kDmaDequant = 1, kDmaSwiglu = 2, kDmaQkv = 3 };
@@ -237,18 +241,24 @@ __device__ __forceinline__ void gemm_wait_vmcnt() {            // s_waitcnt vmcn
 // 23 TB/s into LDS in whole 128-byte lines and 14.5 TB/s in halves.  With 128-byte rows the slot rotation is
 // s ^ ((r >> 1) & 7): two rows span the 64 banks, so 16 consecutive rows of one chunk fall on 16 different bank groups.
 // NW = waves per workgroup, 4 (2x2 wave grid) or 8 (2x4): eight waves let a 256x256 tile keep two waves per SIMD.
-template <int BM, int BN, int EPI, int kDmaStages, int WPE, int BKB, int NW>   // at most 7 stages (the wait below distinguishes up to 5 younger ones)
+// KSPLIT = 2 (with NW = 8): two groups of four waves work on the same output tile, group g on the stages
+// kt with kt % 2 == g, each with its own ring of LDS stages; the second group's accumulators are added to the first's
+// through LDS before the epilogue (integer sums: exact in any order).  For outputs too narrow to give every CU two
+// workgroups (down projection: 256 tiles of 64x128) this puts two independent load pipelines on a CU all the same.
+template <int BM, int BN, int EPI, int kDmaStages, int WPE, int BKB, int NW, int KSPLIT>   // at most 7 stages (the wait below distinguishes up to 5 younger ones)
 __global__ __launch_bounds__(NW * 64, WPE) void gemm_i8_dma_kernel(const int8_t* __restrict__ a, const int8_t* __restrict__ w,
                                                           int32_t* __restrict__ c_out, const float* __restrict__ s_x,
                                                           const float* __restrict__ w_s, const float* __restrict__ residual,
                                                           float* __restrict__ y, int m, int k, int n, int tiles_m, int tiles_n,
                                                           QkvEpiArgs qa) {
     static_assert(NW == 4 || NW == 8, "four or eight waves");
-    constexpr int WGN = NW / 2;                               // waves along N
+    static_assert(KSPLIT == 1 || (KSPLIT == 2 && NW == 8 && EPI != kDmaQkv), "two k-groups need eight waves");
+    constexpr int GW = NW / KSPLIT;                           // waves per k-group
+    constexpr int WGN = GW / 2;                               // waves along N
     constexpr int WM = BM / 2, WN = BN / WGN, TM = WM / 32, TN = WN / 32;
     static_assert(BKB == 64 || BKB == 128, "64 or 128 k-bytes per row and stage");
     constexpr int CPR = BKB / 16, RPI = 64 / CPR;             // 16-byte chunks per row; rows per direct load (1 KiB)
-    constexpr int A_INSTR = BM / (NW * RPI), B_INSTR = BN / (NW * RPI);   // direct loads per wave per stage
+    constexpr int A_INSTR = BM / (GW * RPI), B_INSTR = BN / (GW * RPI);   // direct loads per wave per stage
     static_assert(A_INSTR >= 1 && B_INSTR >= 1 && TM >= 1 && TN >= 1, "tile too small for this wave count");
     constexpr int STAGE = (BM + BN) * BKB, KS = BKB / 32;     // KS MFMA k-steps per stage
     auto rot = [](int r) { return BKB == 64 ? (r >> 2) & 3 : (r >> 1) & 7; };
@@ -265,8 +275,10 @@ __global__ __launch_bounds__(NW * 64, WPE) void gemm_i8_dma_kernel(const int8_t*
     }
     int row0 = tm * BM, col0 = tn * BN;
     const int t = threadIdx.x, lane = t & 63;
-    const int wave = __builtin_amdgcn_readfirstlane(t >> 6);
+    const int wave_wg = __builtin_amdgcn_readfirstlane(t >> 6);
+    const int grp = wave_wg / GW, wave = wave_wg % GW;         // k-group, wave within the group
     const int wm = (wave / WGN) * WM, wn = (wave % WGN) * WN;
+    int8_t* const ring = gemm_smem + grp * (kDmaStages * STAGE);
 
     // per-lane global offsets of this wave's direct loads (without the k offset, which is uniform)
     unsigned offa[A_INSTR], offb[B_INSTR];
@@ -280,13 +292,15 @@ __global__ __launch_bounds__(NW * 64, WPE) void gemm_i8_dma_kernel(const int8_t*
         const int r = (wave * B_INSTR + j) * RPI + lane / CPR;
         offb[j] = (unsigned)min(col0 + r, n - 1) * (unsigned)k + (unsigned)(((lane % CPR) ^ rot(r)) * 16);
     }
-    const unsigned lds0 = (unsigned)(uintptr_t)(__attribute__((address_space(3))) void*)gemm_smem;
+    const unsigned lds0 = (unsigned)(uintptr_t)(__attribute__((address_space(3))) void*)ring;
+    // kt counts the stages of this k-group; the group's stage kt is stage kt * KSPLIT + grp of the whole K range
     auto issue_stage = [&](int kt) {
         const unsigned sb = lds0 + (unsigned)(kt % kDmaStages) * STAGE;
+        const size_t koff = (size_t)(kt * KSPLIT + grp) * BKB;
 #pragma unroll
-        for (int j = 0; j < A_INSTR; j++) gemm_dma_issue(a + (size_t)kt * BKB, offa[j], sb + (wave * A_INSTR + j) * 1024);
+        for (int j = 0; j < A_INSTR; j++) gemm_dma_issue(a + koff, offa[j], sb + (wave * A_INSTR + j) * 1024);
 #pragma unroll
-        for (int j = 0; j < B_INSTR; j++) gemm_dma_issue(w + (size_t)kt * BKB, offb[j], sb + BM * BKB + (wave * B_INSTR + j) * 1024);
+        for (int j = 0; j < B_INSTR; j++) gemm_dma_issue(w + koff, offb[j], sb + BM * BKB + (wave * B_INSTR + j) * 1024);
     };
 
     i32x16 acc[TM][TN];
@@ -297,7 +311,7 @@ __global__ __launch_bounds__(NW * 64, WPE) void gemm_i8_dma_kernel(const int8_t*
 #pragma unroll
             for (int r = 0; r < 16; r++) acc[i][j][r] = 0;
 
-    const int nk = k / BKB;
+    const int nk = k / (BKB * KSPLIT);                         // stages per k-group (the launcher checks divisibility)
     constexpr int PER = A_INSTR + B_INSTR;                     // direct loads per wave per stage
 #pragma unroll
     for (int s0 = 0; s0 < kDmaStages - 1; s0++)
@@ -305,7 +319,7 @@ __global__ __launch_bounds__(NW * 64, WPE) void gemm_i8_dma_kernel(const int8_t*
     // fragment addressing: lane l reads row (l % 32) of a 32-row tile, k-chunk 2*ks + l/32, from its rotated slot
     const int fr = lane & 31, fg = lane >> 5;
     auto read_frags = [&](int kt, int ks, i32x4 (&fa)[TM], i32x4 (&fb)[TN]) {
-        const int8_t* sa = gemm_smem + (kt % kDmaStages) * STAGE;
+        const int8_t* sa = ring + (kt % kDmaStages) * STAGE;
         const int8_t* sb = sa + BM * BKB;
 #pragma unroll
         for (int i = 0; i < TM; i++) {
@@ -370,6 +384,26 @@ __global__ __launch_bounds__(NW * 64, WPE) void gemm_i8_dma_kernel(const int8_t*
     // (32 x 36 words) and then owns 4 consecutive columns of a row: 16-byte loads of the residual, 16-byte stores
     // (8 bytes for the SiLU*up pairs), 128 contiguous bytes per row.
     __syncthreads();                                           // all waves are done with the stage buffers
+    if constexpr (KSPLIT == 2) {
+        // the second k-group hands its accumulators over, lane-contiguous (conflict-free), behind the patch area
+        int* xch = reinterpret_cast<int*>(gemm_smem) + NW * 32 * 36 + wave * (TM * TN * 16 * 64) + lane;
+        if (grp == 1) {
+#pragma unroll
+            for (int i = 0; i < TM; i++)
+#pragma unroll
+                for (int j = 0; j < TN; j++)
+#pragma unroll
+                    for (int r = 0; r < 16; r++) xch[((i * TN + j) * 16 + r) * 64] = acc[i][j][r];
+        }
+        __syncthreads();
+        if (grp == 1) return;
+#pragma unroll
+        for (int i = 0; i < TM; i++)
+#pragma unroll
+            for (int j = 0; j < TN; j++)
+#pragma unroll
+                for (int r = 0; r < 16; r++) acc[i][j][r] += xch[((i * TN + j) * 16 + r) * 64];
+    }
     if constexpr (EPI == kDmaQkv) {
         static_assert(EPI != kDmaQkv || (BM == 64 && BN == 64 && NW == 4), "the q/k/v epilogue works on 64x64 tiles with four waves");
         constexpr int TP = 65;                                 // odd pitch: a column walk hits every bank once
@@ -507,17 +541,17 @@ __global__ __launch_bounds__(NW * 64, WPE) void gemm_i8_dma_kernel(const int8_t*
     }
 }
 
-template <int BM, int BN, int EPI, int STAGES = 3, int WPE = 1, int BKB = 64, int NW = 4>
+template <int BM, int BN, int EPI, int STAGES = 3, int WPE = 1, int BKB = 64, int NW = 4, int KSPLIT = 1>
 inline int launch_gemm_dma(const int8_t* a, const int8_t* w, int32_t* c, const float* s_x, const float* w_s,
                            const float* residual, float* y, int m, int k, int n, hipStream_t st, QkvEpiArgs qa = QkvEpiArgs()) {
     static bool opted_in = false;             // more than the default 64 KiB of LDS per workgroup
     if (!opted_in) {
-        FX_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_i8_dma_kernel<BM, BN, EPI, STAGES, WPE, BKB, NW>),
-                                   hipFuncAttributeMaxDynamicSharedMemorySize, gemm_dma_lds_bytes(BM, BN, STAGES, BKB, NW)));
+        FX_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_i8_dma_kernel<BM, BN, EPI, STAGES, WPE, BKB, NW, KSPLIT>),
+                                   hipFuncAttributeMaxDynamicSharedMemorySize, gemm_dma_lds_bytes(BM, BN, STAGES, BKB, NW, KSPLIT)));
         opted_in = true;
     }
     const int tm = (m + BM - 1) / BM, tn = (n + BN - 1) / BN;
-    gemm_i8_dma_kernel<BM, BN, EPI, STAGES, WPE, BKB, NW><<<tm * tn, NW * 64, gemm_dma_lds_bytes(BM, BN, STAGES, BKB, NW), st>>>(a, w, c, s_x, w_s, residual, y, m, k, n, tm, tn, qa);
+    gemm_i8_dma_kernel<BM, BN, EPI, STAGES, WPE, BKB, NW, KSPLIT><<<tm * tn, NW * 64, gemm_dma_lds_bytes(BM, BN, STAGES, BKB, NW, KSPLIT), st>>>(a, w, c, s_x, w_s, residual, y, m, k, n, tm, tn, qa);
     FX_LAUNCH_CHECK();
     return FLEXLLM_OK;
 }
@@ -528,7 +562,8 @@ inline int launch_gemm(const int8_t* a, const int8_t* w, int32_t* c, const float
     // Measured on MI355X at M=1024: the direct-load kernel wins wherever it applies; 128x128 tiles once they fill
     // the chip about three times over, 64x64 tiles for the narrow projections.  FLEXLLM_GEMM_TILE forces a variant
     // (0..2: register-staged 128x128 / 64x128 / 64x64; direct-load: 11 = 128x128, 13 = 64x64, 19 = 64x128 four
-    // stages, all with 64-byte rows; 36 = 64x64 four stages and 38 = 64x64 three stages with 128-byte rows).
+    // stages, all with 64-byte rows; 36 = 64x64 four stages and 38 = 64x64 three stages with 128-byte rows; 60 = 64x128
+    // three stages with 128-byte rows and two k-groups).
     auto tiles = [&](int bm, int bn) { return ((m + bm - 1) / bm) * ((n + bn - 1) / bn); };
     static const char* force = getenv("FLEXLLM_GEMM_TILE");
     // the direct-load kernel needs 32-bit element offsets into both operands and 16-byte aligned output rows
@@ -536,6 +571,9 @@ inline int launch_gemm(const int8_t* a, const int8_t* w, int32_t* c, const float
     int mode = dma_ok ? (tiles(128, 128) >= 768 ? 11 : (k >= 4096 && tiles(64, 128) >= 256) ? 19 : 13) : (tiles(128, 128) >= 1024 ? 0 : 2);
     // whole 128-byte lines per row and stage where K allows: three workgroups of 48 KiB per CU when the grid has
     // that many, else two of 64 KiB with a fourth stage (the narrow projections stream their weights cold)
+    // Long K and an output too narrow for two workgroups per CU (down projection): 64x128 tiles, two k-groups of
+    // four waves per workgroup (32 us against 36 us for 64x64 tiles, two workgroups per CU).
+    if (mode == 19 && k % 256 == 0) mode = 60;
     if ((mode == 13 || mode == 19) && k % 128 == 0) mode = tiles(64, 64) >= 768 ? 38 : 36;
     if (force) mode = atoi(force);
     if (mode >= 10 && !dma_ok) mode = 2;
@@ -547,6 +585,9 @@ inline int launch_gemm(const int8_t* a, const int8_t* w, int32_t* c, const float
         if (k % 128 == 0) {
             if (mode == 36) return launch_gemm_dma<64, 64, DE, 4, 2, 128>(a, w, c, s_x, w_s, residual, y, m, k, n, st);
             if (mode == 38) return launch_gemm_dma<64, 64, DE, 3, 3, 128>(a, w, c, s_x, w_s, residual, y, m, k, n, st);
+            if (k % 256 == 0) {
+                if (mode == 60) return launch_gemm_dma<64, 128, DE, 3, 2, 128, 8, 2>(a, w, c, s_x, w_s, residual, y, m, k, n, st);
+            }
         }
         return launch_gemm_dma<64, 64, DE>(a, w, c, s_x, w_s, residual, y, m, k, n, st);
     }

@@ -24,6 +24,22 @@ def test_gemm_int32_exact(fx, m, k, n):
     assert np.array_equal(acc, ref)
 
 
+def test_gemm_down_projection_shape(fx, oracle):
+    """1024 x 8192 -> 2048, the shape that takes 64x128 tiles with two k-groups per workgroup: raw int32 and the
+    dequantised + residual epilogue.  float64 BLAS is exact here (|sum| < 2^31)."""
+    m, k, n = 1024, 8192, 2048
+    a = rng.integers(-128, 128, (m, k)).astype(np.int8)
+    w = rng.integers(-128, 128, (n, k)).astype(np.int8)
+    ref = (a.astype(np.float64) @ w.astype(np.float64).T).astype(np.int64).astype(np.int32)
+    da, dw = fx.to_device(a), fx.to_device(w)
+    assert np.array_equal(fx.ops.linear_i8_gemm(da, dw).numpy(), ref)
+    s_x = rng.uniform(0.01, 0.02, m).astype(np.float32)
+    w_s = rng.uniform(1e-3, 1e-2, n).astype(np.float32)
+    res = rng.standard_normal((m, n)).astype(np.float32)
+    y = fx.ops.linear_i8_gemm_dequant(da, fx.to_device(s_x), dw, fx.to_device(w_s), residual=fx.to_device(res)).numpy()
+    assert np.array_equal(y, oracle.residual(oracle.dequant(ref, s_x, w_s), res))
+
+
 def test_gemm_all_tile_shapes_and_extremes(fx):
     # 128x128 tiles (>= 512 workgroups), 64x128 and 64x64 paths; saturated operands
     for m, k, n in [(1024, 128, 8192), (512, 128, 4096), (256, 128, 256)]:
