@@ -1,0 +1,151 @@
+"""Reads and writes a model in the reference's on-disk parameter format (directory `parameters/`).
+
+What the reference's testbench reads (SpinQuant_Llama_32_1B/SpinQuant_Prefilling_Decoding_mem_opt_tb.cpp):
+  * `<proj>_L%02d.bin` for proj in q_proj, k_proj, v_proj, o_proj, gate_proj, up_proj, down_proj: one signed byte
+    per weight, row-major [out_channel][in_channel] (:30-47, :385-429)
+  * `model_embed_tokens_fp32.bin`: fp32 [vocab][hidden], one row per token id (:150-172, :579)
+  * generated headers with C arrays (:435-443): `w_<proj>_s_sum.h` holding `w_<proj>_s[layers][out]` (per-channel
+    weight scale) and `w_<proj>_sum[layers][out]` (row sums, used by the asymmetric 4-bit path only),
+    `w_rmsnorm.h` holding `RMSNorm_weight[2*layers+1][hidden]` (:485-486, :727-734: rows 2l and 2l+1 are layer l's
+    two norms, the last row the final norm)
+  * `Q_s.h`, `K_s.h`, `V_s.h`, `A_s.h`: static attention scales `Q_s[layers][q_heads]`, `K_s[layers][kv_heads]`,
+    `V_s[layers][kv_heads]`, `A_s[layers][q_heads]` (SpinQuant_Llama_32_1B/MHA_i8xi8.h:11-14, :32, :63, :245)
+
+The reference tree ships none of these files, so the header syntax is taken from how the arrays are indexed: any C
+initialiser `name[d0][d1] = { ... }` (or one-dimensional) is accepted, numbers may carry an `f` suffix.  The rotary
+table (`parameters/RoPE_sin_cos.h`) is regenerated from the formula, and the output head is the embedding matrix
+in fp16 (tied), so `lm_head.bin` / `w_lm_head_lm_head.h` are not read.
+
+`save_reference_parameters` writes the same files from a host weight dictionary, e.g. to hand a synthetic model to
+the reference's own testbench.
+"""
+import os
+import re
+
+import numpy as np
+
+from .device import to_device
+from .ops import rope_table
+
+_PROJ_FILES = dict(q="q_proj", k="k_proj", v="v_proj", o="o_proj", g="gate_proj", u="up_proj", d="down_proj")
+_PROJ_DIMS = dict(q=("hidden", "hidden"), k=("kv_hidden", "hidden"), v=("kv_hidden", "hidden"), o=("hidden", "hidden"),
+                  g=("inter", "hidden"), u=("inter", "hidden"), d=("hidden", "inter"))
+_STATIC = dict(q_s=("Q_s", "q_heads"), k_s=("K_s", "kv_heads"), v_s=("V_s", "kv_heads"), a_s=("A_s", "q_heads"))
+_NUM = re.compile(r"[-+]?(?:\d+\.\d*|\.\d+|\d+)(?:[eE][-+]?\d+)?")
+
+
+class ParameterError(ValueError):
+    pass
+
+
+def parse_c_array(text, name):
+    """The float32 array initialised as `name[d0]...[dn] = { ... }` in C source `text`, shaped by its declared
+    dimensions when all of them are integer literals, flat otherwise.  Comments are ignored."""
+    text = re.sub(r"/\*.*?\*/", " ", text, flags=re.S)
+    text = re.sub(r"//[^\n]*", " ", text)
+    m = re.search(r"\b" + re.escape(name) + r"\s*((?:\[\s*\w*\s*\]\s*)+)=\s*\{", text)
+    if not m:
+        raise ParameterError("array %s not found" % name)
+    dims = re.findall(r"\[\s*(\w*)\s*\]", m.group(1))
+    depth, i = 1, m.end()
+    while depth and i < len(text):
+        depth += {"{": 1, "}": -1}.get(text[i], 0)
+        i += 1
+    if depth:
+        raise ParameterError("array %s: unbalanced braces" % name)
+    body = text[m.end():i - 1]
+    vals = np.array([float(v) for v in _NUM.findall(re.sub(r"(?<=[\d.])[fF]\b", "", body))], dtype=np.float64)
+    vals = vals.astype(np.float32)
+    if not all(d.isdigit() for d in dims):
+        return vals                                # sizes given by macros or left open: flat, the caller knows the shape
+    shape = [int(d) for d in dims]
+    if vals.size != int(np.prod(shape)):
+        raise ParameterError("array %s: %d values do not fit %s" % (name, vals.size, shape))
+    return vals.reshape(shape)
+
+
+def _read_header_array(param_dir, fname, name, shape):
+    path = os.path.join(param_dir, fname)
+    if not os.path.exists(path):
+        raise ParameterError("missing %s" % path)
+    with open(path) as f:
+        arr = parse_c_array(f.read(), name)
+    if arr.size != int(np.prod(shape)):
+        raise ParameterError("%s: %s has %d values, expected %s" % (path, name, arr.size, shape))
+    return np.ascontiguousarray(arr.reshape(shape))
+
+
+def load_reference_parameters(param_dir, cfg, device=True):
+    """Weight dictionary for `llama.Llama` from a reference `parameters/` directory.  device=False returns numpy
+    arrays (the layout of `llama.synth_weights(device=False)`)."""
+    L, H = cfg["layers"], cfg["hidden"]
+    w = {}
+    for key, stem in _PROJ_FILES.items():
+        n, k = cfg[_PROJ_DIMS[key][0]], cfg[_PROJ_DIMS[key][1]]
+        mats = []
+        for l in range(L):
+            path = os.path.join(param_dir, "%s_L%02d.bin" % (stem, l))
+            if not os.path.exists(path):
+                raise ParameterError("missing %s" % path)
+            if os.path.getsize(path) != n * k:
+                raise ParameterError("%s: %d bytes, expected %d x %d" % (path, os.path.getsize(path), n, k))
+            mats.append(np.fromfile(path, dtype=np.int8).reshape(n, k))
+        w["w" + key] = mats
+        s = _read_header_array(param_dir, "w_%s_s_sum.h" % stem, "w_%s_s" % stem, (L, n))
+        w["s" + key] = [np.ascontiguousarray(s[l]) for l in range(L)]
+    w["gamma"] = _read_header_array(param_dir, "w_rmsnorm.h", "RMSNorm_weight", (2 * L + 1, H))
+    for key, (name, heads) in _STATIC.items():
+        w[key] = _read_header_array(param_dir, name + ".h", name, (L, cfg[heads]))
+    path = os.path.join(param_dir, "model_embed_tokens_fp32.bin")
+    if not os.path.exists(path):
+        raise ParameterError("missing %s" % path)
+    if os.path.getsize(path) != 4 * cfg["vocab"] * H:
+        raise ParameterError("%s: %d bytes, expected fp32 %d x %d" % (path, os.path.getsize(path), cfg["vocab"], H))
+    embed = np.memmap(path, dtype=np.float32, mode="r", shape=(cfg["vocab"], H))
+    w["embed"] = np.asarray(embed).astype(np.float16).view(np.uint16)      # tied fp16 table (round to nearest even)
+    w["rope_sin"], w["rope_cos"] = rope_table(cfg["max_pos"], cfg["head_dim"])
+    if not device:
+        return w
+    dev = {}
+    for key, val in w.items():
+        if isinstance(val, list):
+            dev[key] = [to_device(a) for a in val]
+        elif key == "embed":
+            dev[key] = to_device(val.view(np.float16))
+        else:
+            dev[key] = to_device(val)
+    return dev
+
+
+def _fmt(v):
+    t = "%.9g" % v                                 # nine significant digits reproduce a float32 exactly
+    return t + "f" if ("." in t or "e" in t or "n" in t) else t + ".0f"
+
+
+def _write_header(path, arrays):
+    with open(path, "w") as f:
+        for name, arr in arrays:
+            arr = np.asarray(arr, dtype=np.float32)
+            f.write("static const float %s%s = {\n" % (name, "".join("[%d]" % d for d in arr.shape)))
+            for r in arr.reshape(-1, arr.shape[-1]):
+                row = ", ".join(_fmt(v) for v in r)
+                f.write("  {%s},\n" % row if arr.ndim > 1 else "  %s,\n" % row)
+            f.write("};\n\n")
+
+
+def save_reference_parameters(param_dir, cfg, w):
+    """Writes host weights `w` (layout of `llama.synth_weights(device=False)`) as a reference `parameters/` directory."""
+    os.makedirs(param_dir, exist_ok=True)
+    L = cfg["layers"]
+    for key, stem in _PROJ_FILES.items():
+        for l in range(L):
+            np.ascontiguousarray(w["w" + key][l], dtype=np.int8).tofile(os.path.join(param_dir, "%s_L%02d.bin" % (stem, l)))
+        s = np.stack([np.asarray(w["s" + key][l], dtype=np.float32) for l in range(L)])
+        sums = np.stack([np.asarray(w["w" + key][l], dtype=np.int64).sum(1).astype(np.float32) for l in range(L)])
+        _write_header(os.path.join(param_dir, "w_%s_s_sum.h" % stem), [("w_%s_s" % stem, s), ("w_%s_sum" % stem, sums)])
+    _write_header(os.path.join(param_dir, "w_rmsnorm.h"), [("RMSNorm_weight", w["gamma"])])
+    for key, (name, _) in _STATIC.items():
+        _write_header(os.path.join(param_dir, name + ".h"), [(name, w[key])])
+    embed = np.asarray(w["embed"])
+    embed = embed.view(np.float16) if embed.dtype == np.uint16 else embed
+    embed.astype(np.float32).tofile(os.path.join(param_dir, "model_embed_tokens_fp32.bin"))
