@@ -250,6 +250,23 @@ def main():
     modules = None
     if not args.no_modules:
         modules = module_legs(fx, lib, synth, ops, stream, Event)
+        if not args.no_prefill and cfg["max_pos"] >= 1024:
+            # HMT plug-in at the reference's segment sizes (990 tokens, summary 495, recurrent 32, 64 memory slots):
+            # one middle segment = stage 0 (512 rows) + retrieval + stage 1 (1024 rows) + memory update
+            from flexllm_amd import hmt
+            wq = synth.device_uniform_f32((H, H), 9401, -0.02, 0.02); wk = synth.device_uniform_f32((H, H), 9402, -0.02, 0.02)
+            t_emb = synth.device_uniform_f32((H,), 9403, -1.0, 1.0)
+            emb = synth.device_uniform_f32((3 * 990, H), 9404, -1.7, 1.7)
+            plug = hmt.Hmt(model, wq, wk, t_emb)
+            plug.run(emb, stream=stream); stream.sync()
+            h0, h1 = Event(), Event()
+            h0.record(stream)
+            plug.run(emb, stream=stream)
+            h1.record(stream); h1.sync()
+            ms = h0.elapsed_ms(h1)
+            modules["hmt_3_segments_of_990"] = {"ms": round(ms, 3), "prefill_passes": 5, "tokens_per_s": round(3 * 990 / ms * 1e3, 1),
+                                                "note": "segment loop incl. host sequencing: 3 stage-1 passes of 1024 rows and 2 stage-0 passes of 512 rows through the 16 layers"}
+            del plug, wq, wk, emb
 
     # ---- CPU baseline: the oracle (scalar C port of the reference modules), bounded sample --------------
     cpu = None

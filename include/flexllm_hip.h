@@ -312,6 +312,28 @@ int flexllm_llama_decode_sample(flexllm_llama* m, int* token_io, int pos0, int s
  * writes the residual stream to hidden_out (device [s][hidden], may be NULL). */
 int flexllm_llama_prefill_hidden(flexllm_llama* m, const float* x_in, int s, float* hidden_out, void* stream);
 
+/* ---- HMT long-context plug-in (Modules/HMT.h, HMT_SpinQuant_Llama_32_1B/HMT_SpinQuant_Unit.h) ----------------
+ * The plug-in runs the layer stack (flexllm_llama_prefill_hidden) twice per segment on assembled sequences and
+ * keeps a ring of memory embeddings; these entry points are its fp32 pieces.  All pointers are device pointers. */
+/* y[n] = sum_k w[n][k] * x[k] in fp32 (w row-major [n][k], k % 4 == 0).  dec_Linear_Layer_fp32xfp32
+ * (Modules/Linear_Layer.h:1041-1100), used for the query Q_n = Wq S_n and the key K_n = Wk M_n
+ * (Modules/HMT.h:289-292, :306-311). */
+int flexllm_linear_f32_gemv(const float* x, const float* w, float* y, int k, int n, void* stream);
+/* Memory retrieval: a[j] = q . kmem[j] over ALL mem_num slots (empty slots are zero rows and take part),
+ * a_sft = softmax((a - max) / scale), p_out[c] = sum_j a_sft[j] * mmem[j][c].  kmem, mmem: [mem_num][hidden].
+ * hmt_Linear_Layer_fp32xfp32_qk_attn_template (Modules/HMT.h:278-316) + hmt_attn_softmax with enable_scale,
+ * enable_sub_max (HMT_SpinQuant_Unit.h:96-105; Modules/Softmax.h:262-360).  mem_num <= 1024. */
+int flexllm_hmt_retrieve(const float* q, const float* kmem, const float* mmem, float* a_sft, float* p_out, int mem_num,
+                         int hidden, float scale, void* stream);
+/* Input sequence of one stage of hmt_segment_loader_sync_template (Modules/HMT.h:48-98 stage 0, :125-170 stage 1),
+ * written to x_out [rows][hidden], rows beyond the sequence zero:
+ *   stage 0: [t_embed, emb[seq_off .. seq_off+cur_sum_len), t_embed]
+ *   stage 1: [p_buf, emb[seq_off-rec_len .. seq_off) (zero rows before the text), emb[seq_off .. seq_off+cur_len),
+ *             p_buf if tail_p]
+ * emb: [seq_len][hidden] token embeddings. */
+int flexllm_hmt_stage_input(const float* emb, const float* t_embed, const float* p_buf, float* x_out, int stage, int seq_off,
+                            int cur_len, int cur_sum_len, int rec_len, int tail_p, int rows, int hidden, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

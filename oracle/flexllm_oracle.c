@@ -251,6 +251,53 @@ void fxo_softmax(const float* x, int rows, int dim, float* y) {
     for (int r = 0; r < rows; r++) softmax_row(x + (size_t)r * dim, dim, y + (size_t)r * dim);
 }
 
+/* dec_Softmax (Softmax.h:262-360), the vector form used outside attention: the dim inputs are block-partitioned over
+ * bp lanes (lane i holds elements i*dim/bp ... ), exp((x - max) / scale) when enable_scale (:313), partial sums per
+ * lane and per k % 4 (:316), lane sums (p0+p1)+(p2+p3) (:337-342), lanes added in order (:344-347), one reciprocal (:349). */
+void fxo_softmax_dec(const float* x, int dim, int bp, int enable_scale, float scale, float* y) {
+    float mx = (float)-1e32;                                              /* :287 */
+    for (int k = 0; k < dim; k++) mx = x[k] > mx ? x[k] : mx;             /* :297-305 */
+    const int per = dim / bp;
+    float total = 0.0f;
+    for (int i = 0; i < bp; i++) {
+        float p[4] = {0, 0, 0, 0};
+        for (int k = 0; k < per; k++) {
+            const float d = x[i * per + k] - mx;
+            const float t = enable_scale ? expf(d / scale) : expf(d);
+            y[i * per + k] = t;
+            p[k % 4] += t;
+        }
+        total += (p[0] + p[1]) + (p[2] + p[3]);
+    }
+    const float cd = 1.0f / total;
+    for (int k = 0; k < dim; k++) y[k] = y[k] * cd;                       /* :351-360 */
+}
+
+/* dec_Linear_Layer_fp32xfp32 (Linear_Layer.h:1041-1100) on PE_fp32xfp32_pack_1x2_1D (PE.h:709-752): y[n] = sum_k
+ * w[n][k] * x[k] in fp32 with four partial sums by k % 4 joined as (p0+p1)+(p2+p3) (tree_adder_4, PE.h:86-90). */
+void fxo_linear_f32(const float* x, const float* w, int k, int n, float* y) {
+    for (int r = 0; r < n; r++) {
+        float p[4] = {0, 0, 0, 0};
+        for (int i = 0; i < k; i++) p[i % 4] += x[i] * w[(size_t)r * k + i];
+        y[r] = (p[0] + p[1]) + (p[2] + p[3]);
+    }
+}
+
+/* Memory retrieval of the HMT plug-in (HMT.h:278-316, HMT_SpinQuant_Unit.h:96-105): scores a[j] = q . kmem[j] over ALL
+ * mem_num slots (empty slots hold zeros and take part), softmax((a - max) / scale) over the slots, p = sum_j a[j] *
+ * mmem[j] computed as a linear layer whose weight row c is column c of the memory matrix. */
+void fxo_hmt_retrieve(const float* q, const float* kmem, const float* mmem, int mem_num, int hidden, int bp,
+                      float scale, float* a_sft, float* p_out) {
+    float a[1024];
+    fxo_linear_f32(q, kmem, hidden, mem_num, a);
+    fxo_softmax_dec(a, mem_num, bp, 1, scale, a_sft);
+    for (int c = 0; c < hidden; c++) {
+        float p[4] = {0, 0, 0, 0};
+        for (int j = 0; j < mem_num; j++) p[j % 4] += a_sft[j] * mmem[(size_t)j * hidden + c];
+        p_out[c] = (p[0] + p[1]) + (p[2] + p[3]);
+    }
+}
+
 void fxo_causal_mask(const float* x, int rows, int heads, int dim, float* y) {
     for (int r = 0; r < rows; r++)
         for (int h = 0; h < heads; h++)

@@ -79,6 +79,13 @@ void fxo_residual(const float* a, const float* b, int n, float* y); /* Modules/R
 /* ---- Softmax.h / MHA.h ---------------------------------------------------- */
 /* Modules/Softmax.h:6-163 and :456-635 (non-versal, enable_sub_max, no scale); ragged dim allowed. */
 void fxo_softmax(const float* x, int rows, int dim, float* y);
+/* Softmax.h:262-360 dec_Softmax on a block-partitioned vector, optional division of the exponent by `scale` */
+void fxo_softmax_dec(const float* x, int dim, int bp, int enable_scale, float scale, float* y);
+/* Linear_Layer.h:1041-1100 + PE.h:709-752: fp32 GEMV, four partial sums by k % 4 */
+void fxo_linear_f32(const float* x, const float* w, int k, int n, float* y);
+/* HMT.h:278-316: scores over all memory slots, scaled softmax, weighted sum of the memories (mem_num <= 1024) */
+void fxo_hmt_retrieve(const float* q, const float* kmem, const float* mmem, int mem_num, int hidden, int bp,
+                      float scale, float* a_sft, float* p_out);
 /* Modules/MHA.h:246-273: y[q][k] = k<=q ? x : -1e32 ; x is [rows][heads][dim]. */
 void fxo_causal_mask(const float* x, int rows, int heads, int dim, float* y);
 

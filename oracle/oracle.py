@@ -180,6 +180,81 @@ def softmax(x):
     lib().fxo_softmax(_p(x), rows, dim, _p(y)); return y
 
 
+def softmax_dec(x, block_parallel=4, scale=None):
+    """dec_Softmax on one block-partitioned vector; `scale` divides the exponent (enable_scale)."""
+    x = _f32(x); y = np.empty(x.shape, np.float32)
+    lib().fxo_softmax_dec(_p(x), x.size, block_parallel, 0 if scale is None else 1, C.c_float(1.0 if scale is None else scale), _p(y))
+    return y
+
+
+def linear_f32(x, w):
+    """fp32 GEMV y = W x with the reference's four partial sums (dec_Linear_Layer_fp32xfp32)."""
+    x = _f32(x); w = _f32(w); n, k = w.shape
+    y = np.empty(n, np.float32)
+    lib().fxo_linear_f32(_p(x), _p(w), k, n, _p(y)); return y
+
+
+def hmt_retrieve(q, kmem, mmem, scale, block_parallel=4):
+    """(softmaxed scores over all memory slots, retrieved memory embedding P) for query q."""
+    q = _f32(q); kmem = _f32(kmem); mmem = _f32(mmem)
+    mem_num, hidden = mmem.shape
+    assert mem_num % block_parallel == 0 and mem_num <= 1024, "memory slots come in whole blocks"
+    a = np.empty(mem_num, np.float32); p_out = np.empty(hidden, np.float32)
+    lib().fxo_hmt_retrieve(_p(q), _p(kmem), _p(mmem), mem_num, hidden, block_parallel, C.c_float(scale), _p(a), _p(p_out))
+    return a, p_out
+
+
+def hmt_stage_lengths(seq_len, seg_id, seg_num, seg_len, sum_seg_len, rec_seg_len, pad):
+    """(current segment length, stage-0 length, stage-1 length), lengths padded up to a multiple of `pad`
+    (Modules/HMT.h:39-45)."""
+    cur = seg_len if seg_id < seg_num - 1 else seq_len - seg_id * seg_len
+    cur_sum = min(cur, sum_seg_len)
+    up = lambda n: (n + pad - 1) // pad * pad
+    return cur, up(1 + cur_sum + 1), up(1 + rec_seg_len + cur + 1)
+
+
+def hmt_run(backbone, emb, t_embed, wq, wk, seg_len, sum_seg_len, rec_seg_len, mem_num, scale, pad=8, block_parallel=4):
+    """The segment loop of the HMT plug-in (Modules/HMT.h:8-195 feeding :198-474) around `backbone`, a function
+    [S][hidden] -> [S][hidden] (the layer stack without the final norm).  `emb` holds the token embeddings, `t_embed`
+    the summary-prompt embedding stored ahead of them (HMT.h:10).  Returns (list of stage-1 hidden states of each
+    segment's own tokens, memory matrix, key matrix, list of retrieved embeddings P_n)."""
+    emb = _f32(emb); seq_len, hidden = emb.shape
+    seg_num = (seq_len + seg_len - 1) // seg_len
+    mmem = np.zeros((mem_num, hidden), np.float32)                 # HMT.h:369-378, :428-437: caches start at zero
+    kmem = np.zeros((mem_num, hidden), np.float32)
+    p_buf = np.zeros(hidden, np.float32)                           # HMT.h:29-35
+    outs, ps = [], []
+    for seg in range(seg_num):
+        cur, len0, len1 = hmt_stage_lengths(seq_len, seg, seg_num, seg_len, sum_seg_len, rec_seg_len, pad)
+        cur_sum = min(cur, sum_seg_len)
+        off = seg * seg_len
+        if seg > 0:                                                # stage 0: [T, first cur_sum tokens, T] (HMT.h:48-98)
+            x0 = np.zeros((len0, hidden), np.float32)
+            x0[0] = t_embed
+            x0[1:1 + cur_sum] = emb[off:off + cur_sum]
+            x0[1 + cur_sum] = t_embed
+            s_n = backbone(x0)[1 + cur_sum]                        # HMT.h:101-105
+            q_n = linear_f32(s_n, wq)                              # HMT.h:289-292
+            _, p_buf = hmt_retrieve(q_n, kmem, mmem, scale, block_parallel)     # HMT.h:294-302
+            ps.append(p_buf.copy())
+        x1 = np.zeros((len1, hidden), np.float32)                  # stage 1 (HMT.h:125-170)
+        x1[0] = p_buf
+        for j in range(rec_seg_len):                               # the tokens just before the segment, zeros before the text
+            src = off - rec_seg_len + j
+            if src >= 0:
+                x1[1 + j] = emb[src]
+        x1[1 + rec_seg_len:1 + rec_seg_len + cur] = emb[off:off + cur]
+        if seg < seg_num - 1:
+            x1[1 + rec_seg_len + cur] = p_buf
+        h1 = backbone(x1)
+        outs.append(h1[1 + rec_seg_len:1 + rec_seg_len + cur].copy())
+        if seg < seg_num - 1:                                      # HMT.h:176-190, :397-406, :456-472
+            m_n = h1[1 + rec_seg_len + cur]
+            mmem[seg % mem_num] = m_n
+            kmem[seg % mem_num] = linear_f32(m_n, wk)              # HMT.h:306-311
+    return outs, mmem, kmem, ps
+
+
 def causal_mask(x):
     x = _f32(x)
     rows, heads, dim = x.shape

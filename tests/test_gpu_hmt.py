@@ -1,0 +1,96 @@
+"""HMT plug-in: its fp32 pieces against the oracle, and the whole segment loop around the GPU prefill against the
+oracle's segment loop around the oracle's prefill (one layer, real hidden sizes, short segments)."""
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+rng = np.random.default_rng(77)
+
+
+@pytest.fixture(scope="module")
+def fx():
+    import flexllm_amd as fx
+    fx.lib()
+    return fx
+
+
+def test_linear_f32_gemv_and_retrieve_vs_oracle(fx, oracle):
+    from flexllm_amd import hmt
+    hidden, mem_num = 2048, 64
+    x = rng.standard_normal(hidden).astype(np.float32)
+    w = (rng.standard_normal((hidden, hidden)) / 45).astype(np.float32)
+    y = hmt.linear_f32_gemv(fx.to_device(x), fx.to_device(w)).numpy()
+    ref = oracle.linear_f32(x, w)
+    np.testing.assert_allclose(y, ref, rtol=0, atol=2e-5 * np.abs(ref).max())          # fp32 sums, different association
+    kmem = np.zeros((mem_num, hidden), np.float32); mmem = np.zeros((mem_num, hidden), np.float32)
+    kmem[:9] = rng.standard_normal((9, hidden)); mmem[:9] = rng.standard_normal((9, hidden)) * 3     # 55 empty slots
+    q = rng.standard_normal(hidden).astype(np.float32)
+    scale = float(np.sqrt(hidden))
+    a, p = hmt.hmt_retrieve(fx.to_device(q), fx.to_device(kmem), fx.to_device(mmem), scale)
+    a_ref, p_ref = oracle.hmt_retrieve(q, kmem, mmem, scale)
+    np.testing.assert_allclose(a.numpy(), a_ref, rtol=1e-4)
+    np.testing.assert_allclose(p.numpy(), p_ref, rtol=0, atol=1e-4 * np.abs(p_ref).max())
+    assert abs(float(a.numpy().sum()) - 1.0) < 1e-5 and a.numpy()[9:].min() > 0          # empty slots keep their share
+
+
+def test_stage_inputs_are_the_oracles_sequences_bit_for_bit(fx, oracle):
+    from flexllm_amd import hmt
+    hidden, seg_len, sum_len, rec = 256, 10, 5, 3
+    emb = rng.standard_normal((34, hidden)).astype(np.float32)
+    t_embed = rng.standard_normal(hidden).astype(np.float32)
+    wq = (rng.standard_normal((hidden, hidden)) / 16).astype(np.float32)
+    seen = []
+
+    def backbone(x):
+        seen.append(x.copy())
+        return x + np.float32(1.0)
+
+    _, _, _, ps = oracle.hmt_run(backbone, emb, t_embed, wq, wq, seg_len, sum_len, rec, 4, 16.0, pad=32)
+    d_emb, d_t = fx.to_device(emb), fx.to_device(t_embed)
+    i = 0
+    for seg in range(4):
+        cur = 10 if seg < 3 else 4
+        p_prev = ps[seg - 2] if seg >= 2 else np.zeros(hidden, np.float32)
+        if seg > 0:
+            x0 = hmt.hmt_stage_input(d_emb, d_t, fx.to_device(p_prev), 0, seg * seg_len, cur, min(cur, sum_len), rec, False, 32)
+            assert np.array_equal(x0.numpy(), seen[i]); i += 1
+        p_now = ps[seg - 1] if seg >= 1 else np.zeros(hidden, np.float32)
+        x1 = hmt.hmt_stage_input(d_emb, d_t, fx.to_device(p_now), 1, seg * seg_len, cur, min(cur, sum_len), rec, seg < 3, 32)
+        assert np.array_equal(x1.numpy(), seen[i]); i += 1
+    assert i == len(seen) == 7
+
+
+def test_segment_loop_vs_oracle_on_the_real_layer_stack(fx, oracle):
+    from flexllm_amd import hmt, llama
+    cfg = llama.make_config(layers=1, vocab=512, max_pos=256)
+    host_w = llama.synth_weights(cfg, seed=5, device=False)
+    model = llama.Llama(cfg, llama.synth_weights(cfg, seed=5, device=True))
+    om = oracle.OracleModel(cfg, host_w)
+    hidden = cfg["hidden"]
+    seg_len, sum_len, rec, mem_num = 24, 12, 4, 4
+    emb = rng.standard_normal((60, hidden)).astype(np.float32)                 # segments of 24, 24, 12 tokens
+    t_embed = rng.standard_normal(hidden).astype(np.float32)
+    wq = (rng.standard_normal((hidden, hidden)) / 45).astype(np.float32)
+    wk = (rng.standard_normal((hidden, hidden)) / 45).astype(np.float32)
+    scale = float(np.sqrt(hidden))
+
+    def backbone(x):
+        kc, vc = om.new_caches()
+        print("oracle prefill of", x.shape[0], "rows", flush=True)
+        return om.prefill(x, kc, vc)
+
+    outs_ref, mmem_ref, kmem_ref, ps_ref = oracle.hmt_run(backbone, emb, t_embed, wq, wk, seg_len, sum_len, rec, mem_num, scale, pad=32)
+    plug = hmt.Hmt(model, fx.to_device(wq), fx.to_device(wk), fx.to_device(t_embed), seg_len, sum_len, rec, mem_num)
+    outs, ps = plug.run(fx.to_device(emb))
+    model.check()
+    assert len(outs) == 3 and len(ps) == 2
+    # same bound as the layer-graph tests: int8 rounding ties may flip a step, hidden states agree to 2e-3 of their scale
+    for o, r in zip(outs, outs_ref):
+        assert o.shape == r.shape
+        assert np.abs(o.numpy() - r).max() <= 2e-3 * np.abs(r).max()
+    for pn, r in zip(ps, ps_ref):
+        assert np.abs(pn.numpy() - r).max() <= 2e-3 * np.abs(r).max()
+    assert np.abs(plug.mmem.numpy() - mmem_ref).max() <= 2e-3 * np.abs(mmem_ref).max()
+    assert np.abs(plug.kmem.numpy() - kmem_ref).max() <= 2e-3 * np.abs(kmem_ref).max()
+    assert not plug.mmem.numpy()[2:].any() and plug.mmem.numpy()[:2].any()      # two memories stored, slots 2 and 3 empty
+    model.close()

@@ -324,3 +324,87 @@ def test_sample_topk_tie_order_is_the_insertion_order(oracle):
     tok, idx, val, prob = oracle.sample_topk(x, 3, 0.0, 4)
     assert list(idx) == [1, 9, 2] and np.all(val == 7.0)
     np.testing.assert_allclose(prob, [1 / 3] * 3, rtol=1e-6)
+
+
+# ------------------------------------------------------------------ HMT plug-in (Modules/HMT.h)
+def test_linear_f32_and_scaled_softmax_against_float64(oracle):
+    x = rng.standard_normal(2048).astype(np.float32)
+    w = rng.standard_normal((96, 2048)).astype(np.float32)
+    y = oracle.linear_f32(x, w)
+    ref = w.astype(np.float64) @ x.astype(np.float64)
+    np.testing.assert_allclose(y, ref, rtol=0, atol=2e-4)                  # ~45 * 2048 * 2^-24 worst-case growth
+    assert np.array_equal(oracle.linear_f32(np.ones(8, np.float32), np.arange(16, dtype=np.float32).reshape(2, 8)),
+                          np.array([28, 92], np.float32))                  # exact in any order
+    a = (rng.standard_normal(64) * 30).astype(np.float32)
+    p = oracle.softmax_dec(a, 4, scale=45.2548339959)
+    ref = scipy.special.softmax(a.astype(np.float64) / 45.2548339959)      # the scale divides the exponent
+    np.testing.assert_allclose(p, ref, rtol=2e-6)
+    assert abs(float(p.sum()) - 1.0) < 1e-6
+    p1 = oracle.softmax_dec(a, 4)                                          # without scale: plain softmax
+    np.testing.assert_allclose(p1, scipy.special.softmax(a.astype(np.float64)), rtol=2e-6, atol=1e-30)
+
+
+def test_hmt_retrieve_counts_empty_slots_and_is_a_convex_combination(oracle):
+    hidden, mem_num = 256, 8
+    mmem = np.zeros((mem_num, hidden), np.float32); kmem = np.zeros((mem_num, hidden), np.float32)
+    mmem[:3] = rng.standard_normal((3, hidden)); kmem[:3] = rng.standard_normal((3, hidden))
+    q = rng.standard_normal(hidden).astype(np.float32)
+    scale = 16.0
+    a, p = oracle.hmt_retrieve(q, kmem, mmem, scale)
+    s = kmem.astype(np.float64) @ q.astype(np.float64)                     # empty slots score exactly 0 and take part
+    ref_a = scipy.special.softmax(s / scale)
+    np.testing.assert_allclose(a, ref_a, rtol=1e-5)
+    np.testing.assert_allclose(p, ref_a @ mmem.astype(np.float64), rtol=0, atol=1e-5)
+    assert a[3:].min() > 0 and np.allclose(a[3:], a[3])                    # five empty slots share equal, non-zero weight
+    # a zero query weighs all slots equally: P is the mean over ALL slots, empty ones included
+    a0, p0 = oracle.hmt_retrieve(np.zeros(hidden, np.float32), kmem, mmem, scale)
+    assert np.allclose(a0, 1.0 / mem_num)
+    np.testing.assert_allclose(p0, mmem.sum(0) / mem_num, rtol=0, atol=1e-6)
+
+
+def test_hmt_stage_lengths_match_the_reference_comments(oracle):
+    # Modules/HMT.h:47 "1 + 495 + 1 = 497" and :125 "1 + 32 + 990 + 1 = 1024" for a full segment, before padding to
+    # the token-parallel factor (8): 497 -> 504, 1024 -> 1024
+    cur, l0, l1 = oracle.hmt_stage_lengths(3000, 1, 4, 990, 495, 32, 8)
+    assert (cur, l0, l1) == (990, 504, 1024)
+    cur, l0, l1 = oracle.hmt_stage_lengths(3000, 3, 4, 990, 495, 32, 8)    # last segment: 3000 - 3*990 = 30 tokens
+    assert (cur, l0, l1) == (30, 32, 64)
+
+
+def test_hmt_segment_flow_with_a_transparent_backbone(oracle):
+    """With the reference's own stand-in backbone (hmt_dummy_prefilling, Modules/HMT.h:494-521: x + 1) every quantity
+    of the segment loop has a closed form: S_n = T + 1, M_n = P_n + 1, slot = n % mem_num."""
+    hidden, seg_len, sum_len, rec, mem_num = 64, 10, 5, 3, 2
+    emb = rng.standard_normal((34, hidden)).astype(np.float32)             # 4 segments: 10, 10, 10, 4
+    t_embed = rng.standard_normal(hidden).astype(np.float32)
+    wq = (rng.standard_normal((hidden, hidden)) / 8).astype(np.float32)
+    wk = (rng.standard_normal((hidden, hidden)) / 8).astype(np.float32)
+    seen = []
+
+    def backbone(x):
+        seen.append(x.copy())
+        return x + np.float32(1.0)
+
+    outs, mmem, kmem, ps = oracle.hmt_run(backbone, emb, t_embed, wq, wk, seg_len, sum_len, rec, mem_num, 8.0, pad=4, block_parallel=2)
+    assert [o.shape[0] for o in outs] == [10, 10, 10, 4] and len(ps) == 3 and len(seen) == 7
+    for n, o in enumerate(outs):                                           # stage-1 rows of the segment's own tokens
+        assert np.array_equal(o, emb[n * seg_len:n * seg_len + o.shape[0]] + np.float32(1.0))
+    # stage-1 input of segment 0: zero P, zero recurrent rows (nothing precedes the text), tokens, zero P, zero padding
+    x1 = seen[0]
+    assert x1.shape[0] == 16 and not x1[0].any() and not x1[1:4].any() and np.array_equal(x1[4:14], emb[:10]) and not x1[14:].any()
+    # stage-0 input of segment 1: [T, first 5 tokens of the segment, T] padded to 8
+    x0 = seen[1]
+    assert x0.shape[0] == 8 and np.array_equal(x0[0], t_embed) and np.array_equal(x0[1:6], emb[10:15]) and np.array_equal(x0[6], t_embed) and not x0[7].any()
+    # stage-1 input of segment 1: P_1, the 3 tokens before the segment, the segment, P_1
+    x1 = seen[2]
+    assert np.array_equal(x1[0], ps[0]) and np.array_equal(x1[1:4], emb[7:10]) and np.array_equal(x1[4:14], emb[10:20]) and np.array_equal(x1[14], ps[0])
+    # last segment: no trailing P row
+    assert not seen[6][1 + rec + 4:].any()
+    # memories: M_0 = 0 + 1 went to slot 0, M_1 = P_1 + 1 to slot 1, M_2 = P_2 + 1 overwrote slot 0 (ring of 2)
+    assert np.array_equal(mmem[1], ps[0] + np.float32(1.0)) and np.array_equal(mmem[0], ps[1] + np.float32(1.0))
+    np.testing.assert_allclose(kmem[0], wk.astype(np.float64) @ mmem[0].astype(np.float64), rtol=0, atol=1e-5)
+    # P_1 from first principles in float64: only slot 0 is filled (ones), slot 1 empty
+    q1 = wq.astype(np.float64) @ (t_embed.astype(np.float64) + 1.0)
+    k0 = wk.astype(np.float64) @ np.ones(hidden)
+    wts = scipy.special.softmax(np.array([q1 @ k0, 0.0]) / 8.0)
+    np.testing.assert_allclose(ps[0], wts[0] * np.ones(hidden), rtol=0, atol=1e-5)
