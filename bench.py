@@ -114,21 +114,23 @@ def module_legs(fx, lib, synth, ops, stream, Event):
                       "mfma_frac": round(tot_ops / tot_us / 1e6 / INT8_PEAK_TOPS, 4)}
     out["prefill_linear_stack_M1024"] = stack
     del wq, wo, wg, wd
-    # (4) prefill attention, S = 1024, 32/8 heads, reading the int8 cache
-    S, QH, KVH = 1024, 32, 8
-    q8 = synth.device_i8((S, QH, 64), 9400)
-    kc, vc = ops.kv_cache(KVH, S)
-    lib.flexllm_rt_fill_i8(P(kc), C.c_size_t(kc.size), C.c_uint64(9401), -100, 100, stream.handle)
-    lib.flexllm_rt_fill_i8(P(vc), C.c_size_t(vc.size), C.c_uint64(9402), -100, 100, stream.handle)
+    # (4) prefill attention, S = 1024 and the maximum context 4096, 32/8 heads, reading the int8 cache
+    QH, KVH = 32, 8
     scl = ops.Scales(np.full(QH, 4e-3, np.float32), np.full(KVH, 0.03, np.float32), np.full(KVH, 0.03, np.float32), np.full(QH, 1.0 / 255, np.float32))
-    o = fx.empty((S, QH, 64), np.float32)
-    def leg4(i):
-        lib.flexllm_mha_i8_prefill(P(q8), P(kc), P(vc), scl.ref(), P(o), None, S, QH, KVH, 64, S, stream.handle)
-    us = _time(stream, Event, leg4, 20)
-    ops4 = 2 * 2 * QH * S * S * 64
-    out["attention_prefill_S1024"] = {"us": round(us, 2), "GOP_full_S2": round(ops4 / 1e9, 2), "TOPs_full_S2": round(ops4 / us / 1e6, 1),
-                                      "mfma_frac_full_S2": round(ops4 / us / 1e6 / INT8_PEAK_TOPS, 4),
-                                      "note": "causal half computed, scores twice (two-pass softmax); bound by exp/division per probability"}
+    for S in (1024, 4096):
+        q8 = synth.device_i8((S, QH, 64), 9400)
+        kc, vc = ops.kv_cache(KVH, S)
+        lib.flexllm_rt_fill_i8(P(kc), C.c_size_t(kc.size), C.c_uint64(9401), -100, 100, stream.handle)
+        lib.flexllm_rt_fill_i8(P(vc), C.c_size_t(vc.size), C.c_uint64(9402), -100, 100, stream.handle)
+        o = fx.empty((S, QH, 64), np.float32)
+        def leg4(i):
+            lib.flexllm_mha_i8_prefill(P(q8), P(kc), P(vc), scl.ref(), P(o), None, S, QH, KVH, 64, S, stream.handle)
+        us = _time(stream, Event, leg4, 20 if S == 1024 else 5)
+        ops4 = 2 * 2 * QH * S * S * 64
+        out["attention_prefill_S%d" % S] = {"us": round(us, 2), "GOP_full_S2": round(ops4 / 1e9, 2), "TOPs_full_S2": round(ops4 / us / 1e6, 1),
+                                            "mfma_frac_full_S2": round(ops4 / us / 1e6 / INT8_PEAK_TOPS, 4),
+                                            "note": "causal half computed, scores twice (two-pass softmax); bound by the exponential and rounding per probability"}
+        del q8, kc, vc, o
     return out
 
 
@@ -230,6 +232,7 @@ def main():
 
     # ---- prefill: 1024 synthetic tokens through the 16 layers ------------------------------------------
     prefill_ms = None
+    prefill_ms_4096 = None
     if not args.no_prefill:
         try:
             S = 1024
@@ -243,6 +246,16 @@ def main():
             p1.record(stream)
             p1.sync()
             prefill_ms = p0.elapsed_ms(p1) / 3
+            if cfg["max_pos"] >= 4096:                       # the maximum context in one pass
+                x4 = synth.device_uniform_f32((4096, H), 4244, -1.7, 1.7)
+                model.prefill_hidden(x4, stream=stream)
+                stream.sync()
+                p0.record(stream)
+                model.prefill_hidden(x4, stream=stream)
+                p1.record(stream)
+                p1.sync()
+                prefill_ms_4096 = p0.elapsed_ms(p1)
+                del x4
         except Exception as e:  # prefill path not available in this build
             print("prefill leg skipped: %s" % e, file=sys.stderr)
 
@@ -309,6 +322,7 @@ def main():
                    "hbm_frac": round(token_gbs / HBM_PEAK_GBS, 4), "event_ms_per_step": round(ev_ms / K, 5),
                    "last_tokens": out.numpy()[-4:].tolist()},
         "prefill_ms_1024": None if prefill_ms is None else round(prefill_ms, 3),
+        "prefill_ms_4096": None if prefill_ms_4096 is None else round(prefill_ms_4096, 3),
         # dominant kernel: the persistent decode kernel (all layers + lm_head + arg-max of every token of a
         # launch); algorithmic bytes per launch = bytes_per_token x tokens in the launch, duration from HIP
         # events around the timed launches (nothing else runs between them).  `traffic` is per launch too.

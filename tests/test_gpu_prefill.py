@@ -170,11 +170,12 @@ def test_mha_prefill_vs_oracle(fx, oracle, s, qh, kvh):
     assert np.all(np.abs(o.numpy().astype(np.float64) - ref["o"]) <= 1e-6 * np.abs(ref["o"]) + flips * tol + 1e-9)
 
 
-def test_mha_prefill_rows_equal_decode(fx):
-    """Size-independent property at full size (1024 tokens, 32/8 heads): prefill row i equals decode of query i
-    against the first i+1 cache positions, in the probability bytes and hence bit for bit in the output,
-    except where the two kernels' row sums differ in the last bit (reported as a one-step probability flip)."""
-    s, qh, kvh, hd = 1024, 32, 8, 64
+@pytest.mark.parametrize("s", [1024, 4096])
+def test_mha_prefill_rows_equal_decode(fx, s):
+    """Size-independent property at full size (1024 tokens and the maximum context 4096, 32/8 heads): prefill row i
+    equals decode of query i against the first i+1 cache positions, in the probability bytes and hence bit for bit in
+    the output, except where the two kernels' row sums differ in the last bit (a one-step probability flip)."""
+    qh, kvh, hd = 32, 8, 64
     q_s, k_s, v_s, a_s = mha_scales(qh, kvh)
     sc = fx.ops.Scales(q_s, k_s, v_s, a_s)
     q8 = rng.integers(-128, 128, (s, qh, hd)).astype(np.int8)
@@ -184,7 +185,7 @@ def test_mha_prefill_rows_equal_decode(fx):
     fx.ops.kv_store_i8(fx.to_device(k8), fx.to_device(v8), kc, vc, 0)
     o, _ = fx.ops.mha_i8_prefill(fx.to_device(q8), kc, vc, sc)
     oh = o.numpy()
-    for i in (0, 31, 32, 500, 1023):
+    for i in (0, 31, 32, 500, s - 1):
         od, _ = fx.ops.mha_i8_decode(fx.to_device(q8[i]), kc, vc, sc, i + 1)
         tol = (a_s * np.repeat(v_s, qh // kvh) * 128 * 2)[:, None]
         assert np.all(np.abs(od.numpy() - oh[i]) <= 1e-6 * np.abs(oh[i]) + tol)
