@@ -76,6 +76,7 @@ class Llama:
             setattr(w, n, C.cast(arr, C.c_void_p))
         for n in ("gamma", "q_s", "k_s", "v_s", "a_s", "rope_sin", "rope_cos", "embed"):
             setattr(w, n, weights[n].ptr)
+        self._gamma, self._embed = weights["gamma"], weights["embed"]
         h = C.c_void_p()
         check(lib().flexllm_llama_create(C.byref(h), C.byref(c), C.byref(w)))
         self.handle = h
@@ -101,6 +102,31 @@ class Llama:
         """Top-k sampling loop; rands: device float32 [steps] in [0,1)."""
         check(lib().flexllm_llama_decode_sample(self.handle, C.c_void_p(token_io.ptr), int(pos0), int(steps),
                                                 C.c_void_p(rands.ptr), int(top_k), C.c_void_p(tokens_out.ptr), _s(stream)))
+
+    def generate_int4_head(self, token, pos0, steps, rands, top_k, head, embed_f32=None):
+        """The reference's generation loop with its int4 output head and top-k sampling (SpinQuant_Decoding_mem_opt.h:
+        924-940, Modules/Logits.h:145-279), sequenced from the host: embedding -> layer stack -> final RMSNorm ->
+        `ops.lm_head_u4i4` -> `ops.sample_topk_f32` -> next token.  head = (w4, w_s, w_sum) device arrays
+        (nibble-packed int4 [vocab_pad][hidden/2], fp32 [vocab_pad] each); rands: host floats in [0,1), one per step;
+        embed_f32: optional device fp32 [vocab][hidden] table (the reference's embedding file), else the model's fp16
+        table.  Returns the sampled token ids (host list)."""
+        from . import ops
+        hidden = self.cfg["hidden"]
+        w4, w_s, w_sum = head
+        gamma_final = self._gamma.view(2 * self.cfg["layers"] * hidden * 4, (hidden,), np.float32)
+        out = []
+        tok = int(token)
+        for i in range(int(steps)):
+            if embed_f32 is not None:
+                x = embed_f32.view(tok * hidden * 4, (hidden,), np.float32)
+            else:
+                x = ops.embed_f16(self._embed, to_device(np.array([tok], np.int32)))
+            hid, _ = self.decode_hidden(x, pos0 + i, want_logits=False)
+            n_vec = ops.rmsnorm_f32(hid.view(0, (1, hidden)), gamma_final, eps=self.cfg["eps"])
+            logits = ops.lm_head_u4i4(n_vec.view(0, (hidden,)), w4, w_s, w_sum)
+            tok, _, _, _ = ops.sample_topk_f32(logits, top_k=top_k, rand=float(rands[i]))
+            out.append(tok)
+        return out
 
     def set_decode_mode(self, mode):
         """0: persistent one-kernel-per-token schedule (default), 1: one kernel per stage."""

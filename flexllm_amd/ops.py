@@ -151,6 +151,16 @@ def linear_u4i4_gemm_dequant(a4, s_x, b_x, w4, w_s, w_sum, residual=None, stream
 
 
 # ---------------------------------------------------------------- FHT.h
+def lm_head_u4i4(n_vec, w4, w_s, w_sum, stream=None):
+    """The reference's output head (SpinQuant_Decoding_mem_opt.h:363-365, config D6): the normalised hidden vector is
+    quantised to asymmetric uint4, multiplied with the int4 head weights (nibble-packed [vocab_pad][hidden/2]) and
+    dequantised with zero point x row sum.  Returns fp32 logits [vocab_pad]."""
+    hidden = n_vec.shape[-1]
+    q, s, b = quant_asym_u8(n_vec.view(0, (1, hidden)), bits=4, stream=stream)
+    a4 = pack_nibbles(q, stream=stream)
+    return linear_u4i4_gemv_dequant(a4.view(0, (hidden // 2,)), s, b, w4, w_s, w_sum, stream=stream)
+
+
 def fht_f32(x, scale=1.0, stream=None, out=None):
     y = out if out is not None else DeviceArray(x.shape, np.float32)
     check(lib().flexllm_fht_f32(_p(x), _p(y), _rows(x), x.shape[-1], C.c_float(scale), _s(stream)))

@@ -93,3 +93,61 @@ def test_w4a4_layer_like_the_reference_testbench(fx, oracle):
     gold = x_fq.astype(np.float64) @ w_deq.astype(np.float64).T
     big = np.abs(gold) > 1.0
     assert np.max(np.abs(y[big] - gold[big]) / np.abs(gold[big])) < 1e-2
+
+
+def test_int4_lm_head_at_the_padded_vocabulary(fx, oracle):
+    """The reference's output head: 131072 x 2048 int4 weights (vocabulary padded), asymmetric uint4 activation.
+    Logits bit-exact against the oracle chain (quant -> exact integer product -> dequant with zero point x row sum),
+    and the sampler on those logits picks the oracle's token."""
+    vocab_pad, hidden = 131072, 2048
+    r = np.random.default_rng(99)
+    n_vec = r.standard_normal(hidden).astype(np.float32)
+    q_w = r.integers(-8, 8, (vocab_pad, hidden)).astype(np.int8)
+    w_s = r.uniform(1e-3, 1e-2, vocab_pad).astype(np.float32)
+    w_sum = (q_w.sum(1, dtype=np.int64).astype(np.float32) * w_s).astype(np.float32)
+    w4 = fx.to_device(pack(q_w))
+    logits = fx.ops.lm_head_u4i4(fx.to_device(n_vec), w4, fx.to_device(w_s), fx.to_device(w_sum)).numpy()
+    q_ref, s_ref, b_ref = oracle.quant_asym(n_vec[None, :], bits=4)
+    acc = np.empty(vocab_pad, np.int32)
+    xq = q_ref[0].astype(np.float32)
+    for i in range(0, vocab_pad, 16384):                                  # fp32 BLAS is exact here (|sum| < 2^24)
+        acc[i:i + 16384] = (q_w[i:i + 16384].astype(np.float32) @ xq).astype(np.int32)
+    ref = oracle.dequant(acc[None, :], s_ref, w_s, b_x=b_ref, w_sum=w_sum)[0]
+    assert np.array_equal(logits, ref)
+    tok, idx, val, prob = fx.ops.sample_topk_f32(fx.to_device(logits), top_k=5, rand=0.37)
+    tok_ref, idx_ref, val_ref, prob_ref = oracle.sample_topk(ref, top_k=5, rand=0.37)
+    assert tok == tok_ref and np.array_equal(idx, idx_ref)
+
+
+def test_generation_loop_with_int4_head(fx, oracle):
+    """Host-sequenced generation (embedding -> layers -> final norm -> int4 head -> top-k sampling): first step against
+    the oracle chain to the layer-graph tolerance, the whole loop deterministic and in range."""
+    from flexllm_amd import llama
+    cfg = llama.make_config(layers=2, vocab=4096, max_pos=256)
+    host_w = llama.synth_weights(cfg, seed=21, device=False)
+    model = llama.Llama(cfg, llama.synth_weights(cfg, seed=21, device=True))
+    hidden, vocab_pad = cfg["hidden"], 8192
+    r = np.random.default_rng(5)
+    q_w = r.integers(-8, 8, (vocab_pad, hidden)).astype(np.int8)
+    w_s = r.uniform(1e-3, 1e-2, vocab_pad).astype(np.float32)
+    w_sum = (q_w.sum(1, dtype=np.int64).astype(np.float32) * w_s).astype(np.float32)
+    head = (fx.to_device(pack(q_w)), fx.to_device(w_s), fx.to_device(w_sum))
+    rands = [0.11, 0.52, 0.93, 0.30, 0.76, 0.05]
+    toks = model.generate_int4_head(77, 0, len(rands), rands, 5, head)
+    model.check()
+    assert len(toks) == len(rands) and all(0 <= t < vocab_pad for t in toks)
+    # oracle chain for the first step
+    om = oracle.OracleModel(cfg, host_w)
+    kc, vc = om.new_caches()
+    x = oracle.embed(host_w["embed"], 77)
+    hid_ref, _ = om.decode_token(x, 0, kc, vc, want_logits=False)
+    n_ref = oracle.rmsnorm_dec(hid_ref, host_w["gamma"][2 * cfg["layers"]])
+    q_ref, s_ref, b_ref = oracle.quant_asym(n_ref[None, :], bits=4)
+    acc = (q_w.astype(np.float32) @ q_ref[0].astype(np.float32)).astype(np.int32)
+    logits_ref = oracle.dequant(acc[None, :], s_ref, w_s, b_x=b_ref, w_sum=w_sum)[0]
+    tok_ref, idx_ref, _, prob_ref = oracle.sample_topk(logits_ref, top_k=5, rand=rands[0])
+    assert toks[0] in idx_ref.tolist()                                    # a 4-bit rounding tie may reorder near-equal candidates
+    # the loop is deterministic: a second model run from the same state gives the same ids
+    model2 = llama.Llama(cfg, llama.synth_weights(cfg, seed=21, device=True))
+    assert model2.generate_int4_head(77, 0, len(rands), rands, 5, head) == toks
+    model.close(); model2.close()
