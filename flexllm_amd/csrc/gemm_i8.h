@@ -188,15 +188,16 @@ __global__ __launch_bounds__(256) void gemm_i8_kernel(const int8_t* __restrict__
 }
 
 // ---------------------------------------------------------------------------------------------------------
-// Second kernel: tiles go global -> LDS by direct loads (global_load_lds_dwordx4), bypassing registers, three
-// stages deep.  Tile BM x BN x 64, 4 waves (2x2), wave tile (BM/2)x(BN/2); at 256x256 every fragment read from
-// LDS feeds four MFMAs, which halves the LDS traffic per operation of the 128x128 tile.
+// Second kernel: tiles go global -> LDS by direct loads (global_load_lds_dwordx4), bypassing registers, two to four
+// stages deep.  Tile BM x BN, BKB = 64 or 128 k-bytes per row and stage, four waves (2x2) or eight (2x4, or two
+// k-groups of 2x2); the wave tile is a grid of 32x32 MFMA tiles, and the wider it is the more MFMAs every fragment
+// read from LDS feeds (a 128x64 wave tile: six reads for eight MFMAs).
 //
-// LDS stage layout: row-major, 64 bytes (= four 16-byte k-chunks) per tile row.  A direct load writes lane i
-// at base + 16*i, i.e. four lanes per row, which is also the coalesced order in global memory.  To keep the
-// MFMA fragment reads (32 rows x one chunk) free of bank conflicts the chunks of a row are stored rotated:
-// slot s of row r holds k-chunk s ^ ((r >> 2) & 3).  The rotation is applied on the global side of the
-// direct load (the LDS side is fixed by the hardware).
+// LDS stage layout: row-major, BKB bytes (= BKB/16 16-byte k-chunks) per tile row.  A direct load writes lane i
+// at base + 16*i, i.e. 64/(BKB/16) rows per instruction, which is also the coalesced order in global memory.  To
+// keep the MFMA fragment reads (32 rows x one chunk) free of bank conflicts the chunks of a row are stored rotated:
+// slot s of row r holds k-chunk s ^ ((r >> 2) & 3) for 64-byte rows, s ^ ((r >> 1) & 7) for 128-byte rows.  The
+// rotation is applied on the global side of the direct load (the LDS side is fixed by the hardware).
 //
 // The loads are issued from inline assembly: the compiler does not track them, so the k-loop waits for them
 // with explicit counters (results return in issue order).
