@@ -126,3 +126,33 @@ def test_topk_sampling_loop_matches_oracle(small):
         ref.append(t)
     assert out.numpy().tolist() == ref
     assert int(tok.numpy()[0]) == ref[-1]
+
+
+@pytest.mark.parametrize("mode", [0, 1], ids=["persistent", "per_stage"])
+def test_decode_at_the_maximum_context(mode):
+    """The benchmark's situation checked against the oracle: context 4096 (all 32 key chunks of every KV head active),
+    caches pre-filled in cache layout, tokens decoded at positions 4030 (a chunk partly filled) and 4095 (the last)."""
+    import flexllm_amd as fx
+    from flexllm_amd import llama, synth
+    from oracle import oracle
+    cfg = llama.make_config(layers=2, vocab=1024, max_pos=4096)
+    host_w = llama.synth_weights(cfg, seed=9, device=False)
+    model = llama.Llama(cfg, llama.synth_weights(cfg, seed=9, device=True))
+    model.set_decode_mode(mode)
+    om = oracle.OracleModel(cfg, host_w)
+    for pos in (4030, 4095):
+        kc, vc = om.new_caches()
+        kc[:, :pos] = synth.host_i8((cfg["layers"], pos, cfg["kv_hidden"]), 177, -100, 100)
+        vc[:, :pos] = synth.host_i8((cfg["layers"], pos, cfg["kv_hidden"]), 178, -100, 100)
+        model.load_caches_token_major(kc, vc)
+        x = synth.host_normal_f32((cfg["hidden"],), 950 + pos)
+        print("decode at position", pos, flush=True)
+        hid, logits = model.decode_hidden(fx.to_device(x), pos, want_logits=True)
+        hid_ref, logits_ref = om.decode_token(x, pos, kc, vc)
+        assert np.abs(hid.numpy() - hid_ref).max() <= 2e-3 * np.abs(hid_ref).max()
+        assert np.abs(logits.numpy() - logits_ref).max() <= 2e-3 * np.abs(logits_ref).max()
+        k_gpu, v_gpu = model.caches_token_major()
+        close_int8(k_gpu[:, pos], kc[:, pos], "appended k row")
+        close_int8(v_gpu[:, pos], vc[:, pos], "appended v row")
+    model.check()
+    model.close()
