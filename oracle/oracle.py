@@ -204,6 +204,45 @@ def hmt_retrieve(q, kmem, mmem, scale, block_parallel=4):
     return a, p_out
 
 
+def w4a4_linear(x, w_q, w_s, w_sum, residual_in=None):
+    """One W4A4 linear of the reference: asymmetric uint4 quantisation per token, exact integer product, dequantisation
+    with zero point x row sum (quant.h:53-82, Linear_Layer.h i4 PEs, quant.h:147-152), optional residual."""
+    q, s, b = quant_asym(x, bits=4)
+    y = dequant(linear_i8(q, w_q), s, w_s, b_x=b, w_sum=w_sum)
+    return y if residual_in is None else residual(y, residual_in)
+
+
+def w4a4_layer(cfg, w, l, x, pos0, k_cache, v_cache):
+    """One decoder layer of the shipped W4A4 configuration on S tokens starting at pos0 (S > 1: prefill from 0; S == 1:
+    decode), stage order of SpinQuant_Prefilling.h:807-1050 / SpinQuant_Decoding_mem_opt.h:947-1128.  k_cache, v_cache:
+    int8 [max_pos][kv_hidden] of this layer, updated in place."""
+    S, H = x.shape
+    qh, kvh, hd = cfg["q_heads"], cfg["kv_heads"], cfg["head_dim"]
+    norm = rmsnorm_pref if S > 1 else (lambda t, g, eps: rmsnorm_dec(t[0], g, eps=eps)[None, :])
+    n = norm(x, w["gamma"][2 * l], cfg["eps"])
+    q = w4a4_linear(n, w["wq"][l], w["sq"][l], w["sumq"][l])
+    k = w4a4_linear(n, w["wk"][l], w["sk"][l], w["sumk"][l])
+    v = w4a4_linear(n, w["wv"][l], w["sv"][l], w["sumv"][l])
+    q = rope(q.reshape(S, qh, hd), w["rope_sin"], w["rope_cos"], pos0)
+    k = rope(k.reshape(S, kvh, hd), w["rope_sin"], w["rope_cos"], pos0)
+    if S > 1:
+        r = mha_prefill(q, k, v.reshape(S, kvh, hd), w["q_s"][l], w["k_s"][l], w["v_s"][l], w["a_s"][l])
+        k_cache[:S] = r["k8"].reshape(S, -1); v_cache[:S] = r["v8"].reshape(S, -1)
+        o = r["o"]
+    else:
+        q8 = static_quant(q, w["q_s"][l], factor=8.0)
+        k_cache[pos0] = static_quant(k, w["k_s"][l]).reshape(-1)
+        v_cache[pos0] = static_quant(v.reshape(1, kvh, hd), w["v_s"][l]).reshape(-1)
+        o, _ = mha_decode(q8[0], k_cache[:pos0 + 1].reshape(pos0 + 1, kvh, hd), v_cache[:pos0 + 1].reshape(pos0 + 1, kvh, hd),
+                          w["q_s"][l], w["k_s"][l], w["v_s"][l], w["a_s"][l])
+    x2 = w4a4_linear(o.reshape(S, H), w["wo"][l], w["so"][l], w["sumo"][l], residual_in=x)
+    n2 = norm(x2, w["gamma"][2 * l + 1], cfg["eps"])
+    g = w4a4_linear(n2, w["wg"][l], w["sg"][l], w["sumg"][l])
+    u = w4a4_linear(n2, w["wu"][l], w["su"][l], w["sumu"][l])
+    h = gate(u, swish(g))
+    return w4a4_linear(fht(h, cfg["fht_scale"]), w["wd"][l], w["sd"][l], w["sumd"][l], residual_in=x2)
+
+
 def hmt_stage_lengths(seq_len, seg_id, seg_num, seg_len, sum_seg_len, rec_seg_len, pad):
     """(current segment length, stage-0 length, stage-1 length), lengths padded up to a multiple of `pad`
     (Modules/HMT.h:39-45)."""
