@@ -194,8 +194,9 @@ __device__ __forceinline__ int quant_round(float x, float s) { return (int)round
 __device__ __forceinline__ bool quant_fast_ok(float s) { return s >= 0x1p-100f && s <= 0x1p100f; }
 __device__ __forceinline__ int quant_round_fast(float x, float rs, bool& near_tie) {
     const float q = x * rs;
-    near_tie |= fabsf(__builtin_amdgcn_fractf(fabsf(q)) - 0.5f) < 1e-4f;
-    return (int)(q + copysignf(0.5f, q));            // conversion truncates toward zero: round half away from zero
+    const float r = __builtin_rintf(q);              // nearest integer (ties to even: a tie is redone by the caller anyway)
+    near_tie |= fabsf(q - r) > 0.4999f;              // within 1e-4 of k + 0.5
+    return (int)r;
 }
 template <int N>
 __device__ __forceinline__ void quant_vector(const float (&v)[N], float s, int (&n)[N]) {
