@@ -640,7 +640,17 @@ __global__ __launch_bounds__(kMegaT, 1) void decode_mega_kernel(MegaParams p) {
                 if (lane < 8) L.hst[sw * 8 + (ridx >> 1)] = other * silu_f(mine);   // lanes 0..7 hold the (even) gate rows
             }
             __syncthreads();
-            if (t < 32) st_f(&p.h[wg * 32 + t], L.hst[t]);           // stored by a wave with no prefetch in flight
+            if (t < 64) {
+                // This workgroup's 32 values are the indices 32*wg .. 32*wg+31 of the 8192-vector: the first four stages
+                // of the transform (index bits 1..4, in that order) pair elements inside the block, so wave 0 does them
+                // here once instead of every workgroup doing them on the whole vector in phase 6.
+                float hv = L.hst[t & 31];
+                hv = lane_butterfly_s<2>(hv, lane_sign<2>(t));
+                hv = lane_butterfly_s<4>(hv, lane_sign<4>(t));
+                hv = lane_butterfly_s<8>(hv, lane_sign<8>(t));
+                hv = lane_butterfly_s<16>(hv, lane_sign<16>(t));
+                if (t < 32) st_f(&p.h[wg * 32 + t], hv);             // stored by a wave with no prefetch in flight
+            }
             stamp();
             bar.arrive(!is_s);
         }
@@ -653,7 +663,7 @@ __global__ __launch_bounds__(kMegaT, 1) void decode_mega_kernel(MegaParams p) {
             stamp();
             if (is_s && lane == 0) { xres[0] = ld_f(&p.x2[wg * 8 + sw * 2]); xres[1] = ld_f(&p.x2[wg * 8 + sw * 2 + 1]); }
             // 8192-point transform on all 512 threads, stage order bits 1,2,...,12,0 (bit-exact order, see
-            // fht_kernels.h).  A: i = j*2048 + t*4 + e   -> stage 1 in registers, 2..7 across lanes
+            // fht_kernels.h).  A: i = j*2048 + t*4 + e   -> stages 1..4 came done from phase 5, 5..7 across lanes
             //                  B: i = (t>>8)*4096 + r*256 + (t&255) -> stages 8..11 in registers
             //                  C: i = r*512 + t          -> stage 12 in registers, stage 0 across lanes
             float4 a[4];
@@ -661,11 +671,6 @@ __global__ __launch_bounds__(kMegaT, 1) void decode_mega_kernel(MegaParams p) {
             for (int j = 0; j < 4; j++) {
                 const float* src = p.h + j * 2048 + t * 4;
                 a[j] = make_float4(ld_f(src), ld_f(src + 1), ld_f(src + 2), ld_f(src + 3));
-            }
-#pragma unroll
-            for (int j = 0; j < 4; j++) {
-                const float u0 = a[j].x, v0 = a[j].z, u1 = a[j].y, v1 = a[j].w;
-                a[j].x = u0 + v0; a[j].z = u0 - v0; a[j].y = u1 + v1; a[j].w = u1 - v1;
             }
 #define FX_MEGA_STAGE(MASK)                                                                   \
     {                                                                                         \
@@ -677,10 +682,10 @@ __global__ __launch_bounds__(kMegaT, 1) void decode_mega_kernel(MegaParams p) {
             a[j].w = lane_butterfly_s<MASK>(a[j].w, sg);                                      \
         }                                                                                     \
     }
-            __builtin_amdgcn_s_waitcnt(0x0F70);               // vmcnt(0): the h loads, which stage 1 has consumed, are complete
+            __builtin_amdgcn_s_waitcnt(0x0F70);               // vmcnt(0): the h loads are complete
             if (is_s) mega_row_to_lds(w.wd, wg * 8 + sw * 2 + 1, lane, L.wd[sw * 2 + 1]);
             if (l == 1) fine();
-            FX_MEGA_STAGE(1) FX_MEGA_STAGE(2) FX_MEGA_STAGE(4) FX_MEGA_STAGE(8) FX_MEGA_STAGE(16) FX_MEGA_STAGE(32)
+            FX_MEGA_STAGE(8) FX_MEGA_STAGE(16) FX_MEGA_STAGE(32)
 #undef FX_MEGA_STAGE
             if (l == 1) fine();
 #pragma unroll
