@@ -61,7 +61,15 @@ static __global__ __launch_bounds__(256) void hmt_weighted_sum_kernel(const floa
     const int c = blockIdx.x * 256 + threadIdx.x;
     if (c >= hidden) return;
     float p[4] = {0.0f, 0.0f, 0.0f, 0.0f};
-    for (int j = 0; j < mem_num; j++) p[j & 3] += a_sft[j] * mmem[(size_t)j * hidden + c];
+    int j = 0;
+    for (; j + 8 <= mem_num; j += 8) {                       // eight loads in flight, summed in slot order
+        float m[8];
+#pragma unroll
+        for (int u = 0; u < 8; u++) m[u] = mmem[(size_t)(j + u) * hidden + c];
+#pragma unroll
+        for (int u = 0; u < 8; u++) p[u & 3] += a_sft[j + u] * m[u];
+    }
+    for (; j < mem_num; j++) p[j & 3] += a_sft[j] * mmem[(size_t)j * hidden + c];
     p_out[c] = (p[0] + p[1]) + (p[2] + p[3]);
 }
 
