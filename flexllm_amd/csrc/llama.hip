@@ -186,8 +186,11 @@ static int launch_mega(flexllm_llama* m, int* token, const float* x_in, float* l
                                    (int)sizeof(MegaLds)));
         lds_opted_in = true;
     }
-    decode_mega_kernel<<<kMegaWG, kMegaT, sizeof(MegaLds), st>>>(p);
-    FX_LAUNCH_CHECK();
+    // Cooperative launch: the runtime places all 256 workgroups at once or refuses the launch, which is what the
+    // kernel's grid barriers assume.
+    void* args[] = {&p};
+    FX_HIP(hipLaunchCooperativeKernel(reinterpret_cast<const void*>(decode_mega_kernel), dim3(kMegaWG), dim3(kMegaT), args,
+                                      (unsigned)sizeof(MegaLds), st));
     return FLEXLLM_OK;
 }
 
