@@ -186,11 +186,11 @@ static int launch_mega(flexllm_llama* m, int* token, const float* x_in, float* l
                                    (int)sizeof(MegaLds)));
         lds_opted_in = true;
     }
-    // Cooperative launch: the runtime places all 256 workgroups at once or refuses the launch, which is what the
-    // kernel's grid barriers assume.
-    void* args[] = {&p};
-    FX_HIP(hipLaunchCooperativeKernel(reinterpret_cast<const void*>(decode_mega_kernel), dim3(kMegaWG), dim3(kMegaT), args,
-                                      (unsigned)sizeof(MegaLds), st));
+    // An ordinary launch: one workgroup per CU fits by construction (mega_ok checks the CU count), and every barrier
+    // and poll in the kernel is bounded, so work of other streams that delays some workgroups costs time, not a hang.
+    // (A cooperative launch gives the same timing, but rocprofv3 of this ROCm release crashes at exit after one.)
+    decode_mega_kernel<<<kMegaWG, kMegaT, sizeof(MegaLds), st>>>(p);
+    FX_LAUNCH_CHECK();
     return FLEXLLM_OK;
 }
 
