@@ -33,7 +33,7 @@ __device__ __forceinline__ i32x16 zero16() {
 //
 // Work per query block grows linearly with its index (causal), and workgroups b, b+P, b+2P, ... (P = number of
 // CUs) end up resident on the same CU.  The (block, head) items are therefore taken in order of decreasing
-// length and dealt out in snake order (round 0 forwards, round 1 backwards, ...): every CU gets the same total.
+// length and dealt out in snake order (first deal forwards, second backwards, ...): every CU gets the same total.
 constexpr int kPfWaves = 4;        // waves per workgroup (8 measured slower: the kernel is bound by VALU throughput, not by the longest block)
 static __global__ __launch_bounds__(64 * kPfWaves) void pf_attention_kernel(const int8_t* __restrict__ q8, const int8_t* __restrict__ kc,
                                                                   const int8_t* __restrict__ vc, const float* __restrict__ q_s,

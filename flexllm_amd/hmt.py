@@ -26,10 +26,10 @@ def _p(a):
     return C.c_void_p(a.ptr) if a is not None else None
 
 
-def linear_f32_gemv(x, w, stream=None):
+def linear_f32_gemv(x, w, stream=None, out=None):
     """y = W x in fp32 (dec_Linear_Layer_fp32xfp32, Modules/Linear_Layer.h:1041-1100); w: [n][k]."""
     n, k = w.shape
-    y = DeviceArray((n,), np.float32)
+    y = out if out is not None else DeviceArray((n,), np.float32)
     check(lib().flexllm_linear_f32_gemv(_p(x), _p(w), _p(y), k, n, _s(stream)))
     return y
 
@@ -43,10 +43,10 @@ def hmt_retrieve(q, kmem, mmem, scale, stream=None):
     return a, p
 
 
-def hmt_stage_input(emb, t_embed, p_buf, stage, seq_off, cur_len, cur_sum_len, rec_len, tail_p, rows, stream=None):
+def hmt_stage_input(emb, t_embed, p_buf, stage, seq_off, cur_len, cur_sum_len, rec_len, tail_p, rows, stream=None, out=None):
     """Assembled input sequence [rows][hidden] of one stage (Modules/HMT.h:48-98, :125-170)."""
     hidden = emb.shape[1]
-    x = DeviceArray((rows, hidden), np.float32)
+    x = out if out is not None else DeviceArray((rows, hidden), np.float32)
     check(lib().flexllm_hmt_stage_input(_p(emb), _p(t_embed), _p(p_buf), _p(x), stage, seq_off, cur_len, cur_sum_len, rec_len,
                                         int(bool(tail_p)), rows, hidden, _s(stream)))
     return x
@@ -68,6 +68,12 @@ class Hmt:
         self.model, self.wq, self.wk, self.t_embed = model, wq, wk, t_embed
         self.seg_len, self.sum_seg_len, self.rec_seg_len, self.mem_num = seg_len, sum_seg_len, rec_seg_len, mem_num
         self.scale = float(scale) if scale is not None else math.sqrt(hidden)     # sqrt_HIDDEN_DIM (HMT_SpinQuant_Unit.h:103)
+        # Stage buffers live as long as the plug-in: freeing device memory waits for the device, which would stall
+        # the host between the stages of every segment.
+        self._x = DeviceArray((longest, hidden), np.float32)
+        self._h = DeviceArray((longest, hidden), np.float32)
+        self._q = DeviceArray((hidden,), np.float32)
+        self._k = DeviceArray((hidden,), np.float32)
         self.reset()
 
     def reset(self):
@@ -94,15 +100,18 @@ class Hmt:
             off = seg * self.seg_len
             last = seg == seg_num - 1
             if seg > 0:
-                x0 = hmt_stage_input(emb, self.t_embed, self.p_buf, 0, off, cur, cur_sum, self.rec_seg_len, False, up(1 + cur_sum + 1), stream)
-                h0 = self.model.prefill_hidden(x0, stream=stream)
-                q_n = linear_f32_gemv(self._row(h0, 1 + cur_sum), self.wq, stream)
+                rows0 = up(1 + cur_sum + 1)
+                x0 = hmt_stage_input(emb, self.t_embed, self.p_buf, 0, off, cur, cur_sum, self.rec_seg_len, False, rows0, stream,
+                                     out=self._x.view(0, (rows0, hidden)))
+                h0 = self.model.prefill_hidden(x0, stream=stream, out=self._h.view(0, (rows0, hidden)))
+                q_n = linear_f32_gemv(self._row(h0, 1 + cur_sum), self.wq, stream, out=self._q)
                 _, p_n = hmt_retrieve(q_n, self.kmem, self.mmem, self.scale, stream)
                 self.p_buf = p_n
                 ps.append(p_n)
-            x1 = hmt_stage_input(emb, self.t_embed, self.p_buf, 1, off, cur, cur_sum, self.rec_seg_len, not last,
-                                 up(1 + self.rec_seg_len + cur + 1), stream)
-            h1 = self.model.prefill_hidden(x1, stream=stream)
+            rows1 = up(1 + self.rec_seg_len + cur + 1)
+            x1 = hmt_stage_input(emb, self.t_embed, self.p_buf, 1, off, cur, cur_sum, self.rec_seg_len, not last, rows1, stream,
+                                 out=self._x.view(0, (rows1, hidden)))
+            h1 = self.model.prefill_hidden(x1, stream=stream, out=self._h.view(0, (rows1, hidden)))
             out = DeviceArray((cur, hidden), np.float32)
             check(copy(_p(out), C.c_void_p(h1.ptr + (1 + self.rec_seg_len) * hidden * 4), C.c_size_t(cur * hidden * 4), _s(stream)))
             outs.append(out)
@@ -110,6 +119,6 @@ class Hmt:
                 slot = seg % self.mem_num                                       # HMT.h:403, :465-466
                 m_row = self._row(h1, 1 + self.rec_seg_len + cur)
                 check(copy(C.c_void_p(self.mmem.ptr + slot * hidden * 4), _p(m_row), C.c_size_t(hidden * 4), _s(stream)))
-                k_n = linear_f32_gemv(m_row, self.wk, stream)
+                k_n = linear_f32_gemv(m_row, self.wk, stream, out=self._k)
                 check(copy(C.c_void_p(self.kmem.ptr + slot * hidden * 4), _p(k_n), C.c_size_t(hidden * 4), _s(stream)))
         return outs, ps

@@ -136,9 +136,11 @@ class Llama:
         """Synchronise and raise if the persistent decode kernel reported a barrier time-out."""
         check(lib().flexllm_llama_check(self.handle))
 
-    def prefill_hidden(self, x_in, stream=None):
+    def prefill_hidden(self, x_in, stream=None, out=None):
         s = x_in.shape[0]
-        hidden = DeviceArray((s, self.cfg["hidden"]), np.float32)
+        hidden = out if out is not None else DeviceArray((s, self.cfg["hidden"]), np.float32)
+        if hidden.shape != (s, self.cfg["hidden"]) or hidden.dtype != np.float32:
+            raise ValueError("out must be float32 [%d][%d]" % (s, self.cfg["hidden"]))
         check(lib().flexllm_llama_prefill_hidden(self.handle, C.c_void_p(x_in.ptr), s, C.c_void_p(hidden.ptr), _s(stream)))
         return hidden
 
