@@ -56,7 +56,8 @@ def _time(stream, Event, fn, reps):
 def module_legs(fx, lib, synth, ops, stream, Event):
     """Single-module timings on seeded synthetic inputs, weights cycled through rings larger than the 256 MB
     memory-side cache: (1) decode linear 2048x2048, (2) Hadamard + per-token quantisation of 1024 tokens,
-    (3) the prefill linear stack of one layer at M=1024, (4) prefill attention at S=1024."""
+    (3) the prefill linear stack of one layer at M=1024, (4) prefill attention at S=1024 and 4096, (5) the W4A4
+    linears (decode GEMV and prefill GEMM on nibble-packed operands)."""
     P = lambda a: C.c_void_p(a.ptr) if a is not None else None
     out = {}
     # (1) quantise -> GEMV -> dequant, 1 x 2048 against 2048 x 2048
@@ -129,8 +130,36 @@ def module_legs(fx, lib, synth, ops, stream, Event):
         ops4 = 2 * 2 * QH * S * S * 64
         out["attention_prefill_S%d" % S] = {"us": round(us, 2), "GOP_full_S2": round(ops4 / 1e9, 2), "TOPs_full_S2": round(ops4 / us / 1e6, 1),
                                             "mfma_frac_full_S2": round(ops4 / us / 1e6 / INT8_PEAK_TOPS, 4),
-                                            "note": "causal half computed, scores twice (two-pass softmax); bound by the exponential and rounding per probability"}
+                                            "note": ("causal half computed, scores kept in registers between the two softmax passes"
+                                                     if S <= 1024 else "causal half computed, scores twice (two-pass softmax)")
+                                                    + "; bound by the exponential and rounding per probability"}
         del q8, kc, vc, o
+    # (5) W4A4 linears (the reference's shipped precision): decode GEMV 2048 -> 8192 on nibble-packed weights
+    # (half the bytes of the int8 path) and the prefill GEMM at M = 1024
+    K, N = 2048, 8192
+    ring4 = [synth.device_i8((N, K // 2), 9500 + i) for i in range(48)]                  # 48 x 8.4 MB = 403 MB
+    x4 = synth.device_i8((K // 2,), 9550)
+    sx = fx.to_device(np.array([0.1], np.float32)); bx = fx.to_device(np.array([-0.7], np.float32))
+    w_s = synth.device_uniform_f32((N,), 9551, 1e-3, 1e-2); w_sum = synth.device_uniform_f32((N,), 9552, -1, 1)
+    y = fx.empty((N,), np.float32)
+    def leg5(i):
+        lib.flexllm_linear_u4i4_gemv_dequant(P(x4), P(sx), P(bx), P(ring4[i % len(ring4)]), P(w_s), P(w_sum), None, P(y), K, N, stream.handle)
+    us = _time(stream, Event, leg5, 96)
+    b5 = N * K // 2 + 8 * N + K // 2 + 4 * N
+    out["w4a4_linear_decode_2048x8192"] = {"bytes": b5, "us": round(us, 2), "GBs": round(b5 / us / 1e3, 1),
+                                           "hbm_frac": round(b5 / us / 1e3 / HBM_PEAK_GBS, 4)}
+    M = 1024
+    a4 = synth.device_i8((M, K // 2), 9560)
+    sxm = synth.device_uniform_f32((M,), 9561, 0.05, 0.1); bxm = synth.device_uniform_f32((M,), 9562, -1, 0)
+    ym = fx.empty((M, N), np.float32)
+    def leg5b(i):
+        lib.flexllm_linear_u4i4_gemm_dequant(P(a4), P(sxm), P(bxm), P(ring4[i % len(ring4)]), P(w_s), P(w_sum), None, P(ym), M, K, N, stream.handle)
+    us = _time(stream, Event, leg5b, 24)
+    ops5 = 2 * M * K * N
+    out["w4a4_linear_prefill_M1024_2048x8192"] = {"us": round(us, 2), "TOPs": round(ops5 / us / 1e6, 1),
+                                                  "mfma_frac": round(ops5 / us / 1e6 / INT8_PEAK_TOPS, 4),
+                                                  "note": "nibbles widened to int8 on the way to LDS, int8 MFMA (gfx950 has no int4 MFMA)"}
+    del ring4
     return out
 
 
@@ -280,6 +309,17 @@ def main():
             modules["hmt_3_segments_of_990"] = {"ms": round(ms, 3), "prefill_passes": 5, "tokens_per_s": round(3 * 990 / ms * 1e3, 1),
                                                 "note": "segment loop incl. host sequencing: 3 stage-1 passes of 1024 rows and 2 stage-0 passes of 512 rows through the 16 layers"}
             del plug, wq, wk, emb
+        # top-k sampling loop (the reference's own generation loop): one launch sequence per token, top_k = 5
+        n_s = 32
+        rands = fx.to_device(np.random.default_rng(7).random(n_s).astype(np.float32))
+        tok_s_io = fx.to_device(np.array([12345], np.int32)); out_s = fx.zeros((n_s,), np.int32)
+        model.decode_sample(tok_s_io, cfg["max_pos"] - 2 * n_s, n_s, rands, 5, out_s, stream=stream); stream.sync()
+        s0, s1 = Event(), Event()
+        s0.record(stream)
+        model.decode_sample(tok_s_io, cfg["max_pos"] - n_s, n_s, rands, 5, out_s, stream=stream)
+        s1.record(stream); s1.sync()
+        ms = s0.elapsed_ms(s1)
+        modules["decode_top5_sampling_ctx4096"] = {"ms_per_token": round(ms / n_s, 4), "tokens_per_s": round(n_s / ms * 1e3, 1), "steps": n_s}
 
     # ---- CPU baseline: the oracle (scalar C port of the reference modules), bounded sample --------------
     cpu = None

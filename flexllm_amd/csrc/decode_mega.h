@@ -74,6 +74,16 @@ struct MegaParams {
 };
 
 __device__ __forceinline__ float ld_f(const float* p) { return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
+// Two / four consecutive floats with 64-bit coherent loads (p 8-byte aligned): half the vector-memory instructions
+// of single loads, and the lanes of a wave cover whole cache lines.
+__device__ __forceinline__ float2 ld_f2(const float* p) {
+    const unsigned long long w = __hip_atomic_load(reinterpret_cast<const unsigned long long*>(p), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    return make_float2(__int_as_float((int)(unsigned)w), __int_as_float((int)(unsigned)(w >> 32)));
+}
+__device__ __forceinline__ void ld_f4(const float* p, float* v) {
+    const float2 a = ld_f2(p), b = ld_f2(p + 2);
+    v[0] = a.x; v[1] = a.y; v[2] = b.x; v[3] = b.y;
+}
 __device__ __forceinline__ void st_f(float* p, float v) { __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
 __device__ __forceinline__ int ld_i(const int* p) { return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
 __device__ __forceinline__ void st_i(int* p, int v) { __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
@@ -372,8 +382,7 @@ __global__ __launch_bounds__(kMegaT, 1) void decode_mega_kernel(MegaParams p) {
                     for (int i = 0; i < 4; i++) v[i] = __half2float(p.embed[(size_t)tok * H + 4 * t + i]);
                 }
             } else {
-#pragma unroll
-                for (int i = 0; i < 4; i++) v[i] = ld_f(&p.x[4 * t + i]);
+                ld_f4(&p.x[4 * t], v);
             }
             const float sx = norm_quant_2048(v, gam, true, p.eps, L, [&]() { gu_slice(0); });
             if (!is_s) {
@@ -555,7 +564,11 @@ __global__ __launch_bounds__(kMegaT, 1) void decode_mega_kernel(MegaParams p) {
             // the stream waves' previous slice has landed long ago, so they can share the activation loads
             float v[4], xr[2] = {0.0f, 0.0f};
 #pragma unroll
-            for (int i = 0; i < 4; i++) v[i] = (float)ld_i(&p.o_acc[4 * t + i]) * osa * osv;
+            for (int i = 0; i < 2; i++) {
+                const unsigned long long w2 = ld_u64(reinterpret_cast<const unsigned long long*>(p.o_acc + 4 * t + 2 * i));
+                v[2 * i] = (float)(int)(unsigned)w2 * osa * osv;
+                v[2 * i + 1] = (float)(int)(unsigned)(w2 >> 32) * osa * osv;
+            }
             if (!is_s && lane == 0) {                                 // residual inputs, fetched with the activations
 #pragma unroll
                 for (int j = 0; j < 2; j++) {
@@ -588,8 +601,7 @@ __global__ __launch_bounds__(kMegaT, 1) void decode_mega_kernel(MegaParams p) {
             stamp();
             if (t < 8) st_i(&p.o_acc[wg * 8 + t], 0);                // every reader of o_acc has passed the barrier
             float v[4];
-#pragma unroll
-            for (int i = 0; i < 4; i++) v[i] = ld_f(&p.x2[4 * t + i]);
+            ld_f4(&p.x2[4 * t], v);
             const float sx = norm_quant_2048(v, gam, true, p.eps, L, [&]() {
                 __builtin_amdgcn_s_waitcnt(0x0F70);                   // vmcnt(0): see gu_slice
                 if (is_s) mega_row_to_lds(w.wd, wg * 8 + sw * 2, lane, L.wd[sw * 2]);
@@ -669,8 +681,8 @@ __global__ __launch_bounds__(kMegaT, 1) void decode_mega_kernel(MegaParams p) {
             float4 a[4];
 #pragma unroll
             for (int j = 0; j < 4; j++) {
-                const float* src = p.h + j * 2048 + t * 4;
-                a[j] = make_float4(ld_f(src), ld_f(src + 1), ld_f(src + 2), ld_f(src + 3));
+                const float2 lo = ld_f2(p.h + j * 2048 + t * 4), hi = ld_f2(p.h + j * 2048 + t * 4 + 2);
+                a[j] = make_float4(lo.x, lo.y, hi.x, hi.y);
             }
 #define FX_MEGA_STAGE(MASK)                                                                   \
     {                                                                                         \
@@ -792,8 +804,7 @@ __global__ __launch_bounds__(kMegaT, 1) void decode_mega_kernel(MegaParams p) {
         bar.wait();
         stamp();
         float v[4];
-#pragma unroll
-        for (int i = 0; i < 4; i++) v[i] = ld_f(&p.x[4 * t + i]);
+        ld_f4(&p.x[4 * t], v);
         float ss = (v[0] * v[0] + v[1] * v[1]) + (v[2] * v[2] + v[3] * v[3]);
         ss = block_sum<kMegaWaves>(ss, L.red);
         const float rms = 1.0f / sqrtf(ss / 2048.0f + p.eps);
