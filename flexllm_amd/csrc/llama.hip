@@ -35,6 +35,8 @@ struct flexllm_llama {
     int* state = nullptr;           // [0] position of the token being processed, [1] step index
     float* am_v = nullptr;
     int* am_i = nullptr;
+    float* topk_val = nullptr;      // sampler: per-workgroup candidates of the first selection stage
+    int* topk_idx = nullptr;
     hipGraphExec_t graph_exec = nullptr;
     int* graph_token_io = nullptr;
     int* graph_tokens_out = nullptr;
@@ -308,6 +310,8 @@ int flexllm_llama_create(flexllm_llama** out, const flexllm_llama_config* cfg, c
     FX_TRY_HIP(hipMemset(m->stats_tag, 0xFF, sizeof(unsigned long long) * 2 * (size_t)c.q_heads * kMaxChunks));
     FX_TRY(dev_alloc(m, (void**)&m->state, sizeof(int) * 4));
     FX_TRY(dev_alloc(m, (void**)&m->am_v, sizeof(float) * kArgmaxParts));
+    FX_TRY(dev_alloc(m, (void**)&m->topk_val, sizeof(float) * kTopKParts * kTopKMax));
+    FX_TRY(dev_alloc(m, (void**)&m->topk_idx, sizeof(int) * kTopKParts * kTopKMax));
     FX_TRY(dev_alloc(m, (void**)&m->am_i, sizeof(int) * kArgmaxParts));
     FX_TRY(dev_alloc(m, (void**)&m->layers_dev, sizeof(LayerW) * L));
     FX_TRY_HIP(hipMemcpy(m->layers_dev, m->layers.data(), sizeof(LayerW) * L, hipMemcpyHostToDevice));
@@ -476,7 +480,9 @@ int flexllm_llama_decode_sample(flexllm_llama* m, int* token_io, int pos0, int s
                 if ((rc = decode_layer(m, l, st))) return rc;
             if ((rc = decode_head(m, m->logits, st))) return rc;
         }
-        topk_sample_kernel<<<1, kTopKThreads, 0, st>>>(m->logits, c.vocab, top_k, rands, 1, 1, out);
+        // two stages: 128 workgroups pick the top_k of their share of the vocabulary, one workgroup picks among those
+        topk_partial_kernel<<<kTopKParts, kTopKPartThreads, 0, st>>>(m->logits, c.vocab, top_k, m->topk_val, m->topk_idx);
+        topk_sample_kernel<<<1, kTopKThreads, 0, st>>>(m->topk_val, m->topk_idx, kTopKParts * top_k, top_k, rands, 1, 1, out);
         FX_LAUNCH_CHECK();
     }
     return FLEXLLM_OK;

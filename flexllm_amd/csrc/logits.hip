@@ -33,7 +33,16 @@ int flexllm_sample_topk_f32(const float* logits, int n, int top_k, const float* 
     FX_REQUIRE(logits && rand && token, "sample_topk: null pointer");
     FX_REQUIRE(n > 0 && top_k >= 1 && top_k <= kTopKMax && top_k <= n, "sample_topk: n=%d top_k=%d (1..%d)", n, top_k, kTopKMax);
     TopKOut out = {token, top_idx, top_val, top_prob, nullptr, nullptr, nullptr};
-    topk_sample_kernel<<<1, kTopKThreads, 0, as_stream(stream)>>>(logits, n, top_k, rand, 0, enable_sub_max, out);
+    if (n >= 4096) {
+        if (!g_tv) {
+            FX_HIP(hipMalloc(&g_tv, kTopKParts * kTopKMax * sizeof(float)));
+            FX_HIP(hipMalloc(&g_ti, kTopKParts * kTopKMax * sizeof(int)));
+        }
+        topk_partial_kernel<<<kTopKParts, kTopKPartThreads, 0, as_stream(stream)>>>(logits, n, top_k, g_tv, g_ti);
+        topk_sample_kernel<<<1, kTopKThreads, 0, as_stream(stream)>>>(g_tv, g_ti, kTopKParts * top_k, top_k, rand, 0, enable_sub_max, out);
+    } else {
+        topk_sample_kernel<<<1, kTopKThreads, 0, as_stream(stream)>>>(logits, nullptr, n, top_k, rand, 0, enable_sub_max, out);
+    }
     FX_LAUNCH_CHECK();
     return FLEXLLM_OK;
 }

@@ -93,9 +93,11 @@ static __global__ __launch_bounds__(64) void argmax_final_kernel(const float* __
 }
 
 // ---- top-k sampling (Modules/Logits.h:145-279) ------------------------------------------------------------
-// One workgroup of 1024 threads.  Each thread keeps the k best (value, index) of its strided share, ordered by
-// value descending then index ascending; k rounds of a block-wide arg-max over the threads' current heads pop the
-// global top-k in that order.  Thread 0 then does what the reference does with the k candidates: softmax with
+// Each thread keeps the k best (value, index) of its share, ordered by value descending then index ascending; k
+// rounds of a block-wide arg-max over the threads' current heads pop the top-k in that order.  Long rows go through
+// two stages (128 workgroups over contiguous shares of the row, then one workgroup over their candidates: 12 us
+// for 128256 logits where a single workgroup needs 230 us), short rows through the last stage alone.
+// Thread 0 then does what the reference does with the k candidates: softmax with
 // two partial sums (exp(v_k - v_0)), cumulative distribution, first k with rand < cdf[k] (else the last one).
 // The reference orders EQUAL logits by its lane scan order instead of by index; the candidates' values, hence the
 // probabilities, are the same either way, only which of two equal logits is reported can differ.
@@ -105,31 +107,15 @@ struct TopKOut { int* token; int* top_idx; float* top_val; float* top_prob; int*
 
 __device__ __forceinline__ bool topk_better(float v, int i, float bv, int bi) { return v > bv || (v == bv && i < bi); }
 
-static __global__ __launch_bounds__(kTopKThreads) void topk_sample_kernel(const float* __restrict__ logits, int n, int top_k,
-                                                                         const float* __restrict__ rand_ptr, int rand_index_from_state,
-                                                                         int enable_sub_max, TopKOut out) {
-    __shared__ float s_val[kTopKThreads / 64];
-    __shared__ int s_idx[kTopKThreads / 64], s_own[kTopKThreads / 64];
-    __shared__ float f_val[kTopKMax];
-    __shared__ int f_idx[kTopKMax];
+// Block-wide selection: every thread holds a list sorted by (value descending, index ascending); top_k rounds of an
+// arg-max over the threads' current heads pop the block's top_k in that order into f_val / f_idx (shared memory).
+template <int THREADS>
+__device__ __forceinline__ void topk_block_select(const float (&val)[kTopKMax], const int (&idx)[kTopKMax], int top_k,
+                                                  float* f_val, int* f_idx) {
+    __shared__ float s_val[THREADS / 64];
+    __shared__ int s_idx[THREADS / 64], s_own[THREADS / 64];
     __shared__ int s_winner;
     const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
-    float val[kTopKMax];
-    int idx[kTopKMax];
-#pragma unroll
-    for (int k = 0; k < kTopKMax; k++) { val[k] = -1e32f; idx[k] = 0x7fffffff; }
-    for (int i = t; i < n; i += kTopKThreads) {
-        // insertion into the sorted list (k is small; statically indexed so that the lists stay in registers)
-        float cv = logits[i];
-        int ci = i;
-#pragma unroll
-        for (int k = 0; k < kTopKMax; k++) {
-            if (k < top_k && topk_better(cv, ci, val[k], idx[k])) {
-                const float tv = val[k]; const int ti = idx[k];
-                val[k] = cv; idx[k] = ci; cv = tv; ci = ti;
-            }
-        }
-    }
     int head = 0;                                   // this thread's best not yet taken
     for (int r = 0; r < top_k; r++) {
         float bv = -1e32f; int bi = 0x7fffffff, bo = t;
@@ -145,14 +131,65 @@ static __global__ __launch_bounds__(kTopKThreads) void topk_sample_kernel(const 
         __syncthreads();
         if (t == 0) {
             float wv = s_val[0]; int wi = s_idx[0], wo = s_own[0];
-            for (int w = 1; w < kTopKThreads / 64; w++)
+            for (int w = 1; w < THREADS / 64; w++)
                 if (topk_better(s_val[w], s_idx[w], wv, wi) || (s_val[w] == wv && s_idx[w] == wi && s_own[w] < wo)) { wv = s_val[w]; wi = s_idx[w]; wo = s_own[w]; }
-            f_val[r] = wv; f_idx[r] = wi == 0x7fffffff ? -1 : wi; s_winner = wo;
+            f_val[r] = wv; f_idx[r] = wi; s_winner = wo;
         }
         __syncthreads();
         if (t == s_winner) head++;
         __syncthreads();
     }
+}
+
+// Sorted insertion of one candidate (k is small; statically indexed so that the lists stay in registers).
+__device__ __forceinline__ void topk_insert(float (&val)[kTopKMax], int (&idx)[kTopKMax], int top_k, float cv, int ci) {
+#pragma unroll
+    for (int k = 0; k < kTopKMax; k++) {
+        if (k < top_k && topk_better(cv, ci, val[k], idx[k])) {
+            const float tv = val[k]; const int ti = idx[k];
+            val[k] = cv; idx[k] = ci; cv = tv; ci = ti;
+        }
+    }
+}
+
+// First stage for long rows: workgroup g selects the top_k of its contiguous share of the logits and writes them,
+// in order, to cand_val / cand_idx [g * top_k ...]; unused places carry the sentinel (-1e32, 0x7fffffff).  The global
+// top_k is a subset of the union, and the second stage (topk_sample_kernel with in_idx) orders it the same way.
+constexpr int kTopKParts = 128;
+constexpr int kTopKPartThreads = 256;
+static __global__ __launch_bounds__(kTopKPartThreads) void topk_partial_kernel(const float* __restrict__ logits, int n, int top_k,
+                                                                              float* __restrict__ cand_val, int* __restrict__ cand_idx) {
+    __shared__ float f_val[kTopKMax];
+    __shared__ int f_idx[kTopKMax];
+    const int chunk = (n + gridDim.x - 1) / gridDim.x;
+    const int begin = blockIdx.x * chunk, end = min(n, begin + chunk);
+    float val[kTopKMax];
+    int idx[kTopKMax];
+#pragma unroll
+    for (int k = 0; k < kTopKMax; k++) { val[k] = -1e32f; idx[k] = 0x7fffffff; }
+    for (int i = begin + threadIdx.x; i < end; i += kTopKPartThreads) topk_insert(val, idx, top_k, logits[i], i);
+    topk_block_select<kTopKPartThreads>(val, idx, top_k, f_val, f_idx);
+    if (threadIdx.x < top_k) {
+        cand_val[blockIdx.x * top_k + threadIdx.x] = f_val[threadIdx.x];
+        cand_idx[blockIdx.x * top_k + threadIdx.x] = f_idx[threadIdx.x];
+    }
+}
+
+// in_idx == NULL: logits[i] is the logit of token i.  Otherwise (second stage) logits / in_idx are n candidates.
+static __global__ __launch_bounds__(kTopKThreads) void topk_sample_kernel(const float* __restrict__ logits, const int* __restrict__ in_idx,
+                                                                         int n, int top_k, const float* __restrict__ rand_ptr,
+                                                                         int rand_index_from_state, int enable_sub_max, TopKOut out) {
+    __shared__ float f_val[kTopKMax];
+    __shared__ int f_idx[kTopKMax];
+    const int t = threadIdx.x;
+    float val[kTopKMax];
+    int idx[kTopKMax];
+#pragma unroll
+    for (int k = 0; k < kTopKMax; k++) { val[k] = -1e32f; idx[k] = 0x7fffffff; }
+    for (int i = t; i < n; i += kTopKThreads) topk_insert(val, idx, top_k, logits[i], in_idx ? in_idx[i] : i);
+    topk_block_select<kTopKThreads>(val, idx, top_k, f_val, f_idx);
+    if (t < top_k && f_idx[t] == 0x7fffffff) f_idx[t] = -1;
+    __syncthreads();
     if (t == 0) {
         float prob[kTopKMax], cdf[kTopKMax];
         float sum_partial[2] = {0.0f, 0.0f};
@@ -186,8 +223,12 @@ static __global__ __launch_bounds__(kTopKThreads) void topk_sample_kernel(const 
 }
 
 constexpr int kArgmaxParts = 256;
+// Process-wide candidate buffers of the stand-alone arg-max and sampling entry points (allocated on first use;
+// calls that overlap on different streams would share them, a model object owns buffers of its own).
 inline float* g_pv = nullptr;
 inline int* g_pi = nullptr;
+inline float* g_tv = nullptr;
+inline int* g_ti = nullptr;
 
 inline int argmax_launch(const float* x, int n, int* result, float* pv, int* pi, hipStream_t st) {
     argmax_partial_kernel<<<kArgmaxParts, 256, 0, st>>>(x, n, pv, pi);
