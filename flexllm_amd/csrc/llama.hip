@@ -482,7 +482,7 @@ int flexllm_llama_decode_sample(flexllm_llama* m, int* token_io, int pos0, int s
         }
         // two stages: 128 workgroups pick the top_k of their share of the vocabulary, one workgroup picks among those
         topk_partial_kernel<<<kTopKParts, kTopKPartThreads, 0, st>>>(m->logits, c.vocab, top_k, m->topk_val, m->topk_idx);
-        topk_sample_kernel<<<1, kTopKThreads, 0, st>>>(m->topk_val, m->topk_idx, kTopKParts * top_k, top_k, rands, 1, 1, out);
+        topk_sample_kernel<256><<<1, 256, 0, st>>>(m->topk_val, m->topk_idx, kTopKParts * top_k, top_k, rands, 1, 1, out);
         FX_LAUNCH_CHECK();
     }
     return FLEXLLM_OK;

@@ -39,9 +39,9 @@ int flexllm_sample_topk_f32(const float* logits, int n, int top_k, const float* 
             FX_HIP(hipMalloc(&g_ti, kTopKParts * kTopKMax * sizeof(int)));
         }
         topk_partial_kernel<<<kTopKParts, kTopKPartThreads, 0, as_stream(stream)>>>(logits, n, top_k, g_tv, g_ti);
-        topk_sample_kernel<<<1, kTopKThreads, 0, as_stream(stream)>>>(g_tv, g_ti, kTopKParts * top_k, top_k, rand, 0, enable_sub_max, out);
+        topk_sample_kernel<256><<<1, 256, 0, as_stream(stream)>>>(g_tv, g_ti, kTopKParts * top_k, top_k, rand, 0, enable_sub_max, out);
     } else {
-        topk_sample_kernel<<<1, kTopKThreads, 0, as_stream(stream)>>>(logits, nullptr, n, top_k, rand, 0, enable_sub_max, out);
+        topk_sample_kernel<kTopKThreads><<<1, kTopKThreads, 0, as_stream(stream)>>>(logits, nullptr, n, top_k, rand, 0, enable_sub_max, out);
     }
     FX_LAUNCH_CHECK();
     return FLEXLLM_OK;

@@ -95,7 +95,7 @@ static __global__ __launch_bounds__(64) void argmax_final_kernel(const float* __
 // ---- top-k sampling (Modules/Logits.h:145-279) ------------------------------------------------------------
 // Each thread keeps the k best (value, index) of its share, ordered by value descending then index ascending; k
 // rounds of a block-wide arg-max over the threads' current heads pop the top-k in that order.  Long rows go through
-// two stages (128 workgroups over contiguous shares of the row, then one workgroup over their candidates: 12 us
+// two stages (128 workgroups over contiguous shares of the row, then one workgroup over their candidates: 23 us
 // for 128256 logits where a single workgroup needs 230 us), short rows through the last stage alone.
 // Thread 0 then does what the reference does with the k candidates: softmax with
 // two partial sums (exp(v_k - v_0)), cumulative distribution, first k with rand < cdf[k] (else the last one).
@@ -112,9 +112,12 @@ __device__ __forceinline__ bool topk_better(float v, int i, float bv, int bi) { 
 template <int THREADS>
 __device__ __forceinline__ void topk_block_select(const float (&val)[kTopKMax], const int (&idx)[kTopKMax], int top_k,
                                                   float* f_val, int* f_idx) {
-    __shared__ float s_val[THREADS / 64];
-    __shared__ int s_idx[THREADS / 64], s_own[THREADS / 64];
-    __shared__ int s_winner;
+    constexpr int NW = THREADS / 64;
+    static_assert((NW & (NW - 1)) == 0 && NW <= 64, "waves per workgroup: a power of two");
+    // wave winners of a round, double-buffered by round parity: a buffer is rewritten two rounds later, after the
+    // barrier of the round in between, which no thread passes before it has read this round's entries
+    __shared__ float s_val[2][NW];
+    __shared__ int s_idx[2][NW], s_own[2][NW];
     const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
     int head = 0;                                   // this thread's best not yet taken
     for (int r = 0; r < top_k; r++) {
@@ -127,18 +130,20 @@ __device__ __forceinline__ void topk_block_select(const float (&val)[kTopKMax], 
             const float ov = __shfl_xor(bv, m); const int oi = __shfl_xor(bi, m); const int oo = __shfl_xor(bo, m);
             if (topk_better(ov, oi, bv, bi) || (ov == bv && oi == bi && oo < bo)) { bv = ov; bi = oi; bo = oo; }
         }
-        if (lane == 0) { s_val[wave] = bv; s_idx[wave] = bi; s_own[wave] = bo; }
+        if (lane == 0) { s_val[r & 1][wave] = bv; s_idx[r & 1][wave] = bi; s_own[r & 1][wave] = bo; }
         __syncthreads();
-        if (t == 0) {
-            float wv = s_val[0]; int wi = s_idx[0], wo = s_own[0];
-            for (int w = 1; w < THREADS / 64; w++)
-                if (topk_better(s_val[w], s_idx[w], wv, wi) || (s_val[w] == wv && s_idx[w] == wi && s_own[w] < wo)) { wv = s_val[w]; wi = s_idx[w]; wo = s_own[w]; }
-            f_val[r] = wv; f_idx[r] = wi; s_winner = wo;
+        // every wave reduces the NW wave winners itself (each group of NW lanes holds all of them), so every thread
+        // learns the round's winner without a second exchange
+        bv = s_val[r & 1][lane & (NW - 1)]; bi = s_idx[r & 1][lane & (NW - 1)]; bo = s_own[r & 1][lane & (NW - 1)];
+#pragma unroll
+        for (int m = 1; m < NW; m <<= 1) {
+            const float ov = __shfl_xor(bv, m); const int oi = __shfl_xor(bi, m); const int oo = __shfl_xor(bo, m);
+            if (topk_better(ov, oi, bv, bi) || (ov == bv && oi == bi && oo < bo)) { bv = ov; bi = oi; bo = oo; }
         }
-        __syncthreads();
-        if (t == s_winner) head++;
-        __syncthreads();
+        if (t == 0) { f_val[r] = bv; f_idx[r] = bi; }
+        if (t == bo) head++;
     }
+    __syncthreads();
 }
 
 // Sorted insertion of one candidate (k is small; statically indexed so that the lists stay in registers).
@@ -167,7 +172,15 @@ static __global__ __launch_bounds__(kTopKPartThreads) void topk_partial_kernel(c
     int idx[kTopKMax];
 #pragma unroll
     for (int k = 0; k < kTopKMax; k++) { val[k] = -1e32f; idx[k] = 0x7fffffff; }
-    for (int i = begin + threadIdx.x; i < end; i += kTopKPartThreads) topk_insert(val, idx, top_k, logits[i], i);
+    // four loads in flight per thread (a share of the 128256-entry vocabulary is 1002 logits: one batch)
+    for (int i0 = begin + threadIdx.x; i0 < end; i0 += 4 * kTopKPartThreads) {
+        float lv[4];
+#pragma unroll
+        for (int u = 0; u < 4; u++) lv[u] = i0 + u * kTopKPartThreads < end ? logits[i0 + u * kTopKPartThreads] : 0.0f;
+#pragma unroll
+        for (int u = 0; u < 4; u++)
+            if (i0 + u * kTopKPartThreads < end) topk_insert(val, idx, top_k, lv[u], i0 + u * kTopKPartThreads);
+    }
     topk_block_select<kTopKPartThreads>(val, idx, top_k, f_val, f_idx);
     if (threadIdx.x < top_k) {
         cand_val[blockIdx.x * top_k + threadIdx.x] = f_val[threadIdx.x];
@@ -176,9 +189,12 @@ static __global__ __launch_bounds__(kTopKPartThreads) void topk_partial_kernel(c
 }
 
 // in_idx == NULL: logits[i] is the logit of token i.  Otherwise (second stage) logits / in_idx are n candidates.
-static __global__ __launch_bounds__(kTopKThreads) void topk_sample_kernel(const float* __restrict__ logits, const int* __restrict__ in_idx,
-                                                                         int n, int top_k, const float* __restrict__ rand_ptr,
-                                                                         int rand_index_from_state, int enable_sub_max, TopKOut out) {
+// THREADS: 1024 for a whole short row, 256 for the few hundred candidates of the second stage (the selection rounds
+// cost issue slots per wave, and all waves of the one workgroup share a CU).
+template <int THREADS>
+static __global__ __launch_bounds__(THREADS) void topk_sample_kernel(const float* __restrict__ logits, const int* __restrict__ in_idx,
+                                                                    int n, int top_k, const float* __restrict__ rand_ptr,
+                                                                    int rand_index_from_state, int enable_sub_max, TopKOut out) {
     __shared__ float f_val[kTopKMax];
     __shared__ int f_idx[kTopKMax];
     const int t = threadIdx.x;
@@ -186,32 +202,44 @@ static __global__ __launch_bounds__(kTopKThreads) void topk_sample_kernel(const 
     int idx[kTopKMax];
 #pragma unroll
     for (int k = 0; k < kTopKMax; k++) { val[k] = -1e32f; idx[k] = 0x7fffffff; }
-    for (int i = t; i < n; i += kTopKThreads) topk_insert(val, idx, top_k, logits[i], in_idx ? in_idx[i] : i);
-    topk_block_select<kTopKThreads>(val, idx, top_k, f_val, f_idx);
+    for (int i = t; i < n; i += THREADS) topk_insert(val, idx, top_k, logits[i], in_idx ? in_idx[i] : i);
+    topk_block_select<THREADS>(val, idx, top_k, f_val, f_idx);
     if (t < top_k && f_idx[t] == 0x7fffffff) f_idx[t] = -1;
     __syncthreads();
     if (t == 0) {
+        // loops over the compile-time maximum with a predicate: the small arrays stay in registers
         float prob[kTopKMax], cdf[kTopKMax];
         float sum_partial[2] = {0.0f, 0.0f};
-        for (int k = 0; k < top_k; k++) {
-            const float e = enable_sub_max ? expf(f_val[k] - f_val[0]) : expf(f_val[k]);
-            prob[k] = e;
-            sum_partial[k % 2] += e;
+        const float v0 = f_val[0];
+#pragma unroll
+        for (int k = 0; k < kTopKMax; k++) {
+            prob[k] = 0.0f;
+            if (k < top_k) {
+                const float e = enable_sub_max ? expf(f_val[k] - v0) : expf(f_val[k]);
+                prob[k] = e;
+                sum_partial[k % 2] += e;
+            }
         }
         const float sum = sum_partial[0] + sum_partial[1];
-        for (int k = 0; k < top_k; k++) prob[k] = prob[k] / sum;
+#pragma unroll
+        for (int k = 0; k < kTopKMax; k++) if (k < top_k) prob[k] = prob[k] / sum;
         cdf[0] = prob[0];
-        for (int k = 1; k < top_k; k++) cdf[k] = prob[k] + cdf[k - 1];
+#pragma unroll
+        for (int k = 1; k < kTopKMax; k++) cdf[k] = k < top_k ? prob[k] + cdf[k - 1] : cdf[k - 1];
         const float rnd = rand_ptr[rand_index_from_state && out.state ? out.state[1] : 0];
         int selected = top_k - 1;
-        for (int k = 0; k < top_k; k++)
-            if (rnd < cdf[k] && selected == top_k - 1) selected = k;
+#pragma unroll
+        for (int k = kTopKMax - 1; k >= 0; k--)
+            if (k < top_k && rnd < cdf[k]) selected = k;                    // ends on the first k with rnd < cdf[k]
         const int tok = f_idx[selected];
         if (out.token) out.token[0] = tok;
-        for (int k = 0; k < top_k; k++) {
-            if (out.top_idx) out.top_idx[k] = f_idx[k];
-            if (out.top_val) out.top_val[k] = f_val[k];
-            if (out.top_prob) out.top_prob[k] = prob[k];
+#pragma unroll
+        for (int k = 0; k < kTopKMax; k++) {
+            if (k < top_k) {
+                if (out.top_idx) out.top_idx[k] = f_idx[k];
+                if (out.top_val) out.top_val[k] = f_val[k];
+                if (out.top_prob) out.top_prob[k] = prob[k];
+            }
         }
         if (out.state) {                            // generation loop: hand the token over and advance position / step
             out.token_io[0] = tok;

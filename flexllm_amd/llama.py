@@ -116,7 +116,11 @@ class Llama:
         gamma_final = self._gamma.view(2 * self.cfg["layers"] * hidden * 4, (hidden,), np.float32)
         out = []
         tok = int(token)
+        rows = embed_f32.shape[0] if embed_f32 is not None else self._embed.shape[0]
         for i in range(int(steps)):
+            if not 0 <= tok < rows:
+                # the head may have more rows than the embedding table (padding rows): such an id has no embedding
+                raise ValueError("step %d: token id %d outside the embedding table (%d rows)" % (i, tok, rows))
             if embed_f32 is not None:
                 x = embed_f32.view(tok * hidden * 4, (hidden,), np.float32)
             else:

@@ -126,7 +126,7 @@ def test_generation_loop_with_int4_head(fx, oracle):
     cfg = llama.make_config(layers=2, vocab=4096, max_pos=256)
     host_w = llama.synth_weights(cfg, seed=21, device=False)
     model = llama.Llama(cfg, llama.synth_weights(cfg, seed=21, device=True))
-    hidden, vocab_pad = cfg["hidden"], 8192
+    hidden, vocab_pad = cfg["hidden"], cfg["vocab"]          # every id the head can produce has an embedding row
     r = np.random.default_rng(5)
     q_w = r.integers(-8, 8, (vocab_pad, hidden)).astype(np.int8)
     w_s = r.uniform(1e-3, 1e-2, vocab_pad).astype(np.float32)
@@ -150,4 +150,7 @@ def test_generation_loop_with_int4_head(fx, oracle):
     # the loop is deterministic: a second model run from the same state gives the same ids
     model2 = llama.Llama(cfg, llama.synth_weights(cfg, seed=21, device=True))
     assert model2.generate_int4_head(77, 0, len(rands), rands, 5, head) == toks
+    # an id without an embedding row (a head may carry padding rows beyond the vocabulary) is refused, not looked up
+    with pytest.raises(ValueError, match="outside the embedding table"):
+        model2.generate_int4_head(cfg["vocab"] + 3, 6, 1, [0.0], 1, head)
     model.close(); model2.close()
