@@ -303,6 +303,10 @@ __global__ __launch_bounds__(kMegaT, 1) void decode_mega_kernel(MegaParams p) {
     auto fine = [&]() {};
 #endif
     int tok = p.x_in ? 0 : p.token[0];
+    if ((unsigned)tok >= (unsigned)p.vocab) {                      // never look up a row outside the table: report and use token 0
+        if (wg == 0 && threadIdx.x == 0) st_i(&p.state[3], 2);
+        tok = 0;
+    }
     const bool greedy = p.tokens_out != nullptr;
 
     // Greedy mode runs several tokens in one launch: after the lm_head every workgroup reduces the per-workgroup

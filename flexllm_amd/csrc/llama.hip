@@ -201,7 +201,7 @@ static inline bool use_mega(const flexllm_llama* m) { return m->mega_ok && m->de
 // One greedy step: embedding of *token_io -> layers -> head -> argmax -> *token_io, tokens_out[step], pos++.
 static int greedy_step(flexllm_llama* m, int* token_io, int* tokens_out, hipStream_t st) {
     const flexllm_llama_config& c = m->cfg;
-    embed_kernel<<<(c.hidden + 255) / 256, 256, 0, st>>>(reinterpret_cast<const __half*>(m->embed), token_io, m->x, c.hidden);
+    embed_kernel<<<(c.hidden + 255) / 256, 256, 0, st>>>(reinterpret_cast<const __half*>(m->embed), token_io, m->x, c.hidden, c.vocab, &m->state[3]);
     int rc;
     for (int l = 0; l < c.layers; l++)
         if ((rc = decode_layer(m, l, st))) return rc;
@@ -374,6 +374,10 @@ int flexllm_llama_check(flexllm_llama* m) {
     FX_HIP(hipMemcpy(st, m->state, sizeof(st), hipMemcpyDeviceToHost));
     if (st[3] != 0) {
         (void)hipMemset(&m->state[3], 0, sizeof(int));
+        if (st[3] == 2) {
+            set_error("decode: a token id outside the vocabulary (%d entries) was fed in; token 0 was used instead", m->cfg.vocab);
+            return FLEXLLM_EINVAL;
+        }
         set_error("persistent decode kernel: a grid barrier timed out (were all %d workgroups resident?)", kMegaWG);
         return FLEXLLM_EHIP;
     }
@@ -475,7 +479,7 @@ int flexllm_llama_decode_sample(flexllm_llama* m, int* token_io, int pos0, int s
         if (use_mega(m)) {
             if ((rc = launch_mega(m, token_io, nullptr, m->logits, 1, st))) return rc;
         } else {
-            embed_kernel<<<(c.hidden + 255) / 256, 256, 0, st>>>(reinterpret_cast<const __half*>(m->embed), token_io, m->x, c.hidden);
+            embed_kernel<<<(c.hidden + 255) / 256, 256, 0, st>>>(reinterpret_cast<const __half*>(m->embed), token_io, m->x, c.hidden, c.vocab, &m->state[3]);
             for (int l = 0; l < c.layers; l++)
                 if ((rc = decode_layer(m, l, st))) return rc;
             if ((rc = decode_head(m, m->logits, st))) return rc;

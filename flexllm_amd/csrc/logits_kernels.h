@@ -7,9 +7,15 @@ namespace fx {
 
 using h16x8 = _Float16 __attribute__((ext_vector_type(8)));
 
+// vocab > 0: a token id outside [0, vocab) is replaced by 0 and reported through *err = 2 (never looked up).
 static __global__ __launch_bounds__(256) void embed_kernel(const __half* __restrict__ table, const int* __restrict__ token,
-                                                    float* __restrict__ y, int hidden) {
-    const size_t base = (size_t)token[0] * hidden;
+                                                    float* __restrict__ y, int hidden, int vocab = 0, int* __restrict__ err = nullptr) {
+    int tk = token[0];
+    if (vocab > 0 && (unsigned)tk >= (unsigned)vocab) {
+        if (err && blockIdx.x == 0 && threadIdx.x == 0) err[0] = 2;
+        tk = 0;
+    }
+    const size_t base = (size_t)tk * hidden;
     for (int i = blockIdx.x * 256 + threadIdx.x; i < hidden; i += gridDim.x * 256) y[i] = __half2float(table[base + i]);
 }
 

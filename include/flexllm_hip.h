@@ -249,7 +249,8 @@ int flexllm_argmax_f32(const float* x, int n, int* result, void* stream);
  * reference ranks them by its lane scan order; values and probabilities are the same).  1 <= top_k <= 16. */
 int flexllm_sample_topk_f32(const float* logits, int n, int top_k, const float* rand, int enable_sub_max, int* token,
                             int* top_idx, float* top_val, float* top_prob, void* stream);
-/* y = fp32(E[token]) with the token id read from device memory. */
+/* y = fp32(E[token]) with the token id read from device memory.  The table's row count is not known here: the
+ * caller guarantees 0 <= token < rows (the model entry points below check ids against their vocabulary). */
 int flexllm_embed_f16(const uint16_t* embed, const int* token, float* y, int hidden, void* stream);
 
 /* ---- whole model: Llama-3.2-1B W8A8 SpinQuant graph ------------------------------------- */
@@ -286,7 +287,9 @@ int flexllm_llama_set_decode_mode(flexllm_llama* m, int mode);
  * stamps of the last persistent decode step: per layer 6 x (stage start after the barrier, stage end before the
  * next arrive), then the head's start and end. */
 int flexllm_llama_stage_timeline(flexllm_llama* m, long long* host_out, int max_entries);
-/* Synchronises the device and reports a failed run of the persistent kernel (a grid barrier that timed out). */
+/* Synchronises the device and reports what a decode run flagged on the device: a grid barrier of the persistent
+ * kernel that timed out (FLEXLLM_EHIP), or an input token id outside the vocabulary (FLEXLLM_EINVAL; token 0 was
+ * used in its place, no row outside the embedding table is ever read).  Clears the flag. */
 int flexllm_llama_check(flexllm_llama* m);
 /* Device pointers to the int8 caches ([layers][max_pos][kv_hidden]) for inspection / pre-filling. */
 int flexllm_llama_kv_cache(flexllm_llama* m, int8_t** k_cache, int8_t** v_cache);

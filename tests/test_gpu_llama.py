@@ -128,6 +128,28 @@ def test_topk_sampling_loop_matches_oracle(small):
     assert int(tok.numpy()[0]) == ref[-1]
 
 
+def test_token_id_outside_the_vocabulary_is_reported(small):
+    """An id without an embedding row is never looked up: token 0 is used in its place and check() reports it."""
+    fx, cfg, model, om, host_w = small
+    from flexllm_amd._lib import FlexLLMError
+    stream = fx.Stream()
+    model.k_cache.zero_(); model.v_cache.zero_()
+    out = fx.zeros((2,), np.int32)
+    tok = fx.to_device(np.array([cfg["vocab"] + 7], np.int32))
+    model.decode_greedy(tok, 0, 2, out, use_graph=False, stream=stream)
+    stream.sync()
+    with pytest.raises(FlexLLMError, match="outside the vocabulary"):
+        model.check()
+    bad = out.numpy().tolist()
+    # the same two steps from token 0 give the same ids, and the flag is clear again
+    model.k_cache.zero_(); model.v_cache.zero_()
+    tok0 = fx.to_device(np.array([0], np.int32))
+    model.decode_greedy(tok0, 0, 2, out, use_graph=False, stream=stream)
+    stream.sync()
+    model.check()
+    assert out.numpy().tolist() == bad
+
+
 @pytest.mark.parametrize("mode", [0, 1], ids=["persistent", "per_stage"])
 def test_decode_at_the_maximum_context(mode):
     """The benchmark's situation checked against the oracle: context 4096 (all 32 key chunks of every KV head active),
