@@ -159,7 +159,16 @@ def module_legs(fx, lib, synth, ops, stream, Event):
     out["w4a4_linear_prefill_M1024_2048x8192"] = {"us": round(us, 2), "TOPs": round(ops5 / us / 1e6, 1),
                                                   "mfma_frac": round(ops5 / us / 1e6 / INT8_PEAK_TOPS, 4),
                                                   "note": "nibbles widened to int8 on the way to LDS, int8 MFMA (gfx950 has no int4 MFMA)"}
-    del ring4
+    # the same product with both operands held one value per byte, on the direct-load kernel of the int8 path
+    ring8 = [synth.device_i8((N, K), 9600 + i, -8, 7) for i in range(24)]                # 24 x 16.8 MB = 403 MB
+    a8 = synth.device_i8((M, K), 9650, 0, 15)
+    def leg5c(i):
+        lib.flexllm_linear_i8_gemm_dequant_asym(P(a8), P(sxm), P(bxm), P(ring8[i % len(ring8)]), P(w_s), P(w_sum), None, P(ym), M, K, N, stream.handle)
+    us = _time(stream, Event, leg5c, 24)
+    out["w4a4_linear_prefill_M1024_2048x8192_byte_held"] = {"us": round(us, 2), "TOPs": round(ops5 / us / 1e6, 1),
+                                                            "mfma_frac": round(ops5 / us / 1e6 / INT8_PEAK_TOPS, 4),
+                                                            "note": "4-bit values one per byte (weights widened once at load time): direct global-to-LDS loads, int8 MFMA"}
+    del ring4, ring8
     return out
 
 

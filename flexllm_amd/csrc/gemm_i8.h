@@ -209,7 +209,7 @@ __host__ __device__ constexpr int gemm_dma_lds_bytes(int bm, int bn, int stages,
     return rings > epi ? rings : epi;
 }
 
-enum GemmDmaEpi { kDmaRaw = 0, kDmaDequant = 1, kDmaSwiglu = 2, kDmaQkv = 3 };
+enum GemmDmaEpi { kDmaRaw = 0, kDmaDequant = 1, kDmaSwiglu = 2, kDmaQkv = 3, kDmaDequantAsym = 4 };
 
 // Arguments of the q/k/v epilogue: the 64-column tile of the fused [q | k | v] projection is one attention head,
 // so RoPE (pairs k, k+32), the static int8 quantisation and the store into q8 / the K cache / the transposed V
@@ -218,6 +218,7 @@ struct QkvEpiArgs {
     const float *sin_t, *cos_t, *q_s, *k_s, *v_s;
     int8_t *q8, *kc, *vc;
     int pos0, q_heads, kv_heads, max_pos;
+    const float *b_x, *w_sum;          // kDmaDequantAsym only: zero point per row, weight row sum (times its scale) per column
 };
 
 __device__ __forceinline__ void gemm_dma_issue(const int8_t* base, unsigned voff, unsigned lds_dst) {
@@ -465,6 +466,8 @@ __global__ __launch_bounds__(NW * 64, WPE) void gemm_i8_dma_kernel(const int8_t*
     // together with the stores issued before it (one counter covers both), once per group of rows.
     float sxv[TM][4];
     float4 wsv[TN];
+    float bxv[EPI == kDmaDequantAsym ? TM : 1][4];
+    float4 wsumv[EPI == kDmaDequantAsym ? TN : 1];
     if constexpr (EPI != kDmaRaw) {
 #pragma unroll
         for (int i = 0; i < TM; i++)
@@ -476,6 +479,17 @@ __global__ __launch_bounds__(NW * 64, WPE) void gemm_i8_dma_kernel(const int8_t*
             wsv[j] = col < n ? *reinterpret_cast<const float4*>(w_s + col) : make_float4(0.0f, 0.0f, 0.0f, 0.0f);
         }
     }
+    if constexpr (EPI == kDmaDequantAsym) {
+#pragma unroll
+        for (int i = 0; i < TM; i++)
+#pragma unroll
+            for (int p = 0; p < 4; p++) bxv[i][p] = qa.b_x[min(row0 + wm + i * 32 + p * 8 + pr, m - 1)];
+#pragma unroll
+        for (int j = 0; j < TN; j++) {
+            const int col = col0 + wn + j * 32 + pc;
+            wsumv[j] = col < n ? *reinterpret_cast<const float4*>(qa.w_sum + col) : make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+        }
+    }
 #pragma unroll
     for (int j = 0; j < TN; j++) {
         const int col = col0 + wn + j * 32 + pc;               // n is a multiple of 4 (checked by the launcher)
@@ -484,7 +498,7 @@ __global__ __launch_bounds__(NW * 64, WPE) void gemm_i8_dma_kernel(const int8_t*
         for (int i = 0; i < TM; i++) {
             float4 rs[4];                                      // the tile's residual rows, in flight during the turn through LDS
             bool has_res = false;
-            if constexpr (EPI == kDmaDequant) {
+            if constexpr (EPI == kDmaDequant || EPI == kDmaDequantAsym) {
                 has_res = residual != nullptr;
                 if (has_res) {
 #pragma unroll
@@ -523,7 +537,12 @@ __global__ __launch_bounds__(NW * 64, WPE) void gemm_i8_dma_kernel(const int8_t*
                     float4 o;
                     o.x = (float)v[0] * sx * ws.x; o.y = (float)v[1] * sx * ws.y;
                     o.z = (float)v[2] * sx * ws.z; o.w = (float)v[3] * sx * ws.w;
-                    if constexpr (EPI == kDmaDequant) {
+                    if constexpr (EPI == kDmaDequantAsym) {      // + zero point x row sum of the dequantised weights
+                        const float bx = bxv[i][p];
+                        const float4 wq = wsumv[j];
+                        o.x = o.x + bx * wq.x; o.y = o.y + bx * wq.y; o.z = o.z + bx * wq.z; o.w = o.w + bx * wq.w;
+                    }
+                    if constexpr (EPI == kDmaDequant || EPI == kDmaDequantAsym) {
                         if (has_res) { o.x = o.x + rs[p].x; o.y = o.y + rs[p].y; o.z = o.z + rs[p].z; o.w = o.w + rs[p].w; }
                         if (ok) *reinterpret_cast<float4*>(y + (size_t)row * n + col) = o;
                     } else {
@@ -562,7 +581,8 @@ inline int launch_gemm(const int8_t* a, const int8_t* w, int32_t* c, const float
                        const float* residual, float* y, int m, int k, int n, hipStream_t st) {
     // Measured on MI355X at M=1024: the direct-load kernel wins wherever it applies; 128x128 tiles once they fill
     // the chip about three times over, 64x64 tiles for the narrow projections.  FLEXLLM_GEMM_TILE forces a variant
-    // (0..2: register-staged 128x128 / 64x128 / 64x64; direct-load: 11 = 128x128, 13 = 64x64, 19 = 64x128 four
+    // (0..2: register-staged 128x128 / 64x128 / 64x64; direct-load: 11 = 128x128, 12 = 128x128 with two stages of
+    // 128-byte rows, 13 = 64x64, 19 = 64x128 four
     // stages, all with 64-byte rows; 36 = 64x64 four stages and 38 = 64x64 three stages with 128-byte rows; 60 = 64x128
     // three stages with 128-byte rows and two k-groups).
     auto tiles = [&](int bm, int bn) { return ((m + bm - 1) / bm) * ((n + bn - 1) / bn); };
@@ -574,6 +594,10 @@ inline int launch_gemm(const int8_t* a, const int8_t* w, int32_t* c, const float
     // that many, else two of 64 KiB with a fourth stage (the narrow projections stream their weights cold)
     // Long K and an output too narrow for two workgroups per CU (down projection): 64x128 tiles, two k-groups of
     // four waves per workgroup (32 us against 36 us for 64x64 tiles, two workgroups per CU).
+    // 384..767 tiles of 128x128 (o and down projections from M = 3072): two stages of 128-byte rows, two workgroups
+    // per CU.  At M = 4096: 36 us against 47 us (o) and 102 us against 133 us (down) for the narrow-tile choices below;
+    // at M = 3072: 30 / 87 us against 35 / 109 us; at M = 2048 (256 tiles) the narrow tiles are level or ahead.
+    if (dma_ok && mode != 11 && k % 128 == 0 && tiles(128, 128) >= 384) mode = 12;
     if (mode == 19 && k % 256 == 0) mode = 60;
     if ((mode == 13 || mode == 19) && k % 128 == 0) mode = tiles(64, 64) >= 768 ? 38 : 36;
     if (force) mode = atoi(force);
@@ -581,6 +605,7 @@ inline int launch_gemm(const int8_t* a, const int8_t* w, int32_t* c, const float
     const int nk = k / kGemmBK;
     if (mode >= 10) {
         constexpr int DE = EPI == kGemmDequant ? kDmaDequant : kDmaRaw;
+        if (mode == 12 && k % 128 == 0) return launch_gemm_dma<128, 128, DE, 2, 2, 128>(a, w, c, s_x, w_s, residual, y, m, k, n, st);
         if (mode == 11) return launch_gemm_dma<128, 128, DE>(a, w, c, s_x, w_s, residual, y, m, k, n, st);
         if (mode == 19) return launch_gemm_dma<64, 128, DE, 4, 2>(a, w, c, s_x, w_s, residual, y, m, k, n, st);
         if (k % 128 == 0) {
@@ -604,6 +629,33 @@ inline int launch_gemm(const int8_t* a, const int8_t* w, int32_t* c, const float
 #undef FX_GEMM_LAUNCH
     FX_LAUNCH_CHECK();
     return FLEXLLM_OK;
+}
+
+// Asymmetric activations held one value per byte (0..127, e.g. the uint4 values of the W4A4 path before packing) times
+// int8 weights on the direct-load kernel: y = (float(acc) * s_x) * w_s + b_x * w_sum (+ residual).
+inline int launch_gemm_asym(const int8_t* a, const int8_t* w, const float* s_x, const float* b_x, const float* w_s,
+                            const float* w_sum, const float* residual, float* y, int m, int k, int n, hipStream_t st) {
+    FX_REQUIRE((size_t)m * k < (1ull << 31) && (size_t)n * k < (1ull << 31) && n % 4 == 0,
+               "linear_i8_gemm_dequant_asym: m=%d k=%d n=%d outside the direct-load kernel's range", m, k, n);
+    auto tiles = [&](int bm, int bn) { return ((m + bm - 1) / bm) * ((n + bn - 1) / bn); };
+    QkvEpiArgs qa = QkvEpiArgs();
+    qa.b_x = b_x; qa.w_sum = w_sum;
+    constexpr int DE = kDmaDequantAsym;
+    static const char* force = getenv("FLEXLLM_GEMM_TILE");
+    const int fm = force ? atoi(force) : 0;
+    // Wide outputs (the separate gate and up projections of the W4A4 graph, 2048 -> 8192 at M = 1024), measured (us):
+    // 128x128 tiles, two stages of 128-byte rows 26.7; 128x128, three stages of 64-byte rows 31.8; 128x256 on four
+    // waves 38.7; 64x64 tiles 41.0.
+    if (k % 128 == 0 && (fm == 12 || (!fm && tiles(128, 128) >= 384)))
+        return launch_gemm_dma<128, 128, DE, 2, 2, 128>(a, w, nullptr, s_x, w_s, residual, y, m, k, n, st, qa);
+    if (fm == 11 || (!fm && tiles(128, 128) >= 768)) return launch_gemm_dma<128, 128, DE>(a, w, nullptr, s_x, w_s, residual, y, m, k, n, st, qa);
+    if (k % 256 == 0 && k >= 4096 && tiles(64, 128) >= 256 && (!fm || fm == 60))
+        return launch_gemm_dma<64, 128, DE, 3, 2, 128, 8, 2>(a, w, nullptr, s_x, w_s, residual, y, m, k, n, st, qa);
+    if (k % 128 == 0) {
+        if (tiles(64, 64) >= 768) return launch_gemm_dma<64, 64, DE, 3, 3, 128>(a, w, nullptr, s_x, w_s, residual, y, m, k, n, st, qa);
+        return launch_gemm_dma<64, 64, DE, 4, 2, 128>(a, w, nullptr, s_x, w_s, residual, y, m, k, n, st, qa);
+    }
+    return launch_gemm_dma<64, 64, DE>(a, w, nullptr, s_x, w_s, residual, y, m, k, n, st, qa);
 }
 
 // W4A4 prefill GEMM on nibble-packed operands (register-staged kernel, nibbles widened on the way to LDS).

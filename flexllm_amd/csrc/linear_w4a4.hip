@@ -53,4 +53,13 @@ int flexllm_linear_u4i4_gemm_dequant(const uint8_t* a4, const float* s_x, const 
     return launch_gemm_u4i4<kGemmDequantAsym>(a4, w4, nullptr, s_x, b_x, w_s, w_sum, residual, y, m, k, n, as_stream(stream));
 }
 
+int flexllm_linear_i8_gemm_dequant_asym(const int8_t* a, const float* s_x, const float* b_x, const int8_t* w, const float* w_s,
+                                        const float* w_sum, const float* residual, float* y, int m, int k, int n, void* stream) {
+    FX_REQUIRE(a && s_x && b_x && w && w_s && w_sum && y, "linear_i8_gemm_dequant_asym: null pointer");
+    FX_REQUIRE(k > 0 && k % kGemmBK == 0, "linear_i8_gemm_dequant_asym: k=%d must be a multiple of 64", k);
+    FX_REQUIRE(m >= 0 && n >= 0 && n % 4 == 0, "linear_i8_gemm_dequant_asym: m=%d n=%d (n a multiple of 4)", m, n);
+    if (m == 0 || n == 0) return FLEXLLM_OK;
+    return launch_gemm_asym(a, w, s_x, b_x, w_s, w_sum, residual, y, m, k, n, as_stream(stream));
+}
+
 }  // extern "C"

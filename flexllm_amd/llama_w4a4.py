@@ -27,7 +27,10 @@ class LlamaW4A4:
         q,k,v,o,g,u,d; gamma [2L+1][hidden]; q_s, k_s, v_s, a_s [L][heads]; rope_sin, rope_cos."""
         self.cfg = cfg
         L = cfg["layers"]
-        self.w4 = {p: [ops.pack_nibbles(to_device(np.ascontiguousarray(w["w" + p][l], np.int8))) for l in range(L)] for p in _PROJ}
+        # decode streams the nibble-packed weights (half the bytes); prefill multiplies the same values held one per
+        # byte on the direct-load MFMA kernel of the int8 path
+        self.w8 = {p: [to_device(np.ascontiguousarray(w["w" + p][l], np.int8)) for l in range(L)] for p in _PROJ}
+        self.w4 = {p: [ops.pack_nibbles(self.w8[p][l]) for l in range(L)] for p in _PROJ}
         self.ws = {p: [to_device(np.asarray(w["s" + p][l], np.float32)) for l in range(L)] for p in _PROJ}
         self.wsum = {p: [to_device(np.asarray(w["sum" + p][l], np.float32)) for l in range(L)] for p in _PROJ}
         self.gamma = [to_device(np.ascontiguousarray(w["gamma"][i], np.float32)) for i in range(2 * L + 1)]
@@ -39,6 +42,8 @@ class LlamaW4A4:
     # one W4A4 linear: per-token asymmetric uint4 quantisation, int4 x uint4 product, dequantisation (+ residual)
     def _linear(self, x, p, l, residual=None):
         q, s, b = ops.quant_asym_u8(x, bits=4)
+        if x.shape[0] > 1 and self.w8[p][l].shape[0] % 4 == 0:
+            return ops.linear_i8_gemm_dequant_asym(q, s, b, self.w8[p][l], self.ws[p][l], self.wsum[p][l], residual=residual)
         a4 = ops.pack_nibbles(q)
         if x.shape[0] == 1:
             k2 = a4.shape[-1]

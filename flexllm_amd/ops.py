@@ -151,6 +151,17 @@ def linear_u4i4_gemm_dequant(a4, s_x, b_x, w4, w_s, w_sum, residual=None, stream
 
 
 # ---------------------------------------------------------------- FHT.h
+def linear_i8_gemm_dequant_asym(a, s_x, b_x, w, w_s, w_sum, residual=None, stream=None):
+    """W4A4-style product on operands held one value per byte: a [m][k] unsigned values (0..127) in int8/uint8
+    containers, w [n][k] int8; y = (float(acc) * s_x) * w_s + b_x * w_sum (+ residual)."""
+    m, k = a.shape
+    n = w.shape[0]
+    y = DeviceArray((m, n), np.float32)
+    check(lib().flexllm_linear_i8_gemm_dequant_asym(_p(a), _p(s_x), _p(b_x), _p(w), _p(w_s), _p(w_sum), _p(residual), _p(y),
+                                                    m, k, n, _s(stream)))
+    return y
+
+
 def lm_head_u4i4(n_vec, w4, w_s, w_sum, stream=None):
     """The reference's output head (SpinQuant_Decoding_mem_opt.h:363-365, config D6): the normalised hidden vector is
     quantised to asymmetric uint4, multiplied with the int4 head weights (nibble-packed [vocab_pad][hidden/2]) and

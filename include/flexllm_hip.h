@@ -141,6 +141,13 @@ int flexllm_linear_u4i4_gemm(const uint8_t* a4, const uint8_t* w4, int32_t* acc,
 int flexllm_linear_u4i4_gemm_dequant(const uint8_t* a4, const float* s_x, const float* b_x, const uint8_t* w4,
                                      const float* w_s, const float* w_sum, const float* residual, float* y, int m, int k,
                                      int n, void* stream);
+/* The same product on operands held one value per byte: a [m][k] with the unsigned activation values (0..127, e.g.
+ * the uint4 output of flexllm_quant_asym_u8 before packing) in int8 containers, w [n][k] int8 (e.g. int4 weights
+ * widened once at load time).  Same integer sums and the same dequantisation as flexllm_linear_u4i4_gemm_dequant, on
+ * the direct-load MFMA kernel of the int8 path (twice the operand bytes, about half the time at M = 1024).
+ * k % 64 == 0, n % 4 == 0.  Replaces pref_Linear_Layer_i4xi4 + the asymmetric dequant like the entry point above. */
+int flexllm_linear_i8_gemm_dequant_asym(const int8_t* a, const float* s_x, const float* b_x, const int8_t* w, const float* w_s,
+                                        const float* w_sum, const float* residual, float* y, int m, int k, int n, void* stream);
 
 /* ---- FHT.h ---------------------------------------------------------------------------- */
 /* y = H_n x / scale (Sylvester order, butterfly stage order of the reference's omega network, so

@@ -51,6 +51,22 @@ def test_gemm_all_tile_shapes_and_extremes(fx):
     assert np.all(fx.ops.linear_i8_gemm(fx.to_device(a), fx.to_device(w)).numpy() == 8192 * 128 * 128)
 
 
+@pytest.mark.parametrize("m,k,n", [(4096, 2048, 2048), (2048, 128, 4096), (2000, 384, 4100), (3072, 256, 2048)])
+def test_gemm_long_prefill_shapes(fx, oracle, m, k, n):
+    """Shapes with 384..767 tiles of 128x128 (the o projection of a 4096-token prefill, shallow ones, a ragged one):
+    the 128x128 variant with two stages of 128-byte rows.  Raw int32 and dequantised + residual, float64 BLAS as the
+    exact reference (|sum| < 2^31)."""
+    a = rng.integers(-128, 128, (m, k)).astype(np.int8)
+    w = rng.integers(-128, 128, (n, k)).astype(np.int8)
+    ref = (a.astype(np.float64) @ w.astype(np.float64).T).astype(np.int64).astype(np.int32)
+    da, dw = fx.to_device(a), fx.to_device(w)
+    assert np.array_equal(fx.ops.linear_i8_gemm(da, dw).numpy(), ref)
+    s_x = rng.uniform(0.01, 0.02, m).astype(np.float32); w_s = rng.uniform(1e-3, 1e-2, n).astype(np.float32)
+    res = rng.standard_normal((m, n)).astype(np.float32)
+    y = fx.ops.linear_i8_gemm_dequant(da, fx.to_device(s_x), dw, fx.to_device(w_s), residual=fx.to_device(res)).numpy()
+    assert np.array_equal(y, oracle.residual(oracle.dequant(ref, s_x, w_s), res))
+
+
 def test_gemm_dequant_residual_bit_exact(fx, oracle):
     m, k, n = 160, 2048, 384
     x = rng.standard_normal((m, k)).astype(np.float32)

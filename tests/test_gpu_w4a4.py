@@ -59,6 +59,34 @@ def test_gemm_u4i4_exact(fx, m, k, n):
     assert np.array_equal(acc, a.astype(np.int32) @ w.astype(np.int32).T)
 
 
+@pytest.mark.parametrize("m,k,n", [(1024, 2048, 8192), (1024, 8192, 2048), (1024, 2048, 2048), (160, 2048, 384), (96, 64, 132),
+                                   (33, 128, 260), (1, 64, 4)])
+def test_gemm_on_byte_held_operands_equals_the_packed_path(fx, oracle, m, k, n):
+    """W4A4 values held one per byte on the direct-load kernel (every tile variant its launcher picks, ragged edges):
+    bit for bit the oracle's dequantised product, hence the nibble-packed entry point's result too."""
+    a = rng.integers(0, 16, (m, k)).astype(np.uint8)
+    w = rng.integers(-8, 8, (n, k)).astype(np.int8)
+    s_x = rng.uniform(0.05, 0.2, m).astype(np.float32); b_x = rng.uniform(-2, 0, m).astype(np.float32)
+    w_s = rng.uniform(0.01, 0.05, n).astype(np.float32)
+    w_sum = (w.sum(1, dtype=np.int64).astype(np.float32) * w_s).astype(np.float32)
+    res = rng.standard_normal((m, n)).astype(np.float32)
+    da, dw = fx.to_device(a), fx.to_device(w)
+    dev = [fx.to_device(v) for v in (s_x, b_x, w_s, w_sum)]
+    y = fx.ops.linear_i8_gemm_dequant_asym(da, dev[0], dev[1], dw, dev[2], dev[3]).numpy()
+    y_res = fx.ops.linear_i8_gemm_dequant_asym(da, dev[0], dev[1], dw, dev[2], dev[3], residual=fx.to_device(res)).numpy()
+    acc = a.astype(np.int32) @ w.astype(np.int32).T
+    ref = oracle.dequant(acc, s_x, w_s, b_x=b_x, w_sum=w_sum)
+    assert np.array_equal(y, ref)
+    assert np.array_equal(y_res, oracle.residual(ref, res))
+    if m * n <= 1024 * 2048:
+        y_packed = fx.ops.linear_u4i4_gemm_dequant(fx.to_device(pack(a)), dev[0], dev[1], fx.to_device(pack(w)), dev[2], dev[3]).numpy()
+        assert np.array_equal(y, y_packed)
+    # the largest byte value the container admits, against the most negative weight
+    a2 = np.full((m, k), 127, np.uint8); w2 = np.full((n, k), -128, np.int8)
+    y2 = fx.ops.linear_i8_gemm_dequant_asym(fx.to_device(a2), dev[0], dev[1], fx.to_device(w2), dev[2], dev[3]).numpy()
+    assert np.array_equal(y2, oracle.dequant(np.full((m, n), -127 * 128 * k, np.int32), s_x, w_s, b_x=b_x, w_sum=w_sum))
+
+
 def test_w4a4_layer_like_the_reference_testbench(fx, oracle):
     """quant (asym uint4) -> linear -> dequant with zero point, decode and prefill shapes: bit-exact against the oracle
     chain, and within the testbench's own 1e-2 criterion of the fake-quant golden (…_tb.cpp:215-236)."""
