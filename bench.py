@@ -328,6 +328,15 @@ def main():
         model.decode_sample(tok_s_io, cfg["max_pos"] - n_s, n_s, rands, 5, out_s, stream=stream)
         s1.record(stream); s1.sync()
         ms = s0.elapsed_ms(s1)
+        # prompt -> tokens (the reference's combined prefill + decode harness): 1025-token prompt, 64 greedy tokens
+        n_p, n_g = 1025, 64
+        prompt = fx.to_device(np.random.default_rng(11).integers(0, cfg["vocab"], n_p).astype(np.int32))
+        out_g = fx.zeros((n_g,), np.int32)
+        gen = lambda: fx.check(lib.flexllm_llama_generate(model.handle, C.c_void_p(prompt.ptr), n_p, n_g, None, 0, C.c_void_p(out_g.ptr), stream.handle))
+        gen(); stream.sync()
+        g0, g1 = Event(), Event()
+        g0.record(stream); gen(); g1.record(stream); g1.sync()
+        modules["generate_prompt1025_greedy64"] = {"ms": round(g0.elapsed_ms(g1), 3), "prefilled_tokens": n_p - 1, "generated_tokens": n_g}
         modules["decode_top5_sampling_ctx4096"] = {"ms_per_token": round(ms / n_s, 4), "tokens_per_s": round(n_s / ms * 1e3, 1), "steps": n_s}
 
     # ---- CPU baseline: the oracle (scalar C port of the reference modules), bounded sample --------------

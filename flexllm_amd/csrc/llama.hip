@@ -37,6 +37,9 @@ struct flexllm_llama {
     int* am_i = nullptr;
     float* topk_val = nullptr;      // sampler: per-workgroup candidates of the first selection stage
     int* topk_idx = nullptr;
+    float* gen_x = nullptr;         // generate: embeddings of the prompt, [gen_rows][hidden] (allocated on first use)
+    int gen_rows = 0;
+    int* gen_token = nullptr;       // generate: the token fed back between decode steps
     hipGraphExec_t graph_exec = nullptr;
     int* graph_token_io = nullptr;
     int* graph_tokens_out = nullptr;
@@ -490,6 +493,39 @@ int flexllm_llama_decode_sample(flexllm_llama* m, int* token_io, int pos0, int s
         FX_LAUNCH_CHECK();
     }
     return FLEXLLM_OK;
+}
+
+int flexllm_llama_generate(flexllm_llama* m, const int* prompt, int n_prompt, int steps, const float* rands, int top_k,
+                           int* tokens_out, void* stream) {
+    FX_REQUIRE(m && prompt && tokens_out, "llama_generate: null pointer");
+    FX_REQUIRE(n_prompt >= 1 && steps >= 0 && n_prompt - 1 + steps <= m->cfg.max_pos,
+               "llama_generate: prompt of %d tokens + %d steps exceed max_pos=%d", n_prompt, steps, m->cfg.max_pos);
+    FX_REQUIRE(top_k == 0 || rands, "llama_generate: sampling (top_k=%d) needs the uniform numbers", top_k);
+    hipStream_t st = as_stream(stream);
+    const flexllm_llama_config& c = m->cfg;
+    const int s = n_prompt - 1;                               // prefilled tokens: all but the last one
+    const int rows = (s + 31) / 32 * 32;                      // the prefill works on tiles of 32 rows
+    FX_REQUIRE(rows <= c.max_pos, "llama_generate: %d prompt rows (padded to 32) exceed max_pos=%d", rows, c.max_pos);
+    if (!m->gen_token) FX_ALLOC(m, m->gen_token, sizeof(int));
+    if (rows > 0) {
+        if (!m->gen_x) {                                      // once, for the longest prompt the cache admits
+            m->gen_rows = (c.max_pos + 31) / 32 * 32;
+            FX_ALLOC(m, m->gen_x, sizeof(float) * (size_t)m->gen_rows * c.hidden);
+        }
+        embed_rows_kernel<<<rows, 256, 0, st>>>(reinterpret_cast<const __half*>(m->embed), prompt, s, m->gen_x, c.hidden, c.vocab,
+                                                &m->state[3]);
+        FX_LAUNCH_CHECK();
+        // rows s..rows-1 are zero padding: they write cache rows at positions >= s, which the decode steps below
+        // overwrite one by one before any of them is read
+        int rc = llama_prefill_run(c, m->layers.data(), m->gamma, m->q_s, m->k_s, m->v_s, m->a_s, m->rope_sin, m->rope_cos,
+                                   m->k_cache, m->v_cache, m->cache_layer_bytes, &m->pws, m->gen_x, rows, nullptr, st);
+        if (rc) return rc;
+    }
+    copy_int_kernel<<<1, 1, 0, st>>>(prompt + s, m->gen_token);
+    FX_LAUNCH_CHECK();
+    if (steps == 0) return FLEXLLM_OK;
+    if (top_k == 0) return flexllm_llama_decode_greedy(m, m->gen_token, s, steps, tokens_out, 0, stream);
+    return flexllm_llama_decode_sample(m, m->gen_token, s, steps, rands, top_k, tokens_out, stream);
 }
 
 int flexllm_llama_prefill_hidden(flexllm_llama* m, const float* x_in, int s, float* hidden_out, void* stream) {

@@ -19,6 +19,27 @@ static __global__ __launch_bounds__(256) void embed_kernel(const __half* __restr
     for (int i = blockIdx.x * 256 + threadIdx.x; i < hidden; i += gridDim.x * 256) y[i] = __half2float(table[base + i]);
 }
 
+// Embeddings of a prompt: out[r] = fp32(E[tokens[r]]) for r < n, zero rows for n <= r < rows (padding to the prefill
+// tile).  Ids outside [0, vocab) are replaced by 0 and reported through *err = 2.  One workgroup per row.
+static __global__ __launch_bounds__(256) void embed_rows_kernel(const __half* __restrict__ table, const int* __restrict__ tokens,
+                                                         int n, float* __restrict__ out, int hidden, int vocab, int* __restrict__ err) {
+    const int r = blockIdx.x;
+    float* dst = out + (size_t)r * hidden;
+    if (r >= n) {
+        for (int i = threadIdx.x; i < hidden; i += 256) dst[i] = 0.0f;
+        return;
+    }
+    int tk = tokens[r];
+    if ((unsigned)tk >= (unsigned)vocab) {
+        if (err && threadIdx.x == 0) err[0] = 2;
+        tk = 0;
+    }
+    const __half* src = table + (size_t)tk * hidden;
+    for (int i = threadIdx.x; i < hidden; i += 256) dst[i] = __half2float(src[i]);
+}
+
+static __global__ void copy_int_kernel(const int* __restrict__ src, int* __restrict__ dst) { dst[0] = src[0]; }
+
 // One wave per run of rows; lane reads 16-byte chunks (8 halves) lane, lane+64, ... of the row.
 template <int NCH>
 __global__ __launch_bounds__(256) void lm_head_kernel(const __half* __restrict__ table, const float* __restrict__ n,

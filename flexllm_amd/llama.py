@@ -103,6 +103,24 @@ class Llama:
         check(lib().flexllm_llama_decode_sample(self.handle, C.c_void_p(token_io.ptr), int(pos0), int(steps),
                                                 C.c_void_p(rands.ptr), int(top_k), C.c_void_p(tokens_out.ptr), _s(stream)))
 
+    def generate(self, prompt, steps, top_k=0, rands=None, stream=None):
+        """Prompt (host sequence of token ids) -> `steps` generated ids (host list): prefill of all prompt tokens but
+        the last, then the decode loop from the last one, greedy (top_k = 0) or top-k sampling with the host-supplied
+        uniform numbers `rands` - the flow of SpinQuant_Prefilling_Decoding_mem_opt_tb.cpp:753-930."""
+        prompt = np.ascontiguousarray(prompt, np.int32).reshape(-1)
+        d_prompt = to_device(prompt)
+        out = DeviceArray((max(int(steps), 1),), np.int32)
+        d_rands = to_device(np.ascontiguousarray(rands, np.float32)) if top_k else None
+        if top_k and d_rands.size < steps:
+            raise ValueError("%d uniform numbers for %d steps" % (d_rands.size, steps))
+        check(lib().flexllm_llama_generate(self.handle, C.c_void_p(d_prompt.ptr), int(prompt.size), int(steps),
+                                           C.c_void_p(d_rands.ptr) if d_rands is not None else None, int(top_k),
+                                           C.c_void_p(out.ptr), _s(stream)))
+        if stream is not None:
+            stream.sync()
+        self.check()
+        return out.numpy()[:int(steps)].tolist()
+
     def generate_int4_head(self, token, pos0, steps, rands, top_k, head, embed_f32=None):
         """The reference's generation loop with its int4 output head and top-k sampling (SpinQuant_Decoding_mem_opt.h:
         924-940, Modules/Logits.h:145-279), sequenced from the host: embedding -> layer stack -> final RMSNorm ->

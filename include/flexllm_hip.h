@@ -318,6 +318,15 @@ int flexllm_llama_decode_greedy(flexllm_llama* m, int* token_io, int pos0, int s
  * token_io (device int, holds the first input token on entry). */
 int flexllm_llama_decode_sample(flexllm_llama* m, int* token_io, int pos0, int steps, const float* rands, int top_k,
                                 int* tokens_out, void* stream);
+/* Prompt to tokens, the flow of the reference's combined harness (SpinQuant_Prefilling_Decoding_mem_opt_tb.cpp:753-930):
+ * all prompt tokens but the last are embedded and prefilled (positions 0..n_prompt-2; the rows are padded to the
+ * prefill tile with zero rows, whose cache entries the decode steps overwrite before they are read), the last prompt
+ * token is the first input of the decode loop at position n_prompt-1, and `steps` tokens are generated into
+ * tokens_out (device): greedy when top_k == 0, else top-k sampling with rands[step] (device, `steps` floats in [0,1)).
+ * prompt: device int [n_prompt], n_prompt >= 1, n_prompt - 1 + steps <= max_pos.  Token ids outside the vocabulary are
+ * reported by flexllm_llama_check. */
+int flexllm_llama_generate(flexllm_llama* m, const int* prompt, int n_prompt, int steps, const float* rands, int top_k,
+                           int* tokens_out, void* stream);
 /* Prefill s tokens at positions 0..s-1 from fp32 embeddings x_in (device [s][hidden]); fills the KV cache,
  * writes the residual stream to hidden_out (device [s][hidden], may be NULL). */
 int flexllm_llama_prefill_hidden(flexllm_llama* m, const float* x_in, int s, float* hidden_out, void* stream);

@@ -213,3 +213,31 @@ def test_full_size_schedules_agree_at_the_maximum_context():
     a.check()
     assert np.array_equal(a.k_cache.numpy(), b.k_cache.numpy()) and np.array_equal(a.v_cache.numpy(), b.v_cache.numpy())
     a.close(); b.close()
+
+
+@pytest.mark.parametrize("n_prompt", [1, 2, 33, 70])
+def test_generate_from_a_prompt_matches_the_oracle_flow(small, n_prompt):
+    """The reference's combined flow: prefill of prompt[:-1], decode from prompt[-1] at position len-1, greedy.  Prompts of
+    1 token (no prefill), 2 (one prefilled row, 31 rows of padding), 33 (exactly one tile) and 70 tokens."""
+    fx, cfg, model, om, host_w = small
+    from oracle import oracle
+    r = np.random.default_rng(100 + n_prompt)
+    prompt = r.integers(0, cfg["vocab"], n_prompt).astype(np.int32)
+    steps = 5
+    model.k_cache.copy_from(r.integers(-128, 128, model.k_cache.shape).astype(np.int8))      # stale cache contents must not matter
+    model.v_cache.copy_from(r.integers(-128, 128, model.v_cache.shape).astype(np.int8))
+    got = model.generate(prompt, steps)
+    kc, vc = om.new_caches()
+    if n_prompt > 1:
+        x = np.stack([oracle.embed(host_w["embed"], int(t)) for t in prompt[:-1]])
+        om.prefill(x, kc, vc)
+    t, ref = int(prompt[-1]), []
+    for i in range(steps):
+        _, logits = om.decode_token(oracle.embed(host_w["embed"], t), n_prompt - 1 + i, kc, vc)
+        t = int(np.argmax(logits))
+        ref.append(t)
+    assert got == ref
+    # sampling variant: deterministic, in range, and equal to the greedy ids when only one candidate is kept
+    assert model.generate(prompt, steps, top_k=1, rands=np.full(steps, 0.5, np.float32)) == ref
+    with pytest.raises(Exception, match="max_pos"):
+        model.generate(prompt, cfg["max_pos"] + 1)
