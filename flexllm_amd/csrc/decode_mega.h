@@ -37,6 +37,7 @@
 #pragma once
 #include "attn_decode_kernels.h"
 #include "gemv_i8.h"
+#include "logits_kernels.h"
 #include "prefill.h"
 #include <hip/hip_fp16.h>
 
@@ -68,6 +69,11 @@ struct MegaParams {
     const float* x_in;             // optional fp32 input embedding
     float* am_v;                   // [kMegaWG] argmax candidates
     int* am_i;
+    // top-k sampling instead of arg-max (top_k > 0): step s draws with rands[state[1] + s]; per-workgroup candidates
+    int top_k;
+    const float* rands;
+    float* cand_v;                 // [kMegaWG][kTopKMax]
+    int* cand_i;
     int n_layers, max_pos, vocab, want_head;
     float eps, fht_scale;
     long long* timeline;           // optional [n_layers*6+2][2] wall-clock stamps of workgroup 0 (after wait, before arrive)
@@ -173,6 +179,9 @@ struct MegaLds {
     float bestv[kMegaWaves];
     int besti[kMegaWaves];
     float hst[32];                                     // SiLU(gate)*up of this workgroup's 32 row pairs, stream waves -> store wave
+    float tk_val[kTopKMax];                            // sampling: the selected candidates (this workgroup's, then the global ones)
+    int tk_idx[kTopKMax];
+    int tk_tok;
     __attribute__((aligned(16))) int8_t wd[8][8192];   // this workgroup's 8 down rows, filled by global->LDS direct loads (64 KiB);
                                                        // the odd rows first hold gate/up rows 12..15 of their stream wave
     __attribute__((aligned(16))) int8_t gu2[4][8192];  // gate/up rows 8..11 of each stream wave (32 KiB)
@@ -308,6 +317,7 @@ __global__ __launch_bounds__(kMegaT, 1) void decode_mega_kernel(MegaParams p) {
         tok = 0;
     }
     const bool greedy = p.tokens_out != nullptr;
+    const bool sampling = greedy && p.top_k > 0;
 
     // Greedy mode runs several tokens in one launch: after the lm_head every workgroup reduces the per-workgroup
     // candidates itself, so all of them know the next token and position without a further exchange.
@@ -839,7 +849,10 @@ __global__ __launch_bounds__(kMegaT, 1) void decode_mega_kernel(MegaParams p) {
                 const float s = wave_sum(acc[u]);
                 const int row = r + u * kMegaWaves;
                 if (row < row_end) {
-                    if (lane == 0) p.logits[row] = s;
+                    if (lane == 0) {
+                        p.logits[row] = s;
+                        if (sampling) L.f[4096 + (row - row_begin)] = s;      // L.f[0..2047] holds the normalised vector
+                    }
                     if (s > best || (s == best && row < bi)) { best = s; bi = row; }
                 }
             }
@@ -853,7 +866,37 @@ __global__ __launch_bounds__(kMegaT, 1) void decode_mega_kernel(MegaParams p) {
             st_i(&p.am_i[wg], bi);
         }
         stamp();
-        if (greedy) {
+        if (sampling) {
+            // Top-k sampling (Modules/Logits.h:145-279) without leaving the kernel: this workgroup's top_k logits ->
+            // grid barrier -> every workgroup selects the global top_k among the kMegaWG * top_k candidates and draws
+            // the same token from them (same inputs, same arithmetic), so the next step needs no further exchange.
+            float val[kTopKMax];
+            int idx[kTopKMax];
+#pragma unroll
+            for (int k = 0; k < kTopKMax; k++) { val[k] = -1e32f; idx[k] = 0x7fffffff; }
+            for (int i = t; i < row_end - row_begin; i += kMegaT) topk_insert(val, idx, p.top_k, L.f[4096 + i], row_begin + i);
+            topk_block_select<kMegaT>(val, idx, p.top_k, L.tk_val, L.tk_idx);
+            if (t < p.top_k) { st_f(&p.cand_v[wg * kTopKMax + t], L.tk_val[t]); st_i(&p.cand_i[wg * kTopKMax + t], L.tk_idx[t]); }
+            bar.arrive();
+            bar.wait();
+#pragma unroll
+            for (int k = 0; k < kTopKMax; k++) { val[k] = -1e32f; idx[k] = 0x7fffffff; }
+            for (int i = t; i < kMegaWG * p.top_k; i += kMegaT) {
+                const int slot = (i / p.top_k) * kTopKMax + i % p.top_k;
+                topk_insert(val, idx, p.top_k, ld_f(&p.cand_v[slot]), ld_i(&p.cand_i[slot]));
+            }
+            topk_block_select<kMegaT>(val, idx, p.top_k, L.tk_val, L.tk_idx);
+            if (t == 0) {
+                float prob[kTopKMax];
+                const int sel = topk_sample_rank(L.tk_val, p.top_k, p.rands[p.state[1] + step], 1, prob);
+                const int chosen = L.tk_idx[sel];
+                L.tk_tok = chosen == 0x7fffffff ? 0 : chosen;
+            }
+            __syncthreads();
+            tok = __builtin_amdgcn_readfirstlane(L.tk_tok);
+            if (wg == 0 && t == 0) p.tokens_out[p.state[1] + step] = tok;
+            __syncthreads();                                        // L.tk_* and L.f are reused by the next step
+        } else if (greedy) {
             // every workgroup picks the winner among the kMegaWG candidates (largest value, then smallest index)
             bar.arrive();
             bar.wait();

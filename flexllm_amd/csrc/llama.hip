@@ -171,7 +171,7 @@ static int decode_head(flexllm_llama* m, float* logits, hipStream_t st) {
 
 // tokens_out != NULL: greedy mode, `steps` tokens in this launch (argmax, token hand-over and position advance inside the kernel)
 static int launch_mega(flexllm_llama* m, int* token, const float* x_in, float* logits, int want_head, hipStream_t st,
-                       int* tokens_out = nullptr, int steps = 1) {
+                       int* tokens_out = nullptr, int steps = 1, const float* rands = nullptr, int top_k = 0) {
     const flexllm_llama_config& c = m->cfg;
     MegaParams p;
     p.layers = m->layers_dev;
@@ -183,6 +183,7 @@ static int launch_mega(flexllm_llama* m, int* token, const float* x_in, float* l
     p.stats = m->stats; p.stats_tag = m->stats_tag; p.qkv_tag = m->qkv_tag; p.o_acc = m->o_acc; p.state = m->state; p.bar = m->bar;
     p.token = token; p.tokens_out = tokens_out; p.n_steps = steps; p.x_in = x_in; p.am_v = m->am_v; p.am_i = m->am_i;
     p.n_layers = c.layers; p.max_pos = c.max_pos; p.vocab = c.vocab; p.want_head = want_head;
+    p.top_k = top_k; p.rands = rands; p.cand_v = m->topk_val; p.cand_i = m->topk_idx;
     p.eps = c.eps; p.fht_scale = c.fht_scale;
     p.timeline = m->timeline;
     static bool lds_opted_in = false;     // the kernel's LDS block exceeds the default 64 KiB per workgroup
@@ -313,8 +314,10 @@ int flexllm_llama_create(flexllm_llama** out, const flexllm_llama_config* cfg, c
     FX_TRY_HIP(hipMemset(m->stats_tag, 0xFF, sizeof(unsigned long long) * 2 * (size_t)c.q_heads * kMaxChunks));
     FX_TRY(dev_alloc(m, (void**)&m->state, sizeof(int) * 4));
     FX_TRY(dev_alloc(m, (void**)&m->am_v, sizeof(float) * kArgmaxParts));
-    FX_TRY(dev_alloc(m, (void**)&m->topk_val, sizeof(float) * kTopKParts * kTopKMax));
-    FX_TRY(dev_alloc(m, (void**)&m->topk_idx, sizeof(int) * kTopKParts * kTopKMax));
+    // per-workgroup sampling candidates: of the persistent kernel's workgroups or of the stand-alone first stage
+    constexpr int kCandGroups = kMegaWG > kTopKParts ? kMegaWG : kTopKParts;
+    FX_TRY(dev_alloc(m, (void**)&m->topk_val, sizeof(float) * kCandGroups * kTopKMax));
+    FX_TRY(dev_alloc(m, (void**)&m->topk_idx, sizeof(int) * kCandGroups * kTopKMax));
     FX_TRY(dev_alloc(m, (void**)&m->am_i, sizeof(int) * kArgmaxParts));
     FX_TRY(dev_alloc(m, (void**)&m->layers_dev, sizeof(LayerW) * L));
     FX_TRY_HIP(hipMemcpy(m->layers_dev, m->layers.data(), sizeof(LayerW) * L, hipMemcpyHostToDevice));
@@ -474,19 +477,25 @@ int flexllm_llama_decode_sample(flexllm_llama* m, int* token_io, int pos0, int s
     const flexllm_llama_config& c = m->cfg;
     set_state_kernel<<<1, 1, 0, st>>>(m->state, pos0, 0);
     FX_LAUNCH_CHECK();
-    // per token: layers + lm_head into m->logits, then the sampler picks the token (rands[step]), hands it over
-    // through token_io and advances position and step in device memory
+    if (use_mega(m) && (c.vocab + kMegaWG - 1) / kMegaWG <= 4096) {
+        // the persistent kernel samples by itself (per-workgroup candidates, one more grid barrier, every workgroup
+        // draws the same token): up to kMegaMaxSteps tokens per launch, as in greedy mode
+        for (int s = 0; s < steps; s += kMegaMaxSteps) {
+            int rc = launch_mega(m, token_io, nullptr, nullptr, 1, st, tokens_out, steps - s < kMegaMaxSteps ? steps - s : kMegaMaxSteps,
+                                 rands, top_k);
+            if (rc) return rc;
+        }
+        return FLEXLLM_OK;
+    }
+    // one kernel per stage: layers + lm_head into m->logits, then the sampler picks the token (rands[step]), hands it
+    // over through token_io and advances position and step in device memory
     TopKOut out = {nullptr, nullptr, nullptr, nullptr, token_io, tokens_out, m->state};
     for (int s = 0; s < steps; s++) {
         int rc;
-        if (use_mega(m)) {
-            if ((rc = launch_mega(m, token_io, nullptr, m->logits, 1, st))) return rc;
-        } else {
-            embed_kernel<<<(c.hidden + 255) / 256, 256, 0, st>>>(reinterpret_cast<const __half*>(m->embed), token_io, m->x, c.hidden, c.vocab, &m->state[3]);
-            for (int l = 0; l < c.layers; l++)
-                if ((rc = decode_layer(m, l, st))) return rc;
-            if ((rc = decode_head(m, m->logits, st))) return rc;
-        }
+        embed_kernel<<<(c.hidden + 255) / 256, 256, 0, st>>>(reinterpret_cast<const __half*>(m->embed), token_io, m->x, c.hidden, c.vocab, &m->state[3]);
+        for (int l = 0; l < c.layers; l++)
+            if ((rc = decode_layer(m, l, st))) return rc;
+        if ((rc = decode_head(m, m->logits, st))) return rc;
         // two stages: 128 workgroups pick the top_k of their share of the vocabulary, one workgroup picks among those
         topk_partial_kernel<<<kTopKParts, kTopKPartThreads, 0, st>>>(m->logits, c.vocab, top_k, m->topk_val, m->topk_idx);
         topk_sample_kernel<256><<<1, 256, 0, st>>>(m->topk_val, m->topk_idx, kTopKParts * top_k, top_k, rands, 1, 1, out);

@@ -134,8 +134,36 @@ struct TopKOut { int* token; int* top_idx; float* top_val; float* top_prob; int*
 
 __device__ __forceinline__ bool topk_better(float v, int i, float bv, int bi) { return v > bv || (v == bv && i < bi); }
 
+// (value, index) as one 64-bit key whose unsigned order is "larger value first, then smaller index": the value's bits
+// mapped monotonically to unsigned (sign bit flipped for positives, all bits for negatives; -0 is canonicalised to +0
+// so that it ties with +0 as the float comparison does), the index complemented.
+__device__ __forceinline__ unsigned long long topk_key(float v, int i) {
+    const unsigned b = (unsigned)__float_as_int(v + 0.0f);
+    const unsigned ord = b ^ ((b >> 31) ? 0xFFFFFFFFu : 0x80000000u);
+    return ((unsigned long long)ord << 32) | (unsigned)~i;
+}
+__device__ __forceinline__ float topk_key_value(unsigned long long k) {
+    const unsigned ord = (unsigned)(k >> 32);
+    return __int_as_float((int)(ord ^ ((ord >> 31) ? 0x80000000u : 0xFFFFFFFFu)));
+}
+__device__ __forceinline__ int topk_key_index(unsigned long long k) { return (int)~(unsigned)k; }
+template <int MASK>
+__device__ __forceinline__ unsigned long long topk_key_max_xor(unsigned long long k) {
+    const unsigned lo = (unsigned)lane_xor_i<MASK>((int)(unsigned)k), hi = (unsigned)lane_xor_i<MASK>((int)(unsigned)(k >> 32));
+    const unsigned long long o = ((unsigned long long)hi << 32) | lo;
+    return o > k ? o : k;
+}
+__device__ __forceinline__ unsigned long long topk_key_wave_max(unsigned long long k) {
+    k = topk_key_max_xor<1>(k); k = topk_key_max_xor<2>(k); k = topk_key_max_xor<4>(k);
+    k = topk_key_max_xor<8>(k); k = topk_key_max_xor<16>(k); k = topk_key_max_xor<32>(k);
+    return k;
+}
+
 // Block-wide selection: every thread holds a list sorted by (value descending, index ascending); top_k rounds of an
 // arg-max over the threads' current heads pop the block's top_k in that order into f_val / f_idx (shared memory).
+// Indices are distinct, so the winner's key identifies its owner: the thread whose head equals it advances.  (When
+// fewer than top_k real entries exist the winner is the sentinel, which every exhausted list shows; advancing those
+// changes nothing.)
 template <int THREADS>
 __device__ __forceinline__ void topk_block_select(const float (&val)[kTopKMax], const int (&idx)[kTopKMax], int top_k,
                                                   float* f_val, int* f_idx) {
@@ -143,32 +171,29 @@ __device__ __forceinline__ void topk_block_select(const float (&val)[kTopKMax], 
     static_assert((NW & (NW - 1)) == 0 && NW <= 64, "waves per workgroup: a power of two");
     // wave winners of a round, double-buffered by round parity: a buffer is rewritten two rounds later, after the
     // barrier of the round in between, which no thread passes before it has read this round's entries
-    __shared__ float s_val[2][NW];
-    __shared__ int s_idx[2][NW], s_own[2][NW];
+    __shared__ unsigned long long s_key[2][NW];
     const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
     int head = 0;                                   // this thread's best not yet taken
     for (int r = 0; r < top_k; r++) {
-        float bv = -1e32f; int bi = 0x7fffffff, bo = t;
+        float bv = -1e32f; int bi = 0x7fffffff;
 #pragma unroll
         for (int k = 0; k < kTopKMax; k++) if (k == head) { bv = val[k]; bi = idx[k]; }
         if (head >= top_k) { bv = -1e32f; bi = 0x7fffffff; }
-#pragma unroll
-        for (int m = 1; m < 64; m <<= 1) {
-            const float ov = __shfl_xor(bv, m); const int oi = __shfl_xor(bi, m); const int oo = __shfl_xor(bo, m);
-            if (topk_better(ov, oi, bv, bi) || (ov == bv && oi == bi && oo < bo)) { bv = ov; bi = oi; bo = oo; }
-        }
-        if (lane == 0) { s_val[r & 1][wave] = bv; s_idx[r & 1][wave] = bi; s_own[r & 1][wave] = bo; }
+        const unsigned long long mine = topk_key(bv, bi);
+        const unsigned long long wmax = topk_key_wave_max(mine);
+        if (lane == 0) s_key[r & 1][wave] = wmax;
         __syncthreads();
         // every wave reduces the NW wave winners itself (each group of NW lanes holds all of them), so every thread
         // learns the round's winner without a second exchange
-        bv = s_val[r & 1][lane & (NW - 1)]; bi = s_idx[r & 1][lane & (NW - 1)]; bo = s_own[r & 1][lane & (NW - 1)];
-#pragma unroll
-        for (int m = 1; m < NW; m <<= 1) {
-            const float ov = __shfl_xor(bv, m); const int oi = __shfl_xor(bi, m); const int oo = __shfl_xor(bo, m);
-            if (topk_better(ov, oi, bv, bi) || (ov == bv && oi == bi && oo < bo)) { bv = ov; bi = oi; bo = oo; }
-        }
-        if (t == 0) { f_val[r] = bv; f_idx[r] = bi; }
-        if (t == bo) head++;
+        unsigned long long win = s_key[r & 1][lane & (NW - 1)];
+        if constexpr (NW > 1) win = topk_key_max_xor<1>(win);
+        if constexpr (NW > 2) win = topk_key_max_xor<2>(win);
+        if constexpr (NW > 4) win = topk_key_max_xor<4>(win);
+        if constexpr (NW > 8) win = topk_key_max_xor<8>(win);
+        if constexpr (NW > 16) win = topk_key_max_xor<16>(win);
+        if constexpr (NW > 32) win = topk_key_max_xor<32>(win);
+        if (t == 0) { f_val[r] = topk_key_value(win); f_idx[r] = topk_key_index(win); }
+        if (mine == win) head++;
     }
     __syncthreads();
 }
@@ -182,6 +207,36 @@ __device__ __forceinline__ void topk_insert(float (&val)[kTopKMax], int (&idx)[k
             val[k] = cv; idx[k] = ci; cv = tv; ci = ti;
         }
     }
+}
+
+// What the reference does with the k candidates (values in rank order): softmax with two partial sums of
+// exp(v_k - v_0), cumulative distribution, the first k with rnd < cdf[k] (else the last one).  Returns the rank of the
+// sampled candidate; prob receives the probabilities.  Loops run over the compile-time maximum with a predicate so
+// that the small arrays stay in registers.  One thread calls this.
+__device__ __forceinline__ int topk_sample_rank(const float* f_val, int top_k, float rnd, int enable_sub_max, float (&prob)[kTopKMax]) {
+    float cdf[kTopKMax];
+    float sum_partial[2] = {0.0f, 0.0f};
+    const float v0 = f_val[0];
+#pragma unroll
+    for (int k = 0; k < kTopKMax; k++) {
+        prob[k] = 0.0f;
+        if (k < top_k) {
+            const float e = enable_sub_max ? expf(f_val[k] - v0) : expf(f_val[k]);
+            prob[k] = e;
+            sum_partial[k % 2] += e;
+        }
+    }
+    const float sum = sum_partial[0] + sum_partial[1];
+#pragma unroll
+    for (int k = 0; k < kTopKMax; k++) if (k < top_k) prob[k] = prob[k] / sum;
+    cdf[0] = prob[0];
+#pragma unroll
+    for (int k = 1; k < kTopKMax; k++) cdf[k] = k < top_k ? prob[k] + cdf[k - 1] : cdf[k - 1];
+    int selected = top_k - 1;
+#pragma unroll
+    for (int k = kTopKMax - 1; k >= 0; k--)
+        if (k < top_k && rnd < cdf[k]) selected = k;                    // ends on the first k with rnd < cdf[k]
+    return selected;
 }
 
 // First stage for long rows: workgroup g selects the top_k of its contiguous share of the logits and writes them,
@@ -234,30 +289,9 @@ static __global__ __launch_bounds__(THREADS) void topk_sample_kernel(const float
     if (t < top_k && f_idx[t] == 0x7fffffff) f_idx[t] = -1;
     __syncthreads();
     if (t == 0) {
-        // loops over the compile-time maximum with a predicate: the small arrays stay in registers
-        float prob[kTopKMax], cdf[kTopKMax];
-        float sum_partial[2] = {0.0f, 0.0f};
-        const float v0 = f_val[0];
-#pragma unroll
-        for (int k = 0; k < kTopKMax; k++) {
-            prob[k] = 0.0f;
-            if (k < top_k) {
-                const float e = enable_sub_max ? expf(f_val[k] - v0) : expf(f_val[k]);
-                prob[k] = e;
-                sum_partial[k % 2] += e;
-            }
-        }
-        const float sum = sum_partial[0] + sum_partial[1];
-#pragma unroll
-        for (int k = 0; k < kTopKMax; k++) if (k < top_k) prob[k] = prob[k] / sum;
-        cdf[0] = prob[0];
-#pragma unroll
-        for (int k = 1; k < kTopKMax; k++) cdf[k] = k < top_k ? prob[k] + cdf[k - 1] : cdf[k - 1];
+        float prob[kTopKMax];
         const float rnd = rand_ptr[rand_index_from_state && out.state ? out.state[1] : 0];
-        int selected = top_k - 1;
-#pragma unroll
-        for (int k = kTopKMax - 1; k >= 0; k--)
-            if (k < top_k && rnd < cdf[k]) selected = k;                    // ends on the first k with rnd < cdf[k]
+        const int selected = topk_sample_rank(f_val, top_k, rnd, enable_sub_max, prob);
         const int tok = f_idx[selected];
         if (out.token) out.token[0] = tok;
 #pragma unroll

@@ -28,9 +28,11 @@ def _seed(base, layer, tensor):
     return (base * 1000003 + layer * 101 + tensor) & 0xFFFFFFFFFFFF
 
 
-def synth_weights(cfg, seed=1, device=False):
+def synth_weights(cfg, seed=1, device=False, embed_range=1.7):
     """Random-init int8 weights U[-127,127] with per-channel scales sized so that activations stay O(1),
-    RMSNorm gains U[0.5,1.5], static attention scales with a seeded +-20% jitter per head, fp16 embedding.
+    RMSNorm gains U[0.5,1.5], static attention scales with a seeded +-20% jitter per head, fp16 embedding
+    U[-embed_range, embed_range] (with the default range a token's own row wins the tied head by a wide margin; a
+    range of a few hundredths gives logits of order one and top-k distributions with several live candidates).
     device=False -> numpy arrays on the host; device=True -> DeviceArrays filled on the GPU by the
     same counter-based generator."""
     i8 = synth.device_i8 if device else synth.host_i8
@@ -48,7 +50,7 @@ def synth_weights(cfg, seed=1, device=False):
     w["k_s"] = f32((L, cfg["kv_heads"]), _seed(seed, 99, 3), 0.8 * 0.03, 1.2 * 0.03)
     w["v_s"] = f32((L, cfg["kv_heads"]), _seed(seed, 99, 4), 0.8 * 0.03, 1.2 * 0.03)
     w["a_s"] = f32((L, cfg["q_heads"]), _seed(seed, 99, 5), 1.0 / 255, 1.0 / 255)
-    w["embed"] = f16((cfg["vocab"], cfg["hidden"]), _seed(seed, 99, 6), -1.7, 1.7)
+    w["embed"] = f16((cfg["vocab"], cfg["hidden"]), _seed(seed, 99, 6), -embed_range, embed_range)
     sin_t, cos_t = rope_table(cfg["max_pos"], cfg["head_dim"])
     if device:
         w["rope_sin"], w["rope_cos"] = to_device(sin_t), to_device(cos_t)

@@ -315,7 +315,8 @@ int flexllm_llama_decode_greedy(flexllm_llama* m, int* token_io, int pos0, int s
  * dec_Sampling_Embedding_Layer, Modules/Logits.h:145-279; host random numbers as in
  * SpinQuant_Prefilling_Decoding_mem_opt_tb.cpp:827-830): for step s the token is drawn from the top_k logits
  * with rands[s] (device array of `steps` floats in [0,1)), written to tokens_out[s] (device) and fed back through
- * token_io (device int, holds the first input token on entry). */
+ * token_io (device int, holds the first input token on entry).  On the persistent-kernel schedule the selection and
+ * the draw happen inside the kernel, up to 64 tokens per launch. */
 int flexllm_llama_decode_sample(flexllm_llama* m, int* token_io, int pos0, int steps, const float* rands, int top_k,
                                 int* tokens_out, void* stream);
 /* Prompt to tokens, the flow of the reference's combined harness (SpinQuant_Prefilling_Decoding_mem_opt_tb.cpp:753-930):
