@@ -101,15 +101,17 @@ def test_greedy_loop_graph_replay_equals_eager_and_oracle(small):
     assert outs[0].tolist() == ref
 
 
+@pytest.mark.parametrize("vocab", [4096, 600], ids=["vocab4096", "vocab600"])
 @pytest.mark.parametrize("mode", [0, 1], ids=["persistent", "per_stage"])
-def test_topk_sampling_loop_matches_oracle(mode):
+def test_topk_sampling_loop_matches_oracle(mode, vocab):
     """The reference's generation loop: top-5 sampling with host-supplied uniform numbers, token fed back.  The embedding
     table is scaled down so that the logits are of order one and several candidates carry probability (with the default
-    table a token's own row takes probability 1 and sampling would equal arg-max)."""
+    table a token's own row takes probability 1 and sampling would equal arg-max).  With 600 entries a workgroup of the
+    persistent kernel owns three logits, fewer than top_k, and the last workgroups none."""
     import flexllm_amd as fx
     from flexllm_amd import llama
     from oracle import oracle
-    cfg = llama.make_config(layers=2, vocab=4096, max_pos=256)
+    cfg = llama.make_config(layers=2, vocab=vocab, max_pos=256)
     host_w = llama.synth_weights(cfg, seed=3, device=False, embed_range=0.03)
     model = llama.Llama(cfg, llama.synth_weights(cfg, seed=3, device=True, embed_range=0.03))
     model.set_decode_mode(mode)
