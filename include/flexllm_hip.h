@@ -14,6 +14,11 @@
  *    their inputs.  fp32 results follow the reference's operation order except for
  *    reductions over a row (sum of squares, sum of exponentials), whose association
  *    differs; those agree to <=1e-3 relative.
+ *  - Three stand-alone entry points keep small scratch buffers that the library allocates on first use and shares
+ *    process-wide: flexllm_argmax_f32, flexllm_sample_topk_f32 (rows of 4096 logits and more) and
+ *    flexllm_mha_i8_decode.  Calls to one of them that may run at the same time on different streams must be
+ *    serialised by the caller.  A flexllm_llama object owns all of its buffers; use one object from one stream at a
+ *    time.
  *
  * Reference citations are relative to the reference tree root.
  */
