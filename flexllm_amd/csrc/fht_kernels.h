@@ -7,13 +7,17 @@
 // stages in that order (bits 1,2,...,log2(n)-1, then 0) reproduces the reference's fp32 result bit for
 // bit, so the int8 tensor quantised from it is exact as well.
 //
-// One workgroup of 256 threads transforms one row:
-//   layout A: element i = j*1024 + t*4 + e   (float4 loads, e = bits 0-1, lane = bits 2-7, wave = bits 8-9,
-//             j = bits 10+)      -> stage bit 1 in registers, bits 2..7 as cross-lane butterflies (DPP
-//             quad_perm / ds_swizzle / bpermute), no memory traffic
-//   one transpose through LDS
-//   layout B: element i = r*256 + t          (r = bits 8+, t = bits 0-7)
-//                                -> stages bits 8.. in registers, then bit 0 as a DPP butterfly.
+// One workgroup of 256 threads transforms one row of n = 256 * NR elements, NR = 2^P values per thread:
+//   layout A: element i = j*1024 + t*4 + e   (float4 loads; e = bits 0-1, t = bits 2-9, j = bits 10+)
+//             -> stage bit 1 in registers, bits 2..7-P as cross-lane butterflies on lane bits 0..5-P (DPP only:
+//             one stage at n = 8192, four at n = 1024)
+//   through LDS to layout M: i = hi*256 + r*2^(8-P) + lo, thread = (hi, lo), r = bits 8-P..7
+//             -> stages bits 8-P..7 in registers
+//   through LDS to layout B: i = r*256 + t   (r = bits 8+, t = bits 0-7)
+//             -> stages bits 8.. in registers, then bit 0 as a DPP butterfly.
+// A butterfly between registers is one add or subtract; across lanes it costs a data movement as well, so all but a
+// few stages run between registers, at the price of a second pass through LDS.  Each 256-element block of the LDS row
+// is followed by 2^(8-P) floats of padding, which spreads layout M's reads over all banks.
 #pragma once
 #include "common.h"
 
@@ -26,8 +30,11 @@ __global__ __launch_bounds__(kFhtBlock) void fht_kernel(const float* __restrict_
                                                         int8_t* __restrict__ q, float* __restrict__ s, float scale) {
     constexpr int N = 1 << LOG2N;
     constexpr int NJ = N / 1024;   // float4 vectors per thread in layout A
-    constexpr int NR = N / 256;    // floats per thread in layout B
-    __shared__ float lds[N];
+    constexpr int NR = N / 256;    // floats per thread in layouts M and B
+    constexpr int P = LOG2N - 8;   // log2(NR)
+    constexpr int PAD = 1 << (8 - P);
+    static_assert(P >= 2 && P <= 5, "1024 <= n <= 8192");
+    __shared__ float lds[N + PAD * NR];
     __shared__ float red[kFhtBlock / kWave];
     const int t = threadIdx.x;
     const int lane = t & 63;
@@ -57,7 +64,7 @@ __global__ __launch_bounds__(kFhtBlock) void fht_kernel(const float* __restrict_
         a[j].x = u0 + v0; a[j].z = u0 - v0;
         a[j].y = u1 + v1; a[j].w = u1 - v1;
     }
-    // stages: bits 2..7 = lane bits 0..5
+    // stages: bits 2..7-P = lane bits 0..5-P
 #define FX_LANE_STAGE(MASK)                                             \
     {                                                                   \
         const unsigned sg = lane_sign<MASK>(lane);                      \
@@ -69,20 +76,44 @@ __global__ __launch_bounds__(kFhtBlock) void fht_kernel(const float* __restrict_
         }                                                               \
     }
     FX_LANE_STAGE(1)
-    FX_LANE_STAGE(2)
-    FX_LANE_STAGE(4)
-    FX_LANE_STAGE(8)
-    FX_LANE_STAGE(16)
-    FX_LANE_STAGE(32)
+    if constexpr (P < 5) FX_LANE_STAGE(2)
+    if constexpr (P < 4) FX_LANE_STAGE(4)
+    if constexpr (P < 3) FX_LANE_STAGE(8)
 #undef FX_LANE_STAGE
 
-    // transpose A -> B through LDS
+    // A -> M through LDS (float4 stores: conflict-free whatever the padding)
 #pragma unroll
-    for (int j = 0; j < NJ; j++) reinterpret_cast<float4*>(lds)[j * 256 + t] = a[j];
+    for (int j = 0; j < NJ; j++) {
+        const int i = j * 1024 + t * 4;
+        *reinterpret_cast<float4*>(&lds[i + PAD * (i >> 8)]) = a[j];
+    }
     __syncthreads();
     float b[NR];
+    {
+        constexpr int LOB = 8 - P;                               // low index bits that stay with the thread
+        const int base = (t >> LOB) * (256 + PAD) + (t & ((1 << LOB) - 1));
 #pragma unroll
-    for (int r = 0; r < NR; r++) b[r] = lds[r * 256 + t];
+        for (int r = 0; r < NR; r++) b[r] = lds[base + (r << LOB)];
+        // stages: bits 8-P..7 = register index bits 0..P-1
+#pragma unroll
+        for (int bit = 1; bit < NR; bit <<= 1) {
+#pragma unroll
+            for (int r = 0; r < NR; r++) {
+                if ((r & bit) == 0) {
+                    const float u = b[r], v = b[r | bit];
+                    b[r] = u + v;
+                    b[r | bit] = u - v;
+                }
+            }
+        }
+        // every thread rewrites exactly the slots it read, so no barrier is needed before these stores
+#pragma unroll
+        for (int r = 0; r < NR; r++) lds[base + (r << LOB)] = b[r];
+    }
+    __syncthreads();
+    // M -> B
+#pragma unroll
+    for (int r = 0; r < NR; r++) b[r] = lds[r * (256 + PAD) + t];
 
     // stages: bits 8..LOG2N-1 = register index bits 0..
 #pragma unroll
