@@ -689,39 +689,39 @@ __global__ __launch_bounds__(kMegaT, 1) void decode_mega_kernel(MegaParams p) {
             stamp();
             if (is_s && lane == 0) { xres[0] = ld_f(&p.x2[wg * 8 + sw * 2]); xres[1] = ld_f(&p.x2[wg * 8 + sw * 2 + 1]); }
             // 8192-point transform on all 512 threads, stage order bits 1,2,...,12,0 (bit-exact order, see
-            // fht_kernels.h).  A: i = j*2048 + t*4 + e   -> stages 1..4 came done from phase 5, 5..7 across lanes
-            //                  B: i = (t>>8)*4096 + r*256 + (t&255) -> stages 8..11 in registers
-            //                  C: i = r*512 + t          -> stage 12 in registers, stage 0 across lanes
+            // fht_kernels.h).  Every remaining stage is a butterfly between registers of one thread, with two passes
+            // through LDS between the three layouts:
+            //   A: i = (t>>3)*128 + j*32 + (t&7)*4 + e -> stages 1..4 came done from phase 5; here 5 and 6 (j)
+            //   B: i = (t>>7)*2048 + r*128 + (t&127)   -> stages 7..10 (r)
+            //   C: i = q*2048 + 4t + e                 -> stages 11 and 12 (q), then 0 (e)
             float4 a[4];
+            const int abase = (t >> 3) * 128 + (t & 7) * 4;
 #pragma unroll
             for (int j = 0; j < 4; j++) {
-                const float2 lo = ld_f2(p.h + j * 2048 + t * 4), hi = ld_f2(p.h + j * 2048 + t * 4 + 2);
+                const float2 lo = ld_f2(p.h + abase + j * 32), hi = ld_f2(p.h + abase + j * 32 + 2);
                 a[j] = make_float4(lo.x, lo.y, hi.x, hi.y);
             }
-#define FX_MEGA_STAGE(MASK)                                                                   \
-    {                                                                                         \
-        const unsigned sg = lane_sign<MASK>(lane);                                            \
-        _Pragma("unroll") for (int j = 0; j < 4; j++) {                                       \
-            a[j].x = lane_butterfly_s<MASK>(a[j].x, sg);                                      \
-            a[j].y = lane_butterfly_s<MASK>(a[j].y, sg);                                      \
-            a[j].z = lane_butterfly_s<MASK>(a[j].z, sg);                                      \
-            a[j].w = lane_butterfly_s<MASK>(a[j].w, sg);                                      \
-        }                                                                                     \
-    }
             __builtin_amdgcn_s_waitcnt(0x0F70);               // vmcnt(0): the h loads are complete
             if (is_s) mega_row_to_lds(w.wd, wg * 8 + sw * 2 + 1, lane, L.wd[sw * 2 + 1]);
             if (l == 1) fine();
-            FX_MEGA_STAGE(8) FX_MEGA_STAGE(16) FX_MEGA_STAGE(32)
-#undef FX_MEGA_STAGE
+#pragma unroll
+            for (int bit = 1; bit < 4; bit <<= 1)                                                                       // bits 5, 6
+#pragma unroll
+                for (int j = 0; j < 4; j++)
+                    if ((j & bit) == 0) {
+                        const float4 u = a[j], v = a[j | bit];
+                        a[j] = make_float4(u.x + v.x, u.y + v.y, u.z + v.z, u.w + v.w);
+                        a[j | bit] = make_float4(u.x - v.x, u.y - v.y, u.z - v.z, u.w - v.w);
+                    }
             if (l == 1) fine();
 #pragma unroll
-            for (int j = 0; j < 4; j++) reinterpret_cast<float4*>(L.f)[j * 512 + t] = a[j];
+            for (int j = 0; j < 4; j++) reinterpret_cast<float4*>(L.f)[(abase >> 2) + j * 8] = a[j];
             __syncthreads();
             if (l == 1) fine();
             float b[16];
-            const int bbase = (t >> 8) * 4096 + (t & 255);
+            const int bbase = (t >> 7) * 2048 + (t & 127);
 #pragma unroll
-            for (int r = 0; r < 16; r++) b[r] = L.f[bbase + r * 256];
+            for (int r = 0; r < 16; r++) b[r] = L.f[bbase + r * 128];
 #pragma unroll
             for (int bit = 1; bit < 16; bit <<= 1)
 #pragma unroll
@@ -729,13 +729,19 @@ __global__ __launch_bounds__(kMegaT, 1) void decode_mega_kernel(MegaParams p) {
                     if ((r & bit) == 0) { const float u = b[r], v = b[r | bit]; b[r] = u + v; b[r | bit] = u - v; }
             // each thread re-writes exactly the slots it read, so no barrier is needed before this store
 #pragma unroll
-            for (int r = 0; r < 16; r++) L.f[bbase + r * 256] = b[r];
+            for (int r = 0; r < 16; r++) L.f[bbase + r * 128] = b[r];
             __syncthreads();
-            // last pass in the layout of the first one (i = q*2048 + 4t + e): bit 12 pairs q with q^2, bit 0 pairs e with
-            // e^1, both inside the thread, and the quantised bytes of a thread are four consecutive ones per q
+            // last pass (i = q*2048 + 4t + e): bit 11 pairs q with q^1, bit 12 q with q^2, bit 0 pairs e with e^1, all
+            // inside the thread, and the quantised bytes of a thread are four consecutive ones per q
             float4 c4[4];
 #pragma unroll
             for (int q = 0; q < 4; q++) c4[q] = reinterpret_cast<const float4*>(L.f)[q * 512 + t];
+#pragma unroll
+            for (int q = 0; q < 4; q += 2) {                                                                          // bit 11
+                const float4 u = c4[q], v = c4[q + 1];
+                c4[q] = make_float4(u.x + v.x, u.y + v.y, u.z + v.z, u.w + v.w);
+                c4[q + 1] = make_float4(u.x - v.x, u.y - v.y, u.z - v.z, u.w - v.w);
+            }
 #pragma unroll
             for (int q = 0; q < 2; q++) {                                                                             // bit 12
                 const float4 u = c4[q], v = c4[q + 2];
