@@ -607,9 +607,12 @@ __global__ __launch_bounds__(kMegaT, 1) void decode_mega_kernel(MegaParams p) {
 
         // ================= phase 5: RMSNorm + quant -> gate/up rows (64 per workgroup, 16 per stream wave) + SiLU*up =================
         {
-            const int ridx = 8 * (lane & 1) + 4 * ((lane >> 1) & 1) + 2 * ((lane >> 2) & 1) + ((lane >> 3) & 1);
-            float gsc = 0.0f;
-            if (is_s) gsc = w.sgu[wg * 64 + sw * 16 + ridx];          // read before this phase's prefetch is issued
+            // Stream wave s holds rows 0..7 of its 16 gate/up rows in registers and rows 8..15 in LDS; it multiplies the
+            // first eight itself, wave s (of waves 0..3) the other eight.  After the folding below lane L holds the sum
+            // of row ridx of its wave's eight.
+            const int ridx = 4 * (lane & 1) + 2 * ((lane >> 1) & 1) + ((lane >> 2) & 1);
+            const int ow = wave & 3, half = is_s ? 0 : 8;
+            const float gsc = w.sgu[wg * 64 + ow * 16 + half + ridx]; // read before this phase's prefetch is issued
             const float4 gam = reinterpret_cast<const float4*>(g1)[t];
             bar.wait();
             stamp();
@@ -620,52 +623,54 @@ __global__ __launch_bounds__(kMegaT, 1) void decode_mega_kernel(MegaParams p) {
                 __builtin_amdgcn_s_waitcnt(0x0F70);                   // vmcnt(0): see gu_slice
                 if (is_s) mega_row_to_lds(w.wd, wg * 8 + sw * 2, lane, L.wd[sw * 2]);
             });
-            if (is_s) {
-                // sixteen per-lane partial dot products, folded with a transposing butterfly: each step halves
-                // the number of live values, so 15 + 2 cross-lane exchanges replace 16 x 6.  Afterwards lane L
-                // holds the complete sum of row 8*(L&1) + 4*(L>>1 & 1) + 2*(L>>2 & 1) + (L>>3 & 1).
-                int part[16];
+            if (l == 1) fine();
+            {
+                // eight per-lane partial dot products, folded with a transposing butterfly: each step halves the number
+                // of live values, so 7 + 3 cross-lane exchanges replace 8 x 6.  Afterwards lane L holds the complete
+                // sum of row 4*(L&1) + 2*(L>>1 & 1) + (L>>2 & 1).
+                int part[8];
                 {
                     const i32x4 x0 = reinterpret_cast<const i32x4*>(L.xq)[lane], x1 = reinterpret_cast<const i32x4*>(L.xq)[lane + 64];
+                    if (is_s) {
 #pragma unroll
-                    for (int r = 0; r < 8; r++) part[r] = dot16(gu[r][1], x1, dot16(gu[r][0], x0, 0));
-                    // rows 8..15 from LDS (complete: the wait at the head of this phase's prefetch hook covered them)
-                    const i32x4* g2 = reinterpret_cast<const i32x4*>(L.gu2[sw]);
-                    const i32x4* g3 = reinterpret_cast<const i32x4*>(L.wd[sw * 2 + 1]);
+                        for (int r = 0; r < 8; r++) part[r] = dot16(gu[r][1], x1, dot16(gu[r][0], x0, 0));
+                    } else {
+                        // rows 8..15 from LDS (complete and visible: their stream wave waited for them at the head of
+                        // this phase's prefetch hook, before the barrier that ended the quantisation)
+                        const i32x4* g2 = reinterpret_cast<const i32x4*>(L.gu2[ow]);
+                        const i32x4* g3 = reinterpret_cast<const i32x4*>(L.wd[ow * 2 + 1]);
 #pragma unroll
-                    for (int r = 0; r < 4; r++) {
-                        part[8 + r] = dot16(g2[lane + 64 * (2 * r + 1)], x1, dot16(g2[lane + 64 * (2 * r)], x0, 0));
-                        part[12 + r] = dot16(g3[lane + 64 * (2 * r + 1)], x1, dot16(g3[lane + 64 * (2 * r)], x0, 0));
+                        for (int r = 0; r < 4; r++) {
+                            part[r] = dot16(g2[lane + 64 * (2 * r + 1)], x1, dot16(g2[lane + 64 * (2 * r)], x0, 0));
+                            part[4 + r] = dot16(g3[lane + 64 * (2 * r + 1)], x1, dot16(g3[lane + 64 * (2 * r)], x0, 0));
+                        }
                     }
                 }
-                int q8[8], q4[4], q2[2];
+                int q4[4], q2[2];
                 {
                     const bool hi = lane & 1;
 #pragma unroll
-                    for (int i = 0; i < 8; i++) q8[i] = (hi ? part[i + 8] : part[i]) + lane_xor_i<1>(hi ? part[i] : part[i + 8]);
+                    for (int i = 0; i < 4; i++) q4[i] = (hi ? part[i + 4] : part[i]) + lane_xor_i<1>(hi ? part[i] : part[i + 4]);
                 }
                 {
                     const bool hi = lane & 2;
 #pragma unroll
-                    for (int i = 0; i < 4; i++) q4[i] = (hi ? q8[i + 4] : q8[i]) + lane_xor_i<2>(hi ? q8[i] : q8[i + 4]);
-                }
-                {
-                    const bool hi = lane & 4;
-#pragma unroll
-                    for (int i = 0; i < 2; i++) q2[i] = (hi ? q4[i + 2] : q4[i]) + lane_xor_i<4>(hi ? q4[i] : q4[i + 2]);
+                    for (int i = 0; i < 2; i++) q2[i] = (hi ? q4[i + 2] : q4[i]) + lane_xor_i<2>(hi ? q4[i] : q4[i + 2]);
                 }
                 int sum;
                 {
-                    const bool hi = lane & 8;
-                    sum = (hi ? q2[1] : q2[0]) + lane_xor_i<8>(hi ? q2[0] : q2[1]);
+                    const bool hi = lane & 4;
+                    sum = (hi ? q2[1] : q2[0]) + lane_xor_i<4>(hi ? q2[0] : q2[1]);
                 }
+                sum += lane_xor_i<8>(sum);
                 sum += lane_xor_i<16>(sum);
                 sum += lane_xor_i<32>(sum);
                 const float mine = (float)sum * sx * gsc;
-                const float other = lane_xor_f<8>(mine);           // row ridx^1: the other half of the SwiGLU pair
-                if (lane < 8) L.hst[sw * 8 + (ridx >> 1)] = other * silu_f(mine);   // lanes 0..7 hold the (even) gate rows
+                const float other = lane_xor_f<4>(mine);           // row ridx^1: the other half of the SwiGLU pair
+                if (lane < 4) L.hst[ow * 8 + (half >> 1) + (ridx >> 1)] = other * silu_f(mine);   // lanes 0..3 hold the (even) gate rows
             }
             __syncthreads();
+            if (l == 1) fine();
             if (t < 64) {
                 // This workgroup's 32 values are the indices 32*wg .. 32*wg+31 of the 8192-vector: the first four stages
                 // of the transform (index bits 1..4, in that order) pair elements inside the block, so wave 0 does them
@@ -677,6 +682,7 @@ __global__ __launch_bounds__(kMegaT, 1) void decode_mega_kernel(MegaParams p) {
                 hv = lane_butterfly_s<16>(hv, lane_sign<16>(t));
                 if (t < 32) st_f(&p.h[wg * 32 + t], hv);             // stored by a wave with no prefetch in flight
             }
+            if (l == 1) fine();
             stamp();
             bar.arrive(!is_s);
         }
