@@ -687,13 +687,16 @@ __global__ __launch_bounds__(kMegaT, 1) void decode_mega_kernel(MegaParams p) {
             bar.arrive(!is_s);
         }
 
-        // ================= phase 6: Hadamard R4 + quant -> down rows (8 per workgroup, 2 per stream wave) + residual =================
+        // ================= phase 6: Hadamard R4 + quant -> down rows (8 per workgroup, one per wave) + residual =================
         {
-            float dsc[2] = {0.0f, 0.0f}, xres[2] = {0.0f, 0.0f};
-            if (is_s) { dsc[0] = ldc_f(w.sd + wg * 8 + sw * 2); dsc[1] = ldc_f(w.sd + wg * 8 + sw * 2 + 1); }
+            // Each wave multiplies one of the eight rows: stream wave s the even row 2s, wave s (of 0..3) the odd row 2s+1
+            // that stream wave s fetched into LDS.
+            const int drow = wg * 8 + (wave & 3) * 2 + (is_s ? 0 : 1);
+            const float dsc = ldc_f(w.sd + drow);
+            float xres = 0.0f;
             bar.wait();
             stamp();
-            if (is_s && lane == 0) { xres[0] = ld_f(&p.x2[wg * 8 + sw * 2]); xres[1] = ld_f(&p.x2[wg * 8 + sw * 2 + 1]); }
+            if (lane == 0) xres = ld_f(&p.x2[drow]);
             // 8192-point transform on all 512 threads, stage order bits 1,2,...,12,0 (bit-exact order, see
             // fht_kernels.h).  Every remaining stage is a butterfly between registers of one thread, with two passes
             // through LDS between the three layouts:
@@ -788,16 +791,12 @@ __global__ __launch_bounds__(kMegaT, 1) void decode_mega_kernel(MegaParams p) {
                 for (int q = 0; q < 4; q++)
                     reinterpret_cast<uint32_t*>(L.xq)[q * 512 + t] = pack4_i8(n16[4 * q], n16[4 * q + 1], n16[4 * q + 2], n16[4 * q + 3]);
             }
-            __syncthreads();
+            if (is_s) __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): both down rows of this stream wave have landed in LDS
+            __syncthreads();                               // ... and are visible to the wave that multiplies the odd one
             if (l == 1) fine();
-            if (is_s) {
-                __builtin_amdgcn_s_waitcnt(0);        // both down rows of this wave have landed in LDS
-#pragma unroll
-                for (int j = 0; j < 2; j++) {
-                    const int row = wg * 8 + sw * 2 + j;
-                    const int a0 = mega_dot_row_lds(L.wd[sw * 2 + j], L.xq, lane);
-                    if (lane == 0) st_f(&p.x[row], (float)a0 * sx * dsc[j] + xres[j]);
-                }
+            {
+                const int a0 = mega_dot_row_lds(L.wd[(wave & 3) * 2 + (is_s ? 0 : 1)], L.xq, lane);
+                if (lane == 0) st_f(&p.x[drow], (float)a0 * sx * dsc + xres);
             }
             if (l == 1) fine();
             if (l == 1) fine();
