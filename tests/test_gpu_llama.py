@@ -257,3 +257,42 @@ def test_generate_from_a_prompt_matches_the_oracle_flow(small, n_prompt):
     assert model.generate(prompt, steps, top_k=1, rands=np.full(steps, 0.5, np.float32)) == ref
     with pytest.raises(Exception, match="max_pos"):
         model.generate(prompt, cfg["max_pos"] + 1)
+
+
+def test_generate_with_sampling():
+    """Prompt of 40 tokens, then eight tokens drawn with top-5 sampling inside the persistent kernel, on a model whose
+    logits are of order one (several live candidates).  Each drawn id is what the oracle's sampler gives on the logits
+    of that very step (recomputed with decode_hidden from the previous id at the same position, which is bit for bit
+    the same forward pass): this pins the hand-over from the prompt, the indexing of the uniform numbers and the
+    feedback of the ids.  The first id is also among the five candidates of the oracle's own prefill + decode.  (The
+    full oracle flow is not compared id by id: a 40-token prefill carries a few rounding-tie flips, about 1e-2 of
+    the hidden state's scale, and with candidates this close a draw then lands on a neighbour within a few steps;
+    test_generate_from_a_prompt_matches_the_oracle_flow compares the whole flow on well-separated logits.)"""
+    import flexllm_amd as fx
+    from flexllm_amd import llama
+    from oracle import oracle
+    cfg = llama.make_config(layers=2, vocab=4096, max_pos=256)
+    host_w = llama.synth_weights(cfg, seed=13, device=False, embed_range=0.03)
+    model = llama.Llama(cfg, llama.synth_weights(cfg, seed=13, device=True, embed_range=0.03))
+    om = oracle.OracleModel(cfg, host_w)
+    r = np.random.default_rng(21)
+    prompt = r.integers(0, cfg["vocab"], 40).astype(np.int32)
+    steps, k = 8, 5
+    rands = r.uniform(0, 1, steps).astype(np.float32)
+    got = model.generate(prompt, steps, top_k=k, rands=rands)
+    ranks = []
+    for i in range(steps):
+        prev = int(prompt[-1]) if i == 0 else got[i - 1]
+        x = fx.ops.embed_f16(model._embed, fx.to_device(np.array([prev], np.int32)))
+        _, logits = model.decode_hidden(x, len(prompt) - 1 + i, want_logits=True)
+        t_ref, idx, val, prob = oracle.sample_topk(logits.numpy(), k, float(rands[i]), 8)
+        assert np.abs(np.cumsum(prob.astype(np.float64)) - rands[i]).min() > 1e-5
+        assert got[i] == t_ref, "step %d" % i
+        ranks.append(int(np.nonzero(idx == t_ref)[0][0]))
+    assert len(set(ranks)) >= 3, ranks
+    kc, vc = om.new_caches()
+    om.prefill(np.stack([oracle.embed(host_w["embed"], int(t)) for t in prompt[:-1]]), kc, vc)
+    _, logits0 = om.decode_token(oracle.embed(host_w["embed"], int(prompt[-1])), len(prompt) - 1, kc, vc)
+    _, idx0, _, _ = oracle.sample_topk(logits0, k, float(rands[0]), 8)
+    assert got[0] in idx0.tolist()
+    model.close()
