@@ -112,7 +112,9 @@ class Llama:
         prompt = np.ascontiguousarray(prompt, np.int32).reshape(-1)
         d_prompt = to_device(prompt)
         out = DeviceArray((max(int(steps), 1),), np.int32)
-        d_rands = to_device(np.ascontiguousarray(rands, np.float32)) if top_k else None
+        if top_k and rands is None:
+            raise ValueError("top-k sampling needs `rands`, one uniform number in [0,1) per step")
+        d_rands = to_device(np.ascontiguousarray(rands, np.float32).reshape(-1)) if top_k else None
         if top_k and d_rands.size < steps:
             raise ValueError("%d uniform numbers for %d steps" % (d_rands.size, steps))
         check(lib().flexllm_llama_generate(self.handle, C.c_void_p(d_prompt.ptr), int(prompt.size), int(steps),
