@@ -23,10 +23,10 @@ HBM_PEAK_GBS = 8000.0          # MI355X published HBM3E bandwidth
 INT8_PEAK_TOPS = 5000.0        # MI355X published dense int8 MFMA rate
 TOKENS_PER_LAUNCH = 64         # the library's cap on tokens per persistent-kernel launch (kMegaMaxSteps)
 # HBM traffic of the decode_mega_kernel per generated token at context ~4092, from two `rocprofv3 --pmc` runs of this
-# file with --steps 8 --warmup 0 (one 8-token launch: FETCH_SIZE 6,228,019 KiB, WRITE_SIZE 85,469 KiB per dispatch), each
+# file with --steps 8 --warmup 0 (one 8-token launch: FETCH_SIZE 6,228,140 KiB, WRITE_SIZE 71,144 KiB per dispatch), each
 # scaled by the same counter's reading for a plain 1 GiB device copy (FETCH_SIZE reads 524,302 KiB for 1,048,576 KiB
 # fetched -> x2.0; WRITE_SIZE reads 1,048,576 KiB -> x1.0).  Only valid for the default 16-layer model at context 4096.
-MEASURED_TRAFFIC_BYTES_PER_TOKEN = int((6228019.1 * 2.0 + 85469.1 * 1.0) * 1024 / 8)
+MEASURED_TRAFFIC_BYTES_PER_TOKEN = int((6228140.0 * 2.0 + 71144.2 * 1.0) * 1024 / 8)
 
 
 def bytes_per_token(cfg, mean_len):

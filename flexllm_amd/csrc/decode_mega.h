@@ -179,6 +179,7 @@ struct MegaLds {
     float bestv[kMegaWaves];
     int besti[kMegaWaves];
     float hst[32];                                     // SiLU(gate)*up of this workgroup's 32 row pairs, stream waves -> store wave
+    float res8[8];                                     // the workgroup's eight o_proj / down outputs, gathered for one store
     float tk_val[kTopKMax];                            // sampling: the selected candidates (this workgroup's, then the global ones)
     int tk_idx[kTopKMax];
     int tk_tok;
@@ -598,9 +599,13 @@ __global__ __launch_bounds__(kMegaT, 1) void decode_mega_kernel(MegaParams p) {
                 for (int j = 0; j < 2; j++) {
                     const int row = wg * 8 + wave + 4 * j;
                     const int a0 = mega_dot_row<2>(wr[j], L.xq, lane);
-                    if (lane == 0) st_f(&p.x2[row], (float)a0 * sx * wsc[j] + xr[j]);
+                    if (lane == 0) L.res8[wave + 4 * j] = (float)a0 * sx * wsc[j] + xr[j];
                 }
             }
+            // the workgroup's eight outputs leave as one 32-byte store: eight single-lane stores from four waves into
+            // the same sector take longer to be acknowledged, and the barrier waits for that
+            __syncthreads();
+            if (t < 8) st_f(&p.x2[wg * 8 + t], L.res8[t]);
             stamp();
             bar.arrive(!is_s);
         }
@@ -796,8 +801,10 @@ __global__ __launch_bounds__(kMegaT, 1) void decode_mega_kernel(MegaParams p) {
             if (l == 1) fine();
             {
                 const int a0 = mega_dot_row_lds(L.wd[(wave & 3) * 2 + (is_s ? 0 : 1)], L.xq, lane);
-                if (lane == 0) st_f(&p.x[drow], (float)a0 * sx * dsc + xres);
+                if (lane == 0) L.res8[drow - wg * 8] = (float)a0 * sx * dsc + xres;
             }
+            __syncthreads();
+            if (t < 8) st_f(&p.x[wg * 8 + t], L.res8[t]);            // one 32-byte store, as in phase 4
             if (l == 1) fine();
             if (l == 1) fine();
             stamp();
