@@ -47,7 +47,8 @@ constexpr int kMegaWG = 256;       // workgroups (persistent, one per CU)
 constexpr int kMegaT = 512;        // threads per workgroup
 constexpr int kMegaWaves = kMegaT / 64;
 constexpr int kMegaGroup = 32;     // workgroups per first-level barrier counter
-constexpr int kMegaSpinLimit = 1 << 22;
+constexpr int kMegaSpinLimit = 1 << 20;   // polls of ~1 us each: a wait that has not ended after a second never will
+constexpr int kMegaErrPeriod = 64;         // a spinning thread looks at the error flag every so many polls
 constexpr int kMegaMaxSteps = 64;  // tokens per launch in greedy mode (bounds the run time of one launch)
 
 struct MegaParams {
@@ -100,6 +101,14 @@ __device__ __forceinline__ void st_tagged(unsigned long long* p, float v, unsign
 __device__ __forceinline__ unsigned long long ld_u64(const unsigned long long* p) {
     return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
+// Called once per unsuccessful poll (wave-uniform): gives up when the limit is reached (raising the error flag) or when
+// another waiter has already raised it, so that one lost workgroup costs one time-out and not one per wait.
+__device__ __forceinline__ bool spin_should_stop(int it, int* err) {
+    if (it % kMegaErrPeriod != 0) return false;
+    if (ld_i(err) == 1) return true;
+    if (it >= kMegaSpinLimit) { st_i(err, 1); return true; }
+    return false;
+}
 // Polls two tagged words until both carry `tag` in every active lane of the wave (bounded: raises the error flag).
 __device__ __forceinline__ void poll_tagged2(const unsigned long long* a, const unsigned long long* b, unsigned tag,
                                              int* err, float& fa, float& fb) {
@@ -110,7 +119,7 @@ __device__ __forceinline__ void poll_tagged2(const unsigned long long* a, const 
         w1 = ld_u64(b);
         const bool ok = (unsigned)(w0 >> 32) == tag && (unsigned)(w1 >> 32) == tag;
         if (__builtin_amdgcn_ballot_w64(!ok) == 0) break;
-        if (++it > kMegaSpinLimit) { st_i(err, 1); break; }
+        if (spin_should_stop(++it, err)) break;
     }
     fa = __int_as_float((int)(unsigned)w0);
     fb = __int_as_float((int)(unsigned)w1);
@@ -137,6 +146,7 @@ struct GridBarrier {
     unsigned* mem;                              // [0] flag, [64] top counter, [128 + 64*g] group counters
     unsigned epoch;
     int* err;
+    bool dead = false;                          // thread 0 only: a wait timed out or the error flag was seen; later waits return at once
     // drain == false: the calling wave made no global store in this phase and may keep loads in flight
     __device__ __forceinline__ void arrive(bool drain = true) {
         if (drain) __builtin_amdgcn_s_waitcnt(0);          // this thread's stores have been acknowledged
@@ -153,11 +163,11 @@ struct GridBarrier {
         }
     }
     __device__ __forceinline__ void wait() {
-        if (threadIdx.x == 0) {
+        if (threadIdx.x == 0 && !dead) {
             int it = 0;
             // signed distance so that the comparison survives counter wrap-around
             while ((int)(__hip_atomic_load(&mem[0], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) - epoch) < 0) {
-                if (++it > kMegaSpinLimit) { st_i(err, 1); break; }
+                if (spin_should_stop(++it, err)) { dead = true; break; }
             }
         }
         __syncthreads();
@@ -183,6 +193,7 @@ struct MegaLds {
     float tk_val[kTopKMax];                            // sampling: the selected candidates (this workgroup's, then the global ones)
     int tk_idx[kTopKMax];
     int tk_tok;
+    int stop;                                          // set by thread 0 at the end of a step when the error flag is up: the launch ends there
     __attribute__((aligned(16))) int8_t wd[8][8192];   // this workgroup's 8 down rows, filled by global->LDS direct loads (64 KiB);
                                                        // the odd rows first hold gate/up rows 12..15 of their stream wave
     __attribute__((aligned(16))) int8_t gu2[4][8192];  // gate/up rows 8..11 of each stream wave (32 KiB)
@@ -322,7 +333,8 @@ __global__ __launch_bounds__(kMegaT, 1) void decode_mega_kernel(MegaParams p) {
 
     // Greedy mode runs several tokens in one launch: after the lm_head every workgroup reduces the per-workgroup
     // candidates itself, so all of them know the next token and position without a further exchange.
-    for (int step = 0; step < p.n_steps; step++) {
+    int steps_done = 0, stop = 0;
+    for (int step = 0; step < p.n_steps && !stop; step++) {
     const int pos = pos0 + step;
     const int len = pos + 1;
     stamp_i = 0;                                                  // a timeline holds the stamps of the last step
@@ -506,7 +518,7 @@ __global__ __launch_bounds__(kMegaT, 1) void decode_mega_kernel(MegaParams p) {
                             w1 = ld_u64(slot + 1);
                             const bool ok = (unsigned)(w0 >> 32) == bar.epoch && (unsigned)(w1 >> 32) == bar.epoch;
                             if (__builtin_amdgcn_ballot_w64(!ok) == 0) break;
-                            if (++it > kMegaSpinLimit) { if (lane == 0) st_i(bar.err, 1); break; }
+                            if (spin_should_stop(++it, bar.err)) break;
                         }
                         if (lane < nchunks) { m_c = __int_as_float((int)(unsigned)w0); l_c = __int_as_float((int)(unsigned)w1); }
                     }
@@ -597,7 +609,6 @@ __global__ __launch_bounds__(kMegaT, 1) void decode_mega_kernel(MegaParams p) {
             if (!is_s) {
 #pragma unroll
                 for (int j = 0; j < 2; j++) {
-                    const int row = wg * 8 + wave + 4 * j;
                     const int a0 = mega_dot_row<2>(wr[j], L.xq, lane);
                     if (lane == 0) L.res8[wave + 4 * j] = (float)a0 * sx * wsc[j] + xr[j];
                 }
@@ -908,10 +919,12 @@ __global__ __launch_bounds__(kMegaT, 1) void decode_mega_kernel(MegaParams p) {
                 float prob[kTopKMax];
                 const int sel = topk_sample_rank(L.tk_val, p.top_k, p.rands[p.state[1] + step], 1, prob);
                 const int chosen = L.tk_idx[sel];
-                L.tk_tok = chosen == 0x7fffffff ? 0 : chosen;
+                L.tk_tok = (unsigned)chosen < (unsigned)p.vocab ? chosen : 0;   // after a time-out the candidates may be anything
+                L.stop = bar.dead || ld_i(bar.err) == 1;
             }
             __syncthreads();
             tok = __builtin_amdgcn_readfirstlane(L.tk_tok);
+            stop = __builtin_amdgcn_readfirstlane(L.stop);
             if (wg == 0 && t == 0) p.tokens_out[p.state[1] + step] = tok;
             __syncthreads();                                        // L.tk_* and L.f are reused by the next step
         } else if (greedy) {
@@ -921,6 +934,7 @@ __global__ __launch_bounds__(kMegaT, 1) void decode_mega_kernel(MegaParams p) {
             float cv = -INFINITY;
             int ci = 0x7fffffff;
             if (t < kMegaWG) { cv = ld_f(&p.am_v[t]); ci = ld_i(&p.am_i[t]); }
+            if (t == 0) L.stop = bar.dead || ld_i(bar.err) == 1;   // fetched along with the candidates
 #pragma unroll
             for (int m = 1; m < 64; m <<= 1) {
                 const float ov = __shfl_xor(cv, m);
@@ -933,17 +947,19 @@ __global__ __launch_bounds__(kMegaT, 1) void decode_mega_kernel(MegaParams p) {
 #pragma unroll
             for (int i = 1; i < kMegaWG / 64; i++)
                 if (L.bestv[i] > cv || (L.bestv[i] == cv && L.besti[i] < ci)) { cv = L.bestv[i]; ci = L.besti[i]; }
-            tok = __builtin_amdgcn_readfirstlane(ci == 0x7fffffff ? 0 : ci);
+            tok = __builtin_amdgcn_readfirstlane((unsigned)ci < (unsigned)p.vocab ? ci : 0);   // after a time-out the candidates may be anything
+            stop = __builtin_amdgcn_readfirstlane(L.stop);
             if (wg == 0 && t == 0) p.tokens_out[p.state[1] + step] = tok;
             __syncthreads();                                        // L.bestv/besti are reused by the next step
         }
     } else {
         bar.wait();   // keep arrive/wait balanced: the last layer's x is complete when the kernel ends
     }
-    }   // step loop
+    steps_done = step + 1;
+    }   // step loop (left early only after a barrier time-out, which the error flag reports)
     if (wg == 0 && is_t0()) {
         p.state[2] = (int)bar.epoch;
-        if (greedy) { p.token[0] = tok; p.state[0] = pos0 + p.n_steps; p.state[1] += p.n_steps; }
+        if (greedy) { p.token[0] = tok; p.state[0] = pos0 + steps_done; p.state[1] += steps_done; }
     }
 #ifdef FX_MEGA_FINE_STAMPS
     if (p.timeline && is_t0()) p.timeline[p.n_layers * 12 + 2 + 64 + kMegaWG + wg] = wall_clock64();     // workgroup exit

@@ -325,6 +325,10 @@ int flexllm_llama_create(flexllm_llama** out, const flexllm_llama_config* cfg, c
     FX_TRY_HIP(hipMemset(m->bar, 0, sizeof(unsigned) * 64 * (2 + kMegaWG / kMegaGroup)));
     FX_TRY_HIP(hipMemset(m->state, 0, sizeof(int) * 4));
     FX_TRY_HIP(hipMemset(m->o_acc, 0, sizeof(int32_t) * H));
+    FX_TRY_HIP(hipMemset(m->am_v, 0, sizeof(float) * kArgmaxParts));
+    FX_TRY_HIP(hipMemset(m->am_i, 0, sizeof(int) * kArgmaxParts));
+    FX_TRY_HIP(hipMemset(m->topk_val, 0, sizeof(float) * kCandGroups * kTopKMax));
+    FX_TRY_HIP(hipMemset(m->topk_idx, 0, sizeof(int) * kCandGroups * kTopKMax));
     {
         int dev = 0, cus = 0;
         FX_TRY_HIP(hipGetDevice(&dev));
@@ -352,7 +356,13 @@ int flexllm_llama_destroy(flexllm_llama* m) {
 
 int flexllm_llama_set_decode_mode(flexllm_llama* m, int mode) {
     FX_REQUIRE(m && (mode == 0 || mode == 1), "llama_set_decode_mode: mode=%d (0 persistent kernel, 1 one kernel per stage)", mode);
-    if (m->decode_mode != mode && m->graph_exec) { (void)hipGraphExecDestroy(m->graph_exec); m->graph_exec = nullptr; }
+    if (m->decode_mode != mode) {
+        if (m->graph_exec) { (void)hipGraphExecDestroy(m->graph_exec); m->graph_exec = nullptr; }
+        // The persistent kernel only ever adds into the attention accumulators and clears them once they have been read,
+        // so it expects zeros at launch; the per-stage kernels clear them before use and leave the last layer's sums.
+        FX_HIP(hipDeviceSynchronize());
+        FX_HIP(hipMemset(m->o_acc, 0, sizeof(int32_t) * m->cfg.hidden));
+    }
     m->decode_mode = mode;
     return FLEXLLM_OK;
 }

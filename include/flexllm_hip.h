@@ -288,7 +288,9 @@ typedef struct {
 typedef struct flexllm_llama flexllm_llama;
 
 /* Copies/repacks the weights into the library's own device layout (fused qkv and gate/up rows) and
- * allocates the int8 KV cache [layers][max_pos][kv_hidden] x2 and the activation workspace. */
+ * allocates the int8 KV caches (per layer in the head-major layouts given above for flexllm_kv_append_i8:
+ * K [layers][kv_heads][max_pos][64], V [layers][kv_heads][max_pos/64][64 channels][64 positions]) and the
+ * activation workspace. */
 int flexllm_llama_create(flexllm_llama** out, const flexllm_llama_config* cfg, const flexllm_llama_weights* w);
 int flexllm_llama_destroy(flexllm_llama* m);
 /* Decode schedule: 0 (default) = one persistent kernel per token (all layers + lm_head, grid barriers between
@@ -303,7 +305,9 @@ int flexllm_llama_stage_timeline(flexllm_llama* m, long long* host_out, int max_
  * kernel that timed out (FLEXLLM_EHIP), or an input token id outside the vocabulary (FLEXLLM_EINVAL; token 0 was
  * used in its place, no row outside the embedding table is ever read).  Clears the flag. */
 int flexllm_llama_check(flexllm_llama* m);
-/* Device pointers to the int8 caches ([layers][max_pos][kv_hidden]) for inspection / pre-filling. */
+/* Device pointers to the int8 caches for inspection / pre-filling.  They are NOT token-major: layer l starts at byte
+ * l * kv_heads * max_pos * 64 of each, K as [kv_heads][max_pos][64], V as [kv_heads][max_pos/64][64 channels]
+ * [64 positions].  flexllm_kv_store_i8 writes token-major int8 rows [tokens][kv_heads][64] into one layer's pair. */
 int flexllm_llama_kv_cache(flexllm_llama* m, int8_t** k_cache, int8_t** v_cache);
 /* One decode step at position pos from fp32 embedding x_in (device, [hidden]); writes the residual
  * stream after the last layer to hidden_out (device, may be NULL) and, if logits != NULL, the fp32

@@ -6,6 +6,27 @@
 #include <math.h>
 #include <stdlib.h>
 #include <string.h>
+#ifdef _OPENMP
+#include <omp.h>
+#endif
+
+/* The loops over independent outputs (rows of a matrix product, heads and query rows of attention, vocabulary rows)
+ * are OpenMP loops: every output is computed by one thread with the same scalar code, so the results do not depend on
+ * the thread count.  fxo_set_threads(1) gives the single-core baseline. */
+void fxo_set_threads(int n) {
+#ifdef _OPENMP
+    omp_set_num_threads(n > 0 ? n : omp_get_num_procs());
+#else
+    (void)n;
+#endif
+}
+int fxo_max_threads(void) {
+#ifdef _OPENMP
+    return omp_get_max_threads();
+#else
+    return 1;
+#endif
+}
 
 /* ------------------------------------------------------------------ quant.h */
 
@@ -96,6 +117,7 @@ void fxo_head_quant_sym(const float* x, int rows, int heads, int dim, int bits, 
 /* ------------------------------------------------ Linear_Layer.h (int GEMM) */
 
 void fxo_linear_i8(const int8_t* a, const int8_t* w, int m, int k, int n, int32_t* c) {
+#pragma omp parallel for collapse(2) schedule(static)
     for (int i = 0; i < m; i++)
         for (int j = 0; j < n; j++) {
             const int8_t* ar = a + (size_t)i * k;
@@ -107,6 +129,7 @@ void fxo_linear_i8(const int8_t* a, const int8_t* w, int m, int k, int n, int32_
 }
 
 void fxo_linear_u8i8(const uint8_t* a, const int8_t* w, int m, int k, int n, int32_t* c) {
+#pragma omp parallel for collapse(2) schedule(static)
     for (int i = 0; i < m; i++)
         for (int j = 0; j < n; j++) {
             const uint8_t* ar = a + (size_t)i * k;
@@ -320,12 +343,15 @@ void fxo_mha_prefill(const float* q, const float* k, const float* v, int s, int 
     fxo_static_quant(q, s, q_heads, hd, sc->q_s, sqrtf((float)hd), 1, 8, q8);
     fxo_static_quant(k, s, kv_heads, hd, sc->k_s, 1.0f, 1, 8, k8);
     fxo_static_quant(v, s, kv_heads, hd, sc->v_s, 1.0f, 1, 8, v8);
+#pragma omp parallel
+    {
     float* row = (float*)malloc(sizeof(float) * s);
     float* prob = (float*)malloc(sizeof(float) * s);
     uint8_t* p8 = (uint8_t*)malloc((size_t)s);
+#pragma omp for collapse(2) schedule(dynamic, 8)
     for (int h = 0; h < q_heads; h++) {
-        const int kh = h / group;                                         /* MHA.h:96-106 */
         for (int i = 0; i < s; i++) {
+            const int kh = h / group;                                     /* MHA.h:96-106 */
             const int8_t* qi = q8 + ((size_t)i * q_heads + h) * hd;
             for (int j = 0; j < s; j++) {
                 const int8_t* kj = k8 + ((size_t)j * kv_heads + kh) * hd;
@@ -350,19 +376,24 @@ void fxo_mha_prefill(const float* q, const float* k, const float* v, int s, int 
                 }
         }
     }
+    free(row); free(prob); free(p8);
+    }
     if (q8_out) memcpy(q8_out, q8, (size_t)s * q_heads * hd);
     if (k8_out) memcpy(k8_out, k8, (size_t)s * kv_heads * hd);
     if (v8_out) memcpy(v8_out, v8, (size_t)s * kv_heads * hd);
-    free(q8); free(k8); free(v8); free(row); free(prob); free(p8);
+    free(q8); free(k8); free(v8);
 }
 
 void fxo_mha_decode(const int8_t* q8, const int8_t* k_cache, const int8_t* v_cache, int len,
                     int q_heads, int kv_heads, int hd, const fxo_mha_scales* sc,
                     uint8_t* p8_out, float* o) {
     const int group = q_heads / kv_heads;
+#pragma omp parallel
+    {
     float* row = (float*)malloc(sizeof(float) * len);
     float* prob = (float*)malloc(sizeof(float) * len);
     uint8_t* p8 = (uint8_t*)malloc((size_t)len);
+#pragma omp for schedule(static)
     for (int h = 0; h < q_heads; h++) {
         const int kh = h / group;
         const int8_t* qi = q8 + (size_t)h * hd;
@@ -388,6 +419,7 @@ void fxo_mha_decode(const int8_t* q8, const int8_t* k_cache, const int8_t* v_cac
             }
     }
     free(row); free(prob); free(p8);
+    }
 }
 
 /* --------------------------------------------------------- fp16 / lm_head */
@@ -412,6 +444,7 @@ void fxo_embed(const uint16_t* table, int hidden, int token, float* y) {
 }
 
 void fxo_lm_head(const uint16_t* table, int vocab, int hidden, const float* n, float* logits) {
+#pragma omp parallel for schedule(static)
     for (int v = 0; v < vocab; v++) {
         float acc = 0;
         for (int k = 0; k < hidden; k++) acc += fxo_half_to_float(table[(size_t)v * hidden + k]) * n[k];

@@ -24,6 +24,11 @@
 extern "C" {
 #endif
 
+/* Number of OpenMP threads for the loops over independent outputs (n <= 0: all processors).  Results do not depend
+ * on it. */
+void fxo_set_threads(int n);
+int fxo_max_threads(void);
+
 /* ---- quant.h ------------------------------------------------------------ */
 /* Modules/quant.h:6-112 (prefill) and :332-431 (decode), symmetric branch.
  * Pinned by: absmax element maps to +-(2^(b-1)-1), all-zero row gives s=1,

@@ -154,8 +154,11 @@ def mha_scales(qh=32, kvh=8, seed=3):
             r.uniform(0.02, 0.04, kvh).astype(np.float32), np.full(qh, 1.0 / 255, np.float32))
 
 
-@pytest.mark.parametrize("s,qh,kvh", [(32, 4, 1), (64, 8, 2), (160, 32, 8), (256, 32, 8)])
+@pytest.mark.parametrize("s,qh,kvh", [(32, 4, 1), (64, 8, 2), (160, 32, 8), (256, 32, 8), (1024, 32, 8), (1088, 4, 1), (2048, 4, 1)])
 def test_mha_prefill_vs_oracle(fx, oracle, s, qh, kvh):
+    """Probability bytes and outputs against the oracle, up to the benchmark's 1024 tokens x 32/8 heads (every row kept
+    in registers, `pf_attention_cached_kernel`) and, with fewer heads, rows of more than 1024 keys, which take the kernel
+    that recomputes the scores in its second pass (`pf_attention_kernel`)."""
     hd = 64
     q_s, k_s, v_s, a_s = mha_scales(qh, kvh)
     q = rng.standard_normal((s, qh, hd)).astype(np.float32)
@@ -177,8 +180,8 @@ def test_mha_prefill_vs_oracle(fx, oracle, s, qh, kvh):
     assert not np.triu(p, 1).any()                                   # causal: nothing above the diagonal
     # the integer P.V stage is exact given the kernel's own probability bytes
     group = qh // kvh
-    v8 = np.repeat(ref["v8"], group, axis=1).astype(np.int64)       # [s][qh][hd]
-    acc = np.einsum("hqk,khd->qhd", p.astype(np.int64), v8)
+    # (float64 matrix products of integers below 2^53: exact)
+    acc = np.stack([p[h].astype(np.float64) @ ref["v8"][:, h // group].astype(np.float64) for h in range(qh)], axis=1)
     o_from_p = (acc.astype(np.float32) * a_s[None, :, None]) * np.repeat(v_s, group)[None, :, None]
     assert np.array_equal(o.numpy(), o_from_p.astype(np.float32))
     flips = d.sum(-1).T[:, :, None]                                   # [s][qh][1]
