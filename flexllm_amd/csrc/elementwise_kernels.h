@@ -81,11 +81,14 @@ __global__ __launch_bounds__(kBlock) void quant_asym_kernel(const float* __restr
 }
 
 // ------------------------------------------------------------------ RMSNorm (+ optional quant)
-template <int VPT, bool QUANT>
-__global__ __launch_bounds__(kBlock) void rmsnorm_kernel(const float* __restrict__ x, const float* __restrict__ gamma,
+// BLOCK threads per row.  With BLOCK = 512 and VPT = 1 a 2048-row is reduced exactly as the persistent decode kernel
+// reduces it (four values per thread, wave butterflies, the eight wave sums added in order), so the one-kernel-per-
+// stage decode schedule and the persistent kernel agree bit for bit.
+template <int VPT, bool QUANT, int BLOCK = kBlock>
+__global__ __launch_bounds__(BLOCK) void rmsnorm_kernel(const float* __restrict__ x, const float* __restrict__ gamma,
                                                          float* __restrict__ y, int8_t* __restrict__ q,
                                                          float* __restrict__ s, int dim, float eps) {
-    __shared__ float red[kNW];
+    __shared__ float red[BLOCK / kWave];
     const int row = blockIdx.x;
     const int nvec = dim >> 2;
     const float4* xr = reinterpret_cast<const float4*>(x + (size_t)row * dim);
@@ -94,18 +97,18 @@ __global__ __launch_bounds__(kBlock) void rmsnorm_kernel(const float* __restrict
     float ss = 0.0f;
 #pragma unroll
     for (int i = 0; i < VPT; i++) {
-        const int idx = threadIdx.x + i * kBlock;
+        const int idx = threadIdx.x + i * BLOCK;
         if (idx < nvec) {
             v[i] = xr[idx];
             ss += (v[i].x * v[i].x + v[i].y * v[i].y) + (v[i].z * v[i].z + v[i].w * v[i].w);
         }
     }
-    ss = block_sum<kNW>(ss, red);
+    ss = block_sum<BLOCK / kWave>(ss, red);
     const float rms = 1.0f / sqrtf(ss / (float)dim + eps);
     float amax = 0.0f;
 #pragma unroll
     for (int i = 0; i < VPT; i++) {
-        const int idx = threadIdx.x + i * kBlock;
+        const int idx = threadIdx.x + i * BLOCK;
         if (idx < nvec) {
             const float4 g = gr[idx];
             v[i].x = v[i].x * rms * g.x;
@@ -119,13 +122,13 @@ __global__ __launch_bounds__(kBlock) void rmsnorm_kernel(const float* __restrict
         }
     }
     if constexpr (QUANT) {
-        amax = block_max<kNW>(amax, red);
+        amax = block_max<BLOCK / kWave>(amax, red);
         const float sc = sym_scale(amax, 127.0f);
         if (threadIdx.x == 0) s[row] = sc;
         uint32_t* qr = reinterpret_cast<uint32_t*>(q + (size_t)row * dim);
 #pragma unroll
         for (int i = 0; i < VPT; i++) {
-            const int idx = threadIdx.x + i * kBlock;
+            const int idx = threadIdx.x + i * BLOCK;
             if (idx < nvec) {
                 const float f[4] = {v[i].x, v[i].y, v[i].z, v[i].w};
                 int nq[4];

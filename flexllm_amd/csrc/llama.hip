@@ -142,7 +142,7 @@ static int decode_layer(flexllm_llama* m, int l, hipStream_t st) {
     int8_t* vc = m->v_cache + (size_t)l * m->cache_layer_bytes;
     int rc;
     // attention block
-    rmsnorm_kernel<2, true><<<1, kBlock, 0, st>>>(m->x, g0, nullptr, m->xq, m->xs, H, c.eps);
+    rmsnorm_kernel<1, true, 512><<<1, 512, 0, st>>>(m->x, g0, nullptr, m->xq, m->xs, H, c.eps);
     if ((rc = launch_gemv<kEpiDequant>(m->xq, w.wqkv, nullptr, m->xs, w.sqkv, nullptr, m->qkv, H, H + 2 * KV, st))) return rc;
     qkv_post_kernel<<<1, 256, 0, st>>>(m->qkv, m->rope_sin, m->rope_cos, q_s, k_s, v_s, m->q8, kc, vc, m->state, 0,
                                        c.q_heads, c.kv_heads, c.max_pos);
@@ -154,7 +154,7 @@ static int decode_layer(flexllm_llama* m, int l, hipStream_t st) {
     dec_out_quant_kernel<8><<<1, 256, 0, st>>>(m->o_acc, a_s, v_s, m->xq, m->xs, H, group);
     if ((rc = launch_gemv<kEpiDequant>(m->xq, w.wo, nullptr, m->xs, w.so, m->x, m->x2, H, H, st))) return rc;
     // feed-forward block
-    rmsnorm_kernel<2, true><<<1, kBlock, 0, st>>>(m->x2, g1, nullptr, m->xq, m->xs, H, c.eps);
+    rmsnorm_kernel<1, true, 512><<<1, 512, 0, st>>>(m->x2, g1, nullptr, m->xq, m->xs, H, c.eps);
     if ((rc = launch_gemv<kEpiSwiglu>(m->xq, w.wgu, nullptr, m->xs, w.sgu, nullptr, m->h, H, 2 * I, st))) return rc;
     fht_kernel<13, true><<<1, kFhtBlock, 0, st>>>(m->h, nullptr, m->xq, m->xs, c.fht_scale);
     if ((rc = launch_gemv<kEpiDequant>(m->xq, w.wd, nullptr, m->xs, w.sd, m->x2, m->x, I, H, st))) return rc;
@@ -164,7 +164,7 @@ static int decode_layer(flexllm_llama* m, int l, hipStream_t st) {
 
 static int decode_head(flexllm_llama* m, float* logits, hipStream_t st) {
     const flexllm_llama_config& c = m->cfg;
-    rmsnorm_kernel<2, false><<<1, kBlock, 0, st>>>(m->x, m->gamma + (size_t)(2 * c.layers) * c.hidden, m->nrm, nullptr,
+    rmsnorm_kernel<1, false, 512><<<1, 512, 0, st>>>(m->x, m->gamma + (size_t)(2 * c.layers) * c.hidden, m->nrm, nullptr,
                                                    nullptr, c.hidden, c.eps);
     return lm_head_launch(m->embed, m->nrm, logits, c.vocab, c.hidden, st);
 }

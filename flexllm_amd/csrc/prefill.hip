@@ -61,7 +61,7 @@ int llama_prefill_run(const flexllm_llama_config& c, const LayerW* layers, const
         int8_t* kc = k_cache + (size_t)l * cache_layer_bytes;
         int8_t* vc = v_cache + (size_t)l * cache_layer_bytes;
         // attention block
-        rmsnorm_kernel<2, true><<<s, kBlock, 0, st>>>(b.x, g0, nullptr, b.xq, b.xs, H, c.eps);
+        rmsnorm_kernel<1, true, 512><<<s, 512, 0, st>>>(b.x, g0, nullptr, b.xq, b.xs, H, c.eps);
         {   // q/k/v projection with RoPE, static quantisation and the cache stores in the GEMM epilogue
             QkvEpiArgs qa;
             qa.sin_t = rope_sin; qa.cos_t = rope_cos; qa.q_s = q_s; qa.k_s = k_s; qa.v_s = v_s;
@@ -73,7 +73,7 @@ int llama_prefill_run(const flexllm_llama_config& c, const LayerW* layers, const
         quant_sym_kernel<2><<<s, kBlock, 0, st>>>(b.att, b.xq, b.xs, H);
         if ((rc = launch_gemm<kGemmDequant>(b.xq, w.wo, nullptr, b.xs, w.so, b.x, b.x2, s, H, H, st))) return rc;
         // feed-forward block
-        rmsnorm_kernel<2, true><<<s, kBlock, 0, st>>>(b.x2, g1, nullptr, b.xq, b.xs, H, c.eps);
+        rmsnorm_kernel<1, true, 512><<<s, 512, 0, st>>>(b.x2, g1, nullptr, b.xq, b.xs, H, c.eps);
         if ((rc = launch_gemm_swiglu(b.xq, w.wgu, b.xs, w.sgu, b.gu, s, H, 2 * I, st))) return rc;     // b.gu = SiLU(gate)*up [s][I]
         fht_kernel<13, true, false><<<s, kFhtBlock, 0, st>>>(b.gu, nullptr, b.xq, b.xs, c.fht_scale);
         if ((rc = launch_gemm<kGemmDequant>(b.xq, w.wd, nullptr, b.xs, w.sd, b.x2, b.x, s, I, H, st))) return rc;

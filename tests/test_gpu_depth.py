@@ -126,7 +126,7 @@ def test_prefill_16_layers_teacher_forced(full):
     r = np.random.default_rng(42)
     x = r.standard_normal((S, H)).astype(np.float32)
     cfg1 = llama.make_config(layers=1, vocab=256, max_pos=128)
-    flipped_tokens, worst = 0, 0.0
+    beyond, worst, medians = 0, 0.0, []
     for l in range(L):
         print("layer", l, flush=True)
         hw = layer_views(cfg, host_w, l, 256, device=False)
@@ -142,12 +142,18 @@ def test_prefill_16_layers_teacher_forced(full):
         kg, vg = m1.caches_token_major()
         dk = np.abs(kg[0, :S].astype(int) - k1[0, :S]); dv = np.abs(vg[0, :S].astype(int) - v1[0, :S])
         assert dk.max() <= 1 and dv.max() <= 1
-        n_flip = int((e > 2e-5).sum())
-        print("  tokens beyond fp32 rounding: %d, worst %.1e, cache bytes off by one: %d" % (n_flip, e.max(), int((dk != 0).sum() + (dv != 0).sum())), flush=True)
-        flipped_tokens += n_flip; worst = max(worst, float(e.max()))
+        n_beyond = int((e > 2e-5).sum())
+        print("  tokens beyond fp32 rounding: %d, median %.1e, worst %.1e, cache bytes off by one: %d"
+              % (n_beyond, np.median(e), e.max(), int((dk != 0).sum() + (dv != 0).sum())), flush=True)
+        beyond += n_beyond; worst = max(worst, float(e.max())); medians.append(float(np.median(e)))
         m1.close()
         x = y_ref
-    assert flipped_tokens <= 0.1 * L * S and worst <= 2e-2, (flipped_tokens, worst)
+    # A layer makes about 1.1 million roundings to int8 / uint8 on 64 tokens; the few that sit on a tie may fall the other
+    # way (one step), and a flipped byte of a token's K or V row also touches every later token of that layer through
+    # attention, by much less.  So: most tokens exact to fp32 rounding, every layer's typical token exact (at most one
+    # layer where an early token's cache byte flipped), nothing beyond the effect of single steps.
+    assert beyond <= 0.2 * L * S and worst <= 2e-2, (beyond, worst)
+    assert sum(m <= 2e-5 for m in medians) >= L - 1, medians
 
 
 def test_256_token_greedy_run_both_schedules(full):
@@ -195,10 +201,12 @@ def two_layer():
 def test_run_across_a_key_chunk_boundary(two_layer, top_k):
     """80 tokens from position 100 on the persistent kernel: the first launch (64 tokens) crosses position 127 -> 128,
     where a second workgroup per KV head becomes active and takes over the new token's cache row in mid-launch; the
-    run spans two launches.  Checked (a) against the one-kernel-per-stage schedule (ids and cache bytes identical)
-    and (b) against the oracle, teacher-forced on the device's ids: at every step the device's id must be the
-    oracle's choice, or - where a rounding tie moved the device's logits - a candidate the oracle's logits put within
-    the tie effect of its choice; the oracle's cache rows must equal the device's up to single steps."""
+    run spans two launches.  Checked (a) against the one-kernel-per-stage schedule (ids and cache bytes identical);
+    (b) step by step: a third model is fed the run's ids one decode step at a time, which is bit for bit the same forward
+    pass - its logits must select the run's next id (arg-max, or the oracle's sampler on those logits with the same
+    uniform number), which pins the in-kernel selection, the hand-over of the id and the indexing of the uniform numbers;
+    (c) against the oracle, teacher-forced on the same ids and cache bytes: logits to fp32 rounding at the typical
+    step and within the tie effect at every step, appended cache rows equal up to single steps."""
     fx, llama, oracle, cfg, dev_w, host_w = two_layer
     steps, pos0, first = 80, 100, 333
     r = np.random.default_rng(5)
@@ -226,25 +234,42 @@ def test_run_across_a_key_chunk_boundary(two_layer, top_k):
     assert len(set(ga.tolist())) > 10
     om = oracle.OracleModel(cfg, host_w)
     kr, vr = kc.copy(), vc.copy()
-    t, near = first, 0
+    step_model = llama.Llama(cfg, dev_w)
+    step_model.load_caches_token_major(kc, vc)
+    t, errs, skipped, row_flips = first, [], 0, 0
     for i in range(steps):
-        _, logits = om.decode_token(oracle.embed(host_w["embed"], t), pos0 + i, kr, vr)
+        x = fx.ops.embed_f16(step_model._embed, fx.to_device(np.array([t], np.int32)))
+        _, lg = step_model.decode_hidden(x, pos0 + i, want_logits=True)
+        lg = lg.numpy()
         if top_k:
-            want, idx, val, prob = oracle.sample_topk(logits, top_k, float(rands[i]), 8)
-            ok = int(ga[i]) == want
-            if not ok:      # a draw next to a boundary of the cumulative distribution, or a candidate list reordered by a tie
-                assert int(ga[i]) in idx.tolist(), "step %d: %d is not among the oracle's candidates %s" % (i, ga[i], idx)
+            want, idx, val, prob = oracle.sample_topk(lg, top_k, float(rands[i]), 8)
+            if np.abs(np.cumsum(prob.astype(np.float64)) - rands[i]).min() > 1e-5:      # device expf against glibc at a boundary
+                assert int(ga[i]) == want, "step %d" % i
+            else:
+                skipped += 1
         else:
-            want = int(np.argmax(logits))
-            ok = int(ga[i]) == want
-            if not ok:
-                assert logits[want] - logits[int(ga[i])] <= 2e-2 * np.abs(logits).max(), "step %d: %d against %d" % (i, ga[i], want)
-        near += not ok
+            assert int(ga[i]) == int(np.argmax(lg)), "step %d" % i
+        _, logits = om.decode_token(oracle.embed(host_w["embed"], t), pos0 + i, kr, vr)
+        errs.append(float(token_err(lg[None], logits[None])[0]))
+        # the cache rows this step appended: equal up to a single step where a rounding tie fell the other way; the
+        # oracle then continues on the device's bytes, so that each step is judged on identical history
+        ks, vs = step_model.caches_token_major()
+        for dev, ref in ((ks, kr), (vs, vr)):
+            d = np.abs(dev[:, pos0 + i].astype(int) - ref[:, pos0 + i])
+            assert d.max() <= 1
+            row_flips += int((d != 0).sum())
+            ref[:, pos0 + i] = dev[:, pos0 + i]
         t = int(ga[i])
-    assert near <= 3, "%d steps disagree with the oracle's first choice" % near
+    step_model.check()
+    errs = np.array(errs)
+    print("logit errors against the oracle: median %.1e, max %.1e, steps beyond 2e-3: %d; cache bytes off by one: %d"
+          % (np.median(errs), errs.max(), (errs > 2e-3).sum(), row_flips), flush=True)
     n = pos0 + steps
-    dk = np.abs(ka[:, :n].astype(int) - kr[:, :n]); dv = np.abs(va[:, :n].astype(int) - vr[:, :n])
-    assert dk.max() <= 1 and dv.max() <= 1 and (dk != 0).mean() < 2e-3 and (dv != 0).mean() < 2e-3
+    assert skipped <= 1 and np.median(errs) <= 1e-4 and errs.max() <= 3e-2 and (errs > 2e-3).mean() <= 0.1
+    assert row_flips <= 5e-3 * steps * 2 * cfg["layers"] * cfg["kv_hidden"]       # a flip in layer 0 moves many bytes of layer 1's rows
+    ks, vs = step_model.caches_token_major()
+    assert np.array_equal(ks, ka) and np.array_equal(vs, va)                             # the same forward passes indeed
+    step_model.close()
     assert not ka[:, n:].any() and not va[:, n:].any()
 
 
