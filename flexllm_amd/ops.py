@@ -293,6 +293,15 @@ def mha_i8_decode(q8, k_cache, v_cache, scales, length, want_p=False, stream=Non
     return o, p8
 
 
+def mha_i8_decode_noalloc(q8, k_cache, v_cache, scales, length, o, p8=None, stream=None):
+    """flexllm_mha_i8_decode on the library's built-in scratch: the caller passes the outputs, nothing is allocated."""
+    qh, hd = q8.shape
+    kvh, max_pos, _ = k_cache.shape
+    check(lib().flexllm_mha_i8_decode_noalloc(_p(q8), _p(k_cache), _p(v_cache), scales.ref(), _p(o), _p(p8), length, qh, kvh,
+                                              hd, max_pos, _s(stream)))
+    return o, p8
+
+
 def mha_i8_prefill(q8, k_cache, v_cache, scales, want_p=False, stream=None):
     s, qh, hd = q8.shape
     kvh, max_pos, _ = k_cache.shape

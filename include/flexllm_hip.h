@@ -237,6 +237,16 @@ int flexllm_kv_store_i8(const int8_t* k8, const int8_t* v8, int8_t* k_cache, int
 int flexllm_mha_i8_decode(const int8_t* q8, const int8_t* k_cache, const int8_t* v_cache,
                           const flexllm_mha_scales* sc, float* o, uint8_t* p8_out, int len, int q_heads,
                           int kv_heads, int head_dim, int max_pos, void* stream);
+/* flexllm_mha_i8_decode for callers that cannot allocate device memory (code under HIP graph capture, serving loops,
+ * harnesses that forbid hipMalloc): same arguments, same kernels and bit-identical results, but the scratch (scores,
+ * chunk statistics, accumulators: 1 072 KiB) is a fixed array inside the loaded library, one copy per GPU, and the call
+ * makes no hipMalloc / hipFree.  It has no counterpart in the reference.  Limits: q_heads <= 32, len <= 8192; larger
+ * sizes are rejected with FLEXLLM_EINVAL.  All calls on one GPU share that GPU's array: calls that may overlap on one
+ * GPU (different streams) race and must be serialised by the caller.  The first call on a device looks up the array's
+ * address (no allocation); make it outside a graph capture. */
+int flexllm_mha_i8_decode_noalloc(const int8_t* q8, const int8_t* k_cache, const int8_t* v_cache,
+                                  const flexllm_mha_scales* sc, float* o, uint8_t* p8_out, int len, int q_heads,
+                                  int kv_heads, int head_dim, int max_pos, void* stream);
 /* Prefill causal attention over s tokens (positions 0..s-1): q8 [s][q_heads][64] int8; K and V are read from
  * the cache layouts above (filled by flexllm_kv_append_i8 / flexllm_kv_store_i8); o fp32 [s][q_heads][64].
  * Replaces SpinQuant_Llama_32_1B/MHA_i8xi8.h:369-427 from the qxk stage on (pref_MHA_i8xi8_qxk_template,
