@@ -19,6 +19,11 @@ class MhaScales(C.Structure):
     _fields_ = [("q_s", C.c_void_p), ("k_s", C.c_void_p), ("v_s", C.c_void_p), ("a_s", C.c_void_p)]
 
 
+class MhaDynScales(C.Structure):
+    _fields_ = [("q_s", C.c_void_p), ("k_s", C.c_void_p), ("v_s", C.c_void_p), ("v_ch_s", C.c_void_p),
+                ("q_scale_div", C.c_float)]
+
+
 class LlamaConfig(C.Structure):
     _fields_ = [(n, C.c_int) for n in
                 ("layers", "hidden", "kv_hidden", "inter", "q_heads", "kv_heads", "head_dim", "vocab", "max_pos")] + \

@@ -5,7 +5,7 @@ import ctypes as C
 
 import numpy as np
 
-from ._lib import lib, check, MhaScales
+from ._lib import lib, check, MhaScales, MhaDynScales
 from .device import DeviceArray, _s, to_device
 
 
@@ -310,6 +310,36 @@ def mha_i8_prefill(q8, k_cache, v_cache, scales, want_p=False, stream=None):
     check(lib().flexllm_mha_i8_prefill(_p(q8), _p(k_cache), _p(v_cache), scales.ref(), _p(o), _p(p8), s, qh, kvh, hd,
                                        max_pos, _s(stream)))
     return o, p8
+
+
+def _dyn_scales(q_s, k_s, v_s, v_ch_s, q_scale_div):
+    return MhaDynScales(q_s.ptr, k_s.ptr, v_s.ptr, v_ch_s.ptr if v_ch_s is not None else None, float(q_scale_div))
+
+
+def mha_i8_prefill_dyn(q8, q_s, k_cache, k_s, v_cache, v_s, v_ch_s=None, q_scale_div=8.0, want_p=False, stream=None):
+    """Attention with dynamic per-(token, head) scales: q_s [s][qh], k_s / v_s [max_pos][kvh] device arrays of the
+    quantiser's scales.  Returns (o, p8 int8 [qh][s][s] or None, p_s [s][qh])."""
+    s, qh, hd = q8.shape
+    kvh, max_pos, _ = k_cache.shape
+    o = DeviceArray((s, qh, hd), np.float32)
+    p8 = DeviceArray((qh, s, s), np.int8).zero_() if want_p else None
+    p_s = DeviceArray((s, qh), np.float32)
+    sc = _dyn_scales(q_s, k_s, v_s, v_ch_s, q_scale_div)
+    check(lib().flexllm_mha_i8_prefill_dyn(_p(q8), _p(k_cache), _p(v_cache), C.byref(sc), _p(o), _p(p8), _p(p_s), s, qh, kvh, hd,
+                                           max_pos, _s(stream)))
+    return o, p8, p_s
+
+
+def mha_i8_decode_dyn(q8, q_s, k_cache, k_s, v_cache, v_s, length, v_ch_s=None, q_scale_div=8.0, want_p=False, stream=None):
+    qh, hd = q8.shape
+    kvh, max_pos, _ = k_cache.shape
+    o = DeviceArray((qh, hd), np.float32)
+    p8 = DeviceArray((qh, length), np.int8) if want_p else None
+    p_s = DeviceArray((qh,), np.float32)
+    sc = _dyn_scales(q_s, k_s, v_s, v_ch_s, q_scale_div)
+    check(lib().flexllm_mha_i8_decode_dyn(_p(q8), _p(k_cache), _p(v_cache), C.byref(sc), _p(o), _p(p8), _p(p_s), length, qh, kvh,
+                                          hd, max_pos, _s(stream)))
+    return o, p8, p_s
 
 
 # ---------------------------------------------------------------- Logits.h (greedy)

@@ -257,6 +257,33 @@ int flexllm_mha_i8_prefill(const int8_t* q8, const int8_t* k_cache, const int8_t
                            const flexllm_mha_scales* sc, float* o, uint8_t* p8_out, int s, int q_heads,
                            int kv_heads, int head_dim, int max_pos, void* stream);
 
+/* ---- attention with dynamic per-(token, head) scales ---------------------------------------------------------
+ * Q, K and V quantised by flexllm_head_quant_sym_i8 (dec_MHA_quant_layer_fp32_qint<8,false>, Modules/quant.h:527-617):
+ * one scale per token and head.  Scores are dequantised per key, a[i][j] = (float(q8_i.k8_j) * Q_s[i][h]) * K_s[j][kvh]
+ * (the per-token scale streams of Modules/quant.h:165-246 and the K scale cache of Modules/MHA.h:9-71, :393-445) with
+ * Q_s = q_s / q_scale_div (sqrt(head_dim) = 8: the factor the static path folds into Q's scale).  V's per-token scale
+ * is folded into the probabilities before they are quantised with the same symmetric quantiser:
+ * p'[j] = softmax(a)[j] * V_s[j][kvh], s_p = max_j p'[j] / 127, P8 = round(p'/s_p) (int8, 0..127),
+ * o[d] = float(sum_j P8[j]*v8[j][d]) * s_p, times v_ch_s[kvh][d] when the reference library's per-channel V scale
+ * (Modules/MHA.h:713-738) is given.  K and V are read from the cache layouts of flexllm_kv_store_i8. */
+typedef struct {
+    const float* q_s;      /* prefill: [s][q_heads]; decode: [q_heads]: the quantiser's scales of q */
+    const float* k_s;      /* [max_pos][kv_heads]: K scale cache, one scale per position and KV head */
+    const float* v_s;      /* [max_pos][kv_heads]: V scale cache */
+    const float* v_ch_s;   /* optional [kv_heads][64] per-channel factor on the output, or NULL */
+    float q_scale_div;     /* 8.0f for head_dim 64 */
+} flexllm_mha_dyn_scales;
+/* Causal prefill over s tokens (positions 0..s-1); q8 [s][q_heads][64]; o fp32 [s][q_heads][64]; optional outputs
+ * p8_out int8 [q_heads][s][s] (zero-filled by the caller) and p_s_out fp32 [s][q_heads].  s % 32 == 0. */
+int flexllm_mha_i8_prefill_dyn(const int8_t* q8, const int8_t* k_cache, const int8_t* v_cache,
+                               const flexllm_mha_dyn_scales* sc, float* o, int8_t* p8_out, float* p_s_out, int s,
+                               int q_heads, int kv_heads, int head_dim, int max_pos, void* stream);
+/* One query token against len cached positions; q8 [q_heads][64]; optional p8_out int8 [q_heads][len], p_s_out
+ * [q_heads].  len <= 8192, q_heads/kv_heads <= 4.  Uses a library-owned scratch buffer like flexllm_mha_i8_decode. */
+int flexllm_mha_i8_decode_dyn(const int8_t* q8, const int8_t* k_cache, const int8_t* v_cache,
+                              const flexllm_mha_dyn_scales* sc, float* o, int8_t* p8_out, float* p_s_out, int len,
+                              int q_heads, int kv_heads, int head_dim, int max_pos, void* stream);
+
 /* ---- Logits.h (greedy and top-k sampling) ---------------------------------------------- */
 /* logits[v] = sum_k fp16(E[v][k]) * n[k] (fp32 accumulate): tied fp16 lm_head GEMV. */
 int flexllm_lm_head_f16(const uint16_t* embed, const float* n, float* logits, int vocab, int hidden, void* stream);

@@ -422,6 +422,109 @@ void fxo_mha_decode(const int8_t* q8, const int8_t* k_cache, const int8_t* v_cac
     }
 }
 
+/* ------------------------------------- attention with dynamic per-(token, head) scales */
+
+/* One row: scores a[0..n) (masked entries -1e32) -> softmax -> fold V's per-token scale -> symmetric dynamic quant
+ * (quant.h:578-615 on the row: absmax / 127, 0 -> 1) -> P.V -> dequant.  v8/v_s are indexed [j][kvh]. */
+static void dyn_row_tail(const float* row, int n, int n_alloc, const int8_t* v8, const float* v_s, const float* v_ch_s,
+                         int kv_heads, int kh, int hd, float* prob, int8_t* p8, float* p_s_out, float* o) {
+    (void)n_alloc;
+    softmax_row(row, n, prob);
+    float vmax = (float)-1e32, vmin = (float)1e32;
+    for (int j = 0; j < n; j++) {
+        prob[j] = prob[j] * v_s[(size_t)j * kv_heads + kh];
+        if (prob[j] > vmax) vmax = prob[j];                               /* quant.h:548-553 */
+        if (prob[j] < vmin) vmin = prob[j];
+    }
+    float amax = fabsf(vmax), amin = fabsf(vmin);
+    float sp = (amax > amin ? amax : amin) / 127.0f;                      /* quant.h:600-603 */
+    if (sp == 0) sp = 1;
+    for (int j = 0; j < n; j++) p8[j] = (int8_t)(int)roundf(prob[j] / sp); /* quant.h:611-612 */
+    if (p_s_out) *p_s_out = sp;
+    if (o)
+        for (int d = 0; d < hd; d++) {
+            int32_t acc = 0;
+            for (int j = 0; j < n; j++) acc += (int32_t)p8[j] * (int32_t)v8[((size_t)j * kv_heads + kh) * hd + d];
+            float t = (float)acc * sp;                                    /* quant.h:646-647 */
+            o[d] = v_ch_s ? t * v_ch_s[kh * hd + d] : t;
+        }
+}
+
+void fxo_mha_prefill_dyn(const float* q, const float* k, const float* v, int s, int q_heads, int kv_heads, int hd,
+                         const float* v_ch_s, int8_t* q8_out, float* q_s_out, int8_t* k8_out, float* k_s_out,
+                         int8_t* v8_out, float* v_s_out, int8_t* p8_out, float* p_s_out, float* o) {
+    const int group = q_heads / kv_heads;
+    int8_t* q8 = (int8_t*)malloc((size_t)s * q_heads * hd);
+    int8_t* k8 = (int8_t*)malloc((size_t)s * kv_heads * hd);
+    int8_t* v8 = (int8_t*)malloc((size_t)s * kv_heads * hd);
+    float* qs = (float*)malloc(sizeof(float) * (size_t)s * q_heads);
+    float* ks = (float*)malloc(sizeof(float) * (size_t)s * kv_heads);
+    float* vs = (float*)malloc(sizeof(float) * (size_t)s * kv_heads);
+    fxo_head_quant_sym(q, s, q_heads, hd, 8, q8, qs);
+    fxo_head_quant_sym(k, s, kv_heads, hd, 8, k8, ks);
+    fxo_head_quant_sym(v, s, kv_heads, hd, 8, v8, vs);
+    const float root = sqrtf((float)hd);
+    for (int i = 0; i < s * q_heads; i++) qs[i] = qs[i] / root;
+#pragma omp parallel
+    {
+    float* row = (float*)malloc(sizeof(float) * s);
+    float* prob = (float*)malloc(sizeof(float) * s);
+    int8_t* p8 = (int8_t*)malloc((size_t)s);
+#pragma omp for collapse(2) schedule(dynamic, 8)
+    for (int h = 0; h < q_heads; h++)
+        for (int i = 0; i < s; i++) {
+            const int kh = h / group;
+            const int8_t* qi = q8 + ((size_t)i * q_heads + h) * hd;
+            for (int j = 0; j < s; j++) {
+                const int8_t* kj = k8 + ((size_t)j * kv_heads + kh) * hd;
+                int32_t acc = 0;
+                for (int d = 0; d < hd; d++) acc += (int32_t)qi[d] * (int32_t)kj[d];
+                float a = (float)acc * qs[(size_t)i * q_heads + h] * ks[(size_t)j * kv_heads + kh];   /* quant.h:240 */
+                row[j] = (j <= i) ? a : (float)-1e32;
+            }
+            dyn_row_tail(row, s, s, v8, vs, v_ch_s, kv_heads, kh, hd, prob, p8,
+                         p_s_out ? p_s_out + (size_t)i * q_heads + h : NULL,
+                         o ? o + ((size_t)i * q_heads + h) * hd : NULL);
+            if (p8_out) memcpy(p8_out + ((size_t)h * s + i) * s, p8, (size_t)s);
+        }
+    free(row); free(prob); free(p8);
+    }
+    if (q8_out) memcpy(q8_out, q8, (size_t)s * q_heads * hd);
+    if (k8_out) memcpy(k8_out, k8, (size_t)s * kv_heads * hd);
+    if (v8_out) memcpy(v8_out, v8, (size_t)s * kv_heads * hd);
+    if (q_s_out) memcpy(q_s_out, qs, sizeof(float) * (size_t)s * q_heads);
+    if (k_s_out) memcpy(k_s_out, ks, sizeof(float) * (size_t)s * kv_heads);
+    if (v_s_out) memcpy(v_s_out, vs, sizeof(float) * (size_t)s * kv_heads);
+    free(q8); free(k8); free(v8); free(qs); free(ks); free(vs);
+}
+
+void fxo_mha_decode_dyn(const int8_t* q8, const float* q_s, const int8_t* k_cache, const float* k_s,
+                        const int8_t* v_cache, const float* v_s, const float* v_ch_s, int len, int q_heads,
+                        int kv_heads, int hd, int8_t* p8_out, float* p_s_out, float* o) {
+    const int group = q_heads / kv_heads;
+#pragma omp parallel
+    {
+    float* row = (float*)malloc(sizeof(float) * len);
+    float* prob = (float*)malloc(sizeof(float) * len);
+    int8_t* p8 = (int8_t*)malloc((size_t)len);
+#pragma omp for schedule(static)
+    for (int h = 0; h < q_heads; h++) {
+        const int kh = h / group;
+        const int8_t* qi = q8 + (size_t)h * hd;
+        for (int j = 0; j < len; j++) {
+            const int8_t* kj = k_cache + ((size_t)j * kv_heads + kh) * hd;
+            int32_t acc = 0;
+            for (int d = 0; d < hd; d++) acc += (int32_t)qi[d] * (int32_t)kj[d];
+            row[j] = (float)acc * q_s[h] * k_s[(size_t)j * kv_heads + kh];
+        }
+        dyn_row_tail(row, len, len, v_cache, v_s, v_ch_s, kv_heads, kh, hd, prob, p8, p_s_out ? p_s_out + h : NULL,
+                     o ? o + (size_t)h * hd : NULL);
+        if (p8_out) memcpy(p8_out + (size_t)h * len, p8, (size_t)len);
+    }
+    free(row); free(prob); free(p8);
+    }
+}
+
 /* --------------------------------------------------------- fp16 / lm_head */
 
 float fxo_half_to_float(uint16_t h) {

@@ -114,6 +114,31 @@ void fxo_mha_decode(const int8_t* q8, const int8_t* k_cache, const int8_t* v_cac
                     int q_heads, int kv_heads, int head_dim, const fxo_mha_scales* sc,
                     uint8_t* p8, float* o);
 
+/* Attention with DYNAMIC per-(token, head) scales, the library's own quantiser (Modules/quant.h:527-617,
+ * dec_MHA_quant_layer_fp32_qint<8,false>: s = absmax/127, 0 -> 1) applied to Q, K, V and to the probabilities, with the
+ * per-token scale streams of Modules/quant.h:165-246 (pref_static_sym_quant/dequant_layer: score = acc * s_q[token] *
+ * s_k[key]) and the K scale cache of Modules/MHA.h:9-71, :393-445.
+ *   q8, s_q = quant(q[t][h]);  Q_s = s_q / sqrt(head_dim)   (the factor the static path folds into Q's scale)
+ *   k8, K_s[t][kvh];  v8, V_s[t][kvh]
+ *   a[i][j] = (float(q8_i . k8_j) * Q_s[i][h]) * K_s[j][kvh];  causal mask -1e32;  softmax (Softmax.h)
+ *   p'[j] = p[j] * V_s[j][kvh]      V's per-token scale varies along the reduction of P.V, so it is folded into the
+ *                                    probabilities before they are quantised (the reference library keeps V's scale
+ *                                    per channel and static, Modules/MHA.h:713-738, and has no per-token V path)
+ *   P8, s_p = quant(p')              int8 in 0..127, one scale per (query, head)
+ *   o[i][h][d] = float(sum_j P8[j] * v8[j][d]) * s_p  (* v_ch_s[kvh][d] when a per-channel V scale is given)
+ * Outputs (any may be NULL): q8 [s][qh][hd], q_s [s][qh] (= Q_s), k8/v8 [s][kvh][hd], k_s/v_s [s][kvh],
+ * p8 [qh][s][s] int8, p_s [s][qh], o [s][qh][hd].  v_ch_s: optional [kvh][hd] input.
+ * Pinned by: float64 fake-quant golden built like MHA_i8xi8_prefilling_tb.cpp:26-218 with per-token scales (each
+ * of the three facts above switched off once must be noticed), decode == prefill row bit for bit, the per-channel
+ * factor as an exact float32 product. */
+void fxo_mha_prefill_dyn(const float* q, const float* k, const float* v, int s, int q_heads, int kv_heads, int head_dim,
+                         const float* v_ch_s, int8_t* q8, float* q_s, int8_t* k8, float* k_s, int8_t* v8, float* v_s,
+                         int8_t* p8, float* p_s, float* o);
+/* One query against len cached keys: q8 [qh][hd] with Q_s [qh]; caches [len][kvh][hd] with K_s, V_s [len][kvh]. */
+void fxo_mha_decode_dyn(const int8_t* q8, const float* q_s, const int8_t* k_cache, const float* k_s,
+                        const int8_t* v_cache, const float* v_s, const float* v_ch_s, int len, int q_heads,
+                        int kv_heads, int head_dim, int8_t* p8, float* p_s, float* o);
+
 /* ---- Llama-3.2-1B W8A8 layer / model (graph order of SpinQuant_Prefilling.h:940-1049 and
  *      SpinQuant_Decoding_mem_opt.h:1050-1126 with int8 symmetric linear layers) ---- */
 typedef struct {

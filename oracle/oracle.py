@@ -337,6 +337,37 @@ def mha_decode(q8, k_cache, v_cache, q_s, k_s, v_s, a_s, want_p=False):
     return o, p8
 
 
+def mha_prefill_dyn(q, k, v, v_ch_s=None, want_p=False):
+    """Attention with dynamic per-(token, head) scales.  q [s][qh][hd], k/v [s][kvh][hd] fp32 ->
+    dict(q8, q_s, k8, k_s, v8, v_s, p8 (int8 [qh][s][s] or None), p_s [s][qh], o)."""
+    q = _f32(q); k = _f32(k); v = _f32(v)
+    s, qh, hd = q.shape
+    kvh = k.shape[1]
+    vch = _f32(v_ch_s) if v_ch_s is not None else None
+    r = dict(q8=np.empty(q.shape, np.int8), q_s=np.empty((s, qh), np.float32), k8=np.empty(k.shape, np.int8),
+             k_s=np.empty((s, kvh), np.float32), v8=np.empty(v.shape, np.int8), v_s=np.empty((s, kvh), np.float32),
+             p8=np.empty((qh, s, s), np.int8) if want_p else None, p_s=np.empty((s, qh), np.float32),
+             o=np.empty(q.shape, np.float32))
+    lib().fxo_mha_prefill_dyn(_p(q), _p(k), _p(v), s, qh, kvh, hd, _p(vch), _p(r["q8"]), _p(r["q_s"]), _p(r["k8"]), _p(r["k_s"]),
+                              _p(r["v8"]), _p(r["v_s"]), _p(r["p8"]), _p(r["p_s"]), _p(r["o"]))
+    return r
+
+
+def mha_decode_dyn(q8, q_s, k_cache, k_s, v_cache, v_s, v_ch_s=None, want_p=False):
+    """q8 [qh][hd] int8 with Q_s [qh]; caches [len][kvh][hd] int8 with K_s, V_s [len][kvh] -> (o, p8, p_s)."""
+    q8 = np.ascontiguousarray(q8, np.int8); q_s = _f32(q_s)
+    k_cache = np.ascontiguousarray(k_cache, np.int8); v_cache = np.ascontiguousarray(v_cache, np.int8)
+    k_s = _f32(k_s); v_s = _f32(v_s)
+    qh, hd = q8.shape
+    ln, kvh, _ = k_cache.shape
+    vch = _f32(v_ch_s) if v_ch_s is not None else None
+    p8 = np.empty((qh, ln), np.int8) if want_p else None
+    p_s = np.empty(qh, np.float32); o = np.empty((qh, hd), np.float32)
+    lib().fxo_mha_decode_dyn(_p(q8), _p(q_s), _p(k_cache), _p(k_s), _p(v_cache), _p(v_s), _p(vch), ln, qh, kvh, hd,
+                             _p(p8), _p(p_s), _p(o))
+    return o, p8, p_s
+
+
 def half_to_float(h):
     return lib().fxo_half_to_float(int(h))
 

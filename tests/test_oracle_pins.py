@@ -258,6 +258,69 @@ def test_mha_decode_equals_prefill_rows_bit_for_bit(oracle):
         assert np.array_equal(p, out["p8"][:, i, :i + 1])
 
 
+def test_mha_dyn_vs_float64_fake_quant_golden_with_per_token_scales(oracle):
+    """Attention with dynamic per-(token, head) scales: golden built the testbench way (fake-quant tensors, float
+    matmuls, scipy softmax) in float64 with every scale taken per token and head; the three facts the variant adds
+    (1/sqrt(d) folded into Q's scale, K's scale indexed by KEY, V's scale folded into the probabilities) are each
+    switched off once and must be noticed."""
+    S, qh, kvh, hd = 48, 8, 2, 64
+    r = np.random.default_rng(77)
+    q = (r.standard_normal((S, qh, hd)) * r.uniform(0.2, 3, (S, qh, 1))).astype(np.float32)      # scales differ a lot per token
+    k = (r.standard_normal((S, kvh, hd)) * r.uniform(0.2, 3, (S, kvh, 1))).astype(np.float32)
+    v = (r.standard_normal((S, kvh, hd)) * r.uniform(0.2, 3, (S, kvh, 1))).astype(np.float32)
+    out = oracle.mha_prefill_dyn(q, k, v, want_p=True)
+    rnd = lambda t: np.sign(t) * np.floor(np.abs(t) + 0.5)
+    sq = np.abs(q).max(-1) / np.float32(127); sk = np.abs(k).max(-1) / np.float32(127); sv = np.abs(v).max(-1) / np.float32(127)
+    assert np.array_equal(out["q_s"], (sq / np.float32(8)).astype(np.float32)) and np.array_equal(out["k_s"], sk) and np.array_equal(out["v_s"], sv)
+    qf, kf, vf = rnd(q / sq[..., None]), rnd(k / sk[..., None]), rnd(v / sv[..., None])
+    assert np.array_equal(out["q8"], qf) and np.array_equal(out["k8"], kf) and np.array_equal(out["v8"], vf)
+    assert np.abs(out["q8"]).max(-1).min() == 127                       # every (token, head) uses its full range
+
+    def golden(mut=None):
+        o = np.zeros((S, qh, hd)); P = np.zeros((qh, S, S)); ps = np.zeros((S, qh))
+        for h in range(qh):
+            kh = h // (qh // kvh)
+            q_deq = qf[:, h] * (sq[:, h, None].astype(np.float64) / (1.0 if mut == "no_sqrt_d" else 8.0))
+            k_scale = sk[:, kh].astype(np.float64)
+            a = (q_deq @ kf[:, kh].T) * (k_scale[:, None] if mut == "k_scale_by_query" else k_scale[None, :])
+            a[np.triu_indices(S, 1)] = -np.inf
+            p = scipy.special.softmax(a, axis=1)
+            pp = p * (1.0 if mut == "v_scale_not_folded" else sv[None, :, kh].astype(np.float64))
+            ps[:, h] = pp.max(1) / 127.0
+            P[h] = rnd(pp / ps[:, h, None])
+            o[:, h] = (P[h] * ps[:, h, None]) @ vf[:, kh]
+        return o, P, ps
+
+    o_ref, P_ref, ps_ref = golden()
+    np.testing.assert_allclose(out["p_s"], ps_ref, rtol=2e-6)
+    d = np.abs(out["p8"].astype(np.int64) - P_ref)
+    assert d.max() <= 1 and (d != 0).mean() < 2e-3 and out["p8"].min() == 0 and out["p8"].max() == 127
+    assert not np.triu(out["p8"][0], 1).any()
+    np.testing.assert_allclose(out["o"], o_ref, rtol=0, atol=3e-3 * np.abs(o_ref).max())       # P steps of 1/127
+    o_exact = np.stack([(out["p8"][h].astype(np.float64) * out["p_s"][:, h, None].astype(np.float64)) @ vf[:, h // (qh // kvh)]
+                        for h in range(qh)], axis=1)
+    np.testing.assert_allclose(out["o"], o_exact, rtol=1e-5, atol=1e-6)
+    for mut in ("no_sqrt_d", "k_scale_by_query", "v_scale_not_folded"):
+        assert np.abs(golden(mut)[0] - out["o"]).max() > 3e-2 * np.abs(o_ref).max(), mut
+    # per-channel V scale (the reference library's own form, MHA.h:713-738): one more factor per output channel
+    vch = r.uniform(0.5, 2.0, (kvh, hd)).astype(np.float32)
+    o2 = oracle.mha_prefill_dyn(q, k, v, v_ch_s=vch)["o"]
+    assert np.array_equal(o2, (out["o"] * np.repeat(vch, qh // kvh, axis=0)[None]).astype(np.float32))
+
+
+def test_mha_decode_dyn_equals_prefill_dyn_rows_bit_for_bit(oracle):
+    S, qh, kvh, hd = 37, 8, 2, 64
+    r = np.random.default_rng(78)
+    q = r.standard_normal((S, qh, hd)).astype(np.float32); k = r.standard_normal((S, kvh, hd)).astype(np.float32)
+    v = r.standard_normal((S, kvh, hd)).astype(np.float32)
+    out = oracle.mha_prefill_dyn(q, k, v, want_p=True)
+    for i in (0, 1, 5, 20, S - 1):
+        o, p8, p_s = oracle.mha_decode_dyn(out["q8"][i], out["q_s"][i], out["k8"][:i + 1], out["k_s"][:i + 1],
+                                           out["v8"][:i + 1], out["v_s"][:i + 1], want_p=True)
+        assert np.array_equal(o, out["o"][i]) and np.array_equal(p_s, out["p_s"][i])
+        assert np.array_equal(p8, out["p8"][:, i, :i + 1])
+
+
 # ------------------------------------------------------------------ layouts
 def test_prefill_and_decode_stream_layouts_roundtrip_and_index_formula(oracle):
     tokens, dim, tp = 16, 24, 8
