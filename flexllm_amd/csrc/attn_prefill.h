@@ -3,15 +3,15 @@
 // A workgroup owns 32 consecutive queries of one head; its waves split the key tiles (32 keys) up to the
 // diagonal.
 // The score tile is computed TRANSPOSED, S^T = K_tile . Q_tile^T, so that in the 32x32 accumulator layout a
-// lane holds 16 scores of ONE query (column l%32; keys 8a+4g+b for register 4a+b, g = l/32).  That is also
-// the A-operand shape of the second matrix product P.V (row = query l%32, 16 k-values for k-group g), so the
-// quantised probabilities never leave the registers; V's B operand is gathered in the same key order from
-// the cache's transposed 64-position blocks ([channel][position]: four 4-byte runs per lane).
+// lane holds 16 scores of ONE query (column l%32; accumulator rows 8a+4g+b for register 4a+b, g = l/32).  That is
+// also the A-operand shape of the second matrix product P.V (row = query l%32, 16 k-values for k-group g), so the
+// quantised probabilities never leave the registers; the K rows are loaded in a permuted order that makes those 16
+// values 16 consecutive keys, so that V's B operand is one 16-byte run of the cache's transposed 64-position blocks
+// ([channel][position]) per lane and channel.
 //
-// The reference normalises by the full-row sum BEFORE rounding the probabilities to uint8, so the wave makes
-// two passes over its key tiles: pass 1 keeps a running max / running sum of exponentials per query, pass 2
-// recomputes the scores (64-deep dot products: cheap), forms p = exp(s-max)*(1/sum), P = min(255,
-// round(p/A_s)) and accumulates P.V.  P is unsigned and the MFMA is signed x signed: (P-128).V is
+// The reference normalises by the full-row sum BEFORE rounding the probabilities to uint8, so a wave goes over its
+// key tiles in passes (row maximum, row sum, probabilities) and only the last one forms p = exp(s-max)*(1/sum),
+// P = min(255, round(p/A_s)) and accumulates P.V.  P is unsigned and the MFMA is signed x signed: (P-128).V is
 // accumulated and 128*colsum(V) over the same keys is added at the end, both exact in int32.
 #pragma once
 #include "attn_decode_kernels.h"
@@ -28,163 +28,78 @@ __device__ __forceinline__ i32x16 zero16() {
 }
 
 // grid (s/32 * q_heads), 64 * kPfWaves threads: the waves of a workgroup share one block of 32 queries and split
-// its key tiles round-robin (tile kt goes to wave kt % kPfWaves).  Row statistics are merged through LDS after pass 1;
-// the int32 P.V partial accumulators of the waves are added in LDS after pass 2 (integer adds: exact).
+// its key tiles round-robin (tile kt goes to wave kt % kPfWaves).  Row statistics are merged through LDS between the
+// passes; the int32 P.V partial accumulators of the waves are added in LDS at the end (integer adds: exact).
 //
 // Work per query block grows linearly with its index (causal), and workgroups b, b+P, b+2P, ... (P = number of
 // CUs) end up resident on the same CU.  The (block, head) items are therefore taken in order of decreasing
 // length and dealt out in snake order (first deal forwards, second backwards, ...): every CU gets the same total.
-constexpr int kPfWaves = 4;        // waves per workgroup (8 measured slower: the kernel is bound by VALU throughput, not by the longest block)
-static __global__ __launch_bounds__(64 * kPfWaves) void pf_attention_kernel(const int8_t* __restrict__ q8, const int8_t* __restrict__ kc,
-                                                                  const int8_t* __restrict__ vc, const float* __restrict__ q_s,
-                                                                  const float* __restrict__ k_s, const float* __restrict__ v_s,
-                                                                  const float* __restrict__ a_s, float* __restrict__ o,
-                                                                  uint8_t* __restrict__ p8_out, int s, int q_heads, int group,
-                                                                  int max_pos, int period) {
-    __shared__ float lds_m[kPfWaves][32], lds_l[kPfWaves][32];
-    __shared__ int lds_acc[64][35];            // [lane][16 acc0 | 16 acc1 | vsum0 | vsum1], odd pitch against bank conflicts
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+//
+// Key order inside a tile.  Row m of the S^T tile may hold any key of the tile; lane (col, g) loads K row
+// pi(col) = 16*((col>>2)&1) + 4*(col>>3) + (col&3), which makes accumulator register r of a lane the key 16g + r:
+// a lane's 16 probabilities are 16 CONSECUTIVE keys, in the byte order the P.V A operand wants, and the matching B
+// operand (V[key][channel] for the same 16 keys) is one 16-byte load from the cache's [channel][64 positions] block.
+//
+// Rounding P = min(255, round(p / A_s)) without a division per probability: q~ = e * (cd / A_s) is within 4e-5 of the
+// exactly evaluated (e * cd) / A_s, so both round alike unless q~ lies within 1e-4 of a tie; those groups of four are
+// redone with the reference's own expression.  The conversion instruction rounds to nearest (ties to even, which only
+// differs from the reference's half-away rule AT a tie, i.e. in a group that is redone anyway) and saturates at 255.
+constexpr int kPfWaves = 8;        // waves per workgroup
+constexpr int kPfMasked = -0x7fffffff - 1;
+
+struct PfItem {
+    int qb, q0, h, kvh, col, g, query, ntiles;
+};
+__device__ __forceinline__ PfItem pf_item(int s, int q_heads, int group, int period) {
+    const int lane = threadIdx.x & 63;
     const int n_items = (int)gridDim.x, nqb = s / kPfTile;
     const int round = (int)blockIdx.x / period, c = (int)blockIdx.x % period;
     const int in_round = min(period, n_items - round * period);
     const int item = round * period + ((round & 1) ? in_round - 1 - c : c);   // index into the items sorted by decreasing length
-    const int qb = nqb - 1 - item / q_heads;
-    const int q0 = qb * kPfTile;
-    const int h = item % q_heads, kvh = h / group;
-    const int col = lane & 31, g = lane >> 5;
-    const int query = q0 + col;
-    const float sq = q_s[h], sk = k_s[kvh], as = 1.0f * a_s[h];
+    PfItem it;
+    it.qb = nqb - 1 - item / q_heads;
+    it.q0 = it.qb * kPfTile;
+    it.h = item % q_heads;
+    it.kvh = it.h / group;
+    it.col = lane & 31;
+    it.g = lane >> 5;
+    it.query = it.q0 + it.col;
+    it.ntiles = it.qb + 1;
+    return it;
+}
+__device__ __forceinline__ int pf_key_of_row(int m) { return 16 * ((m >> 2) & 1) + 4 * (m >> 3) + (m & 3); }
 
-    // B operand of S^T = K.Q^T: this lane's query row, 16 d-bytes of k-group g, two k-steps (d 0..31, 32..63)
-    const int8_t* qrow = q8 + ((size_t)query * q_heads + h) * kHd;
-    const i32x4 qf0 = *reinterpret_cast<const i32x4*>(qrow + g * 16);
-    const i32x4 qf1 = *reinterpret_cast<const i32x4*>(qrow + 32 + g * 16);
-
-    auto load_k = [&](int k0, i32x4& kf0, i32x4& kf1) {
-        const int8_t* krow = kc + k_index(kvh, k0 + col, max_pos);
-        kf0 = *reinterpret_cast<const i32x4*>(krow + g * 16);
-        kf1 = *reinterpret_cast<const i32x4*>(krow + 32 + g * 16);
-    };
-    auto score_tile = [&](int k0, const i32x4& kf0, const i32x4& kf1, float (&sc)[16]) {
-        i32x16 acc = zero16();
-        acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(kf0, qf0, acc, 0, 0, 0);
-        acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(kf1, qf1, acc, 0, 0, 0);
-        if (k0 == q0) {                                   // only the diagonal tile has keys beyond the query (uniform branch)
+// Four exponentials (already divided by nothing: e = exp(score - max)) -> four probability bytes, biased by 128 for the
+// signed matrix product.  kq = cd / A_s (fast path), cd and as for the exact redo.
+__device__ __forceinline__ int pf_round4(const float (&e)[4], float kq, float cd, float as, bool fast_q, unsigned& bytes) {
+    float qv[4];
 #pragma unroll
-            for (int r = 0; r < 16; r++) {
-                const int key = k0 + (r >> 2) * 8 + g * 4 + (r & 3);
-                const float v = (float)acc[r] * sq * sk;
-                sc[r] = key <= query ? v : -1e32f;
-            }
-        } else {
+    for (int b = 0; b < 4; b++) qv[b] = e[b] * kq;
+    const float d0 = fabsf(__builtin_amdgcn_fractf(qv[0]) - 0.5f), d1 = fabsf(__builtin_amdgcn_fractf(qv[1]) - 0.5f);
+    const float d2 = fabsf(__builtin_amdgcn_fractf(qv[2]) - 0.5f), d3 = fabsf(__builtin_amdgcn_fractf(qv[3]) - 0.5f);
+    const bool redo = !fast_q || fminf(fminf(d0, d1), fminf(d2, d3)) < 1e-4f;
+    unsigned packed = 0;
+    if (redo) {
 #pragma unroll
-            for (int r = 0; r < 16; r++) sc[r] = (float)acc[r] * sq * sk;
+        for (int b = 0; b < 4; b++) {
+            int v = (int)roundf((e[b] * cd) / as);
+            v = v > 255 ? 255 : v;
+            packed |= (unsigned)v << (8 * b);
         }
-    };
+    } else {
+#pragma unroll
+        for (int b = 0; b < 4; b++) packed = __builtin_amdgcn_cvt_pk_u8_f32(qv[b], b, packed);
+    }
+    bytes = packed;                                   // the four probability bytes, key order
+    return (int)(packed ^ 0x80808080u);
+}
 
-    const int ntiles = qb + 1;
-    for (int i = threadIdx.x; i < 64 * 35; i += 64 * kPfWaves) (&lds_acc[0][0])[i] = 0;
-    // ---- pass 1: row max and row sum of exponentials over this wave's tiles ----
-    float m_run = -1e32f, l_run = 0.0f;
-    {
-        i32x4 kf0, kf1, nf0, nf1;
-        if (wave < ntiles) load_k(wave * kPfTile, kf0, kf1);
-        for (int kt = wave; kt < ntiles; kt += kPfWaves) {
-            if (kt + kPfWaves < ntiles) load_k((kt + kPfWaves) * kPfTile, nf0, nf1);
-            float sc[16];
-            score_tile(kt * kPfTile, kf0, kf1, sc);
-            float mt = sc[0];
-#pragma unroll
-            for (int r = 1; r < 16; r++) mt = fmaxf(mt, sc[r]);
-            const float m_new = fmaxf(m_run, mt);
-            float sum = 0.0f;
-#pragma unroll
-            for (int r = 0; r < 16; r++) sum += exp_f<false>(sc[r] - m_new);
-            l_run = l_run * exp_f<false>(m_run - m_new) + sum;
-            m_run = m_new;
-            kf0 = nf0; kf1 = nf1;
-        }
-    }
-    {   // merge the two lanes that share a query, then the waves
-        const float m_o = lane_xor_f<32>(m_run), l_o = lane_xor_f<32>(l_run);
-        const float mw = fmaxf(m_run, m_o);
-        const float lw = l_run * exp_f(m_run - mw) + l_o * exp_f(m_o - mw);
-        if (g == 0) { lds_m[wave][col] = mw; lds_l[wave][col] = lw; }
-    }
-    __syncthreads();
-    float mx = lds_m[0][col];
-#pragma unroll
-    for (int w = 1; w < kPfWaves; w++) mx = fmaxf(mx, lds_m[w][col]);
-    float total = 0.0f;
-#pragma unroll
-    for (int w = 0; w < kPfWaves; w++) total += lds_l[w][col] * exp_f(lds_m[w][col] - mx);
-    const float cd = 1.0f / total;
-    const bool fast_q = quant_fast_ok(as);
-    const float ras = 1.0f / as;
-
-    // ---- pass 2: probabilities, partial P.V over this wave's tiles ----
-    i32x16 oacc0 = zero16(), oacc1 = zero16();
-    int vsum0 = 0, vsum1 = 0;
-    {
-        i32x4 kf0, kf1, nf0, nf1;
-        if (wave < ntiles) load_k(wave * kPfTile, kf0, kf1);
-        for (int kt = wave; kt < ntiles; kt += kPfWaves) {
-            const int k0 = kt * kPfTile;
-            if (kt + kPfWaves < ntiles) load_k((kt + kPfWaves) * kPfTile, nf0, nf1);
-            // B operand of P.V: V[key][d] for this lane's channel d = col (+32) and the lane's 16 keys, gathered
-            // from the cache's [d][64 pos] blocks; issued before the exponentials so that it is in flight
-            const int8_t* vblk = vc + v_index(kvh, k0, 0, max_pos);
-            i32x4 vf0, vf1;
-#pragma unroll
-            for (int a = 0; a < 4; a++) {
-                vf0[a] = *reinterpret_cast<const int*>(vblk + (size_t)col * kVBlock + a * 8 + g * 4);
-                vf1[a] = *reinterpret_cast<const int*>(vblk + (size_t)(col + 32) * kVBlock + a * 8 + g * 4);
-            }
-            float sc[16];
-            score_tile(k0, kf0, kf1, sc);
-            i32x4 pf;
-#pragma unroll
-            for (int a = 0; a < 4; a++) {
-                // four probabilities -> four bytes; round(pr / as) through the reciprocal, redone with the division
-                // for the whole group when one of them comes near a rounding tie
-                float pr[4];
-                int p8[4];
-                bool redo = !fast_q;
-#pragma unroll
-                for (int b = 0; b < 4; b++) {
-                    pr[b] = exp_f<false>(sc[a * 4 + b] - mx) * cd;
-                    const float qv = pr[b] * ras;               // >= 0: round half up = truncate(qv + 0.5)
-                    redo |= fabsf(__builtin_amdgcn_fractf(qv) - 0.5f) < 1e-4f;
-                    p8[b] = (int)(qv + 0.5f);
-                }
-                if (redo) {
-#pragma unroll
-                    for (int b = 0; b < 4; b++) p8[b] = (int)roundf(pr[b] / as);
-                }
-                uint32_t packed = 0;
-#pragma unroll
-                for (int b = 0; b < 4; b++) {
-                    const int pq = p8[b] > 255 ? 255 : p8[b];
-                    if (p8_out) {
-                        const int key = k0 + a * 8 + g * 4 + b;
-                        p8_out[((size_t)h * s + query) * s + key] = (uint8_t)pq;
-                    }
-                    packed |= (uint32_t)((pq ^ 0x80) & 0xff) << (8 * b);
-                }
-                pf[a] = (int)packed;
-            }
-#pragma unroll
-            for (int a = 0; a < 4; a++) {
-                vsum0 = __builtin_amdgcn_sdot4(0x01010101, vf0[a], vsum0, false);
-                vsum1 = __builtin_amdgcn_sdot4(0x01010101, vf1[a], vsum1, false);
-            }
-            oacc0 = __builtin_amdgcn_mfma_i32_32x32x32_i8(pf, vf0, oacc0, 0, 0, 0);
-            oacc1 = __builtin_amdgcn_mfma_i32_32x32x32_i8(pf, vf1, oacc1, 0, 0, 0);
-            kf0 = nf0; kf1 = nf1;
-        }
-    }
-    // add the waves' partial accumulators (lds_acc was zeroed before pass 1; two barriers have passed)
-    if (wave < ntiles) {
+// Adds the waves' partial accumulators in LDS and writes the block's 32 x 64 outputs.
+__device__ __forceinline__ void pf_reduce_store(int (*lds_acc)[35], const i32x16& oacc0, const i32x16& oacc1, int vsum0, int vsum1,
+                                                bool has_tiles, const PfItem& it, float sa, float sv, float* __restrict__ o,
+                                                int q_heads) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    if (has_tiles) {
 #pragma unroll
         for (int r = 0; r < 16; r++) {
             atomicAdd(&lds_acc[lane][r], oacc0[r]);
@@ -196,24 +111,162 @@ static __global__ __launch_bounds__(64 * kPfWaves) void pf_attention_kernel(cons
     __syncthreads();
     const int vs0 = lds_acc[lane][32] + lds_acc[lane ^ 32][32];
     const int vs1 = lds_acc[lane][33] + lds_acc[lane ^ 32][33];
-    const float sv = v_s[kvh], sa = a_s[h];
 #pragma unroll
     for (int rr = 0; rr < 16 / kPfWaves; rr++) {              // each wave writes its share of the 16 accumulator registers
         const int r = wave * (16 / kPfWaves) + rr;
-        const int row = q0 + (r >> 2) * 8 + g * 4 + (r & 3);
-        float* orow = o + ((size_t)row * q_heads + h) * kHd;
-        orow[col] = (float)(lds_acc[lane][r] + 128 * vs0) * sa * sv;
-        orow[col + 32] = (float)(lds_acc[lane][16 + r] + 128 * vs1) * sa * sv;
+        const int row = it.q0 + (r >> 2) * 8 + it.g * 4 + (r & 3);          // accumulator row = query (standard 32x32 layout)
+        float* orow = o + ((size_t)row * q_heads + it.h) * kHd;
+        orow[it.col] = (float)(lds_acc[lane][r] + 128 * vs0) * sa * sv;
+        orow[it.col + 32] = (float)(lds_acc[lane][16 + r] + 128 * vs1) * sa * sv;
     }
+}
+
+// Rows of any length: three passes over the wave's key tiles, the scores recomputed in each (64-deep dot products on
+// the matrix cores).  Pass 0: integer row maximum (the dequantisation is monotonic).  Pass 1: the softmax denominator,
+// with a one-rounding exponent (2^(acc*c - m), c = Q_s*K_s*log2(e)): its error, a few 1e-7 relative on the terms that
+// matter, only moves the common factor 1/sum.  Pass 2: each probability from the accurate exponential of the
+// reference's own score expression, rounded as described above, and P.V.
+static __global__ __launch_bounds__(64 * kPfWaves) void pf_attention_kernel(const int8_t* __restrict__ q8, const int8_t* __restrict__ kc,
+                                                                  const int8_t* __restrict__ vc, const float* __restrict__ q_s,
+                                                                  const float* __restrict__ k_s, const float* __restrict__ v_s,
+                                                                  const float* __restrict__ a_s, float* __restrict__ o,
+                                                                  uint8_t* __restrict__ p8_out, int s, int q_heads, int group,
+                                                                  int max_pos, int period) {
+    __shared__ int lds_mi[kPfWaves][32];
+    __shared__ float lds_l[kPfWaves][32];
+    __shared__ int lds_acc[64][35];            // [lane][16 acc0 | 16 acc1 | vsum0 | vsum1], odd pitch against bank conflicts
+    const int wave = threadIdx.x >> 6;
+    const PfItem it = pf_item(s, q_heads, group, period);
+    const int col = it.col, g = it.g, query = it.query, ntiles = it.ntiles;
+    const float sq = q_s[it.h], sk = k_s[it.kvh], as = 1.0f * a_s[it.h];
+
+    const int8_t* qrow = q8 + ((size_t)query * q_heads + it.h) * kHd;
+    const i32x4 qf0 = *reinterpret_cast<const i32x4*>(qrow + g * 16);
+    const i32x4 qf1 = *reinterpret_cast<const i32x4*>(qrow + 32 + g * 16);
+    const int krow_in_tile = pf_key_of_row(col);
+    auto load_k = [&](int k0, i32x4& kf0, i32x4& kf1) {
+        const int8_t* krow = kc + k_index(it.kvh, k0 + krow_in_tile, max_pos);
+        kf0 = *reinterpret_cast<const i32x4*>(krow + g * 16);
+        kf1 = *reinterpret_cast<const i32x4*>(krow + 32 + g * 16);
+    };
+    // integer scores of one tile: register r is key k0 + 16g + r; keys beyond the query (diagonal tile only) are masked
+    auto int_tile = [&](int kt, const i32x4& kf0, const i32x4& kf1, int (&tv)[16]) {
+        i32x16 acc = zero16();
+        acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(kf0, qf0, acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(kf1, qf1, acc, 0, 0, 0);
+        if (kt == it.qb) {
+#pragma unroll
+            for (int r = 0; r < 16; r++) tv[r] = (it.q0 + 16 * g + r) <= query ? acc[r] : kPfMasked;
+        } else {
+#pragma unroll
+            for (int r = 0; r < 16; r++) tv[r] = acc[r];
+        }
+    };
+
+    for (int i = threadIdx.x; i < 64 * 35; i += 64 * kPfWaves) (&lds_acc[0][0])[i] = 0;
+    // ---- pass 0: integer row maximum ----
+    int imax = kPfMasked;
+    {
+        i32x4 kf0, kf1, nf0, nf1;
+        if (wave < ntiles) load_k(wave * kPfTile, kf0, kf1);
+        for (int kt = wave; kt < ntiles; kt += kPfWaves) {
+            if (kt + kPfWaves < ntiles) load_k((kt + kPfWaves) * kPfTile, nf0, nf1);
+            int tv[16];
+            int_tile(kt, kf0, kf1, tv);
+#pragma unroll
+            for (int r = 0; r < 16; r++) imax = max(imax, tv[r]);
+            kf0 = nf0; kf1 = nf1;
+        }
+    }
+    imax = max(imax, lane_xor_i<32>(imax));
+    if (g == 0) lds_mi[wave][col] = imax;
+    __syncthreads();
+    int im = lds_mi[0][col];
+#pragma unroll
+    for (int w = 1; w < kPfWaves; w++) im = max(im, lds_mi[w][col]);
+    const float mx = (float)im * sq * sk;                      // int -> float and the positive scales keep the order
+    // ---- pass 1: denominator ----
+    const float c2 = sq * sk * 1.44269502162933349609375f;
+    const float m2 = (float)im * c2;
+    float lsum = 0.0f;
+    {
+        i32x4 kf0, kf1, nf0, nf1;
+        if (wave < ntiles) load_k(wave * kPfTile, kf0, kf1);
+        for (int kt = wave; kt < ntiles; kt += kPfWaves) {
+            if (kt + kPfWaves < ntiles) load_k((kt + kPfWaves) * kPfTile, nf0, nf1);
+            int tv[16];
+            int_tile(kt, kf0, kf1, tv);
+            if (kt == it.qb) {
+#pragma unroll
+                for (int r = 0; r < 16; r++)
+                    lsum += tv[r] == kPfMasked ? 0.0f : __builtin_amdgcn_exp2f(fminf(__builtin_fmaf((float)tv[r], c2, -m2), 0.0f));
+            } else {
+#pragma unroll
+                for (int r = 0; r < 16; r++) lsum += __builtin_amdgcn_exp2f(fminf(__builtin_fmaf((float)tv[r], c2, -m2), 0.0f));
+            }
+            kf0 = nf0; kf1 = nf1;
+        }
+    }
+    lsum = lsum + lane_xor_f<32>(lsum);
+    if (g == 0) lds_l[wave][col] = lsum;
+    __syncthreads();
+    float total = lds_l[0][col];
+#pragma unroll
+    for (int w = 1; w < kPfWaves; w++) total += lds_l[w][col];
+    const float cd = 1.0f / total;
+    const bool fast_q = quant_fast_ok(as);
+    const float kq = cd * (1.0f / as);
+
+    // ---- pass 2: probabilities, partial P.V over this wave's tiles ----
+    i32x16 oacc0 = zero16(), oacc1 = zero16();
+    int vsum0 = 0, vsum1 = 0;
+    {
+        i32x4 kf0, kf1, nf0, nf1;
+        if (wave < ntiles) load_k(wave * kPfTile, kf0, kf1);
+        for (int kt = wave; kt < ntiles; kt += kPfWaves) {
+            const int k0 = kt * kPfTile;
+            if (kt + kPfWaves < ntiles) load_k((kt + kPfWaves) * kPfTile, nf0, nf1);
+            // B operand of P.V: V[key][d] for this lane's channels col, col+32 and its 16 consecutive keys
+            const int8_t* vblk = vc + v_index(it.kvh, k0, 0, max_pos) + 16 * g;
+            const i32x4 vf0 = *reinterpret_cast<const i32x4*>(vblk + (size_t)col * kVBlock);
+            const i32x4 vf1 = *reinterpret_cast<const i32x4*>(vblk + (size_t)(col + 32) * kVBlock);
+            int tv[16];
+            int_tile(kt, kf0, kf1, tv);
+            i32x4 pf;
+#pragma unroll
+            for (int a = 0; a < 4; a++) {
+                float e[4];
+                unsigned bytes;
+                if (kt == it.qb) {                             // uniform: only the diagonal tile has masked keys
+#pragma unroll
+                    for (int b = 0; b < 4; b++)                // masked keys: exactly 0 whatever the scales
+                        e[b] = tv[a * 4 + b] == kPfMasked ? 0.0f : exp_f<false>((float)tv[a * 4 + b] * sq * sk - mx);
+                } else {
+#pragma unroll
+                    for (int b = 0; b < 4; b++) e[b] = exp_f<false>((float)tv[a * 4 + b] * sq * sk - mx);
+                }
+                pf[a] = pf_round4(e, kq, cd, as, fast_q, bytes);
+                if (p8_out) *reinterpret_cast<unsigned*>(p8_out + ((size_t)it.h * s + query) * s + k0 + 16 * g + a * 4) = bytes;
+            }
+#pragma unroll
+            for (int a = 0; a < 4; a++) {
+                vsum0 = __builtin_amdgcn_sdot4(0x01010101, vf0[a], vsum0, false);
+                vsum1 = __builtin_amdgcn_sdot4(0x01010101, vf1[a], vsum1, false);
+            }
+            oacc0 = __builtin_amdgcn_mfma_i32_32x32x32_i8(pf, vf0, oacc0, 0, 0, 0);
+            oacc1 = __builtin_amdgcn_mfma_i32_32x32x32_i8(pf, vf1, oacc1, 0, 0, 0);
+            kf0 = nf0; kf1 = nf1;
+        }
+    }
+    pf_reduce_store(lds_acc, oacc0, oacc1, vsum0, vsum1, wave < ntiles, it, a_s[it.h], v_s[it.kvh], o, q_heads);
 }
 
 // The same attention for rows of at most kPfWaves * kPfCachedTiles * 32 = 1024 keys, with every score tile of the
 // wave held in registers (8 tiles x 16 values per lane): the scores are computed ONCE as integers, the row maximum is
 // an integer maximum (the dequantisation is monotonic), the exponentials are computed ONCE with the final maximum and
-// replace the integers in place, and the second pass only scales, rounds and multiplies with V.  This is also the
+// replace the integers in place, and the last pass only scales, rounds and multiplies with V.  This is also the
 // reference's own order (maximum, then exponentials and their sum, then probabilities from the same exponentials).
-// Per probability: one exponential instead of two, one dequantisation instead of two, K read once.
-constexpr int kPfCachedTiles = 8;
+constexpr int kPfCachedTiles = 4;
 static __global__ __launch_bounds__(64 * kPfWaves, 2) void pf_attention_cached_kernel(
     const int8_t* __restrict__ q8, const int8_t* __restrict__ kc, const int8_t* __restrict__ vc, const float* __restrict__ q_s,
     const float* __restrict__ k_s, const float* __restrict__ v_s, const float* __restrict__ a_s, float* __restrict__ o,
@@ -221,33 +274,25 @@ static __global__ __launch_bounds__(64 * kPfWaves, 2) void pf_attention_cached_k
     __shared__ int lds_mi[kPfWaves][32];
     __shared__ float lds_l[kPfWaves][32];
     __shared__ int lds_acc[64][35];            // [lane][16 acc0 | 16 acc1 | vsum0 | vsum1], odd pitch against bank conflicts
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int n_items = (int)gridDim.x, nqb = s / kPfTile;
-    const int round = (int)blockIdx.x / period, c = (int)blockIdx.x % period;
-    const int in_round = min(period, n_items - round * period);
-    const int item = round * period + ((round & 1) ? in_round - 1 - c : c);   // index into the items sorted by decreasing length
-    const int qb = nqb - 1 - item / q_heads;
-    const int q0 = qb * kPfTile;
-    const int h = item % q_heads, kvh = h / group;
-    const int col = lane & 31, g = lane >> 5;
-    const int query = q0 + col;
-    const float sq = q_s[h], sk = k_s[kvh], as = 1.0f * a_s[h];
+    const int wave = threadIdx.x >> 6;
+    const PfItem it = pf_item(s, q_heads, group, period);
+    const int col = it.col, g = it.g, query = it.query, ntiles = it.ntiles;   // ntiles <= kPfWaves * kPfCachedTiles (checked by the launcher)
+    const float sq = q_s[it.h], sk = k_s[it.kvh], as = 1.0f * a_s[it.h];
 
-    const int8_t* qrow = q8 + ((size_t)query * q_heads + h) * kHd;
+    const int8_t* qrow = q8 + ((size_t)query * q_heads + it.h) * kHd;
     const i32x4 qf0 = *reinterpret_cast<const i32x4*>(qrow + g * 16);
     const i32x4 qf1 = *reinterpret_cast<const i32x4*>(qrow + 32 + g * 16);
+    const int krow_in_tile = pf_key_of_row(col);
     auto load_k = [&](int k0, i32x4& kf0, i32x4& kf1) {
-        const int8_t* krow = kc + k_index(kvh, k0 + col, max_pos);
+        const int8_t* krow = kc + k_index(it.kvh, k0 + krow_in_tile, max_pos);
         kf0 = *reinterpret_cast<const i32x4*>(krow + g * 16);
         kf1 = *reinterpret_cast<const i32x4*>(krow + 32 + g * 16);
     };
-    const int ntiles = qb + 1;                                 // <= kPfWaves * kPfCachedTiles (checked by the launcher)
     for (int i = threadIdx.x; i < 64 * 35; i += 64 * kPfWaves) (&lds_acc[0][0])[i] = 0;
 
     // ---- pass 0: integer scores of this wave's tiles (kept), integer row maximum ----
-    constexpr int kMasked = -0x7fffffff - 1;
     int tv[kPfCachedTiles][16];
-    int imax = kMasked;
+    int imax = kPfMasked;
     {
         i32x4 kf0, kf1, nf0, nf1;
         if (wave < ntiles) load_k(wave * kPfTile, kf0, kf1);
@@ -259,9 +304,9 @@ static __global__ __launch_bounds__(64 * kPfWaves, 2) void pf_attention_cached_k
                 i32x16 acc = zero16();
                 acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(kf0, qf0, acc, 0, 0, 0);
                 acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(kf1, qf1, acc, 0, 0, 0);
-                if (kt == qb) {                                // only the diagonal tile has keys beyond the query
+                if (kt == it.qb) {                             // only the diagonal tile has keys beyond the query
 #pragma unroll
-                    for (int r = 0; r < 16; r++) tv[i][r] = (q0 + (r >> 2) * 8 + g * 4 + (r & 3)) <= query ? acc[r] : kMasked;
+                    for (int r = 0; r < 16; r++) tv[i][r] = (it.q0 + 16 * g + r) <= query ? acc[r] : kPfMasked;
                 } else {
 #pragma unroll
                     for (int r = 0; r < 16; r++) tv[i][r] = acc[r];
@@ -286,12 +331,20 @@ static __global__ __launch_bounds__(64 * kPfWaves, 2) void pf_attention_cached_k
     for (int i = 0; i < kPfCachedTiles; i++) {
         const int kt = wave + kPfWaves * i;
         if (kt < ntiles) {
+            if (kt == it.qb) {                                 // uniform: only the diagonal tile has masked keys
 #pragma unroll
-            for (int r = 0; r < 16; r++) {
-                float e = exp_f<false>((float)tv[i][r] * sq * sk - mx);
-                if (kt == qb && tv[i][r] == kMasked) e = 0.0f;  // masked keys count as exp(-1e32 - max) = 0 whatever the scales
-                tv[i][r] = __float_as_int(e);
-                lsum += e;
+                for (int r = 0; r < 16; r++) {                 // they count as exp(-1e32 - max) = 0 whatever the scales
+                    const float e = tv[i][r] == kPfMasked ? 0.0f : exp_f<false>((float)tv[i][r] * sq * sk - mx);
+                    tv[i][r] = __float_as_int(e);
+                    lsum += e;
+                }
+            } else {
+#pragma unroll
+                for (int r = 0; r < 16; r++) {
+                    const float e = exp_f<false>((float)tv[i][r] * sq * sk - mx);
+                    tv[i][r] = __float_as_int(e);
+                    lsum += e;
+                }
             }
         }
     }
@@ -303,7 +356,7 @@ static __global__ __launch_bounds__(64 * kPfWaves, 2) void pf_attention_cached_k
     for (int w = 1; w < kPfWaves; w++) total += lds_l[w][col];
     const float cd = 1.0f / total;
     const bool fast_q = quant_fast_ok(as);
-    const float ras = 1.0f / as;
+    const float kq = cd * (1.0f / as);
 
     // ---- pass 2: probabilities from the kept exponentials, partial P.V ----
     i32x16 oacc0 = zero16(), oacc1 = zero16();
@@ -313,43 +366,17 @@ static __global__ __launch_bounds__(64 * kPfWaves, 2) void pf_attention_cached_k
         const int kt = wave + kPfWaves * i;
         if (kt < ntiles) {
             const int k0 = kt * kPfTile;
-            // B operand of P.V: V[key][d] for this lane's channels col, col+32 and its 16 keys, gathered from the
-            // cache's [d][64 pos] blocks; issued before the rounding work so that it is in flight
-            const int8_t* vblk = vc + v_index(kvh, k0, 0, max_pos);
-            i32x4 vf0, vf1;
-#pragma unroll
-            for (int a = 0; a < 4; a++) {
-                vf0[a] = *reinterpret_cast<const int*>(vblk + (size_t)col * kVBlock + a * 8 + g * 4);
-                vf1[a] = *reinterpret_cast<const int*>(vblk + (size_t)(col + 32) * kVBlock + a * 8 + g * 4);
-            }
+            const int8_t* vblk = vc + v_index(it.kvh, k0, 0, max_pos) + 16 * g;
+            const i32x4 vf0 = *reinterpret_cast<const i32x4*>(vblk + (size_t)col * kVBlock);
+            const i32x4 vf1 = *reinterpret_cast<const i32x4*>(vblk + (size_t)(col + 32) * kVBlock);
             i32x4 pf;
 #pragma unroll
             for (int a = 0; a < 4; a++) {
-                float pr[4];
-                int p8[4];
-                bool redo = !fast_q;
-#pragma unroll
-                for (int b = 0; b < 4; b++) {
-                    pr[b] = __int_as_float(tv[i][a * 4 + b]) * cd;
-                    const float qv = pr[b] * ras;               // >= 0: round half up = truncate(qv + 0.5)
-                    redo |= fabsf(__builtin_amdgcn_fractf(qv) - 0.5f) < 1e-4f;
-                    p8[b] = (int)(qv + 0.5f);
-                }
-                if (redo) {
-#pragma unroll
-                    for (int b = 0; b < 4; b++) p8[b] = (int)roundf(pr[b] / as);
-                }
-                uint32_t packed = 0;
-#pragma unroll
-                for (int b = 0; b < 4; b++) {
-                    const int pq = p8[b] > 255 ? 255 : p8[b];
-                    if (p8_out) {
-                        const int key = k0 + a * 8 + g * 4 + b;
-                        p8_out[((size_t)h * s + query) * s + key] = (uint8_t)pq;
-                    }
-                    packed |= (uint32_t)((pq ^ 0x80) & 0xff) << (8 * b);
-                }
-                pf[a] = (int)packed;
+                const float e[4] = {__int_as_float(tv[i][a * 4]), __int_as_float(tv[i][a * 4 + 1]), __int_as_float(tv[i][a * 4 + 2]),
+                                    __int_as_float(tv[i][a * 4 + 3])};
+                unsigned bytes;
+                pf[a] = pf_round4(e, kq, cd, as, fast_q, bytes);
+                if (p8_out) *reinterpret_cast<unsigned*>(p8_out + ((size_t)it.h * s + query) * s + k0 + 16 * g + a * 4) = bytes;
             }
 #pragma unroll
             for (int a = 0; a < 4; a++) {
@@ -360,27 +387,7 @@ static __global__ __launch_bounds__(64 * kPfWaves, 2) void pf_attention_cached_k
             oacc1 = __builtin_amdgcn_mfma_i32_32x32x32_i8(pf, vf1, oacc1, 0, 0, 0);
         }
     }
-    if (wave < ntiles) {
-#pragma unroll
-        for (int r = 0; r < 16; r++) {
-            atomicAdd(&lds_acc[lane][r], oacc0[r]);
-            atomicAdd(&lds_acc[lane][16 + r], oacc1[r]);
-        }
-        atomicAdd(&lds_acc[lane][32], vsum0);
-        atomicAdd(&lds_acc[lane][33], vsum1);
-    }
-    __syncthreads();
-    const int vs0 = lds_acc[lane][32] + lds_acc[lane ^ 32][32];
-    const int vs1 = lds_acc[lane][33] + lds_acc[lane ^ 32][33];
-    const float sv = v_s[kvh], sa = a_s[h];
-#pragma unroll
-    for (int rr = 0; rr < 16 / kPfWaves; rr++) {
-        const int r = wave * (16 / kPfWaves) + rr;
-        const int row = q0 + (r >> 2) * 8 + g * 4 + (r & 3);
-        float* orow = o + ((size_t)row * q_heads + h) * kHd;
-        orow[col] = (float)(lds_acc[lane][r] + 128 * vs0) * sa * sv;
-        orow[col + 32] = (float)(lds_acc[lane][16 + r] + 128 * vs1) * sa * sv;
-    }
+    pf_reduce_store(lds_acc, oacc0, oacc1, vsum0, vsum1, wave < ntiles, it, a_s[it.h], v_s[it.kvh], o, q_heads);
 }
 
 inline int mha_prefill_launch(const int8_t* q8, const int8_t* kc, const int8_t* vc, const float* q_s, const float* k_s,
