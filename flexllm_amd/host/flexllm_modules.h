@@ -8,7 +8,8 @@
 //
 // Differences from the reference, all forced by the device boundary:
 //  * Weights do not travel through streams: a linear layer takes a DeviceWeight that was uploaded once from
-//    the row-major int8 [N][K] array (the reference's on-disk format), see DeviceWeight / unpack helpers.
+//    the row-major int8 [N][K] array (the reference's on-disk format); flexllm_adapters.h converts the reference's
+//    packed weight words and KV-cache line layouts to and from that form.
 //  * The int8 instantiation (qint_bit = 8, symmetric) is the W8A8 path; function names keep the reference's
 //    spelling with "i8xi8" where the reference says "i4xi4".
 //  * Errors throw fxhost::Error carrying flexllm_last_error() (the reference prints and returns).
@@ -19,7 +20,10 @@
 #include <string>
 #include <type_traits>
 #include <vector>
+#include <array>
+#include <chrono>
 #include "../../include/flexllm_hip.h"
+#include "flexllm_adapters.h"
 #include "stream_types.h"
 
 namespace fxhost {
@@ -417,6 +421,258 @@ void pref_Softmax(IS& input_stream, OS& output_stream, int seq_len = max_seq_len
     fill_pref(output_stream, dx.download(), seq_len, head_num * io_hidden_dim, io_parallel);
 }
 
+// ======================================================================================= decode-side attention modules
+// Head-parallel decode streams carry head_parallel heads per vector: lane m of step H is head m*(head_num/HP) + H
+// (Modules/quant.h:736, :793), dim values per head in sequence.
+template <class T, class IS>
+std::vector<T> drain_heads(IS& in, int head_num, int dim, int head_parallel) {
+    std::vector<T> x((size_t)head_num * dim);
+    const int per = head_num / head_parallel;
+    for (int H = 0; H < per; H++)
+        for (int k = 0; k < dim; k++) {
+            auto pack = in.read();
+            for (int m = 0; m < head_parallel; m++) x[(size_t)(m * per + H) * dim + k] = (T)pack[m];
+        }
+    return x;
+}
+template <class OS, class T>
+void fill_heads(OS& out, const std::vector<T>& x, int head_num, int dim, int head_parallel) {
+    using V = typename OS::value_type;
+    using E = typename std::remove_reference<decltype(std::declval<V&>()[0])>::type;
+    const int per = head_num / head_parallel;
+    for (int H = 0; H < per; H++)
+        for (int k = 0; k < dim; k++) {
+            V pack;
+            for (int m = 0; m < head_parallel; m++) pack[m] = (E)x[(size_t)(m * per + H) * dim + k];
+            out.write(pack);
+        }
+}
+// Modules/RoPE.h:96-103
+template <typename T, int head_parallel, int io_hidden_dim = 64, int max_head_num = 32, int max_sum_seq_len = 2048, class IS, class OS>
+void dec_RoPE_layer(IS& input_stream, OS& output_stream, const T PE_sin[max_sum_seq_len][io_hidden_dim / 2],
+                    const T PE_cos[max_sum_seq_len][io_hidden_dim / 2], int head_num = max_head_num, int seq_id = 0) {
+    auto x = drain_heads<float>(input_stream, head_num, io_hidden_dim, head_parallel);
+    DeviceArray<float> dx(x), dy(x.size()), ds, dc;
+    // only the row of this position is needed on the device; it is passed as a one-row table at position 0
+    ds.upload(&PE_sin[seq_id][0], (size_t)(io_hidden_dim / 2));
+    dc.upload(&PE_cos[seq_id][0], (size_t)(io_hidden_dim / 2));
+    check(flexllm_rope_f32(dx.get(), dy.get(), ds.get(), dc.get(), 1, head_num, io_hidden_dim, 0, nullptr));
+    fill_heads(output_stream, dy.download(), head_num, io_hidden_dim, head_parallel);
+}
+// Modules/Softmax.h:456-461: one row of io_hidden_dim scores per head
+template <typename T, int head_parallel, int max_hidden_dim = 2048, int head_num = 1, bool enable_scale = false, bool enable_sub_max = true,
+          bool is_versal = false, class IS, class OS>
+void dec_MHA_Softmax(IS& input_stream, OS& output_stream, int io_hidden_dim = max_hidden_dim, const T scale_factor = 1.0) {
+    static_assert(!enable_scale && enable_sub_max, "the configuration the shipped graphs use");
+    auto x = drain_heads<float>(input_stream, head_num, io_hidden_dim, head_parallel);
+    DeviceArray<float> dx(x);
+    check(flexllm_softmax_f32(dx.get(), dx.get(), head_num, io_hidden_dim, nullptr));
+    fill_heads(output_stream, dx.download(), head_num, io_hidden_dim, head_parallel);
+}
+// Modules/quant.h:716-724
+template <int qint_bit, int head_parallel, int max_input_dim, int head_num = 1, bool is_signed = true, int decoder_layer_num = 16,
+          class IS, class OS>
+void dec_MHA_static_sym_per_tensor_quant_layer_fp32_qint(IS& input_stream, OS& output_stream,
+                                                         const float input_s[decoder_layer_num][head_num], int block_id,
+                                                         int input_dim = max_input_dim, float mha_scale_factor = 1.0f) {
+    static_assert(qint_bit == 8, "int8 path");
+    auto x = drain_heads<float>(input_stream, head_num, input_dim, head_parallel);
+    DeviceArray<float> dx(x), dsc(std::vector<float>(input_s[block_id], input_s[block_id] + head_num));
+    DeviceArray<int8_t> dq(x.size());
+    check(flexllm_static_quant_i8(dx.get(), dq.get(), dsc.get(), mha_scale_factor, is_signed, 1, head_num, input_dim, nullptr));
+    auto q = dq.download();
+    if (is_signed) fill_heads(output_stream, q, head_num, input_dim, head_parallel);
+    else fill_heads(output_stream, std::vector<uint8_t>(q.begin(), q.end()), head_num, input_dim, head_parallel);
+}
+// Modules/quant.h:758-766: act head a_H = m*(act_heads/HP) + h, weight head a_H / (act_heads / weight_heads)
+template <int qint_bit, int head_parallel, int max_output_dim, int act_head_num = 1, int weight_head_num = 1, int decoder_layer_num = 16,
+          class IS, class OS>
+void dec_MHA_static_sym_per_tensor_dequant_layer_qint_fp32(IS& input_stream, OS& output_stream,
+                                                           const float input_s[decoder_layer_num][act_head_num],
+                                                           const float weight_s[decoder_layer_num][weight_head_num], int block_id,
+                                                           int output_dim = max_output_dim) {
+    auto acc = drain_heads<int32_t>(input_stream, act_head_num, output_dim, head_parallel);
+    DeviceArray<int32_t> dacc(acc);
+    DeviceArray<float> das(std::vector<float>(input_s[block_id], input_s[block_id] + act_head_num)),
+        dws(std::vector<float>(weight_s[block_id], weight_s[block_id] + weight_head_num)), dy(acc.size());
+    check(flexllm_static_dequant_i32_f32(dacc.get(), dy.get(), das.get(), dws.get(), 1, act_head_num, weight_head_num, output_dim, nullptr));
+    fill_heads(output_stream, dy.download(), act_head_num, output_dim, head_parallel);
+}
+// Modules/quant.h:296-305: per token block, heads in order h*(act/weight)+g, output_dim values each
+template <int qint_bit, int io_parallel, int max_output_dim, int act_head_num = 1, int weight_head_num = 1, int max_seq_len = 1024,
+          int decoder_layer_num = 16, class IS, class OS>
+void pref_static_sym_per_tensor_dequant_layer_qint_fp32(IS& input_stream, OS& output_stream,
+                                                        const float input_s[decoder_layer_num][act_head_num],
+                                                        const float weight_s[decoder_layer_num][weight_head_num], int block_id,
+                                                        int seq_len = max_seq_len, int output_dim = max_output_dim) {
+    auto acc = drain_pref<int32_t>(input_stream, seq_len, act_head_num * output_dim, io_parallel);      // [token][head][dim]
+    DeviceArray<int32_t> dacc(acc);
+    DeviceArray<float> das(std::vector<float>(input_s[block_id], input_s[block_id] + act_head_num)),
+        dws(std::vector<float>(weight_s[block_id], weight_s[block_id] + weight_head_num)), dy(acc.size());
+    check(flexllm_static_dequant_i32_f32(dacc.get(), dy.get(), das.get(), dws.get(), seq_len, act_head_num, weight_head_num, output_dim, nullptr));
+    fill_pref(output_stream, dy.download(), seq_len, act_head_num * output_dim, io_parallel);
+}
+// Modules/MHA.h:246-251: entries with key index k beyond the token's own position become -1e32.  A selection without
+// arithmetic: done while re-packing the stream.
+template <typename T, int io_parallel, int max_hidden_dim = 2048, int max_seq_len = 1024, int head_num = 1, class IS, class OS>
+void pref_causal_mask_template(IS& input_stream, OS& output_stream, int seq_len = max_seq_len, int io_hidden_dim = max_hidden_dim) {
+    for (int M = 0; M < seq_len / io_parallel; M++)
+        for (int H = 0; H < head_num; H++)
+            for (int k = 0; k < io_hidden_dim; k++) {
+                auto in = input_stream.read();
+                typename OS::value_type o;
+                for (int i = 0; i < io_parallel; i++) o[i] = k <= M * io_parallel + i ? (T)in[i] : (T)-1e32;
+                output_stream.write(o);
+            }
+}
+// Modules/MHA.h:189-194.  The key stream carries, per token block M and query head H, the keys of that head's KV head in
+// blocks of K_parallel keys, feature-major inside a block (the cache manager's read order, Modules/MHA.h:96-106); the keys
+// are the same in every token block, so the first block's copy is kept and the repeats are read and dropped.
+template <int io_parallel, int K_parallel, int mha_head_num, int mha_head_dim = 64, int log2_mha_head_dim = 6, int max_seq_len = 1024,
+          bool is_uint_input = false, class IS, class IK, class OS>
+void pref_MHA_i8xi8_qxk_template(IS& input_seq, IK& weight_loader, OS& output_seq, int seq_len = max_seq_len) {
+    static_assert(!is_uint_input, "queries are signed");
+    const int hd = mha_head_dim;
+    std::vector<int8_t> q((size_t)mha_head_num * seq_len * hd), kk((size_t)mha_head_num * seq_len * hd);     // [head][token][d]
+    for (int M = 0; M < seq_len / io_parallel; M++)
+        for (int H = 0; H < mha_head_num; H++) {
+            for (int k = 0; k < hd; k++) {
+                auto pack = input_seq.read();
+                for (int m = 0; m < io_parallel; m++) q[((size_t)H * seq_len + M * io_parallel + m) * hd + k] = (int8_t)(int)pack[m];
+            }
+            for (int N = 0; N < seq_len / K_parallel; N++)
+                for (int k = 0; k < hd; k++) {
+                    auto kp = weight_loader.read();
+                    if (M == 0)
+                        for (int j = 0; j < K_parallel; j++) kk[((size_t)H * seq_len + N * K_parallel + j) * hd + k] = (int8_t)(int)kp[j];
+                }
+        }
+    DeviceArray<int8_t> dq(q), dk(kk);
+    DeviceArray<int32_t> dacc((size_t)mha_head_num * seq_len * seq_len);
+    for (int H = 0; H < mha_head_num; H++)
+        check(flexllm_linear_i8_gemm(dq.get() + (size_t)H * seq_len * hd, dk.get() + (size_t)H * seq_len * hd,
+                                     dacc.get() + (size_t)H * seq_len * seq_len, seq_len, hd, seq_len, nullptr));
+    auto acc = dacc.download();
+    for (int M = 0; M < seq_len / io_parallel; M++)
+        for (int H = 0; H < mha_head_num; H++)
+            for (int n = 0; n < seq_len; n++) {
+                typename OS::value_type o;
+                for (int m = 0; m < io_parallel; m++) o[m] = acc[((size_t)H * seq_len + M * io_parallel + m) * seq_len + n];
+                output_seq.write(o);
+            }
+}
+// Modules/MHA.h:339-344: probabilities [token][head][key] (unsigned when is_uint_input), V blocks of V_parallel channels,
+// key-major inside a block, repeated per token block like the keys above.
+template <int io_parallel, int V_parallel, int mha_head_num, int mha_head_dim = 64, int max_seq_len = 1024, int log2_max_seq_len = 10,
+          bool is_uint_input = false, class IS, class IV, class OS>
+void pref_MHA_i8xi8_axv_template(IS& input_seq, IV& weight_loader, OS& output_seq, int seq_len = max_seq_len) {
+    static_assert(is_uint_input, "the probabilities are unsigned 8-bit");
+    const int hd = mha_head_dim;
+    std::vector<uint8_t> p((size_t)mha_head_num * seq_len * seq_len);                                       // [head][token][key]
+    std::vector<int8_t> vt((size_t)mha_head_num * hd * seq_len);                                            // [head][channel][key]
+    for (int M = 0; M < seq_len / io_parallel; M++)
+        for (int H = 0; H < mha_head_num; H++) {
+            for (int k = 0; k < seq_len; k++) {
+                auto pack = input_seq.read();
+                for (int m = 0; m < io_parallel; m++) p[((size_t)H * seq_len + M * io_parallel + m) * seq_len + k] = (uint8_t)(int)pack[m];
+            }
+            for (int N = 0; N < hd / V_parallel; N++)
+                for (int k = 0; k < seq_len; k++) {
+                    auto vp = weight_loader.read();
+                    if (M == 0)
+                        for (int j = 0; j < V_parallel; j++) vt[((size_t)H * hd + N * V_parallel + j) * seq_len + k] = (int8_t)(int)vp[j];
+                }
+        }
+    DeviceArray<uint8_t> dp(p);
+    DeviceArray<int8_t> dv(vt);
+    DeviceArray<int32_t> dacc((size_t)mha_head_num * seq_len * hd);
+    for (int H = 0; H < mha_head_num; H++)
+        check(flexllm_linear_u8i8_gemm(dp.get() + (size_t)H * seq_len * seq_len, dv.get() + (size_t)H * hd * seq_len,
+                                       dacc.get() + (size_t)H * seq_len * hd, seq_len, seq_len, hd, nullptr));
+    auto acc = dacc.download();
+    for (int M = 0; M < seq_len / io_parallel; M++)
+        for (int H = 0; H < mha_head_num; H++)
+            for (int n = 0; n < hd; n++) {
+                typename OS::value_type o;
+                for (int m = 0; m < io_parallel; m++) o[m] = acc[((size_t)H * seq_len + M * io_parallel + m) * hd + n];
+                output_seq.write(o);
+            }
+}
+// Modules/MHA.h:615-620: one query per head; lane i's key stream carries, for each of its heads H, the keys in blocks of
+// K_parallel (the last block padded with whatever the cache line holds), feature-major inside a block.  The scores of the
+// padded keys are produced too, as in the reference (dec_quant_a_discard_template drops them afterwards).
+template <int head_parallel, int K_parallel, int mha_head_num, int mha_head_dim = 64, int log2_mha_head_dim = 6, int max_sum_seq_len = 2048,
+          bool is_uint_input = false, class IS, class IKS, class OS>
+void dec_MHA_i8xi8_qxk_template(IS& input_seq, IKS& weight_loaders, OS& output_seq, int seq_len) {
+    static_assert(!is_uint_input, "queries are signed");
+    const int hd = mha_head_dim, per = mha_head_num / head_parallel;
+    const int padded = (seq_len + K_parallel - 1) / K_parallel * K_parallel;
+    auto q = drain_heads<int8_t>(input_seq, mha_head_num, hd, head_parallel);                               // [head][d]
+    std::vector<int8_t> kk((size_t)mha_head_num * padded * hd);                                             // [head][key][d]
+    for (int H = 0; H < per; H++)
+        for (int N = 0; N < padded / K_parallel; N++)
+            for (int k = 0; k < hd; k++)
+                for (int i = 0; i < head_parallel; i++) {
+                    auto kp = weight_loaders[i].read();
+                    for (int j = 0; j < K_parallel; j++) kk[((size_t)(i * per + H) * padded + N * K_parallel + j) * hd + k] = (int8_t)(int)kp[j];
+                }
+    DeviceArray<int8_t> dq(q), dk(kk);
+    DeviceArray<int32_t> dacc((size_t)mha_head_num * padded);
+    for (int h = 0; h < mha_head_num; h++)
+        check(flexllm_linear_i8_gemv(dq.get() + (size_t)h * hd, dk.get() + (size_t)h * padded * hd, dacc.get() + (size_t)h * padded, hd, padded, nullptr));
+    fill_heads(output_seq, dacc.download(), mha_head_num, padded, head_parallel);
+}
+// Modules/MHA.h:854-859
+template <int head_parallel, int V_parallel, int mha_head_num, int mha_head_dim = 64, int max_sum_seq_len = 2048, int log2_max_sum_seq_len = 11,
+          bool is_uint_input = false, class IS, class IVS, class OS>
+void dec_MHA_i8xi8_axv_template(IS& input_seq, IVS& weight_loaders, OS& output_seq, int seq_len) {
+    static_assert(is_uint_input, "the probabilities are unsigned 8-bit");
+    const int hd = mha_head_dim, per = mha_head_num / head_parallel;
+    const int kpad = (seq_len + 15) / 16 * 16;                                                               // the product wants k % 16 == 0
+    std::vector<uint8_t> p((size_t)mha_head_num * kpad, 0);                                                  // [head][key], zero padding
+    std::vector<int8_t> vt((size_t)mha_head_num * hd * kpad, 0);                                             // [head][channel][key]
+    for (int H = 0; H < per; H++) {
+        for (int k = 0; k < seq_len; k++) {
+            auto pack = input_seq.read();
+            for (int i = 0; i < head_parallel; i++) p[(size_t)(i * per + H) * kpad + k] = (uint8_t)(int)pack[i];
+        }
+        for (int N = 0; N < hd / V_parallel; N++)
+            for (int k = 0; k < seq_len; k++)
+                for (int i = 0; i < head_parallel; i++) {
+                    auto vp = weight_loaders[i].read();
+                    for (int j = 0; j < V_parallel; j++) vt[((size_t)(i * per + H) * hd + N * V_parallel + j) * kpad + k] = (int8_t)(int)vp[j];
+                }
+    }
+    DeviceArray<uint8_t> dp(p);
+    DeviceArray<int8_t> dv(vt);
+    DeviceArray<int32_t> dacc((size_t)mha_head_num * hd);
+    for (int h = 0; h < mha_head_num; h++)
+        check(flexllm_linear_u8i8_gemm(dp.get() + (size_t)h * kpad, dv.get() + (size_t)h * hd * kpad, dacc.get() + (size_t)h * hd, 1, kpad, hd, nullptr));
+    fill_heads(output_seq, dacc.download(), mha_head_num, hd, head_parallel);
+}
+
+// ======================================================================================= launcher
+// tapa::invoke-shaped launcher: `top` is called with the remaining arguments and the elapsed time is returned in
+// nanoseconds, as tapa::invoke does (SpinQuant_Llama_32_1B/MHA_i8xi8_decoding_tb.cpp:241-252).  The bitstream argument is
+// kept for the call shape: "hip" (or an empty string, the reference's software-simulation spelling) runs on the GPU, any
+// other value is refused - there is no other backend.  The *_mmap(...) wrappers of the reference only tell TAPA the copy
+// direction; here they pass the host vectors through.
+template <class T> T& read_only_mmap(T& v) { return v; }
+template <class T> const T& read_only_mmap(const T& v) { return v; }
+template <class T> T& write_only_mmap(T& v) { return v; }
+template <class T> T& read_write_mmap(T& v) { return v; }
+template <class T, size_t N> T (&read_only_mmaps(T (&v)[N]))[N] { return v; }
+template <class T, size_t N> T (&read_write_mmaps(T (&v)[N]))[N] { return v; }
+template <class F, class... A>
+int64_t invoke(F&& top, const std::string& bitstream, A&&... args) {
+    if (!bitstream.empty() && bitstream != "hip") throw Error("fxhost::invoke: unknown bitstream '" + bitstream + "' (only \"hip\")");
+    check_hip(hipDeviceSynchronize());
+    const auto t0 = std::chrono::steady_clock::now();
+    top(std::forward<A>(args)...);
+    check_hip(hipDeviceSynchronize());
+    return (int64_t)std::chrono::duration_cast<std::chrono::nanoseconds>(std::chrono::steady_clock::now() - t0).count();
+}
+
 // ======================================================================================= MHA_i8xi8.h tops
 // MHA_i8xi8_Prefilling_tb (SpinQuant_Llama_32_1B/MHA_i8xi8.h:369-427) for ONE layer: q_mmap/k_mmap/v_mmap and
 // o_mmap use the prefill packing [(token/TP)*dim + feature][token%TP]; scales are that layer's rows of
@@ -452,6 +708,57 @@ int64_t MHA_i8xi8_Prefilling_layer(const std::vector<VF>& q_mmap, const std::vec
     for (int t = 0; t < seq_len; t++)
         for (int j = 0; j < H; j++) o_mmap[(size_t)(t / TP) * H + j][t % TP] = o[(size_t)t * H + j];
     return (int64_t)(ms * 1e6);
+}
+
+// MHA_i8xi8_decoding_tb (SpinQuant_Llama_32_1B/MHA_i8xi8.h:1027-1114) for ONE layer: dec_seq_len tokens are decoded one
+// after another on top of pre_seq_len cached positions.  q_mmap/k_mmap/v_mmap/o_mmap use the decode packing
+// [token*dim/BP + j % (dim/BP)][j / (dim/BP)] of that layer's slice; k_caches/v_caches are the reference's HP lane
+// buffers in its line layouts (all layers; `layer` selects the block), read for positions < pre_seq_len and written back
+// for the decoded positions, as the reference's cache managers do.  Scales: that layer's rows of Q_s/K_s/V_s/A_s.
+template <int BP, int HP, int KP, int VP, int q_heads, int kv_heads, int head_dim, class VF, class VK, class VV>
+void MHA_i8xi8_decoding_layer(const std::vector<VF>& q_mmap, const std::vector<VF>& k_mmap, const std::vector<VF>& v_mmap,
+                              std::vector<VK>* k_caches, std::vector<VV>* v_caches, std::vector<VF>& o_mmap, const float* Q_s,
+                              const float* K_s, const float* V_s, const float* A_s, int layer, int layers, int max_sum_seq_len,
+                              int pre_seq_len, int dec_seq_len, float sqrt_head_dim) {
+    const int H = q_heads * head_dim, KV = kv_heads * head_dim;
+    const CacheGeom geom{layers, kv_heads, head_dim, max_sum_seq_len};
+    const int max_pos = (pre_seq_len + dec_seq_len + 63) / 64 * 64;
+    auto unpack = [&](const std::vector<VF>& mm, int dim, int t) {
+        std::vector<float> x(dim);
+        const int per = dim / BP;
+        for (int j = 0; j < dim; j++) x[j] = mm[(size_t)t * per + j % per][j / per];
+        return x;
+    };
+    // the cached history -> token-major -> the GPU's cache layout
+    std::vector<int8_t> k_hist((size_t)pre_seq_len * KV), v_hist((size_t)pre_seq_len * KV);
+    kcache_decode_to_token_major<HP, KP>(k_caches, geom, layer, pre_seq_len, k_hist.data());
+    vcache_decode_to_token_major<HP, VP>(v_caches, geom, layer, pre_seq_len, v_hist.data());
+    DeviceArray<int8_t> dkh(k_hist), dvh(v_hist), kc((size_t)kv_heads * max_pos * head_dim), vc((size_t)kv_heads * max_pos * head_dim);
+    check_hip(hipMemset(kc.get(), 0, kc.size()));
+    check_hip(hipMemset(vc.get(), 0, vc.size()));
+    if (pre_seq_len > 0) check(flexllm_kv_store_i8(dkh.get(), dvh.get(), kc.get(), vc.get(), pre_seq_len, kv_heads, head_dim, max_pos, 0, nullptr));
+    DeviceArray<float> dqs(std::vector<float>(Q_s, Q_s + q_heads)), dks(std::vector<float>(K_s, K_s + kv_heads)),
+        dvs(std::vector<float>(V_s, V_s + kv_heads)), das(std::vector<float>(A_s, A_s + q_heads));
+    flexllm_mha_scales sc{dqs.get(), dks.get(), dvs.get(), das.get()};
+    DeviceArray<float> dq(H), dk(KV), dv(KV), dout(H);
+    DeviceArray<int8_t> q8(H), k8(KV), v8(KV);
+    for (int t = 0; t < dec_seq_len; t++) {
+        const int pos = pre_seq_len + t;
+        dq.upload(unpack(q_mmap, H, t));
+        dk.upload(unpack(k_mmap, KV, pos));              // the k/v buffers hold all positions; the decoded ones follow the history
+        dv.upload(unpack(v_mmap, KV, pos));
+        check(flexllm_static_quant_i8(dq.get(), q8.get(), dqs.get(), sqrt_head_dim, 1, 1, q_heads, head_dim, nullptr));
+        check(flexllm_static_quant_i8(dk.get(), k8.get(), dks.get(), 1.0f, 1, 1, kv_heads, head_dim, nullptr));
+        check(flexllm_static_quant_i8(dv.get(), v8.get(), dvs.get(), 1.0f, 1, 1, kv_heads, head_dim, nullptr));
+        check(flexllm_kv_store_i8(k8.get(), v8.get(), kc.get(), vc.get(), 1, kv_heads, head_dim, max_pos, pos, nullptr));
+        check(flexllm_mha_i8_decode(q8.get(), kc.get(), vc.get(), &sc, dout.get(), nullptr, pos + 1, q_heads, kv_heads, head_dim, max_pos, nullptr));
+        const auto k_new = k8.download(), v_new = v8.download();
+        kcache_decode_from_token_major<HP, KP>(k_new.data(), geom, layer, pos, 1, k_caches);
+        vcache_decode_from_token_major<HP, VP>(v_new.data(), geom, layer, pos, 1, v_caches);
+        const auto o = dout.download();
+        const int per = H / BP;
+        for (int j = 0; j < H; j++) o_mmap[(size_t)t * per + j % per][j / per] = o[j];
+    }
 }
 
 }  // namespace fxhost

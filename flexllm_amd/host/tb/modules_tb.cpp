@@ -6,8 +6,13 @@
 //   QuantWrapper linear, decode   <-> SpinQuant_Llama_32_1B/Linear_Layer_Decoding_tb.cpp:93-251 (1e-2 relative)
 //   QuantWrapper linear, prefill  <-> SpinQuant_Llama_32_1B/Linear_Layer_Prefilling_tb.cpp (1e-2 relative)
 //   MHA prefill                   <-> SpinQuant_Llama_32_1B/MHA_i8xi8_prefilling_tb.cpp:12-268 (5e-3 relative)
-//   FHT / RMSNorm / Swish / residual / softmax against float64 closed forms
+//   MHA decode                    <-> SpinQuant_Llama_32_1B/MHA_i8xi8_decoding_tb.cpp:12-289 (QK^T 1e-3, attention 5e-3),
+//                                     launched through fxhost::invoke(top, "hip", mmaps..., scalars...) on the reference's
+//                                     own cache line layouts, and stage by stage through the dec_MHA_* module functions
+//   layout adapters               <-> the packed int4 weight words and the KV-cache line layouts of the testbenches
+//   FHT / RMSNorm / Swish / residual / softmax / RoPE against float64 closed forms
 #include <algorithm>
+#include <array>
 #include <cmath>
 #include <cstdio>
 #include <iostream>
@@ -364,6 +369,325 @@ static void pref_MHA_test() {
     verdict("MHA (prefill, int8 q/k/v, uint8 probabilities)", correct);
 }
 
+// Decode attention, shaped like SpinQuant_Llama_32_1B/MHA_i8xi8_decoding_tb.cpp:12-289 for one layer (layer 1 of 2, so
+// that the layer offsets of the cache buffers matter): a history of PRE positions held in the reference's lane buffers,
+// DEC tokens decoded on top.  Checks: (1) q.K^T of the last token against the fake-quant golden at 1e-3 through the
+// dec_MHA_* module functions fed from the cache lines; (2) the whole attention through fxhost::invoke on the top
+// function at 5e-3; (3) the module chain (scores -> softmax -> uint8 quant -> P.V -> dequant) against the top bit for bit.
+static void dec_MHA_test() {
+    constexpr int BP = 16, HP = 8, KP = 32, VP = 32, LAYERS = 2, LAYER = 1, MAX_SUM = 256, PRE = 100, DEC = 4;
+    constexpr int H = HIDDEN_DIM, KV = KV_HIDDEN_DIM, per_q = H / BP, per_kv = KV / BP, hpl = KV_HEAD_NUM / HP;
+    std::default_random_engine gen(42);
+    std::uniform_real_distribution<float> dist(-128.0 / std::sqrt((double)HIDDEN_DIM), 128.0 / std::sqrt((double)HIDDEN_DIM));
+    static float Q_s[LAYERS][Q_HEAD_NUM], K_s[LAYERS][KV_HEAD_NUM], V_s[LAYERS][KV_HEAD_NUM], A_s[LAYERS][Q_HEAD_NUM];
+    for (int l = 0; l < LAYERS; l++) {
+        for (int h = 0; h < Q_HEAD_NUM; h++) { Q_s[l][h] = float(h + 1 + l) / HIDDEN_DIM; A_s[l][h] = 1.0f / 256; }
+        for (int h = 0; h < KV_HEAD_NUM; h++) { K_s[l][h] = float(h + 1 + l) / HIDDEN_DIM * 4; V_s[l][h] = float(h + 2 + l) / HIDDEN_DIM * 4; }
+    }
+    using VF = vec<float, BP>;
+    using VK = vec<int8_t, KP>;
+    using VV = vec<int8_t, VP>;
+    std::vector<VF> q_mmap((size_t)DEC * per_q), k_mmap((size_t)(PRE + DEC) * per_kv), v_mmap((size_t)(PRE + DEC) * per_kv), o_mmap((size_t)DEC * per_q);
+    std::vector<VK> k_caches[HP];
+    std::vector<VV> v_caches[HP];
+    for (int i = 0; i < HP; i++) {
+        k_caches[i].assign((size_t)LAYERS * hpl * MAX_SUM / KP * HEAD_DIM, VK());
+        v_caches[i].assign((size_t)LAYERS * hpl * HEAD_DIM / VP * MAX_SUM, VV());
+    }
+    std::vector<double> q_gold((size_t)DEC * H), k_gold((size_t)(PRE + DEC) * KV), v_gold((size_t)(PRE + DEC) * KV);
+    for (int i = 0; i < DEC; i++)
+        for (int j = 0; j < H; j++) {
+            const float val = dist(gen);
+            q_mmap[(size_t)i * per_q + j % per_q][j / per_q] = val;
+            int qv = (int)std::round(val / 8.0f / Q_s[LAYER][j / HEAD_DIM]);
+            qv = std::max(-128, std::min(127, qv));
+            q_gold[(size_t)i * H + j] = qv * (double)Q_s[LAYER][j / HEAD_DIM];
+        }
+    for (int i = 0; i < PRE + DEC; i++)
+        for (int j = 0; j < KV; j++) {
+            const int h = j / HEAD_DIM, d = j % HEAD_DIM;
+            const float kv = dist(gen), vv = dist(gen);
+            k_mmap[(size_t)i * per_kv + j % per_kv][j / per_kv] = kv;
+            v_mmap[(size_t)i * per_kv + j % per_kv][j / per_kv] = vv;
+            int kq = std::max(-128, std::min(127, (int)std::round(kv / K_s[LAYER][h])));
+            int vq = std::max(-128, std::min(127, (int)std::round(vv / V_s[LAYER][h])));
+            if (i < PRE) {      // the history sits in the lane buffers, written with the testbench's own index formulas (:77-80, :214-216)
+                k_caches[h / hpl][((size_t)(LAYER * hpl + h % hpl) * MAX_SUM + i) / KP * HEAD_DIM + d][i % KP] = (int8_t)kq;
+                v_caches[h / hpl][((size_t)(LAYER * hpl + h % hpl) * HEAD_DIM + d) / VP * MAX_SUM + i][d % VP] = (int8_t)vq;
+            }
+            k_gold[(size_t)i * KV + j] = kq * (double)K_s[LAYER][h];
+            v_gold[(size_t)i * KV + j] = vq * (double)V_s[LAYER][h];
+        }
+    std::cout << "kernel begins running!\n";
+    const int64_t ns = invoke(MHA_i8xi8_decoding_layer<BP, HP, KP, VP, Q_HEAD_NUM, KV_HEAD_NUM, HEAD_DIM, VF, VK, VV>, "hip",
+                              read_only_mmap(q_mmap), read_only_mmap(k_mmap), read_only_mmap(v_mmap), read_write_mmaps(k_caches),
+                              read_write_mmaps(v_caches), write_only_mmap(o_mmap), Q_s[LAYER], K_s[LAYER], V_s[LAYER], A_s[LAYER], LAYER, LAYERS,
+                              MAX_SUM, PRE, DEC, 8.0f);
+    std::cout << "kernel time: " << ns * 1e-9 << " s" << std::endl;
+    // (2) whole attention against the fake-quant golden
+    bool correct = true;
+    std::vector<double> a(PRE + DEC), p(PRE + DEC);
+    for (int i = 0; i < DEC && correct; i++)
+        for (int h = 0; h < Q_HEAD_NUM && correct; h++) {
+            const int kh = h / (Q_HEAD_NUM / KV_HEAD_NUM), len = PRE + i + 1;
+            double mx = -1e300, sum = 0;
+            for (int j = 0; j < len; j++) {
+                double acc = 0;
+                for (int d = 0; d < HEAD_DIM; d++) acc += q_gold[(size_t)i * H + h * HEAD_DIM + d] * k_gold[(size_t)j * KV + kh * HEAD_DIM + d];
+                a[j] = acc; mx = std::max(mx, acc);
+            }
+            for (int j = 0; j < len; j++) { p[j] = std::exp(a[j] - mx); sum += p[j]; }
+            for (int j = 0; j < len; j++) p[j] = std::min(255.0, std::round(p[j] / sum / A_s[LAYER][h])) * A_s[LAYER][h];
+            for (int d = 0; d < HEAD_DIM; d++) {
+                double o = 0;
+                for (int j = 0; j < len; j++) o += p[j] * v_gold[(size_t)j * KV + kh * HEAD_DIM + d];
+                const int jj = h * HEAD_DIM + d;
+                const float my = o_mmap[(size_t)i * per_q + jj % per_q][jj / per_q];
+                if (std::abs(my - o) > 5e-3 * std::abs(o) + 1.5 * A_s[LAYER][h] * 128 * V_s[LAYER][kh]) {
+                    correct = false;
+                    std::cout << "Mismatch at (" << i << ", " << jj << "): My: " << my << ", Ref: " << o << std::endl;
+                    break;
+                }
+            }
+        }
+    verdict("MHA (decode, the reference's cache lines, launched through invoke)", correct);
+    // the decoded rows were written back into the lane buffers: layer 0's block untouched, layer 1 holds PRE + DEC rows
+    {
+        bool ok = true;
+        std::vector<int8_t> k_tm((size_t)(PRE + DEC) * KV), v_tm((size_t)(PRE + DEC) * KV);
+        const CacheGeom geom{LAYERS, KV_HEAD_NUM, HEAD_DIM, MAX_SUM};
+        kcache_decode_to_token_major<HP, KP>(k_caches, geom, LAYER, PRE + DEC, k_tm.data());
+        vcache_decode_to_token_major<HP, VP>(v_caches, geom, LAYER, PRE + DEC, v_tm.data());
+        for (int i = 0; i < PRE + DEC; i++)
+            for (int j = 0; j < KV; j++) {
+                if (std::abs(k_tm[(size_t)i * KV + j] * (double)K_s[LAYER][j / HEAD_DIM] - k_gold[(size_t)i * KV + j]) > 1e-9) ok = false;
+                if (std::abs(v_tm[(size_t)i * KV + j] * (double)V_s[LAYER][j / HEAD_DIM] - v_gold[(size_t)i * KV + j]) > 1e-9) ok = false;
+            }
+        std::vector<int8_t> k0((size_t)MAX_SUM * KV);
+        kcache_decode_to_token_major<HP, KP>(k_caches, geom, 0, MAX_SUM, k0.data());
+        for (int8_t v : k0) if (v != 0) ok = false;
+        verdict("decode cache write-back (rows of the decoded tokens in the reference's line layout)", ok);
+    }
+    // (1) + (3): the last decoded token stage by stage through the module functions, keys and values streamed from the lane buffers
+    {
+        const int t = DEC - 1, len = PRE + DEC, per = Q_HEAD_NUM / HP, padded = (len + KP - 1) / KP * KP;
+        stream<vec<float, HP>> q_s;
+        stream<vec<int8_t, HP>> q8_s;
+        std::vector<float> qv(H);
+        for (int j = 0; j < H; j++) qv[j] = q_mmap[(size_t)t * per_q + j % per_q][j / per_q];
+        for (int Hh = 0; Hh < per; Hh++)
+            for (int k = 0; k < HEAD_DIM; k++) { vec<float, HP> pk; for (int m = 0; m < HP; m++) pk[m] = qv[(size_t)(m * per + Hh) * HEAD_DIM + k]; q_s.write(pk); }
+        dec_MHA_static_sym_per_tensor_quant_layer_fp32_qint<8, HP, HEAD_DIM, Q_HEAD_NUM, true, LAYERS>(q_s, q8_s, Q_s, LAYER, HEAD_DIM, 8.0f);
+        // key streams in the cache manager's read order (Modules/MHA.h:503-513): per lane, its heads, each repeated for the
+        // group's query heads; lane i of the q.K^T module serves query heads i*per + Hh, i.e. KV head (i*per + Hh) / 4
+        std::array<stream<VK>, HP> k_str;
+        for (int Hh = 0; Hh < per; Hh++)
+            for (int N = 0; N < padded / KP; N++)
+                for (int k = 0; k < HEAD_DIM; k++)
+                    for (int i = 0; i < HP; i++) {
+                        const int kh = (i * per + Hh) / (Q_HEAD_NUM / KV_HEAD_NUM);
+                        k_str[i].write(k_caches[kh / hpl][((size_t)(LAYER * hpl + kh % hpl) * MAX_SUM + N * KP) / KP * HEAD_DIM + k]);
+                    }
+        stream<vec<int32_t, HP>> acc_s, acc_trim;
+        dec_MHA_i8xi8_qxk_template<HP, KP, Q_HEAD_NUM, HEAD_DIM, 6, MAX_SUM>(q8_s, k_str, acc_s, len);
+        for (int Hh = 0; Hh < per; Hh++)                                   // dec_quant_a_discard_template: drop the padded keys
+            for (int k = 0; k < padded; k++) { auto pk = acc_s.read(); if (k < len) acc_trim.write(pk); }
+        stream<vec<float, HP>> a_s, sfm_s;
+        dec_MHA_static_sym_per_tensor_dequant_layer_qint_fp32<22, HP, MAX_SUM, Q_HEAD_NUM, KV_HEAD_NUM, LAYERS>(acc_trim, a_s, Q_s, K_s, LAYER, len);
+        // (1) scores against the golden at 1e-3 (MHA_i8xi8_decoding_tb.cpp: qxk check)
+        bool ok1 = true;
+        std::vector<float> scores((size_t)Q_HEAD_NUM * len);
+        stream<vec<float, HP>> a_copy;
+        for (int Hh = 0; Hh < per; Hh++)
+            for (int k = 0; k < len; k++) { auto pk = a_s.read(); a_copy.write(pk); for (int m = 0; m < HP; m++) scores[(size_t)(m * per + Hh) * len + k] = pk[m]; }
+        for (int h = 0; h < Q_HEAD_NUM; h++)
+            for (int j = 0; j < len; j++) {
+                double g = 0;
+                const int kh = h / (Q_HEAD_NUM / KV_HEAD_NUM);
+                for (int d = 0; d < HEAD_DIM; d++) g += q_gold[(size_t)t * H + h * HEAD_DIM + d] * k_gold[(size_t)j * KV + kh * HEAD_DIM + d];
+                if (std::abs(scores[(size_t)h * len + j] - g) > 1e-3 * std::abs(g) + 1e-6) ok1 = false;
+            }
+        verdict("MHA q.K^T (decode modules fed from the cache lines, 1e-3)", ok1);
+        dec_MHA_Softmax<float, HP, MAX_SUM, Q_HEAD_NUM>(a_copy, sfm_s, len);
+        stream<vec<uint8_t, HP>> p8_s;
+        dec_MHA_static_sym_per_tensor_quant_layer_fp32_qint<8, HP, MAX_SUM, Q_HEAD_NUM, false, LAYERS>(sfm_s, p8_s, A_s, LAYER, len, 1.0f);
+        std::array<stream<VV>, HP> v_str;
+        for (int Hh = 0; Hh < per; Hh++)
+            for (int N = 0; N < HEAD_DIM / VP; N++)
+                for (int k = 0; k < len; k++)
+                    for (int i = 0; i < HP; i++) {
+                        const int kh = (i * per + Hh) / (Q_HEAD_NUM / KV_HEAD_NUM);
+                        v_str[i].write(v_caches[kh / hpl][((size_t)(LAYER * hpl + kh % hpl) * HEAD_DIM + N * VP) / VP * MAX_SUM + k]);
+                    }
+        stream<vec<int32_t, HP>> o_acc_s;
+        stream<vec<float, HP>> o_s;
+        dec_MHA_i8xi8_axv_template<HP, VP, Q_HEAD_NUM, HEAD_DIM, MAX_SUM, 8, true>(p8_s, v_str, o_acc_s, len);
+        dec_MHA_static_sym_per_tensor_dequant_layer_qint_fp32<24, HP, HEAD_DIM, Q_HEAD_NUM, KV_HEAD_NUM, LAYERS>(o_acc_s, o_s, A_s, V_s, LAYER, HEAD_DIM);
+        bool ok3 = true;
+        int differing = 0;
+        for (int Hh = 0; Hh < per; Hh++)
+            for (int k = 0; k < HEAD_DIM; k++) {
+                auto pk = o_s.read();
+                for (int m = 0; m < HP; m++) {
+                    const int h = m * per + Hh, jj = h * HEAD_DIM + k;
+                    const float d = std::abs(pk[m] - o_mmap[(size_t)t * per_q + jj % per_q][jj / per_q]);
+                    // identical integer stages; the two softmax sums are associated differently, so a probability byte on a
+                    // rounding tie may differ by one step (a whole head's 64 outputs then move by at most A_s * 128 * V_s)
+                    if (d != 0) differing++;
+                    if (d > 1.5f * A_s[LAYER][h] * 128 * V_s[LAYER][h / (Q_HEAD_NUM / KV_HEAD_NUM)]) ok3 = false;
+                }
+            }
+        if (differing > 2 * HEAD_DIM) ok3 = false;
+        verdict("MHA module chain (scores, softmax, uint8 probabilities, P.V, dequant) against the fused top", ok3);
+    }
+}
+
+// Prefill attention stage by stage through the module functions against the fused top, and the decode RoPE module.
+static void pref_MHA_modules_test() {
+    constexpr int S = 32, TP = TOKEN_PARALLEL, QH = 4, KVH = 2, KP = 16, VP = 16, LAYERS = 1;
+    constexpr int Hd = QH * HEAD_DIM, KVd = KVH * HEAD_DIM;
+    std::default_random_engine gen(5);
+    std::uniform_real_distribution<float> dist(-2.8f, 2.8f);
+    static float Q_s[LAYERS][QH], K_s[LAYERS][KVH], V_s[LAYERS][KVH], A_s[LAYERS][QH];
+    for (int h = 0; h < QH; h++) { Q_s[0][h] = 0.004f + 0.001f * h; A_s[0][h] = 1.0f / 255; }
+    for (int h = 0; h < KVH; h++) { K_s[0][h] = 0.03f + 0.002f * h; V_s[0][h] = 0.025f + 0.003f * h; }
+    using VF = vec<float, TP>;
+    std::vector<VF> q_mmap((size_t)S / TP * Hd), k_mmap((size_t)S / TP * KVd), v_mmap((size_t)S / TP * KVd), o_mmap((size_t)S / TP * Hd);
+    for (auto& pk : q_mmap) for (int m = 0; m < TP; m++) pk[m] = dist(gen);
+    for (auto& pk : k_mmap) for (int m = 0; m < TP; m++) pk[m] = dist(gen);
+    for (auto& pk : v_mmap) for (int m = 0; m < TP; m++) pk[m] = dist(gen);
+    MHA_i8xi8_Prefilling_layer<TP, QH, KVH, HEAD_DIM>(q_mmap, k_mmap, v_mmap, o_mmap, Q_s[0], K_s[0], V_s[0], A_s[0], S, 8.0f);
+    // stage chain: static quant -> q.K^T -> dequant -> mask -> softmax -> uint8 quant -> P.V -> dequant
+    stream<VF> q_in, k_in, v_in;
+    for (auto& pk : q_mmap) q_in.write(pk);
+    for (auto& pk : k_mmap) k_in.write(pk);
+    for (auto& pk : v_mmap) v_in.write(pk);
+    stream<vec<int8_t, TP>> q8_s, k8_s, v8_s;
+    pref_static_sym_per_tensor_quant_layer_fp32_qint<8, TP, HEAD_DIM, QH, true, 1024, LAYERS>(q_in, q8_s, Q_s, 0, S, HEAD_DIM, 8.0f);
+    pref_static_sym_per_tensor_quant_layer_fp32_qint<8, TP, HEAD_DIM, KVH, true, 1024, LAYERS>(k_in, k8_s, K_s, 0, S, HEAD_DIM, 1.0f);
+    pref_static_sym_per_tensor_quant_layer_fp32_qint<8, TP, HEAD_DIM, KVH, true, 1024, LAYERS>(v_in, v8_s, V_s, 0, S, HEAD_DIM, 1.0f);
+    std::vector<int8_t> k8((size_t)S * KVd), v8((size_t)S * KVd);
+    for (int M = 0; M < S / TP; M++)
+        for (int j = 0; j < KVd; j++) {
+            auto kp = k8_s.read(); auto vp = v8_s.read();
+            for (int m = 0; m < TP; m++) { k8[(size_t)(M * TP + m) * KVd + j] = kp[m]; v8[(size_t)(M * TP + m) * KVd + j] = vp[m]; }
+        }
+    // key / value streams in the prefill cache managers' read order (Modules/MHA.h:96-106, :322-333)
+    stream<vec<int8_t, KP>> k_str;
+    stream<vec<int8_t, VP>> v_str;
+    for (int M = 0; M < S / TP; M++)
+        for (int h = 0; h < QH; h++) {
+            const int kh = h / (QH / KVH);
+            for (int N = 0; N < S / KP; N++)
+                for (int d = 0; d < HEAD_DIM; d++) { vec<int8_t, KP> pk; for (int j = 0; j < KP; j++) pk[j] = k8[(size_t)(N * KP + j) * KVd + kh * HEAD_DIM + d]; k_str.write(pk); }
+            for (int N = 0; N < HEAD_DIM / VP; N++)
+                for (int t = 0; t < S; t++) { vec<int8_t, VP> pk; for (int j = 0; j < VP; j++) pk[j] = v8[(size_t)t * KVd + kh * HEAD_DIM + N * VP + j]; v_str.write(pk); }
+        }
+    stream<vec<int32_t, TP>> acc_s, o_acc_s;
+    stream<VF> a_s, masked_s, sfm_s, o_s;
+    stream<vec<uint8_t, TP>> p8_s;
+    pref_MHA_i8xi8_qxk_template<TP, KP, QH, HEAD_DIM, 6, 1024>(q8_s, k_str, acc_s, S);
+    pref_static_sym_per_tensor_dequant_layer_qint_fp32<22, TP, 1024, QH, KVH, 1024, LAYERS>(acc_s, a_s, Q_s, K_s, 0, S, S);
+    pref_causal_mask_template<float, TP, 1024, 1024, QH>(a_s, masked_s, S, S);
+    pref_Softmax<float, TP, 1024, 1024, QH>(masked_s, sfm_s, S, S);
+    pref_static_sym_per_tensor_quant_layer_fp32_qint<8, TP, 1024, QH, false, 1024, LAYERS>(sfm_s, p8_s, A_s, 0, S, S, 1.0f);
+    pref_MHA_i8xi8_axv_template<TP, VP, QH, HEAD_DIM, 1024, 10, true>(p8_s, v_str, o_acc_s, S);
+    pref_static_sym_per_tensor_dequant_layer_qint_fp32<26, TP, HEAD_DIM, QH, KVH, 1024, LAYERS>(o_acc_s, o_s, A_s, V_s, 0, S, HEAD_DIM);
+    bool ok = true;
+    int flips = 0;
+    for (size_t i = 0; i < o_mmap.size(); i++) {
+        auto pk = o_s.read();
+        for (int m = 0; m < TP; m++) {
+            const float d = std::abs(pk[m] - o_mmap[i][m]);
+            if (d != 0) flips++;                                            // the row sums of the two paths are associated differently:
+            if (d > 1.5f * A_s[0][0] * 128 * 0.04f) ok = false;             // a probability byte on a tie may differ by one step
+        }
+    }
+    if (flips > (int)(o_mmap.size() * TP) / 20) ok = false;
+    verdict("MHA module chain (prefill: q.K^T, mask, softmax, uint8 probabilities, P.V) against the fused top", ok);
+    // decode RoPE module against the closed form
+    {
+        constexpr int HP = 8, POS = 37;
+        static float PE_sin[64][HEAD_DIM / 2], PE_cos[64][HEAD_DIM / 2];
+        for (int s0 = 0; s0 < 64; s0++)
+            for (int i = 0; i < HEAD_DIM / 2; i++) { const double f = std::pow(500000.0, -2.0 * i / HEAD_DIM); PE_sin[s0][i] = (float)std::sin(s0 * f); PE_cos[s0][i] = (float)std::cos(s0 * f); }
+        std::vector<float> x((size_t)Q_HEAD_NUM * HEAD_DIM);
+        for (auto& v : x) v = dist(gen);
+        stream<vec<float, HP>> in, out;
+        const int per = Q_HEAD_NUM / HP;
+        for (int Hh = 0; Hh < per; Hh++)
+            for (int k = 0; k < HEAD_DIM; k++) { vec<float, HP> pk; for (int m = 0; m < HP; m++) pk[m] = x[(size_t)(m * per + Hh) * HEAD_DIM + k]; in.write(pk); }
+        dec_RoPE_layer<float, HP, HEAD_DIM, Q_HEAD_NUM, 64>(in, out, PE_sin, PE_cos, Q_HEAD_NUM, POS);
+        bool okr = true;
+        for (int Hh = 0; Hh < per; Hh++)
+            for (int k = 0; k < HEAD_DIM; k++) {
+                auto pk = out.read();
+                for (int m = 0; m < HP; m++) {
+                    const float* xh = &x[(size_t)(m * per + Hh) * HEAD_DIM];
+                    const int kk = k % 32;
+                    const double e = k < 32 ? (double)xh[kk] * PE_cos[POS][kk] - (double)xh[kk + 32] * PE_sin[POS][kk]
+                                            : (double)xh[kk] * PE_sin[POS][kk] + (double)xh[kk + 32] * PE_cos[POS][kk];
+                    if (std::abs(pk[m] - e) > 1e-5) okr = false;
+                }
+            }
+        verdict("RoPE (decode stream, head-parallel lanes)", okr);
+    }
+}
+
+// The layout adapters against the testbenches' index formulas, and as round trips.
+static void adapters_test() {
+    bool ok = true;
+    std::default_random_engine gen(9);
+    std::uniform_int_distribution<int> d4(-8, 7), d8(-128, 127);
+    {   // int4 weight words, decode form (Linear_Layer_Decoding_tb.cpp:176-186) and prefill form (Linear_Layer.h:134-185)
+        constexpr int N = 256, K = 64, BP = 8, WP = 16;
+        std::vector<int8_t> w((size_t)N * K), back((size_t)N * K);
+        for (auto& v : w) v = (int8_t)d4(gen);
+        std::vector<vec<int8_t, WP / 2>> lanes[BP];
+        pack_weight_int4_decode<WP, BP>(w.data(), N, K, lanes);
+        for (int n : {0, 1, 17, 31, 32, 255})
+            for (int k : {0, 5, 63}) {
+                const int I = n / (N / BP), i = n % (N / BP);
+                const unsigned byte = (uint8_t)lanes[I][(size_t)(i / WP) * K + k][(i / 2) % (WP / 2)];
+                if (sext4(byte >> (4 * (i % 2))) != w[(size_t)n * K + k]) ok = false;
+            }
+        unpack_weight_int4_decode<WP, BP>(lanes, N, K, back.data());
+        if (back != w) ok = false;
+        std::vector<vec<int8_t, WP / 2>> flat;
+        pack_weight_int4_prefill<WP>(w.data(), N, K, flat);
+        for (int n : {0, 3, 16, 200})
+            for (int k : {0, 63}) {
+                const unsigned byte = (uint8_t)flat[(size_t)(n / WP) * K + k][(n / 2) % (WP / 2)];
+                if (sext4(byte >> (4 * (n % 2))) != w[(size_t)n * K + k]) ok = false;
+            }
+        std::fill(back.begin(), back.end(), 0);
+        unpack_weight_int4_prefill<WP>(flat, N, K, back.data());
+        if (back != w) ok = false;
+    }
+    {   // KV cache lines, prefill buffers (Modules/MHA.h:74-109, :299-336)
+        constexpr int L = 2, KVH = 2, HD = 64, SMAX = 64, KP = 16, VP = 16, LEN = 40, LAYER = 1;
+        const CacheGeom g{L, KVH, HD, SMAX};
+        std::vector<int8_t> tm((size_t)LEN * KVH * HD), back(tm.size());
+        for (auto& v : tm) v = (int8_t)d8(gen);
+        std::vector<vec<int8_t, KP>> kc((size_t)L * KVH * SMAX / KP * HD);
+        std::vector<vec<int8_t, VP>> vcv((size_t)L * KVH * HD / VP * SMAX);
+        kcache_prefill_from_token_major<KP>(tm.data(), g, LAYER, 0, LEN, kc);
+        vcache_prefill_from_token_major<VP>(tm.data(), g, LAYER, 0, LEN, vcv);
+        for (int t : {0, 15, 16, 39})
+            for (int h = 0; h < KVH; h++)
+                for (int d : {0, 17, 63}) {
+                    if (kc[((size_t)(LAYER * KVH + h) * SMAX / KP + t / KP) * HD + d][t % KP] != tm[((size_t)t * KVH + h) * HD + d]) ok = false;
+                    const int ch = h * HD + d;
+                    if (vcv[((size_t)LAYER * (KVH * HD) / VP + ch / VP) * SMAX + t][ch % VP] != tm[((size_t)t * KVH + h) * HD + d]) ok = false;
+                }
+        kcache_prefill_to_token_major<KP>(kc, g, LAYER, LEN, back.data());
+        if (back != tm) ok = false;
+        vcache_prefill_to_token_major<VP>(vcv, g, LAYER, LEN, back.data());
+        if (back != tm) ok = false;
+    }
+    verdict("layout adapters (packed int4 weight words, prefill KV-cache lines; the decode lines are exercised by the MHA test)", ok);
+}
+
 int main() {
     try {
         QuantWrapper_Linear_Layer_q_decoding_test();
@@ -372,6 +696,9 @@ int main() {
         FHT_test();
         Elementwise_test();
         pref_MHA_test();
+        dec_MHA_test();
+        pref_MHA_modules_test();
+        adapters_test();
     } catch (const std::exception& e) {
         std::cerr << "harness error: " << e.what() << std::endl;
         return 2;

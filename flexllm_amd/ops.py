@@ -71,6 +71,15 @@ def linear_i8_gemv(x, w, stream=None, out=None):
     return acc
 
 
+def linear_u8i8_gemm(a, w, stream=None, out=None):
+    """acc[m][n] = sum_k a[m][k] (uint8) * w[n][k] (int8): the probabilities x V product as a stand-alone module."""
+    m, k = a.shape
+    n = w.shape[0]
+    acc = out if out is not None else DeviceArray((m, n), np.int32)
+    check(lib().flexllm_linear_u8i8_gemm(_p(a), _p(w), _p(acc), m, k, n, _s(stream)))
+    return acc
+
+
 def linear_i8_gemv_dequant(x, s_x, w, w_s, residual=None, stream=None, out=None):
     n, k = w.shape
     y = out if out is not None else DeviceArray((n,), np.float32)

@@ -112,6 +112,12 @@ int flexllm_linear_i8_gemv_swiglu(const int8_t* x, const float* s_x, const int8_
  * pref_Linear_Layer_i4xi4 (Modules/Linear_Layer.h:293-341) with the int8 systolic array
  * (Modules/MHA.h:113-187, Modules/PE.h:526-583).  k % 64 == 0. */
 int flexllm_linear_i8_gemm(const int8_t* a, const int8_t* w, int32_t* acc, int m, int k, int n, void* stream);
+/* The same exact product with UNSIGNED 8-bit activations (0..255), the reference's is_uint_input instantiation of its
+ * int8 arrays (Modules/MHA.h:339-344, :854-859 with is_uint_input = true; Modules/PE.h:526-583, is_uint_A): used for
+ * P.V with the uint8 softmax probabilities as a stand-alone stage.  a [m][k] uint8, w [n][k] int8, acc [m][n] int32;
+ * k % 16 == 0; m = 1 is the decode form.  A plain kernel (one wave per output): the fused attention entry points are
+ * the fast path. */
+int flexllm_linear_u8i8_gemm(const uint8_t* a, const int8_t* w, int32_t* acc, int m, int k, int n, void* stream);
 /* Fused prefill linear: y[m][n] = (float(acc)*s_x[m])*w_s[n] (+ residual[m][n]).
  * = GEMM + pref_dequant_layer_qint_fp32 (Modules/quant.h:115-164) (+ pref_Residual_Layer). */
 int flexllm_linear_i8_gemm_dequant(const int8_t* a, const float* s_x, const int8_t* w, const float* w_s,

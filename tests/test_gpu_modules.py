@@ -139,6 +139,24 @@ def test_gemv_int32_exact(fx, oracle, k, n):
     assert np.array_equal(acc.numpy(), oracle.linear_i8(x[None, :], w)[0])
 
 
+@pytest.mark.parametrize("m,k,n", [(1, 16, 1), (7, 48, 5), (100, 1024, 64), (33, 4096, 64), (1024, 1024, 64)])
+def test_u8i8_gemm_int32_exact(fx, m, k, n):
+    """MHA_i8xi8.h:286-345 (probabilities x V as a module of its own): unsigned 8-bit rows times signed 8-bit rows."""
+    a = rng.integers(0, 256, (m, k)).astype(np.uint8)
+    w = rng.integers(-128, 128, (n, k)).astype(np.int8)
+    a[0, :] = 255; w[0, :] = -128                       # the extreme product, k * 255 * -128, in acc[0][0]
+    acc = fx.ops.linear_u8i8_gemm(fx.to_device(a), fx.to_device(w)).numpy()
+    ref = a.astype(np.int64) @ w.astype(np.int64).T
+    assert np.array_equal(acc, ref.astype(np.int32)) and acc[0, 0] == -k * 255 * 128
+
+
+def test_u8i8_gemm_rejects_a_ragged_inner_size(fx):
+    a = fx.to_device(np.zeros((2, 24), np.uint8)); w = fx.to_device(np.zeros((3, 24), np.int8))
+    from flexllm_amd._lib import FlexLLMError
+    with pytest.raises(FlexLLMError, match="multiple of 16"):
+        fx.ops.linear_u8i8_gemm(a, w)
+
+
 def test_gemv_extreme_values_exact(fx):
     k, n = 8192, 64
     x = np.full(k, -128, np.int8); w = np.full((n, k), -128, np.int8)
