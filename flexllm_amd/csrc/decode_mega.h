@@ -61,8 +61,12 @@ struct MegaParams {
     float2* stats;                 // [q_heads][32] (one-kernel-per-stage path)
     unsigned long long* qkv_tag;   // [H + 2*KV]: q/k/v projection outputs, each with the epoch in its high word
     unsigned long long* stats_tag; // [q_heads][32][2]: chunk max and chunk sum of exponentials, each with the epoch in its high word
-    int32_t* o_acc;                // [H]
-    int* state;                    // [0] pos, [1] step, [2] barrier epoch base, [3] error flag
+    unsigned long long* x_tag;     // [H]: the residual stream after a layer (down projection + residual), tagged with the layer's sequence number
+    unsigned long long* x2_tag;    // [H]: the residual stream after attention (o projection + residual), tagged likewise
+    unsigned* h_flag;              // [kFlagCopies][kFlagStride]: sequence number of the layer pass whose 32 values of h workgroup w has published
+    unsigned* o_flag;              // same shape: ... whose attention parts workgroup w has added to o_acc
+    int32_t* o_acc;                // [H]: attention accumulators (zero at launch, cleared again once read)
+    int* state;                    // [0] pos, [1] step, [2] barrier epoch base, [3] error flag, [4] layer sequence number base
     unsigned* bar;                 // [0] flag, [64] top counter, [128+64g] group counters
     int* token;                    // current token id (device), used when x_in == NULL; greedy mode leaves the last token here
     int* tokens_out;               // greedy mode: generated ids are written to tokens_out[state[1] + step]; NULL otherwise
@@ -123,6 +127,59 @@ __device__ __forceinline__ void poll_tagged2(const unsigned long long* a, const 
     }
     fa = __int_as_float((int)(unsigned)w0);
     fb = __int_as_float((int)(unsigned)w1);
+}
+
+// Polls four consecutive tagged words (p 32-byte aligned per thread) until every active lane of the wave has seen `tag`
+// on all four; a lane that has its values stops loading (its later polls are masked out), so the traffic shrinks
+// as the data arrives.  Bounded like every wait here.
+__device__ __forceinline__ void poll_tagged4(const unsigned long long* p, unsigned tag, int* err, float (&v)[4]) {
+    unsigned long long w[4] = {0, 0, 0, 0};
+    bool ok = false;
+    int it = 0;
+    for (;;) {
+        if (!ok) {
+#pragma unroll
+            for (int i = 0; i < 4; i++) w[i] = ld_u64(p + i);
+            ok = (unsigned)(w[0] >> 32) == tag && (unsigned)(w[1] >> 32) == tag && (unsigned)(w[2] >> 32) == tag &&
+                 (unsigned)(w[3] >> 32) == tag;
+        }
+        if (__builtin_amdgcn_ballot_w64(!ok) == 0) break;
+        if (spin_should_stop(++it, err)) break;
+    }
+#pragma unroll
+    for (int i = 0; i < 4; i++) v[i] = __int_as_float((int)(unsigned)w[i]);
+}
+
+// Per-workgroup "published" flags.  A flag word is written by one workgroup only (a plain coherent store, no
+// read-modify-write), and there are kFlagCopies copies of the 256-word array, 4 KiB apart: a workgroup raises its flag
+// in all of them with one store instruction and polls only copy (workgroup % kFlagCopies), with one wave, so that a
+// poll round puts 32 x 8 line requests on a copy instead of 256 x 8 on one set of lines (which serialises on the
+// memory channel that holds them, microseconds per round).
+constexpr int kFlagCopies = 8, kFlagStride = 1024;      // words between copies
+__device__ __forceinline__ void raise_flag(unsigned* flags, int wg, unsigned tag, int lane) {
+    if (lane < kFlagCopies) __hip_atomic_store(&flags[lane * kFlagStride + wg], tag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+// Wave 0 polls its copy (four flags per lane) until every flag of a workgroup w with (w % 32) < nact carries `tag`; the
+// workgroup barrier hands the result to the other waves.
+__device__ __forceinline__ void wait_flags(const unsigned* flags, int wg, unsigned tag, int nact, int* err) {
+    if (threadIdx.x < 64) {
+        const int lane = threadIdx.x;
+        const unsigned long long* p = reinterpret_cast<const unsigned long long*>(flags + (wg % kFlagCopies) * kFlagStride) + 2 * lane;
+        const int c0 = (4 * lane) % 32;                       // chunk index of this lane's first flag; the four are consecutive
+        bool ok = false;
+        int it = 0;
+        for (;;) {
+            if (!ok) {
+                const unsigned long long a = ld_u64(p), b = ld_u64(p + 1);
+                ok = ((unsigned)a == tag || c0 >= nact) && ((unsigned)(a >> 32) == tag || c0 + 1 >= nact) &&
+                     ((unsigned)b == tag || c0 + 2 >= nact) && ((unsigned)(b >> 32) == tag || c0 + 3 >= nact);
+            }
+            if (__builtin_amdgcn_ballot_w64(!ok) == 0) break;
+            if (spin_should_stop(++it, err)) break;
+            __builtin_amdgcn_s_sleep(1);
+        }
+    }
+    __syncthreads();
 }
 
 // Read-only data at a wave-uniform address (layer table, per-row weight scales): the constant address space
@@ -312,6 +369,7 @@ __global__ __launch_bounds__(kMegaT, 1) void decode_mega_kernel(MegaParams p) {
     constexpr int H = 2048, KV = 512, QH = 32, KVH = 8, GROUP = 4;
     const int pos0 = p.state[0];
     GridBarrier bar{p.bar, (unsigned)p.state[2], &p.state[3]};
+    const unsigned seq0 = (unsigned)p.state[4];
     int stamp_i = 0;
     // 'thread 0 of workgroup 0' from scalars and the hardware lane id: no per-thread value has to stay live for it
     auto is_t0 = [&]() { return wave == 0 && __builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u)) == 0; };
@@ -343,6 +401,7 @@ __global__ __launch_bounds__(kMegaT, 1) void decode_mega_kernel(MegaParams p) {
     const int a_h = wg / 32, a_c = wg % 32;
     const bool a_active = a_c * kChunk < len && a_c * kChunk < p.max_pos;
     const bool a_owner = a_active && (pos / kChunk == a_c);       // this chunk holds the new token
+    const int nchunks = (len + kChunk - 1) / kChunk;              // active chunks per head: the parts every accumulator receives
 
     for (int l = 0; l < p.n_layers; l++) {
         // An opaque per-layer copy of the thread index: without it the compiler hoists every per-thread address
@@ -352,6 +411,8 @@ __global__ __launch_bounds__(kMegaT, 1) void decode_mega_kernel(MegaParams p) {
         asm volatile("" : "+v"(t_opaque));
         const int t = t_opaque, lane = t & 63;
         const LayerW w = ldc_layer(p.layers + l);
+        // sequence number of this layer pass: unique over launches, the tag of everything this pass publishes
+        const unsigned tag = seq0 + (unsigned)(step * p.n_layers + l) + 1u;
         const float* g0 = p.gamma + (size_t)(2 * l) * H;
         const float* g1 = p.gamma + (size_t)(2 * l + 1) * H;
         const float* q_s = p.q_s + l * QH;
@@ -399,17 +460,15 @@ __global__ __launch_bounds__(kMegaT, 1) void decode_mega_kernel(MegaParams p) {
                 }
             }
             const float4 gam = reinterpret_cast<const float4*>(g0)[t];
-            if (l > 0) bar.wait();                                   // x of the previous layer is complete
-            stamp();
             float v[4];
+            if (l > 0) poll_tagged4(&p.x_tag[4 * t], tag - 1u, bar.err, v);   // x of the previous layer, as it arrives
+            stamp();
             if (l == 0) {
                 if (p.x_in) { const float4 q = reinterpret_cast<const float4*>(p.x_in)[t]; v[0] = q.x; v[1] = q.y; v[2] = q.z; v[3] = q.w; }
                 else {
 #pragma unroll
                     for (int i = 0; i < 4; i++) v[i] = __half2float(p.embed[(size_t)tok * H + 4 * t + i]);
                 }
-            } else {
-                ld_f4(&p.x[4 * t], v);
             }
             const float sx = norm_quant_2048(v, gam, true, p.eps, L, [&]() { gu_slice(0); });
             if (!is_s) {
@@ -417,7 +476,7 @@ __global__ __launch_bounds__(kMegaT, 1) void decode_mega_kernel(MegaParams p) {
                 for (int j = 0; j < 3; j++) {
                     const int r = wg * 12 + wave + 4 * j;
                     const int a = mega_dot_row<2>(wr[j], L.xq, lane);
-                    if (lane == 0) st_tagged(&p.qkv_tag[r], (float)a * sx * wsc[j], bar.epoch);
+                    if (lane == 0) st_tagged(&p.qkv_tag[r], (float)a * sx * wsc[j], tag);
                 }
             }
             stamp();
@@ -448,7 +507,7 @@ __global__ __launch_bounds__(kMegaT, 1) void decode_mega_kernel(MegaParams p) {
                 if (t < 128) {                                        // q: 4 heads x 32 pairs
                     const int g = t >> 5, k = t & 31, qh = a_h * GROUP + g;
                     float t0, t1;
-                    poll_tagged2(&p.qkv_tag[qh * kHd + k], &p.qkv_tag[qh * kHd + k + 32], bar.epoch, bar.err, t0, t1);
+                    poll_tagged2(&p.qkv_tag[qh * kHd + k], &p.qkv_tag[qh * kHd + k + 32], tag, bar.err, t0, t1);
                     const float o0 = t0 * cs[k] - t1 * sn[k], o1 = t0 * sn[k] + t1 * cs[k];
                     const float div = 8.0f * (g == 0 ? qs4[0] : g == 1 ? qs4[1] : g == 2 ? qs4[2] : qs4[3]);
                     L.q8[g][k] = (int8_t)static_q8(o0, div);
@@ -456,7 +515,7 @@ __global__ __launch_bounds__(kMegaT, 1) void decode_mega_kernel(MegaParams p) {
                 } else if (t < 160) {                                 // k of the new token: 32 pairs
                     const int k = t - 128;
                     float t0, t1;
-                    poll_tagged2(&p.qkv_tag[H + a_h * kHd + k], &p.qkv_tag[H + a_h * kHd + k + 32], bar.epoch, bar.err, t0, t1);
+                    poll_tagged2(&p.qkv_tag[H + a_h * kHd + k], &p.qkv_tag[H + a_h * kHd + k + 32], tag, bar.err, t0, t1);
                     const float o0 = t0 * cs[k] - t1 * sn[k], o1 = t0 * sn[k] + t1 * cs[k];
                     const float div = 1.0f * ks1;
                     const int8_t b0 = (int8_t)static_q8(o0, div), b1 = (int8_t)static_q8(o1, div);
@@ -465,7 +524,7 @@ __global__ __launch_bounds__(kMegaT, 1) void decode_mega_kernel(MegaParams p) {
                 } else if (t < 224) {                                 // v of the new token
                     const int d = t - 160;
                     float tv, tv_again;
-                    poll_tagged2(&p.qkv_tag[H + KV + a_h * kHd + d], &p.qkv_tag[H + KV + a_h * kHd + d], bar.epoch, bar.err, tv, tv_again);
+                    poll_tagged2(&p.qkv_tag[H + KV + a_h * kHd + d], &p.qkv_tag[H + KV + a_h * kHd + d], tag, bar.err, tv, tv_again);
                     const int8_t b = (int8_t)static_q8(tv, 1.0f * vs1);
                     L.vnew[d] = b;
                     if (a_owner) vc[v_index(a_h, pos, d, p.max_pos)] = b;
@@ -492,8 +551,8 @@ __global__ __launch_bounds__(kMegaT, 1) void decode_mega_kernel(MegaParams p) {
                     sum = wave_sum(sum);
                     if (lane == 0) {
                         unsigned long long* slot = p.stats_tag + (size_t)((a_h * GROUP + wave) * 32 + a_c) * 2;
-                        st_tagged(slot, m, bar.epoch);
-                        st_tagged(slot + 1, sum, bar.epoch);
+                        st_tagged(slot, m, tag);
+                        st_tagged(slot + 1, sum, tag);
                     }
                 }
             } else {
@@ -506,7 +565,6 @@ __global__ __launch_bounds__(kMegaT, 1) void decode_mega_kernel(MegaParams p) {
             // a KV head poll those words directly instead of going through a grid barrier and a load after it; the
             // slot is next written a layer later, three grid barriers after every reader has finished with it.
             if (a_active) {
-                const int nchunks = (len + kChunk - 1) / kChunk;
                 if (wave < GROUP) {
                     float m_c = -1e32f, l_c = 0.0f;
                     {
@@ -516,7 +574,7 @@ __global__ __launch_bounds__(kMegaT, 1) void decode_mega_kernel(MegaParams p) {
                         for (;;) {
                             w0 = ld_u64(slot);
                             w1 = ld_u64(slot + 1);
-                            const bool ok = (unsigned)(w0 >> 32) == bar.epoch && (unsigned)(w1 >> 32) == bar.epoch;
+                            const bool ok = (unsigned)(w0 >> 32) == tag && (unsigned)(w1 >> 32) == tag;
                             if (__builtin_amdgcn_ballot_w64(!ok) == 0) break;
                             if (spin_should_stop(++it, bar.err)) break;
                         }
@@ -586,10 +644,10 @@ __global__ __launch_bounds__(kMegaT, 1) void decode_mega_kernel(MegaParams p) {
                 }
             }
             const float osa = a_s[t >> 4], osv = v_s[t >> 6];         // elements 4t..4t+3 lie in query head t/16
-            bar.wait();
-            stamp();
             // the stream waves' previous slice has landed long ago, so they can share the activation loads
             float v[4], xr[2] = {0.0f, 0.0f};
+            bar.wait();
+            stamp();
 #pragma unroll
             for (int i = 0; i < 2; i++) {
                 const unsigned long long w2 = ld_u64(reinterpret_cast<const unsigned long long*>(p.o_acc + 4 * t + 2 * i));
@@ -601,7 +659,8 @@ __global__ __launch_bounds__(kMegaT, 1) void decode_mega_kernel(MegaParams p) {
                 for (int j = 0; j < 2; j++) {
                     const int row = wg * 8 + wave + 4 * j;
                     if (l == 0) xr[j] = p.x_in ? p.x_in[row] : __half2float(p.embed[(size_t)tok * H + row]);
-                    else xr[j] = ld_f(&p.x[row]);
+                    else xr[j] = L.res8[wave + 4 * j];              // this workgroup's own rows of x, left there by phase 6
+
                 }
             }
             const float4 z4 = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
@@ -616,9 +675,9 @@ __global__ __launch_bounds__(kMegaT, 1) void decode_mega_kernel(MegaParams p) {
             // the workgroup's eight outputs leave as one 32-byte store: eight single-lane stores from four waves into
             // the same sector take longer to be acknowledged, and the barrier waits for that
             __syncthreads();
-            if (t < 8) st_f(&p.x2[wg * 8 + t], L.res8[t]);
+            if (t < 8) st_tagged(&p.x2_tag[wg * 8 + t], L.res8[t], tag);
             stamp();
-            bar.arrive(!is_s);
+            // no grid barrier: the consumers poll the tagged words
         }
 
         // ================= phase 5: RMSNorm + quant -> gate/up rows (64 per workgroup, 16 per stream wave) + SiLU*up =================
@@ -630,11 +689,12 @@ __global__ __launch_bounds__(kMegaT, 1) void decode_mega_kernel(MegaParams p) {
             const int ow = wave & 3, half = is_s ? 0 : 8;
             const float gsc = w.sgu[wg * 64 + ow * 16 + half + ridx]; // read before this phase's prefetch is issued
             const float4 gam = reinterpret_cast<const float4*>(g1)[t];
-            bar.wait();
-            stamp();
-            if (t < 8) st_i(&p.o_acc[wg * 8 + t], 0);                // every reader of o_acc has passed the barrier
             float v[4];
-            ld_f4(&p.x2[4 * t], v);
+            poll_tagged4(&p.x2_tag[4 * t], tag, bar.err, v);
+            stamp();
+            // every workgroup has published x2, so it has read the accumulators; the next parts are added a layer later,
+            // by workgroups that have polled this workgroup's x, which wave 0 stores after this store has been acknowledged
+            if (t < 8) st_i(&p.o_acc[wg * 8 + t], 0);
             const float sx = norm_quant_2048(v, gam, true, p.eps, L, [&]() {
                 __builtin_amdgcn_s_waitcnt(0x0F70);                   // vmcnt(0): see gu_slice
                 if (is_s) mega_row_to_lds(w.wd, wg * 8 + sw * 2, lane, L.wd[sw * 2]);
@@ -712,7 +772,7 @@ __global__ __launch_bounds__(kMegaT, 1) void decode_mega_kernel(MegaParams p) {
             float xres = 0.0f;
             bar.wait();
             stamp();
-            if (lane == 0) xres = ld_f(&p.x2[drow]);
+            if (lane == 0) xres = L.res8[drow - wg * 8];              // this workgroup's own rows of x2, left there by phase 4
             // 8192-point transform on all 512 threads, stage order bits 1,2,...,12,0 (bit-exact order, see
             // fht_kernels.h).  Every remaining stage is a butterfly between registers of one thread, with two passes
             // through LDS between the three layouts:
@@ -815,11 +875,14 @@ __global__ __launch_bounds__(kMegaT, 1) void decode_mega_kernel(MegaParams p) {
                 if (lane == 0) L.res8[drow - wg * 8] = (float)a0 * sx * dsc + xres;
             }
             __syncthreads();
-            if (t < 8) st_f(&p.x[wg * 8 + t], L.res8[t]);            // one 32-byte store, as in phase 4
+            if (t < 8) {
+                __builtin_amdgcn_s_waitcnt(0x0F70);                  // vmcnt(0): the accumulator reset of phase 5 has landed
+                st_tagged(&p.x_tag[wg * 8 + t], L.res8[t], tag);     // one 64-byte store, as in phase 4
+                if (l == p.n_layers - 1) st_f(&p.x[wg * 8 + t], L.res8[t]);   // the hidden state the host reads back
+            }
             if (l == 1) fine();
             if (l == 1) fine();
             stamp();
-            bar.arrive();
         }
     }
 
@@ -844,10 +907,9 @@ __global__ __launch_bounds__(kMegaT, 1) void decode_mega_kernel(MegaParams p) {
         };
         int r = row_begin + wave;
         load_group(r);
-        bar.wait();
-        stamp();
         float v[4];
-        ld_f4(&p.x[4 * t], v);
+        poll_tagged4(&p.x_tag[4 * t], seq0 + (unsigned)((step + 1) * p.n_layers), bar.err, v);
+        stamp();
         float ss = (v[0] * v[0] + v[1] * v[1]) + (v[2] * v[2] + v[3] * v[3]);
         ss = block_sum<kMegaWaves>(ss, L.red);
         const float rms = 1.0f / sqrtf(ss / 2048.0f + p.eps);
@@ -952,13 +1014,12 @@ __global__ __launch_bounds__(kMegaT, 1) void decode_mega_kernel(MegaParams p) {
             if (wg == 0 && t == 0) p.tokens_out[p.state[1] + step] = tok;
             __syncthreads();                                        // L.bestv/besti are reused by the next step
         }
-    } else {
-        bar.wait();   // keep arrive/wait balanced: the last layer's x is complete when the kernel ends
     }
     steps_done = step + 1;
     }   // step loop (left early only after a barrier time-out, which the error flag reports)
     if (wg == 0 && is_t0()) {
         p.state[2] = (int)bar.epoch;
+        p.state[4] = (int)(seq0 + (unsigned)(steps_done * p.n_layers));
         if (greedy) { p.token[0] = tok; p.state[0] = pos0 + steps_done; p.state[1] += steps_done; }
     }
 #ifdef FX_MEGA_FINE_STAMPS

@@ -30,7 +30,10 @@ struct flexllm_llama {
     float* scores = nullptr;
     float2* stats = nullptr;
     unsigned long long* qkv_tag = nullptr;     // persistent kernel: q/k/v outputs tagged with the barrier epoch
-    unsigned long long* stats_tag = nullptr;   // persistent kernel: chunk statistics tagged with the barrier epoch
+    unsigned long long* stats_tag = nullptr;   // persistent kernel: chunk statistics tagged with the layer sequence number
+    unsigned *h_flag = nullptr, *o_flag = nullptr;   // persistent kernel: per-workgroup "my part of h is published / my attention parts are added" flags
+    int32_t* o_mega = nullptr;                 // persistent kernel: its own attention accumulators (zero whenever it is not running)
+    unsigned long long *x_tag = nullptr, *x2_tag = nullptr;   // persistent kernel: the residual stream after a layer / after attention, tagged likewise
     int32_t* o_acc = nullptr;
     int* state = nullptr;           // [0] position of the token being processed, [1] step index
     float* am_v = nullptr;
@@ -180,7 +183,7 @@ static int launch_mega(flexllm_llama* m, int* token, const float* x_in, float* l
     p.embed = reinterpret_cast<const __half*>(m->embed);
     p.k_cache = m->k_cache; p.v_cache = m->v_cache; p.cache_layer_bytes = m->cache_layer_bytes;
     p.x = m->x; p.x2 = m->x2; p.qkv = m->qkv; p.h = m->h; p.logits = logits ? logits : m->logits;
-    p.stats = m->stats; p.stats_tag = m->stats_tag; p.qkv_tag = m->qkv_tag; p.o_acc = m->o_acc; p.state = m->state; p.bar = m->bar;
+    p.stats = m->stats; p.stats_tag = m->stats_tag; p.qkv_tag = m->qkv_tag; p.x_tag = m->x_tag; p.x2_tag = m->x2_tag; p.o_acc = m->o_mega; p.h_flag = m->h_flag; p.o_flag = m->o_flag; p.state = m->state; p.bar = m->bar;
     p.token = token; p.tokens_out = tokens_out; p.n_steps = steps; p.x_in = x_in; p.am_v = m->am_v; p.am_i = m->am_i;
     p.n_layers = c.layers; p.max_pos = c.max_pos; p.vocab = c.vocab; p.want_head = want_head;
     p.top_k = top_k; p.rands = rands; p.cand_v = m->topk_val; p.cand_i = m->topk_idx;
@@ -312,7 +315,17 @@ int flexllm_llama_create(flexllm_llama** out, const flexllm_llama_config* cfg, c
     FX_TRY_HIP(hipMemset(m->qkv_tag, 0xFF, sizeof(unsigned long long) * (size_t)(H + 2 * KV)));   // tag 0xFFFFFFFF: never a live epoch (the first is 0)
     FX_TRY(dev_alloc(m, (void**)&m->stats_tag, sizeof(unsigned long long) * 2 * (size_t)c.q_heads * kMaxChunks));
     FX_TRY_HIP(hipMemset(m->stats_tag, 0xFF, sizeof(unsigned long long) * 2 * (size_t)c.q_heads * kMaxChunks));
-    FX_TRY(dev_alloc(m, (void**)&m->state, sizeof(int) * 4));
+    FX_TRY(dev_alloc(m, (void**)&m->x_tag, sizeof(unsigned long long) * (size_t)H));
+    FX_TRY_HIP(hipMemset(m->x_tag, 0xFF, sizeof(unsigned long long) * (size_t)H));
+    FX_TRY(dev_alloc(m, (void**)&m->x2_tag, sizeof(unsigned long long) * (size_t)H));
+    FX_TRY_HIP(hipMemset(m->x2_tag, 0xFF, sizeof(unsigned long long) * (size_t)H));
+    FX_TRY(dev_alloc(m, (void**)&m->h_flag, sizeof(unsigned) * kFlagCopies * kFlagStride));
+    FX_TRY_HIP(hipMemset(m->h_flag, 0xFF, sizeof(unsigned) * kFlagCopies * kFlagStride));
+    FX_TRY(dev_alloc(m, (void**)&m->o_flag, sizeof(unsigned) * kFlagCopies * kFlagStride));
+    FX_TRY_HIP(hipMemset(m->o_flag, 0xFF, sizeof(unsigned) * kFlagCopies * kFlagStride));
+    FX_TRY(dev_alloc(m, (void**)&m->o_mega, sizeof(int32_t) * (size_t)H));
+    FX_TRY_HIP(hipMemset(m->o_mega, 0, sizeof(int32_t) * (size_t)H));
+    FX_TRY(dev_alloc(m, (void**)&m->state, sizeof(int) * 8));
     FX_TRY(dev_alloc(m, (void**)&m->am_v, sizeof(float) * kArgmaxParts));
     // per-workgroup sampling candidates: of the persistent kernel's workgroups or of the stand-alone first stage
     constexpr int kCandGroups = kMegaWG > kTopKParts ? kMegaWG : kTopKParts;
@@ -323,7 +336,7 @@ int flexllm_llama_create(flexllm_llama** out, const flexllm_llama_config* cfg, c
     FX_TRY_HIP(hipMemcpy(m->layers_dev, m->layers.data(), sizeof(LayerW) * L, hipMemcpyHostToDevice));
     FX_TRY(dev_alloc(m, (void**)&m->bar, sizeof(unsigned) * 64 * (2 + kMegaWG / kMegaGroup)));
     FX_TRY_HIP(hipMemset(m->bar, 0, sizeof(unsigned) * 64 * (2 + kMegaWG / kMegaGroup)));
-    FX_TRY_HIP(hipMemset(m->state, 0, sizeof(int) * 4));
+    FX_TRY_HIP(hipMemset(m->state, 0, sizeof(int) * 8));
     FX_TRY_HIP(hipMemset(m->o_acc, 0, sizeof(int32_t) * H));
     FX_TRY_HIP(hipMemset(m->am_v, 0, sizeof(float) * kArgmaxParts));
     FX_TRY_HIP(hipMemset(m->am_i, 0, sizeof(int) * kArgmaxParts));
@@ -358,10 +371,8 @@ int flexllm_llama_set_decode_mode(flexllm_llama* m, int mode) {
     FX_REQUIRE(m && (mode == 0 || mode == 1), "llama_set_decode_mode: mode=%d (0 persistent kernel, 1 one kernel per stage)", mode);
     if (m->decode_mode != mode) {
         if (m->graph_exec) { (void)hipGraphExecDestroy(m->graph_exec); m->graph_exec = nullptr; }
-        // The persistent kernel only ever adds into the attention accumulators and clears them once they have been read,
-        // so it expects zeros at launch; the per-stage kernels clear them before use and leave the last layer's sums.
-        FX_HIP(hipDeviceSynchronize());
-        FX_HIP(hipMemset(m->o_acc, 0, sizeof(int32_t) * m->cfg.hidden));
+        // (the two schedules keep their attention accumulators apart: the persistent kernel's are back at zero
+        // whenever it ends, the per-stage kernels clear theirs before use)
     }
     m->decode_mode = mode;
     return FLEXLLM_OK;
@@ -394,7 +405,11 @@ int flexllm_llama_check(flexllm_llama* m) {
             set_error("decode: a token id outside the vocabulary (%d entries) was fed in; token 0 was used instead", m->cfg.vocab);
             return FLEXLLM_EINVAL;
         }
-        set_error("persistent decode kernel: a grid barrier timed out (were all %d workgroups resident?)", kMegaWG);
+        // after a time-out the barrier counters and the attention accumulators hold partial counts: start them afresh
+        (void)hipMemset(m->bar, 0, sizeof(unsigned) * 64 * (2 + kMegaWG / kMegaGroup));
+        (void)hipMemset(&m->state[2], 0, sizeof(int));
+        (void)hipMemset(m->o_mega, 0, sizeof(int32_t) * (size_t)m->cfg.hidden);
+        set_error("persistent decode kernel: a wait timed out (were all %d workgroups resident?)", kMegaWG);
         return FLEXLLM_EHIP;
     }
     return FLEXLLM_OK;
