@@ -57,14 +57,18 @@ struct MegaParams {
     const __half* embed;
     int8_t *k_cache, *v_cache;
     size_t cache_layer_bytes;
-    float *x, *x2, *qkv, *h, *logits;
+    float *x, *x2, *qkv, *logits;
+    // SiLU(gate)*up after the workgroup-local Hadamard stages: [kMegaMaxSteps * layers][8192], one slice per layer pass
+    // of a launch.  Every workgroup reads all of it, and with coherent (L2-bypassing) loads the 32 CUs of an XCD would
+    // each pull the 32 KiB through the XCD's fabric port.  Because no address is written twice within a launch, and L2
+    // holds nothing from before the launch, an ordinary load can never see a stale line: the first CU of an XCD to
+    // touch a line (after the barrier that follows its write-through store) fetches it, the others hit in L2.
+    float* h;
     float2* stats;                 // [q_heads][32] (one-kernel-per-stage path)
     unsigned long long* qkv_tag;   // [H + 2*KV]: q/k/v projection outputs, each with the epoch in its high word
     unsigned long long* stats_tag; // [q_heads][32][2]: chunk max and chunk sum of exponentials, each with the epoch in its high word
     unsigned long long* x_tag;     // [H]: the residual stream after a layer (down projection + residual), tagged with the layer's sequence number
     unsigned long long* x2_tag;    // [H]: the residual stream after attention (o projection + residual), tagged likewise
-    unsigned* h_flag;              // [kFlagCopies][kFlagStride]: sequence number of the layer pass whose 32 values of h workgroup w has published
-    unsigned* o_flag;              // same shape: ... whose attention parts workgroup w has added to o_acc
     int32_t* o_acc;                // [H]: attention accumulators (zero at launch, cleared again once read)
     int* state;                    // [0] pos, [1] step, [2] barrier epoch base, [3] error flag, [4] layer sequence number base
     unsigned* bar;                 // [0] flag, [64] top counter, [128+64g] group counters
@@ -81,6 +85,7 @@ struct MegaParams {
     int* cand_i;
     int n_layers, max_pos, vocab, want_head;
     float eps, fht_scale;
+    int timeline_wg;               // the workgroup whose stamps the timeline holds
     long long* timeline;           // optional [n_layers*6+2][2] wall-clock stamps of workgroup 0 (after wait, before arrive)
 };
 
@@ -148,38 +153,6 @@ __device__ __forceinline__ void poll_tagged4(const unsigned long long* p, unsign
     }
 #pragma unroll
     for (int i = 0; i < 4; i++) v[i] = __int_as_float((int)(unsigned)w[i]);
-}
-
-// Per-workgroup "published" flags.  A flag word is written by one workgroup only (a plain coherent store, no
-// read-modify-write), and there are kFlagCopies copies of the 256-word array, 4 KiB apart: a workgroup raises its flag
-// in all of them with one store instruction and polls only copy (workgroup % kFlagCopies), with one wave, so that a
-// poll round puts 32 x 8 line requests on a copy instead of 256 x 8 on one set of lines (which serialises on the
-// memory channel that holds them, microseconds per round).
-constexpr int kFlagCopies = 8, kFlagStride = 1024;      // words between copies
-__device__ __forceinline__ void raise_flag(unsigned* flags, int wg, unsigned tag, int lane) {
-    if (lane < kFlagCopies) __hip_atomic_store(&flags[lane * kFlagStride + wg], tag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-}
-// Wave 0 polls its copy (four flags per lane) until every flag of a workgroup w with (w % 32) < nact carries `tag`; the
-// workgroup barrier hands the result to the other waves.
-__device__ __forceinline__ void wait_flags(const unsigned* flags, int wg, unsigned tag, int nact, int* err) {
-    if (threadIdx.x < 64) {
-        const int lane = threadIdx.x;
-        const unsigned long long* p = reinterpret_cast<const unsigned long long*>(flags + (wg % kFlagCopies) * kFlagStride) + 2 * lane;
-        const int c0 = (4 * lane) % 32;                       // chunk index of this lane's first flag; the four are consecutive
-        bool ok = false;
-        int it = 0;
-        for (;;) {
-            if (!ok) {
-                const unsigned long long a = ld_u64(p), b = ld_u64(p + 1);
-                ok = ((unsigned)a == tag || c0 >= nact) && ((unsigned)(a >> 32) == tag || c0 + 1 >= nact) &&
-                     ((unsigned)b == tag || c0 + 2 >= nact) && ((unsigned)(b >> 32) == tag || c0 + 3 >= nact);
-            }
-            if (__builtin_amdgcn_ballot_w64(!ok) == 0) break;
-            if (spin_should_stop(++it, err)) break;
-            __builtin_amdgcn_s_sleep(1);
-        }
-    }
-    __syncthreads();
 }
 
 // Read-only data at a wave-uniform address (layer table, per-row weight scales): the constant address space
@@ -373,7 +346,7 @@ __global__ __launch_bounds__(kMegaT, 1) void decode_mega_kernel(MegaParams p) {
     int stamp_i = 0;
     // 'thread 0 of workgroup 0' from scalars and the hardware lane id: no per-thread value has to stay live for it
     auto is_t0 = [&]() { return wave == 0 && __builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u)) == 0; };
-    auto stamp = [&]() { if (p.timeline && wg == 0 && is_t0()) p.timeline[stamp_i] = wall_clock64(); stamp_i++; };
+    auto stamp = [&]() { if (p.timeline && wg == p.timeline_wg && is_t0()) p.timeline[stamp_i] = wall_clock64(); stamp_i++; };
 #ifdef FX_MEGA_FINE_STAMPS
     int fine_i = 0;
     auto fine = [&]() { if (p.timeline && wg == 0 && is_t0() && fine_i < 64) p.timeline[p.n_layers * 12 + 2 + fine_i] = wall_clock64(); fine_i++; };
@@ -421,6 +394,8 @@ __global__ __launch_bounds__(kMegaT, 1) void decode_mega_kernel(MegaParams p) {
         const float* a_s = p.a_s + l * QH;
         int8_t* kc = p.k_cache + (size_t)l * p.cache_layer_bytes;
         int8_t* vc = p.v_cache + (size_t)l * p.cache_layer_bytes;
+        // h of this layer pass lives at an address that no other pass of this launch uses (see MegaParams::h)
+        float* hbuf = p.h + (size_t)(step * p.n_layers + l) * 8192;
 
         // Stream waves: 16 gate/up rows (interleaved gate, up) and 2 down rows each, fetched in six slices of
         // 8 KiB per wave, one per phase, each issued once the phase's activation loads have landed.  A slice
@@ -756,7 +731,7 @@ __global__ __launch_bounds__(kMegaT, 1) void decode_mega_kernel(MegaParams p) {
                 hv = lane_butterfly_s<4>(hv, lane_sign<4>(t));
                 hv = lane_butterfly_s<8>(hv, lane_sign<8>(t));
                 hv = lane_butterfly_s<16>(hv, lane_sign<16>(t));
-                if (t < 32) st_f(&p.h[wg * 32 + t], hv);             // stored by a wave with no prefetch in flight
+                if (t < 32) st_f(&hbuf[wg * 32 + t], hv);             // stored by a wave with no prefetch in flight
             }
             if (l == 1) fine();
             stamp();
@@ -783,8 +758,7 @@ __global__ __launch_bounds__(kMegaT, 1) void decode_mega_kernel(MegaParams p) {
             const int abase = (t >> 3) * 128 + (t & 7) * 4;
 #pragma unroll
             for (int j = 0; j < 4; j++) {
-                const float2 lo = ld_f2(p.h + abase + j * 32), hi = ld_f2(p.h + abase + j * 32 + 2);
-                a[j] = make_float4(lo.x, lo.y, hi.x, hi.y);
+                a[j] = *reinterpret_cast<const float4*>(hbuf + abase + j * 32);   // ordinary loads: they may hit in L2
             }
             __builtin_amdgcn_s_waitcnt(0x0F70);               // vmcnt(0): the h loads are complete
             if (is_s) mega_row_to_lds(w.wd, wg * 8 + sw * 2 + 1, lane, L.wd[sw * 2 + 1]);

@@ -31,7 +31,6 @@ struct flexllm_llama {
     float2* stats = nullptr;
     unsigned long long* qkv_tag = nullptr;     // persistent kernel: q/k/v outputs tagged with the barrier epoch
     unsigned long long* stats_tag = nullptr;   // persistent kernel: chunk statistics tagged with the layer sequence number
-    unsigned *h_flag = nullptr, *o_flag = nullptr;   // persistent kernel: per-workgroup "my part of h is published / my attention parts are added" flags
     int32_t* o_mega = nullptr;                 // persistent kernel: its own attention accumulators (zero whenever it is not running)
     unsigned long long *x_tag = nullptr, *x2_tag = nullptr;   // persistent kernel: the residual stream after a layer / after attention, tagged likewise
     int32_t* o_acc = nullptr;
@@ -183,12 +182,17 @@ static int launch_mega(flexllm_llama* m, int* token, const float* x_in, float* l
     p.embed = reinterpret_cast<const __half*>(m->embed);
     p.k_cache = m->k_cache; p.v_cache = m->v_cache; p.cache_layer_bytes = m->cache_layer_bytes;
     p.x = m->x; p.x2 = m->x2; p.qkv = m->qkv; p.h = m->h; p.logits = logits ? logits : m->logits;
-    p.stats = m->stats; p.stats_tag = m->stats_tag; p.qkv_tag = m->qkv_tag; p.x_tag = m->x_tag; p.x2_tag = m->x2_tag; p.o_acc = m->o_mega; p.h_flag = m->h_flag; p.o_flag = m->o_flag; p.state = m->state; p.bar = m->bar;
+    p.stats = m->stats; p.stats_tag = m->stats_tag; p.qkv_tag = m->qkv_tag; p.x_tag = m->x_tag; p.x2_tag = m->x2_tag; p.o_acc = m->o_mega; p.state = m->state; p.bar = m->bar;
     p.token = token; p.tokens_out = tokens_out; p.n_steps = steps; p.x_in = x_in; p.am_v = m->am_v; p.am_i = m->am_i;
     p.n_layers = c.layers; p.max_pos = c.max_pos; p.vocab = c.vocab; p.want_head = want_head;
     p.top_k = top_k; p.rands = rands; p.cand_v = m->topk_val; p.cand_i = m->topk_idx;
     p.eps = c.eps; p.fht_scale = c.fht_scale;
     p.timeline = m->timeline;
+    {   // debug aid: which workgroup's stamps to record (default 0)
+        const char* e = getenv("FLEXLLM_TIMELINE_WG");
+        const int w = e ? atoi(e) : 0;
+        p.timeline_wg = w >= 0 && w < kMegaWG ? w : 0;
+    }
     static bool lds_opted_in = false;     // the kernel's LDS block exceeds the default 64 KiB per workgroup
     if (!lds_opted_in) {
         FX_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(decode_mega_kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -303,7 +307,7 @@ int flexllm_llama_create(flexllm_llama** out, const flexllm_llama_config* cfg, c
     FX_TRY(dev_alloc(m, (void**)&m->x2, sizeof(float) * H));
     FX_TRY(dev_alloc(m, (void**)&m->nrm, sizeof(float) * H));
     FX_TRY(dev_alloc(m, (void**)&m->qkv, sizeof(float) * (H + 2 * KV)));
-    FX_TRY(dev_alloc(m, (void**)&m->h, sizeof(float) * I));
+    FX_TRY(dev_alloc(m, (void**)&m->h, sizeof(float) * I * (size_t)kMegaMaxSteps * L));   // one slice per layer pass of a launch
     FX_TRY(dev_alloc(m, (void**)&m->logits, sizeof(float) * c.vocab));
     FX_TRY(dev_alloc(m, (void**)&m->xq, (size_t)I));
     FX_TRY(dev_alloc(m, (void**)&m->q8, (size_t)H));
@@ -319,10 +323,6 @@ int flexllm_llama_create(flexllm_llama** out, const flexllm_llama_config* cfg, c
     FX_TRY_HIP(hipMemset(m->x_tag, 0xFF, sizeof(unsigned long long) * (size_t)H));
     FX_TRY(dev_alloc(m, (void**)&m->x2_tag, sizeof(unsigned long long) * (size_t)H));
     FX_TRY_HIP(hipMemset(m->x2_tag, 0xFF, sizeof(unsigned long long) * (size_t)H));
-    FX_TRY(dev_alloc(m, (void**)&m->h_flag, sizeof(unsigned) * kFlagCopies * kFlagStride));
-    FX_TRY_HIP(hipMemset(m->h_flag, 0xFF, sizeof(unsigned) * kFlagCopies * kFlagStride));
-    FX_TRY(dev_alloc(m, (void**)&m->o_flag, sizeof(unsigned) * kFlagCopies * kFlagStride));
-    FX_TRY_HIP(hipMemset(m->o_flag, 0xFF, sizeof(unsigned) * kFlagCopies * kFlagStride));
     FX_TRY(dev_alloc(m, (void**)&m->o_mega, sizeof(int32_t) * (size_t)H));
     FX_TRY_HIP(hipMemset(m->o_mega, 0, sizeof(int32_t) * (size_t)H));
     FX_TRY(dev_alloc(m, (void**)&m->state, sizeof(int) * 8));
