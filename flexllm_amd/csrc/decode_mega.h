@@ -346,7 +346,19 @@ __global__ __launch_bounds__(kMegaT, 1) void decode_mega_kernel(MegaParams p) {
     int stamp_i = 0;
     // 'thread 0 of workgroup 0' from scalars and the hardware lane id: no per-thread value has to stay live for it
     auto is_t0 = [&]() { return wave == 0 && __builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u)) == 0; };
+#ifdef FX_MEGA_ALL_STAMPS
+    // debug build: every workgroup records the 12 stamps of one layer (the eighth) behind the other timeline entries
+    int cur_layer = 0;
+    auto stamp = [&]() {
+        if (p.timeline && is_t0()) {
+            if (wg == p.timeline_wg) p.timeline[stamp_i] = wall_clock64();
+            if (cur_layer == 8) p.timeline[p.n_layers * 12 + 2 + 64 + 2 * kMegaWG + wg * 12 + stamp_i % 12] = wall_clock64();
+        }
+        stamp_i++;
+    };
+#else
     auto stamp = [&]() { if (p.timeline && wg == p.timeline_wg && is_t0()) p.timeline[stamp_i] = wall_clock64(); stamp_i++; };
+#endif
 #ifdef FX_MEGA_FINE_STAMPS
     int fine_i = 0;
     auto fine = [&]() { if (p.timeline && wg == 0 && is_t0() && fine_i < 64) p.timeline[p.n_layers * 12 + 2 + fine_i] = wall_clock64(); fine_i++; };
@@ -383,6 +395,9 @@ __global__ __launch_bounds__(kMegaT, 1) void decode_mega_kernel(MegaParams p) {
         int t_opaque = threadIdx.x;
         asm volatile("" : "+v"(t_opaque));
         const int t = t_opaque, lane = t & 63;
+#ifdef FX_MEGA_ALL_STAMPS
+        cur_layer = l;
+#endif
         const LayerW w = ldc_layer(p.layers + l);
         // sequence number of this layer pass: unique over launches, the tag of everything this pass publishes
         const unsigned tag = seq0 + (unsigned)(step * p.n_layers + l) + 1u;
@@ -460,6 +475,8 @@ __global__ __launch_bounds__(kMegaT, 1) void decode_mega_kernel(MegaParams p) {
 
         // ================= phase 2: RoPE/quant/append, scores of this chunk, chunk statistics =================
         {
+            // (Requesting these cache rows any earlier does not pay: ahead of the poll for x they hold that poll's
+            // answers up, which return in issue order, and from phase 6 of the layer before they slow that phase.)
             i32x4 kreg = {0, 0, 0, 0};
             const int key = t >> 2, part = t & 3;
             const int kpos = a_c * kChunk + key;

@@ -380,7 +380,8 @@ int flexllm_llama_set_decode_mode(flexllm_llama* m, int mode) {
 
 int flexllm_llama_stage_timeline(flexllm_llama* m, long long* host_out, int max_entries) {
     FX_REQUIRE(m && host_out && max_entries > 0, "llama_stage_timeline: bad arguments");
-    const int n = m->cfg.layers * 12 + 2 + 64 + 2 * fx::kMegaWG;    // stage stamps, fine stamps, per-workgroup entry and exit
+    // stage stamps, fine stamps, per-workgroup entry and exit, one layer's stamps of every workgroup (debug builds)
+    const int n = m->cfg.layers * 12 + 2 + 64 + 2 * fx::kMegaWG + 12 * fx::kMegaWG;
     if (!m->timeline) {
         int rc = dev_alloc(m, (void**)&m->timeline, sizeof(long long) * n);
         if (rc) return rc;
