@@ -105,41 +105,52 @@ __device__ __forceinline__ float exp_f(float x) {
 // reference's value.  Every kernel that applies SiLU calls this one function, so they agree bit for bit.
 __device__ __forceinline__ float silu_f(float v) { return v * __builtin_amdgcn_rcpf(1.0f + exp_f(-v)); }
 
+// Wave-wide reductions; every lane gets the result.  Inside a row of 16 lanes: the xor butterfly on DPP moves.  Across
+// the four rows: two DPP row broadcasts (lane 15 of rows 0 and 2 into rows 1 and 3, then lane 31 into rows 2 and 3)
+// leave the total in lane 63, which a readlane hands to all lanes as a scalar.  The operands of each addition are the
+// ones the full butterfly (xor 16, xor 32) pairs in lane 63, so sums keep their bits; the row broadcasts are ordinary
+// VALU moves, where the swizzle and the bpermute of the butterfly each take a trip through the LDS pipe.
+__device__ __forceinline__ int row_bcast15_i(int v, int keep) { return __builtin_amdgcn_update_dpp(keep, v, 0x142, 0xA, 0xF, false); }
+__device__ __forceinline__ int row_bcast31_i(int v, int keep) { return __builtin_amdgcn_update_dpp(keep, v, 0x143, 0xC, 0xF, false); }
+__device__ __forceinline__ float row_bcast15_f(float v, float keep) { return __int_as_float(row_bcast15_i(__float_as_int(v), __float_as_int(keep))); }
+__device__ __forceinline__ float row_bcast31_f(float v, float keep) { return __int_as_float(row_bcast31_i(__float_as_int(v), __float_as_int(keep))); }
+__device__ __forceinline__ float lane63_f(float v) { return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 63)); }
+
 __device__ __forceinline__ float wave_max(float v) {
     v = fmaxf(v, lane_xor_f<1>(v));
     v = fmaxf(v, lane_xor_f<2>(v));
     v = fmaxf(v, lane_xor_f<4>(v));
     v = fmaxf(v, lane_xor_f<8>(v));
-    v = fmaxf(v, lane_xor_f<16>(v));
-    v = fmaxf(v, lane_xor_f<32>(v));
-    return v;
+    v = fmaxf(v, row_bcast15_f(v, v));               // rows the broadcast does not write keep their own value
+    v = fmaxf(v, row_bcast31_f(v, v));
+    return lane63_f(v);
 }
 __device__ __forceinline__ float wave_min(float v) {
     v = fminf(v, lane_xor_f<1>(v));
     v = fminf(v, lane_xor_f<2>(v));
     v = fminf(v, lane_xor_f<4>(v));
     v = fminf(v, lane_xor_f<8>(v));
-    v = fminf(v, lane_xor_f<16>(v));
-    v = fminf(v, lane_xor_f<32>(v));
-    return v;
+    v = fminf(v, row_bcast15_f(v, v));
+    v = fminf(v, row_bcast31_f(v, v));
+    return lane63_f(v);
 }
 __device__ __forceinline__ float wave_sum(float v) {
     v += lane_xor_f<1>(v);
     v += lane_xor_f<2>(v);
     v += lane_xor_f<4>(v);
     v += lane_xor_f<8>(v);
-    v += lane_xor_f<16>(v);
-    v += lane_xor_f<32>(v);
-    return v;
+    v += row_bcast15_f(v, 0.0f);                     // lane 63's row is written by both broadcasts: it never adds the 0
+    v += row_bcast31_f(v, 0.0f);
+    return lane63_f(v);
 }
 __device__ __forceinline__ int wave_sum_i(int v) {
     v += lane_xor_i<1>(v);
     v += lane_xor_i<2>(v);
     v += lane_xor_i<4>(v);
     v += lane_xor_i<8>(v);
-    v += lane_xor_i<16>(v);
-    v += lane_xor_i<32>(v);
-    return v;
+    v += row_bcast15_i(v, 0);
+    v += row_bcast31_i(v, 0);
+    return __builtin_amdgcn_readlane(v, 63);
 }
 
 // Block-wide reductions for blocks of NW waves; `red` is NW floats of LDS.  Every thread gets the result.

@@ -61,8 +61,10 @@ struct MegaParams {
     // SiLU(gate)*up after the workgroup-local Hadamard stages: [kMegaMaxSteps * layers][8192], one slice per layer pass
     // of a launch.  Every workgroup reads all of it, and with coherent (L2-bypassing) loads the 32 CUs of an XCD would
     // each pull the 32 KiB through the XCD's fabric port.  Because no address is written twice within a launch, and L2
-    // holds nothing from before the launch, an ordinary load can never see a stale line: the first CU of an XCD to
-    // touch a line (after the barrier that follows its write-through store) fetches it, the others hit in L2.
+    // holds nothing from before the launch (every workgroup starts with an acquire fence at device scope, which
+    // drops the clean lines of its XCD's L2: lines of an earlier launch do survive a kernel boundary otherwise),
+    // an ordinary load can never see a stale line: the first CU of an XCD to touch a line (after the barrier that
+    // follows its write-through store) fetches it, the others hit in L2.
     float* h;
     float2* stats;                 // [q_heads][32] (one-kernel-per-stage path)
     unsigned long long* qkv_tag;   // [H + 2*KV]: q/k/v projection outputs, each with the epoch in its high word
@@ -340,6 +342,7 @@ __global__ __launch_bounds__(kMegaT, 1) void decode_mega_kernel(MegaParams p) {
     const bool is_s = wave >= 4;                        // stream wave (see the file comment)
     const int sw = wave - 4;
     constexpr int H = 2048, KV = 512, QH = 32, KVH = 8, GROUP = 4;
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");   // see MegaParams::h
     const int pos0 = p.state[0];
     GridBarrier bar{p.bar, (unsigned)p.state[2], &p.state[3]};
     const unsigned seq0 = (unsigned)p.state[4];
