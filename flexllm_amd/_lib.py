@@ -36,6 +36,11 @@ class LlamaWeights(C.Structure):
                  "gamma", "q_s", "k_s", "v_s", "a_s", "rope_sin", "rope_cos", "embed")]
 
 
+class LlamaW4A4Weights(C.Structure):
+    _fields_ = [("base", LlamaWeights)] + [(n, C.c_void_p) for n in
+                ("sumq", "sumk", "sumv", "sumo", "sumg", "sumu", "sumd", "head_w", "head_s", "head_sum")]
+
+
 _lib = None
 
 

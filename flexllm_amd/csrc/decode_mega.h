@@ -37,6 +37,7 @@
 #pragma once
 #include "attn_decode_kernels.h"
 #include "gemv_i8.h"
+#include "linear_w4a4.h"
 #include "logits_kernels.h"
 #include "prefill.h"
 #include <hip/hip_fp16.h>
@@ -51,8 +52,18 @@ constexpr int kMegaSpinLimit = 1 << 20;   // polls of ~1 us each: a wait that ha
 constexpr int kMegaErrPeriod = 64;         // a spinning thread looks at the error flag every so many polls
 constexpr int kMegaMaxSteps = 64;  // tokens per launch in greedy mode (bounds the run time of one launch)
 
+// Layer table of the W4A4 variant: the same matrices with two 4-bit weights per byte along K (rows of K/2 bytes), and per
+// output row the sum of its dequantised weights, which the asymmetric activations' zero point multiplies.
+struct LayerW4 {
+    int8_t *wqkv, *wo, *wgu, *wd;
+    float *sqkv, *so, *sgu, *sd;
+    float *mqkv, *mo, *mgu, *md;
+};
+
 struct MegaParams {
-    const LayerW* layers;          // device array [layers]
+    const void* layers;            // device array [layers] of LayerW (W8A8) or LayerW4 (W4A4)
+    const uint8_t* head_w4;        // W4A4: int4 output head, nibble-packed [vocab][hidden/2], with per-row scale and row sum
+    const float *head_s, *head_sum;
     const float *gamma, *q_s, *k_s, *v_s, *a_s, *rope_sin, *rope_cos;
     const __half* embed;
     int8_t *k_cache, *v_cache;
@@ -161,6 +172,15 @@ __device__ __forceinline__ void poll_tagged4(const unsigned long long* p, unsign
 // makes these scalar loads, off the vector-memory queue.
 __device__ __forceinline__ float ldc_f(const float* p) { return *(const float __attribute__((address_space(4)))*)(uintptr_t)p; }
 
+__device__ __forceinline__ LayerW4 ldc_layer4(const LayerW4* p) {
+    static_assert(sizeof(LayerW4) == 12 * sizeof(unsigned long long), "LayerW4 is twelve pointers");
+    const unsigned long long __attribute__((address_space(4)))* q = (const unsigned long long __attribute__((address_space(4)))*)(uintptr_t)p;
+    LayerW4 w;
+    w.wqkv = (int8_t*)q[0]; w.wo = (int8_t*)q[1]; w.wgu = (int8_t*)q[2]; w.wd = (int8_t*)q[3];
+    w.sqkv = (float*)q[4]; w.so = (float*)q[5]; w.sgu = (float*)q[6]; w.sd = (float*)q[7];
+    w.mqkv = (float*)q[8]; w.mo = (float*)q[9]; w.mgu = (float*)q[10]; w.md = (float*)q[11];
+    return w;
+}
 __device__ __forceinline__ LayerW ldc_layer(const LayerW* p) {
     static_assert(sizeof(LayerW) == 8 * sizeof(unsigned long long), "LayerW is eight pointers");
     const unsigned long long __attribute__((address_space(4)))* q = (const unsigned long long __attribute__((address_space(4)))*)(uintptr_t)p;
@@ -210,6 +230,7 @@ struct MegaLds {
     __attribute__((aligned(16))) float f[8192];        // FHT buffer / fp32 staging (32 KiB)
     __attribute__((aligned(16))) int8_t xq[8192];      // quantised activation vector of the current GEMV
     float red[kMegaWaves];                             // two-barrier reductions of the lm_head section
+    float red_min[kMegaWaves];                         // W4A4: the minimum of the asymmetric quantiser
     float red_sum[kMegaWaves], red_max[kMegaWaves];    // one-barrier reductions (a slot is rewritten only several barriers after its last read)
     float sc[4][kChunk];                               // scores of this chunk, 4 query heads
     __attribute__((aligned(16))) int8_t q8[4][kHd];
@@ -283,6 +304,94 @@ __device__ __forceinline__ float norm_quant_2048(float (&v)[4], const float4& g,
     return sc;
 }
 
+template <class Hook>
+__device__ __forceinline__ float mega_block_min_h(float v, float* slot, Hook hook) {
+    v = wave_min(v);
+    if ((threadIdx.x & 63) == 0) slot[threadIdx.x >> 6] = v;
+    __syncthreads();
+    hook();
+    float r = slot[0];
+#pragma unroll
+    for (int i = 1; i < kMegaWaves; i++) r = fminf(r, slot[i]);
+    return r;
+}
+// N values of a thread (N = 4: consecutive elements 4t..; N = 16: four groups of four consecutive ones) quantised to
+// asymmetric uint4 with the given minimum and scale, the arithmetic of quant_asym_kernel: round((x - min) / s) & 15,
+// packed low nibble first.  Returns one 16-bit word per group of four.
+template <int N>
+__device__ __forceinline__ void quant_u4_pack(const float (&v)[N], float vmin, float sc, uint16_t (&out)[N / 4]) {
+    float d[N];
+    int n[N];
+#pragma unroll
+    for (int i = 0; i < N; i++) d[i] = v[i] - vmin;
+    quant_vector(d, sc, n);
+#pragma unroll
+    for (int g = 0; g < N / 4; g++)
+        out[g] = (uint16_t)((n[4 * g] & 15) | ((n[4 * g + 1] & 15) << 4) | ((n[4 * g + 2] & 15) << 8) | ((n[4 * g + 3] & 15) << 12));
+}
+// W4A4 counterpart of norm_quant_2048: RMSNorm (optional) + per-token asymmetric uint4 quantisation; the packed vector
+// (1024 bytes) goes to L.xq, the scale comes back in .x and the zero point (the minimum) in .y.
+template <class Hook>
+__device__ __forceinline__ float2 norm_quant_2048_u4(float (&v)[4], const float4& g, bool do_norm, float eps,
+                                                     MegaLds& L, Hook hook) {
+    const int t = threadIdx.x;
+    if (do_norm) {
+        float ss = (v[0] * v[0] + v[1] * v[1]) + (v[2] * v[2] + v[3] * v[3]);
+        ss = mega_block_sum(ss, L.red_sum, hook);
+        const float rms = 1.0f / sqrtf(ss / 2048.0f + eps);
+        v[0] = v[0] * rms * g.x; v[1] = v[1] * rms * g.y; v[2] = v[2] * rms * g.z; v[3] = v[3] * rms * g.w;
+    }
+    float vmax = fmaxf(fmaxf(v[0], v[1]), fmaxf(v[2], v[3]));
+    float vmin = fminf(fminf(v[0], v[1]), fminf(v[2], v[3]));
+    if (do_norm) vmax = mega_block_max_h(vmax, L.red_max, NoHook());
+    else vmax = mega_block_max_h(vmax, L.red_max, hook);
+    vmin = mega_block_min_h(vmin, L.red_min, NoHook());
+    float sc = (vmax - vmin) / 15.0f;
+    if (sc == 0.0f) sc = 1.0f;
+    uint16_t w16[1];
+    quant_u4_pack(v, vmin, sc, w16);
+    reinterpret_cast<uint16_t*>(L.xq)[t] = w16[0];
+    __syncthreads();
+    return make_float2(sc, vmin);
+}
+// One packed row against the packed activation vector in LDS: the unsigned activations enter the signed 4-bit dot
+// product as a - 8, and 8 x (row sum of the weights, a second dot product with ones) is added back.
+template <int NCH>
+__device__ __forceinline__ int mega_dot_row4(const i32x4 (&wr)[NCH], const int8_t* xq_lds, int lane) {
+    const i32x4 ones = {0x11111111, 0x11111111, 0x11111111, 0x11111111};
+    int acc = 0, wsum = 0;
+#pragma unroll
+    for (int i = 0; i < NCH; i++) {
+        i32x4 xs = reinterpret_cast<const i32x4*>(xq_lds)[lane + 64 * i];
+        xs.x ^= 0x88888888; xs.y ^= 0x88888888; xs.z ^= 0x88888888; xs.w ^= 0x88888888;
+        acc = dot32_i4(wr[i], xs, acc);
+        wsum = dot32_i4(wr[i], ones, wsum);
+    }
+    return wave_sum_i(acc + 8 * wsum);
+}
+// One 4096-byte packed weight row (K = 8192) from global memory straight into LDS, as mega_row_to_lds.
+__device__ __forceinline__ void mega_row4_to_lds(const int8_t* __restrict__ w, int row, int lane, int8_t* lds_row) {
+    const int8_t* base = w + (size_t)row * 4096;
+    const unsigned voff = lane * 16;
+    const unsigned dst = __builtin_amdgcn_readfirstlane((unsigned)(uintptr_t)(__attribute__((address_space(3))) void*)lds_row);
+    unsigned saved_m0;
+    asm volatile("s_mov_b32 %0, m0\n\t"
+                 "s_mov_b32 m0, %3\n\t"
+                 "s_nop 0\n\t"
+                 "global_load_lds_dwordx4 %1, %2\n\t"
+                 "global_load_lds_dwordx4 %1, %2 offset:1024\n\t"
+                 "global_load_lds_dwordx4 %1, %2 offset:2048\n\t"
+                 "global_load_lds_dwordx4 %1, %2 offset:3072\n\t"
+                 "s_mov_b32 m0, %0"
+                 : "=&s"(saved_m0) : "v"(voff), "s"(base), "s"(dst) : "memory");
+}
+__device__ __forceinline__ int mega_dot_row4_lds(const int8_t* w_lds, const int8_t* xq_lds, int lane) {
+    i32x4 wr[4];
+#pragma unroll
+    for (int i = 0; i < 4; i++) wr[i] = reinterpret_cast<const i32x4*>(w_lds)[lane + 64 * i];
+    return mega_dot_row4<4>(wr, xq_lds, lane);
+}
+
 // Weight rows are read through a pointer that is explicitly in the global address space: a generic pointer
 // would make these FLAT loads, which also count on the LDS/scalar counter, and every LDS wait of the wave
 // would then wait for the weight prefetch as well.
@@ -334,7 +443,11 @@ __device__ __forceinline__ int mega_dot_row(const i32x4 (&wr)[NCH], const int8_t
     return wave_sum_i(acc);
 }
 
-__global__ __launch_bounds__(kMegaT, 1) void decode_mega_kernel(MegaParams p) {
+// W4 = false: W8A8 (symmetric int8 activations and weights).  W4 = true: the W4A4 configuration (asymmetric uint4
+// activations, int4 weights two per byte, int4 output head); attention, exchanges and wave roles are the same, the
+// weight rows are half as long: a stream wave then holds all 16 of its gate/up rows in registers.
+template <bool W4>
+__device__ __forceinline__ void decode_mega_body(const MegaParams& p) {
     extern __shared__ __attribute__((aligned(16))) unsigned char mega_smem[];   // sizeof(MegaLds) > the static 64 KiB limit
     MegaLds& L = *reinterpret_cast<MegaLds*>(mega_smem);
     const int t = threadIdx.x, wg = blockIdx.x;
@@ -401,7 +514,9 @@ __global__ __launch_bounds__(kMegaT, 1) void decode_mega_kernel(MegaParams p) {
 #ifdef FX_MEGA_ALL_STAMPS
         cur_layer = l;
 #endif
-        const LayerW w = ldc_layer(p.layers + l);
+        typename std::conditional<W4, LayerW4, LayerW>::type w;
+        if constexpr (W4) w = ldc_layer4(reinterpret_cast<const LayerW4*>(p.layers) + l);
+        else w = ldc_layer(reinterpret_cast<const LayerW*>(p.layers) + l);
         // sequence number of this layer pass: unique over launches, the tag of everything this pass publishes
         const unsigned tag = seq0 + (unsigned)(step * p.n_layers + l) + 1u;
         const float* g0 = p.gamma + (size_t)(2 * l) * H;
@@ -420,12 +535,25 @@ __global__ __launch_bounds__(kMegaT, 1) void decode_mega_kernel(MegaParams p) {
         // (8 MiB over the chip) drains while the phase computes; issuing a whole matrix at once instead fills
         // the memory queues for microseconds, and the barrier's own round trips then queue behind it.
         // Slices 0 and 1 (rows 0..7) wait in registers, slices 2 and 3 and the down rows in LDS.
+        // (W4A4: 16 rows of 1024 bytes each, all of them in registers, four per slice: gu[r >> 1][r & 1] is row r.)
         i32x4 gu[8][2];
         // Only the stream waves ever define these registers.  An empty asm "defines" them for every wave here,
         // or the compiler would carry the stale values of the other waves around the layer and token loops.
 #pragma unroll
         for (int r = 0; r < 8; r++) asm volatile("" : "=v"(gu[r][0]), "=v"(gu[r][1]));
         auto gu_slice = [&](int s) {
+            if constexpr (W4) {
+                __builtin_amdgcn_s_waitcnt(0x0F70);            // vmcnt(0) only, as below
+                if (is_s) {
+#pragma unroll
+                    for (int r = 0; r < 4; r++) {
+                        i32x4 one[1];
+                        mega_load_rows<1>(w.wgu, H / 2, wg * 64 + sw * 16 + 4 * s + r, lane, one);
+                        gu[(4 * s + r) >> 1][(4 * s + r) & 1] = one[0];
+                    }
+                }
+                return;
+            }
             // Every wave first waits for its own older loads (long landed at the points where this is called).
             // Otherwise the wait inserted for such a load after the branch below has to assume the path without
             // the slice, and it would make the stream waves sit out their own prefetch.
@@ -444,11 +572,18 @@ __global__ __launch_bounds__(kMegaT, 1) void decode_mega_kernel(MegaParams p) {
         // ================= phase 1: RMSNorm + quant -> q/k/v rows (12 per workgroup, 3 per wave 0..3) =================
         {
             i32x4 wr[3][2];
-            float wsc[3] = {0.0f, 0.0f, 0.0f};
+            float wsc[3] = {0.0f, 0.0f, 0.0f}, wsm[3] = {0.0f, 0.0f, 0.0f};
             if (!is_s) {
 #pragma unroll
                 for (int j = 0; j < 3; j++) {
-                    mega_load_rows<2>(w.wqkv, H, wg * 12 + wave + 4 * j, lane, wr[j]);
+                    if constexpr (W4) {
+                        i32x4 one[1];
+                        mega_load_rows<1>(w.wqkv, H / 2, wg * 12 + wave + 4 * j, lane, one);
+                        wr[j][0] = one[0];
+                        wsm[j] = ldc_f(w.mqkv + wg * 12 + wave + 4 * j);
+                    } else {
+                        mega_load_rows<2>(w.wqkv, H, wg * 12 + wave + 4 * j, lane, wr[j]);
+                    }
                     wsc[j] = ldc_f(w.sqkv + wg * 12 + wave + 4 * j);
                 }
             }
@@ -463,13 +598,22 @@ __global__ __launch_bounds__(kMegaT, 1) void decode_mega_kernel(MegaParams p) {
                     for (int i = 0; i < 4; i++) v[i] = __half2float(p.embed[(size_t)tok * H + 4 * t + i]);
                 }
             }
-            const float sx = norm_quant_2048(v, gam, true, p.eps, L, [&]() { gu_slice(0); });
+            float sx, bx = 0.0f;
+            if constexpr (W4) { const float2 sb = norm_quant_2048_u4(v, gam, true, p.eps, L, [&]() { gu_slice(0); }); sx = sb.x; bx = sb.y; }
+            else sx = norm_quant_2048(v, gam, true, p.eps, L, [&]() { gu_slice(0); });
             if (!is_s) {
 #pragma unroll
                 for (int j = 0; j < 3; j++) {
                     const int r = wg * 12 + wave + 4 * j;
-                    const int a = mega_dot_row<2>(wr[j], L.xq, lane);
-                    if (lane == 0) st_tagged(&p.qkv_tag[r], (float)a * sx * wsc[j], tag);
+                    float out;
+                    if constexpr (W4) {
+                        const i32x4 one[1] = {wr[j][0]};
+                        out = (float)mega_dot_row4<1>(one, L.xq, lane) * sx * wsc[j];
+                        out = out + bx * wsm[j];
+                    } else {
+                        out = (float)mega_dot_row<2>(wr[j], L.xq, lane) * sx * wsc[j];
+                    }
+                    if (lane == 0) st_tagged(&p.qkv_tag[r], out, tag);
                 }
             }
             stamp();
@@ -630,11 +774,18 @@ __global__ __launch_bounds__(kMegaT, 1) void decode_mega_kernel(MegaParams p) {
         // ================= phase 4: attention dequant + quant -> o_proj rows (8 per workgroup, 2 per wave 0..3) + residual =================
         {
             i32x4 wr[2][2];
-            float wsc[2] = {0.0f, 0.0f};
+            float wsc[2] = {0.0f, 0.0f}, wsm[2] = {0.0f, 0.0f};
             if (!is_s) {
 #pragma unroll
                 for (int j = 0; j < 2; j++) {
-                    mega_load_rows<2>(w.wo, H, wg * 8 + wave + 4 * j, lane, wr[j]);
+                    if constexpr (W4) {
+                        i32x4 one[1];
+                        mega_load_rows<1>(w.wo, H / 2, wg * 8 + wave + 4 * j, lane, one);
+                        wr[j][0] = one[0];
+                        wsm[j] = ldc_f(w.mo + wg * 8 + wave + 4 * j);
+                    } else {
+                        mega_load_rows<2>(w.wo, H, wg * 8 + wave + 4 * j, lane, wr[j]);
+                    }
                     wsc[j] = ldc_f(w.so + wg * 8 + wave + 4 * j);
                 }
             }
@@ -659,12 +810,21 @@ __global__ __launch_bounds__(kMegaT, 1) void decode_mega_kernel(MegaParams p) {
                 }
             }
             const float4 z4 = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
-            const float sx = norm_quant_2048(v, z4, false, p.eps, L, [&]() { gu_slice(3); });
+            float sx, bx = 0.0f;
+            if constexpr (W4) { const float2 sb = norm_quant_2048_u4(v, z4, false, p.eps, L, [&]() { gu_slice(3); }); sx = sb.x; bx = sb.y; }
+            else sx = norm_quant_2048(v, z4, false, p.eps, L, [&]() { gu_slice(3); });
             if (!is_s) {
 #pragma unroll
                 for (int j = 0; j < 2; j++) {
-                    const int a0 = mega_dot_row<2>(wr[j], L.xq, lane);
-                    if (lane == 0) L.res8[wave + 4 * j] = (float)a0 * sx * wsc[j] + xr[j];
+                    if constexpr (W4) {
+                        const i32x4 one[1] = {wr[j][0]};
+                        float out = (float)mega_dot_row4<1>(one, L.xq, lane) * sx * wsc[j];
+                        out = out + bx * wsm[j];
+                        if (lane == 0) L.res8[wave + 4 * j] = out + xr[j];
+                    } else {
+                        const int a0 = mega_dot_row<2>(wr[j], L.xq, lane);
+                        if (lane == 0) L.res8[wave + 4 * j] = (float)a0 * sx * wsc[j] + xr[j];
+                    }
                 }
             }
             // the workgroup's eight outputs leave as one 32-byte store: eight single-lane stores from four waves into
@@ -683,6 +843,13 @@ __global__ __launch_bounds__(kMegaT, 1) void decode_mega_kernel(MegaParams p) {
             const int ridx = 4 * (lane & 1) + 2 * ((lane >> 1) & 1) + ((lane >> 2) & 1);
             const int ow = wave & 3, half = is_s ? 0 : 8;
             const float gsc = w.sgu[wg * 64 + ow * 16 + half + ridx]; // read before this phase's prefetch is issued
+            // W4A4: a stream wave multiplies all 16 of its rows (rows ridx and 8 + ridx per lane after the folding)
+            float gsc_b = 0.0f, gsm_a = 0.0f, gsm_b = 0.0f;
+            if constexpr (W4) {
+                gsc_b = w.sgu[wg * 64 + ow * 16 + 8 + ridx];
+                gsm_a = w.mgu[wg * 64 + ow * 16 + ridx];
+                gsm_b = w.mgu[wg * 64 + ow * 16 + 8 + ridx];
+            }
             const float4 gam = reinterpret_cast<const float4*>(g1)[t];
             float v[4];
             poll_tagged4(&p.x2_tag[4 * t], tag, bar.err, v);
@@ -690,33 +857,21 @@ __global__ __launch_bounds__(kMegaT, 1) void decode_mega_kernel(MegaParams p) {
             // every workgroup has published x2, so it has read the accumulators; the next parts are added a layer later,
             // by workgroups that have polled this workgroup's x, which wave 0 stores after this store has been acknowledged
             if (t < 8) st_i(&p.o_acc[wg * 8 + t], 0);
-            const float sx = norm_quant_2048(v, gam, true, p.eps, L, [&]() {
+            auto down_row_0 = [&]() {
                 __builtin_amdgcn_s_waitcnt(0x0F70);                   // vmcnt(0): see gu_slice
-                if (is_s) mega_row_to_lds(w.wd, wg * 8 + sw * 2, lane, L.wd[sw * 2]);
-            });
-            if (l == 1) fine();
-            {
-                // eight per-lane partial dot products, folded with a transposing butterfly: each step halves the number
-                // of live values, so 7 + 3 cross-lane exchanges replace 8 x 6.  Afterwards lane L holds the complete
-                // sum of row 4*(L&1) + 2*(L>>1 & 1) + (L>>2 & 1).
-                int part[8];
-                {
-                    const i32x4 x0 = reinterpret_cast<const i32x4*>(L.xq)[lane], x1 = reinterpret_cast<const i32x4*>(L.xq)[lane + 64];
-                    if (is_s) {
-#pragma unroll
-                        for (int r = 0; r < 8; r++) part[r] = dot16(gu[r][1], x1, dot16(gu[r][0], x0, 0));
-                    } else {
-                        // rows 8..15 from LDS (complete and visible: their stream wave waited for them at the head of
-                        // this phase's prefetch hook, before the barrier that ended the quantisation)
-                        const i32x4* g2 = reinterpret_cast<const i32x4*>(L.gu2[ow]);
-                        const i32x4* g3 = reinterpret_cast<const i32x4*>(L.wd[ow * 2 + 1]);
-#pragma unroll
-                        for (int r = 0; r < 4; r++) {
-                            part[r] = dot16(g2[lane + 64 * (2 * r + 1)], x1, dot16(g2[lane + 64 * (2 * r)], x0, 0));
-                            part[4 + r] = dot16(g3[lane + 64 * (2 * r + 1)], x1, dot16(g3[lane + 64 * (2 * r)], x0, 0));
-                        }
-                    }
+                if (is_s) {
+                    if constexpr (W4) mega_row4_to_lds(w.wd, wg * 8 + sw * 2, lane, L.wd[sw * 2]);
+                    else mega_row_to_lds(w.wd, wg * 8 + sw * 2, lane, L.wd[sw * 2]);
                 }
+            };
+            float sx, bx = 0.0f;
+            if constexpr (W4) { const float2 sb = norm_quant_2048_u4(v, gam, true, p.eps, L, down_row_0); sx = sb.x; bx = sb.y; }
+            else sx = norm_quant_2048(v, gam, true, p.eps, L, down_row_0);
+            if (l == 1) fine();
+            // eight per-lane partial sums folded with a transposing butterfly: each step halves the number of live
+            // values, so 7 + 3 cross-lane exchanges replace 8 x 6.  Afterwards lane L holds the complete sum of row
+            // 4*(L&1) + 2*(L>>1 & 1) + (L>>2 & 1).
+            auto fold8 = [&](const int (&part)[8]) {
                 int q4[4], q2[2];
                 {
                     const bool hi = lane & 1;
@@ -736,6 +891,51 @@ __global__ __launch_bounds__(kMegaT, 1) void decode_mega_kernel(MegaParams p) {
                 sum += lane_xor_i<8>(sum);
                 sum += lane_xor_i<16>(sum);
                 sum += lane_xor_i<32>(sum);
+                return sum;
+            };
+            if constexpr (W4) {
+                if (is_s) {
+                    const i32x4 ones = {0x11111111, 0x11111111, 0x11111111, 0x11111111};
+                    i32x4 xs = reinterpret_cast<const i32x4*>(L.xq)[lane];
+                    xs.x ^= 0x88888888; xs.y ^= 0x88888888; xs.z ^= 0x88888888; xs.w ^= 0x88888888;   // a -> a - 8
+                    int part_a[8], part_b[8];
+#pragma unroll
+                    for (int r = 0; r < 8; r++) {
+                        const i32x4 wa = gu[r >> 1][r & 1], wb = gu[(8 + r) >> 1][r & 1];
+                        part_a[r] = dot32_i4(wa, xs, 0) + 8 * dot32_i4(wa, ones, 0);
+                        part_b[r] = dot32_i4(wb, xs, 0) + 8 * dot32_i4(wb, ones, 0);
+                    }
+                    const int sum_a = fold8(part_a), sum_b = fold8(part_b);
+                    float mine_a = (float)sum_a * sx * gsc;
+                    mine_a = mine_a + bx * gsm_a;
+                    float mine_b = (float)sum_b * sx * gsc_b;
+                    mine_b = mine_b + bx * gsm_b;
+                    const float other_a = lane_xor_f<4>(mine_a), other_b = lane_xor_f<4>(mine_b);   // row ridx^1: the other half of the SwiGLU pair
+                    if (lane < 4) {                                // lanes 0..3 hold the (even) gate rows
+                        L.hst[ow * 8 + (ridx >> 1)] = other_a * silu_f(mine_a);
+                        L.hst[ow * 8 + 4 + (ridx >> 1)] = other_b * silu_f(mine_b);
+                    }
+                }
+            } else {
+                int part[8];
+                {
+                    const i32x4 x0 = reinterpret_cast<const i32x4*>(L.xq)[lane], x1 = reinterpret_cast<const i32x4*>(L.xq)[lane + 64];
+                    if (is_s) {
+#pragma unroll
+                        for (int r = 0; r < 8; r++) part[r] = dot16(gu[r][1], x1, dot16(gu[r][0], x0, 0));
+                    } else {
+                        // rows 8..15 from LDS (complete and visible: their stream wave waited for them at the head of
+                        // this phase's prefetch hook, before the barrier that ended the quantisation)
+                        const i32x4* g2 = reinterpret_cast<const i32x4*>(L.gu2[ow]);
+                        const i32x4* g3 = reinterpret_cast<const i32x4*>(L.wd[ow * 2 + 1]);
+#pragma unroll
+                        for (int r = 0; r < 4; r++) {
+                            part[r] = dot16(g2[lane + 64 * (2 * r + 1)], x1, dot16(g2[lane + 64 * (2 * r)], x0, 0));
+                            part[4 + r] = dot16(g3[lane + 64 * (2 * r + 1)], x1, dot16(g3[lane + 64 * (2 * r)], x0, 0));
+                        }
+                    }
+                }
+                const int sum = fold8(part);
                 const float mine = (float)sum * sx * gsc;
                 const float other = lane_xor_f<4>(mine);           // row ridx^1: the other half of the SwiGLU pair
                 if (lane < 4) L.hst[ow * 8 + (half >> 1) + (ridx >> 1)] = other * silu_f(mine);   // lanes 0..3 hold the (even) gate rows
@@ -764,6 +964,8 @@ __global__ __launch_bounds__(kMegaT, 1) void decode_mega_kernel(MegaParams p) {
             // that stream wave s fetched into LDS.
             const int drow = wg * 8 + (wave & 3) * 2 + (is_s ? 0 : 1);
             const float dsc = ldc_f(w.sd + drow);
+            float dsm = 0.0f;
+            if constexpr (W4) dsm = ldc_f(w.md + drow);
             float xres = 0.0f;
             bar.wait();
             stamp();
@@ -781,7 +983,10 @@ __global__ __launch_bounds__(kMegaT, 1) void decode_mega_kernel(MegaParams p) {
                 a[j] = *reinterpret_cast<const float4*>(hbuf + abase + j * 32);   // ordinary loads: they may hit in L2
             }
             __builtin_amdgcn_s_waitcnt(0x0F70);               // vmcnt(0): the h loads are complete
-            if (is_s) mega_row_to_lds(w.wd, wg * 8 + sw * 2 + 1, lane, L.wd[sw * 2 + 1]);
+            if (is_s) {
+                if constexpr (W4) mega_row4_to_lds(w.wd, wg * 8 + sw * 2 + 1, lane, L.wd[sw * 2 + 1]);
+                else mega_row_to_lds(w.wd, wg * 8 + sw * 2 + 1, lane, L.wd[sw * 2 + 1]);
+            }
             if (l == 1) fine();
 #pragma unroll
             for (int bit = 1; bit < 4; bit <<= 1)                                                                       // bits 5, 6
@@ -851,10 +1056,25 @@ __global__ __launch_bounds__(kMegaT, 1) void decode_mega_kernel(MegaParams p) {
             }
             amax = amax / p.fht_scale;
             if (l == 1) fine();
-            amax = mega_block_max_h(amax, L.red_max, NoHook());
-            const float sx = sym_scale(amax, 127.0f);
-            if (l == 1) fine();
-            {
+            float sx, bx = 0.0f;
+            if constexpr (W4) {
+                // asymmetric uint4: largest and smallest of the scaled values (the thread's own 16, then the workgroup's)
+                float vmax = b2[0], vmin = b2[0];
+#pragma unroll
+                for (int r = 1; r < 16; r++) { vmax = fmaxf(vmax, b2[r]); vmin = fminf(vmin, b2[r]); }
+                vmax = mega_block_max_h(vmax, L.red_max, NoHook());
+                vmin = mega_block_min_h(vmin, L.red_min, NoHook());
+                sx = (vmax - vmin) / 15.0f;
+                if (sx == 0.0f) sx = 1.0f;
+                bx = vmin;
+                uint16_t w16[4];
+                quant_u4_pack(b2, vmin, sx, w16);
+#pragma unroll
+                for (int q = 0; q < 4; q++) reinterpret_cast<uint16_t*>(L.xq)[q * 512 + t] = w16[q];   // nibble q*2048 + 4t + e
+            } else {
+                amax = mega_block_max_h(amax, L.red_max, NoHook());
+                sx = sym_scale(amax, 127.0f);
+                if (l == 1) fine();
                 int n16[16];
                 quant_vector(b2, sx, n16);
 #pragma unroll
@@ -864,7 +1084,11 @@ __global__ __launch_bounds__(kMegaT, 1) void decode_mega_kernel(MegaParams p) {
             if (is_s) __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): both down rows of this stream wave have landed in LDS
             __syncthreads();                               // ... and are visible to the wave that multiplies the odd one
             if (l == 1) fine();
-            {
+            if constexpr (W4) {
+                float out = (float)mega_dot_row4_lds(L.wd[(wave & 3) * 2 + (is_s ? 0 : 1)], L.xq, lane) * sx * dsc;
+                out = out + bx * dsm;
+                if (lane == 0) L.res8[drow - wg * 8] = out + xres;
+            } else {
                 const int a0 = mega_dot_row_lds(L.wd[(wave & 3) * 2 + (is_s ? 0 : 1)], L.xq, lane);
                 if (lane == 0) L.res8[drow - wg * 8] = (float)a0 * sx * dsc + xres;
             }
@@ -885,11 +1109,52 @@ __global__ __launch_bounds__(kMegaT, 1) void decode_mega_kernel(MegaParams p) {
         int t_head = threadIdx.x;                 // opaque copy, as in the layer loop: nothing per-thread stays live across it
         asm volatile("" : "+v"(t_head));
         const int t = t_head, lane = t & 63;
-        using h16x8 = _Float16 __attribute__((ext_vector_type(8)));
         const int rows_per_wg = (p.vocab + kMegaWG - 1) / kMegaWG;
         const int row_begin = wg * rows_per_wg, row_end = min(p.vocab, row_begin + rows_per_wg);
-        const h16x8* table = reinterpret_cast<const h16x8*>(p.embed);
         constexpr int U = 4;
+        int r = row_begin + wave;
+        float best = -INFINITY;
+        int bi = 0x7fffffff;
+        auto keep_logit = [&](float s, int row) {              // one finished row: wave-uniform s
+            if (row < row_end) {
+                if (lane == 0) {
+                    p.logits[row] = s;
+                    if (sampling) L.f[4096 + (row - row_begin)] = s;      // L.f[0..2047] holds the normalised vector
+                }
+                if (s > best || (s == best && row < bi)) { best = s; bi = row; }
+            }
+        };
+        if constexpr (W4) {
+            // int4 output head: rows of 1024 bytes against the normalised vector quantised to asymmetric uint4
+            i32x4 wv[U][1];
+            auto load_group = [&](int rr) {
+#pragma unroll
+                for (int u = 0; u < U; u++)
+                    mega_load_rows<1>(reinterpret_cast<const int8_t*>(p.head_w4), H / 2, min(rr + u * kMegaWaves, p.vocab - 1), lane, wv[u]);
+            };
+            load_group(r);
+            float v[4];
+            poll_tagged4(&p.x_tag[4 * t], seq0 + (unsigned)((step + 1) * p.n_layers), bar.err, v);
+            stamp();
+            const float4 g = reinterpret_cast<const float4*>(p.gamma + (size_t)(2 * p.n_layers) * H)[t];
+            const float2 sb = norm_quant_2048_u4(v, g, true, p.eps, L, NoHook());
+            for (; r < row_end; r += U * kMegaWaves) {
+                int acc[U];
+#pragma unroll
+                for (int u = 0; u < U; u++) acc[u] = mega_dot_row4<1>(wv[u], L.xq, lane);
+                const int rn = r + U * kMegaWaves;
+                if (rn < row_end) load_group(rn);
+#pragma unroll
+                for (int u = 0; u < U; u++) {
+                    const int row = min(r + u * kMegaWaves, p.vocab - 1);
+                    float s = (float)acc[u] * sb.x * p.head_s[row];
+                    s = s + sb.y * p.head_sum[row];
+                    keep_logit(s, r + u * kMegaWaves);
+                }
+            }
+        } else {
+        using h16x8 = _Float16 __attribute__((ext_vector_type(8)));
+        const h16x8* table = reinterpret_cast<const h16x8*>(p.embed);
         h16x8 wv[U][4];
         auto load_group = [&](int r) {
 #pragma unroll
@@ -899,7 +1164,6 @@ __global__ __launch_bounds__(kMegaT, 1) void decode_mega_kernel(MegaParams p) {
                 for (int i = 0; i < 4; i++) wv[u][i] = __builtin_nontemporal_load(table + (size_t)row * (H / 8) + lane + 64 * i);
             }
         };
-        int r = row_begin + wave;
         load_group(r);
         float v[4];
         poll_tagged4(&p.x_tag[4 * t], seq0 + (unsigned)((step + 1) * p.n_layers), bar.err, v);
@@ -915,8 +1179,6 @@ __global__ __launch_bounds__(kMegaT, 1) void decode_mega_kernel(MegaParams p) {
         for (int i = 0; i < 4; i++)
 #pragma unroll
             for (int e = 0; e < 8; e++) nv[i][e] = L.f[(lane + 64 * i) * 8 + e];
-        float best = -INFINITY;
-        int bi = 0x7fffffff;
         for (; r < row_end; r += U * kMegaWaves) {
             float acc[U];
 #pragma unroll
@@ -930,17 +1192,8 @@ __global__ __launch_bounds__(kMegaT, 1) void decode_mega_kernel(MegaParams p) {
             const int rn = r + U * kMegaWaves;
             if (rn < row_end) load_group(rn);
 #pragma unroll
-            for (int u = 0; u < U; u++) {
-                const float s = wave_sum(acc[u]);
-                const int row = r + u * kMegaWaves;
-                if (row < row_end) {
-                    if (lane == 0) {
-                        p.logits[row] = s;
-                        if (sampling) L.f[4096 + (row - row_begin)] = s;      // L.f[0..2047] holds the normalised vector
-                    }
-                    if (s > best || (s == best && row < bi)) { best = s; bi = row; }
-                }
-            }
+            for (int u = 0; u < U; u++) keep_logit(wave_sum(acc[u]), r + u * kMegaWaves);
+        }
         }
         if (lane == 0) { L.bestv[wave] = best; L.besti[wave] = bi; }
         __syncthreads();
@@ -1020,5 +1273,8 @@ __global__ __launch_bounds__(kMegaT, 1) void decode_mega_kernel(MegaParams p) {
     if (p.timeline && is_t0()) p.timeline[p.n_layers * 12 + 2 + 64 + kMegaWG + wg] = wall_clock64();     // workgroup exit
 #endif
 }
+
+__global__ __launch_bounds__(kMegaT, 1) void decode_mega_kernel(MegaParams p) { decode_mega_body<false>(p); }
+__global__ __launch_bounds__(kMegaT, 1) void decode_mega_w4_kernel(MegaParams p) { decode_mega_body<true>(p); }
 
 }  // namespace fx

@@ -49,6 +49,12 @@ struct flexllm_llama {
     std::vector<void*> owned;
     fx::PrefillWorkspace pws;
     fx::LayerW* layers_dev = nullptr;   // device copy of `layers` for the persistent kernel
+    // W4A4 model (flexllm_llama_create_w4a4): the nibble-packed matrices with their row sums, the int4 output head
+    bool w4 = false;
+    std::vector<fx::LayerW4> layers4;
+    fx::LayerW4* layers4_dev = nullptr;
+    uint8_t* head_w4 = nullptr;
+    float *head_s = nullptr, *head_sum = nullptr;
     unsigned* bar = nullptr;            // grid-barrier counters of the persistent kernel
     bool mega_ok = false;               // shapes match the persistent kernel's compile-time constants
     int decode_mode = 0;                // 0: persistent kernel when possible, 1: one kernel per stage
@@ -176,7 +182,8 @@ static int launch_mega(flexllm_llama* m, int* token, const float* x_in, float* l
                        int* tokens_out = nullptr, int steps = 1, const float* rands = nullptr, int top_k = 0) {
     const flexllm_llama_config& c = m->cfg;
     MegaParams p;
-    p.layers = m->layers_dev;
+    p.layers = m->w4 ? (const void*)m->layers4_dev : (const void*)m->layers_dev;
+    p.head_w4 = m->head_w4; p.head_s = m->head_s; p.head_sum = m->head_sum;
     p.gamma = m->gamma; p.q_s = m->q_s; p.k_s = m->k_s; p.v_s = m->v_s; p.a_s = m->a_s;
     p.rope_sin = m->rope_sin; p.rope_cos = m->rope_cos;
     p.embed = reinterpret_cast<const __half*>(m->embed);
@@ -193,16 +200,19 @@ static int launch_mega(flexllm_llama* m, int* token, const float* x_in, float* l
         const int w = e ? atoi(e) : 0;
         p.timeline_wg = w >= 0 && w < kMegaWG ? w : 0;
     }
-    static bool lds_opted_in = false;     // the kernel's LDS block exceeds the default 64 KiB per workgroup
+    static bool lds_opted_in = false;     // the kernels' LDS block exceeds the default 64 KiB per workgroup
     if (!lds_opted_in) {
         FX_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(decode_mega_kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                   (int)sizeof(MegaLds)));
+        FX_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(decode_mega_w4_kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
                                    (int)sizeof(MegaLds)));
         lds_opted_in = true;
     }
     // An ordinary launch: one workgroup per CU fits by construction (mega_ok checks the CU count), and every barrier
     // and poll in the kernel is bounded, so work of other streams that delays some workgroups costs time, not a hang.
     // (A cooperative launch gives the same timing, but rocprofv3 of this ROCm release crashes at exit after one.)
-    decode_mega_kernel<<<kMegaWG, kMegaT, sizeof(MegaLds), st>>>(p);
+    if (m->w4) decode_mega_w4_kernel<<<kMegaWG, kMegaT, sizeof(MegaLds), st>>>(p);
+    else decode_mega_kernel<<<kMegaWG, kMegaT, sizeof(MegaLds), st>>>(p);
     FX_LAUNCH_CHECK();
     return FLEXLLM_OK;
 }
@@ -357,6 +367,84 @@ int flexllm_llama_create(flexllm_llama** out, const flexllm_llama_config* cfg, c
     return FLEXLLM_OK;
 }
 
+int flexllm_llama_create_w4a4(flexllm_llama** out, const flexllm_llama_config* cfg, const flexllm_llama_w4a4_weights* w) {
+    FX_REQUIRE(out && cfg && w, "llama_create_w4a4: null pointer");
+    FX_REQUIRE(w->sumq && w->sumk && w->sumv && w->sumo && w->sumg && w->sumu && w->sumd && w->head_w && w->head_s && w->head_sum,
+               "llama_create_w4a4: null weight pointer");
+    // The common part (fused q/k/v rows, interleaved gate/up rows, scales, tables, caches, workspace) is that of the
+    // W8A8 model on the same values held one per byte; the matrices are then packed two values per byte.
+    flexllm_llama* m = nullptr;
+    int rc = flexllm_llama_create(&m, cfg, &w->base);
+    if (rc) return rc;
+    const flexllm_llama_config& c = m->cfg;
+    const int H = c.hidden, KV = c.kv_hidden, I = c.inter, L = c.layers;
+    auto fail = [&](int code) { flexllm_llama_destroy(m); return code; };
+    if (!m->mega_ok) {
+        set_error("llama_create_w4a4: the W4A4 decode path is the persistent kernel only (needs >= %d CUs and Llama-3.2-1B shapes)", kMegaWG);
+        return fail(FLEXLLM_EINVAL);
+    }
+#define FX_TRY(expr)                          \
+    do {                                      \
+        int rc__ = (expr);                    \
+        if (rc__) return fail(rc__);          \
+    } while (0)
+#define FX_TRY_HIP(call)                                                               \
+    do {                                                                               \
+        hipError_t e_ = (call);                                                        \
+        if (e_ != hipSuccess) {                                                        \
+            set_error("%s failed: %s", #call, hipGetErrorString(e_));                  \
+            return fail(FLEXLLM_EHIP);                                                 \
+        }                                                                              \
+    } while (0)
+    auto pack = [&](const int8_t* values, int8_t** packed, size_t n_values) -> int {
+        int r = dev_alloc(m, (void**)packed, n_values / 2);
+        if (r) return r;
+        const size_t n_out = n_values / 2;
+        pack_nibbles_kernel<<<(int)((n_out + 255) / 256 < 4096 ? (n_out + 255) / 256 : 4096), 256>>>(
+            reinterpret_cast<const uint8_t*>(values), reinterpret_cast<uint8_t*>(*packed), n_out);
+        return FLEXLLM_OK;
+    };
+    m->layers4.resize(L);
+    for (int l = 0; l < L; l++) {
+        const LayerW& lw = m->layers[l];
+        LayerW4& l4 = m->layers4[l];
+        FX_TRY(pack(lw.wqkv, &l4.wqkv, (size_t)(H + 2 * KV) * H));
+        FX_TRY(pack(lw.wo, &l4.wo, (size_t)H * H));
+        FX_TRY(pack(lw.wgu, &l4.wgu, (size_t)2 * I * H));
+        FX_TRY(pack(lw.wd, &l4.wd, (size_t)H * I));
+        l4.sqkv = lw.sqkv; l4.so = lw.so; l4.sgu = lw.sgu; l4.sd = lw.sd;
+        FX_TRY(dev_alloc(m, (void**)&l4.mqkv, sizeof(float) * (H + 2 * KV)));
+        FX_TRY(dev_alloc(m, (void**)&l4.mo, sizeof(float) * H));
+        FX_TRY(dev_alloc(m, (void**)&l4.mgu, sizeof(float) * 2 * I));
+        FX_TRY(dev_alloc(m, (void**)&l4.md, sizeof(float) * H));
+        FX_TRY_HIP(hipMemcpy(l4.mqkv, w->sumq[l], sizeof(float) * H, hipMemcpyDeviceToDevice));
+        FX_TRY_HIP(hipMemcpy(l4.mqkv + H, w->sumk[l], sizeof(float) * KV, hipMemcpyDeviceToDevice));
+        FX_TRY_HIP(hipMemcpy(l4.mqkv + H + KV, w->sumv[l], sizeof(float) * KV, hipMemcpyDeviceToDevice));
+        FX_TRY_HIP(hipMemcpy(l4.mo, w->sumo[l], sizeof(float) * H, hipMemcpyDeviceToDevice));
+        FX_TRY_HIP(hipMemcpy2D(l4.mgu, 2 * sizeof(float), w->sumg[l], sizeof(float), sizeof(float), I, hipMemcpyDeviceToDevice));
+        FX_TRY_HIP(hipMemcpy2D(l4.mgu + 1, 2 * sizeof(float), w->sumu[l], sizeof(float), sizeof(float), I, hipMemcpyDeviceToDevice));
+        FX_TRY_HIP(hipMemcpy(l4.md, w->sumd[l], sizeof(float) * H, hipMemcpyDeviceToDevice));
+    }
+    {
+        int8_t* hw = nullptr;
+        FX_TRY(pack(w->head_w, &hw, (size_t)c.vocab * H));
+        m->head_w4 = reinterpret_cast<uint8_t*>(hw);
+        FX_TRY(dev_alloc(m, (void**)&m->head_s, sizeof(float) * c.vocab));
+        FX_TRY(dev_alloc(m, (void**)&m->head_sum, sizeof(float) * c.vocab));
+        FX_TRY_HIP(hipMemcpy(m->head_s, w->head_s, sizeof(float) * c.vocab, hipMemcpyDeviceToDevice));
+        FX_TRY_HIP(hipMemcpy(m->head_sum, w->head_sum, sizeof(float) * c.vocab, hipMemcpyDeviceToDevice));
+    }
+    FX_TRY(dev_alloc(m, (void**)&m->layers4_dev, sizeof(LayerW4) * L));
+    FX_TRY_HIP(hipMemcpy(m->layers4_dev, m->layers4.data(), sizeof(LayerW4) * L, hipMemcpyHostToDevice));
+    FX_TRY_HIP(hipDeviceSynchronize());
+    FX_TRY_HIP(hipGetLastError());
+#undef FX_TRY
+#undef FX_TRY_HIP
+    m->w4 = true;
+    *out = m;
+    return FLEXLLM_OK;
+}
+
 int flexllm_llama_destroy(flexllm_llama* m) {
     if (!m) return FLEXLLM_OK;
     (void)hipDeviceSynchronize();
@@ -369,6 +457,7 @@ int flexllm_llama_destroy(flexllm_llama* m) {
 
 int flexllm_llama_set_decode_mode(flexllm_llama* m, int mode) {
     FX_REQUIRE(m && (mode == 0 || mode == 1), "llama_set_decode_mode: mode=%d (0 persistent kernel, 1 one kernel per stage)", mode);
+    FX_REQUIRE(!(m->w4 && mode == 1), "llama_set_decode_mode: a W4A4 model decodes with the persistent kernel only");
     if (m->decode_mode != mode) {
         if (m->graph_exec) { (void)hipGraphExecDestroy(m->graph_exec); m->graph_exec = nullptr; }
         // (the two schedules keep their attention accumulators apart: the persistent kernel's are back at zero
@@ -513,6 +602,7 @@ int flexllm_llama_decode_sample(flexllm_llama* m, int* token_io, int pos0, int s
         }
         return FLEXLLM_OK;
     }
+    FX_REQUIRE(!m->w4, "llama_decode_sample: vocab=%d is too large for the persistent kernel's sampler, the only one a W4A4 model has", c.vocab);
     // one kernel per stage: layers + lm_head into m->logits, then the sampler picks the token (rands[step]), hands it
     // over through token_io and advances position and step in device memory
     TopKOut out = {nullptr, nullptr, nullptr, nullptr, token_io, tokens_out, m->state};
@@ -533,6 +623,7 @@ int flexllm_llama_decode_sample(flexllm_llama* m, int* token_io, int pos0, int s
 int flexllm_llama_generate(flexllm_llama* m, const int* prompt, int n_prompt, int steps, const float* rands, int top_k,
                            int* tokens_out, void* stream) {
     FX_REQUIRE(m && prompt && tokens_out, "llama_generate: null pointer");
+    FX_REQUIRE(!m->w4, "llama_generate: a W4A4 model has no fused prefill (its prefill runs stage by stage over the module entry points)");
     FX_REQUIRE(n_prompt >= 1 && steps >= 0 && n_prompt - 1 + steps <= m->cfg.max_pos,
                "llama_generate: prompt of %d tokens + %d steps exceed max_pos=%d", n_prompt, steps, m->cfg.max_pos);
     FX_REQUIRE(top_k == 0 || rands, "llama_generate: sampling (top_k=%d) needs the uniform numbers", top_k);
@@ -565,6 +656,7 @@ int flexllm_llama_generate(flexllm_llama* m, const int* prompt, int n_prompt, in
 
 int flexllm_llama_prefill_hidden(flexllm_llama* m, const float* x_in, int s, float* hidden_out, void* stream) {
     FX_REQUIRE(m && x_in, "llama_prefill_hidden: null pointer");
+    FX_REQUIRE(!m->w4, "llama_prefill_hidden: a W4A4 model has no fused prefill (its prefill runs stage by stage over the module entry points)");
     return llama_prefill_run(m->cfg, m->layers.data(), m->gamma, m->q_s, m->k_s, m->v_s, m->a_s, m->rope_sin, m->rope_cos,
                              m->k_cache, m->v_cache, m->cache_layer_bytes, &m->pws, x_in, s, hidden_out, as_stream(stream));
 }

@@ -6,7 +6,7 @@ import math
 import numpy as np
 
 from . import synth
-from ._lib import lib, check, LlamaConfig, LlamaWeights
+from ._lib import lib, check, LlamaConfig, LlamaWeights, LlamaW4A4Weights
 from .device import DeviceArray, to_device, _s
 from .ops import rope_table
 
@@ -60,8 +60,41 @@ def synth_weights(cfg, seed=1, device=False, embed_range=1.7):
     return w
 
 
+def synth_weights_w4a4(cfg, seed=1, device=False, embed_range=1.7):
+    """Random-init weights of the W4A4 configuration: int4 values U[-8,7] held one per byte, per-channel scales sized
+    so that activations stay O(1), the row sums of the dequantised weights (`sum<p>`, the generated headers'
+    w_<proj>_sum), an int4 output head (`head_w`, `head_s`, `head_sum`) and everything synth_weights gives besides the
+    matrices.  device as in synth_weights; the row sums of device matrices are taken on the device too (a GEMV with
+    a vector of ones)."""
+    w = synth_weights(cfg, seed, device, embed_range)
+    i8 = synth.device_i8 if device else synth.host_i8
+    f32 = synth.device_uniform_f32 if device else synth.host_uniform_f32
+
+    def row_sums(q, s):
+        if not device:
+            return (q.sum(1, dtype=np.int64).astype(np.float32) * s).astype(np.float32)
+        from . import ops
+        tot = ops.linear_i8_gemv(to_device(np.ones(q.shape[1], np.int8)), q).numpy()
+        return to_device((tot.astype(np.float32) * s.numpy()).astype(np.float32))
+
+    for t, (name, (n_key, k_key)) in enumerate(_PROJ.items()):
+        n, k = cfg[n_key], cfg[k_key]
+        base = 1.0 / (4.6 * math.sqrt(k))
+        w["w" + name] = [i8((n, k), _seed(seed, l, 40 + t), -8, 7) for l in range(cfg["layers"])]
+        w["s" + name] = [f32((n,), _seed(seed, l, 60 + t), 0.5 * base, 1.5 * base) for l in range(cfg["layers"])]
+        w["sum" + name] = [row_sums(w["w" + name][l], w["s" + name][l]) for l in range(cfg["layers"])]
+    V, H = cfg["vocab"], cfg["hidden"]
+    base = 1.0 / (4.6 * math.sqrt(H))
+    w["head_w"] = i8((V, H), _seed(seed, 99, 7), -8, 7)
+    w["head_s"] = f32((V,), _seed(seed, 99, 8), 0.5 * base, 1.5 * base)
+    w["head_sum"] = row_sums(w["head_w"], w["head_s"])
+    return w
+
+
 class Llama:
-    """Device model object.  `weights` holds DeviceArrays (see synth_weights(device=True))."""
+    """Device model object.  `weights` holds DeviceArrays (see synth_weights(device=True)); with the keys of
+    synth_weights_w4a4 (`sum<p>`, `head_w`, ...) it is the W4A4 model (flexllm_llama_create_w4a4), which decodes in the
+    persistent kernel and has no fused prefill."""
 
     def __init__(self, cfg, weights):
         self.cfg = cfg
@@ -80,7 +113,19 @@ class Llama:
             setattr(w, n, weights[n].ptr)
         self._gamma, self._embed = weights["gamma"], weights["embed"]
         h = C.c_void_p()
-        check(lib().flexllm_llama_create(C.byref(h), C.byref(c), C.byref(w)))
+        self.w4a4 = "sumq" in weights
+        if self.w4a4:
+            w4 = LlamaW4A4Weights()
+            w4.base = w
+            for n in ("sumq", "sumk", "sumv", "sumo", "sumg", "sumu", "sumd"):
+                arr = (C.c_void_p * L)(*[weights[n][l].ptr for l in range(L)])
+                keep.append(arr)
+                setattr(w4, n, C.cast(arr, C.c_void_p))
+            for n in ("head_w", "head_s", "head_sum"):
+                setattr(w4, n, weights[n].ptr)
+            check(lib().flexllm_llama_create_w4a4(C.byref(h), C.byref(c), C.byref(w4)))
+        else:
+            check(lib().flexllm_llama_create(C.byref(h), C.byref(c), C.byref(w)))
         self.handle = h
         cache_shape_k = (L, cfg["kv_heads"], cfg["max_pos"], cfg["head_dim"])
         cache_shape_v = (L, cfg["kv_heads"], cfg["max_pos"] // 64, cfg["head_dim"], 64)

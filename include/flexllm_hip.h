@@ -335,6 +335,25 @@ typedef struct flexllm_llama flexllm_llama;
  * K [layers][kv_heads][max_pos][64], V [layers][kv_heads][max_pos/64][64 channels][64 positions]) and the
  * activation workspace. */
 int flexllm_llama_create(flexllm_llama** out, const flexllm_llama_config* cfg, const flexllm_llama_weights* w);
+/* The shipped W4A4 configuration as a model of its own: asymmetric uint4 activations x int4 weights in all seven
+ * projections and in the output head (one int4 engine for every linear layer and an int4 lm_head in
+ * SpinQuant_Llama_32_1B/SpinQuant_Decoding_mem_opt.h:363-365, 415-469), int8 attention as above.  `base` holds the
+ * matrices as int8 arrays of int4 values (-8..7, one per byte, as in parameters/<proj>_L%02d.bin) with their scales,
+ * and the fp16 embedding table that turns a token id into the layer input; sum<p>[l] is the per-output-row sum of
+ * the dequantised weights (the generated headers' w_<proj>_sum), which the activations' zero point multiplies; the
+ * head is int4 [vocab][hidden] one value per byte with per-row scale and row sum.  The library packs the matrices two
+ * values per byte.  Decoding (flexllm_llama_decode_hidden / _decode_greedy / _decode_sample) runs in the persistent
+ * kernel only, which then streams half the weight bytes per token; prefill of this configuration runs stage by stage
+ * over the module entry points (flexllm_amd/llama_w4a4.py), and the entry points that prefill return an error. */
+typedef struct {
+    flexllm_llama_weights base;
+    const float* const* sumq; const float* const* sumk; const float* const* sumv; const float* const* sumo;
+    const float* const* sumg; const float* const* sumu; const float* const* sumd;
+    const int8_t* head_w;               /* device int4 values [vocab][hidden], one per byte */
+    const float* head_s;                /* device [vocab] */
+    const float* head_sum;              /* device [vocab] */
+} flexllm_llama_w4a4_weights;
+int flexllm_llama_create_w4a4(flexllm_llama** out, const flexllm_llama_config* cfg, const flexllm_llama_w4a4_weights* w);
 int flexllm_llama_destroy(flexllm_llama* m);
 /* Decode schedule: 0 (default) = one persistent kernel per token (all layers + lm_head, grid barriers between
  * stages, next stage's weights prefetched across the barrier) when the device has >= 256 CUs and the shapes are
