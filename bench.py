@@ -363,6 +363,38 @@ def main():
         g0.record(stream); gen(); g1.record(stream); g1.sync()
         modules["generate_prompt1025_greedy64"] = {"ms": round(g0.elapsed_ms(g1), 3), "prefilled_tokens": n_p - 1, "generated_tokens": n_g}
         modules["decode_top5_sampling_ctx4096"] = {"ms_per_token": round(ms / n_s, 4), "tokens_per_s": round(n_s / ms * 1e3, 1), "steps": n_s}
+        # the shipped W4A4 configuration decoded by the persistent kernel's W4A4 instance (nibble-packed weights, int4
+        # output head): same loop as the headline, 64 greedy tokens per launch up to the maximum context, with its own
+        # HBM roofline line (half the weight bytes per token)
+        w4 = llama.synth_weights_w4a4(cfg, seed=5, device=True, embed_range=0.03)
+        model4 = llama.Llama(cfg, w4)
+        del w4
+        lib.flexllm_rt_fill_i8(C.c_void_p(model4.k_cache.ptr), C.c_size_t(model4.k_cache.size), C.c_uint64(911), -100, 100, stream.handle)
+        lib.flexllm_rt_fill_i8(C.c_void_p(model4.v_cache.ptr), C.c_size_t(model4.v_cache.size), C.c_uint64(912), -100, 100, stream.handle)
+        n4 = TOKENS_PER_LAUNCH
+        tok4 = fx.to_device(np.array([12345], np.int32)); out4 = fx.zeros((n4,), np.int32)
+        model4.decode_greedy(tok4, cfg["max_pos"] - 2 * n4, n4, out4, use_graph=False, stream=stream); stream.sync()
+        q0, q1 = Event(), Event()
+        q0.record(stream)
+        model4.decode_greedy(tok4, cfg["max_pos"] - n4, n4, out4, use_graph=False, stream=stream)
+        q1.record(stream); q1.sync()
+        model4.check()
+        us4 = q0.elapsed_ms(q1) * 1e3 / n4
+        Hh, KVh, Ih, Lh, Vh = cfg["hidden"], cfg["kv_hidden"], cfg["inter"], cfg["layers"], cfg["vocab"]
+        n_w = Lh * (Hh * Hh + 2 * KVh * Hh + Hh * Hh + 2 * Ih * Hh + Hh * Ih)
+        rows = Lh * (Hh + 2 * KVh + Hh + 2 * Ih + Hh)
+        bytes4 = n_w // 2 + 8 * rows + 4 * (2 * Lh + 1) * Hh + Vh * Hh // 2 + 8 * Vh \
+            + Lh * 2 * KVh * (cfg["max_pos"] - n4 / 2.0) + Lh * 2 * KVh
+        modules["w4a4_decode_ctx4096"] = {
+            "us_per_token": round(us4, 2), "tokens_per_s": round(1e6 / us4, 1), "bytes_per_token": int(bytes4),
+            "roofline": {"bound": "hbm", "kernel": "decode_mega_w4_kernel (1 launch of %d tokens)" % n4,
+                         "achieved": round(bytes4 / us4 / 1e3, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                         "frac": round(bytes4 / us4 / 1e3 / HBM_PEAK_GBS, 4)},
+            "distinct_tokens": int(len(set(out4.numpy().tolist()))),
+            "note": "int4 weights two per byte + scale and row sum per output row, int4 output head, int8 KV cache; "
+                    "the kernel is bound by its exchanges between workgroups, not by bytes"}
+        model4.close()
+        del model4
 
     # ---- CPU baseline: the oracle (scalar C port of the reference modules), measured, not extrapolated -----
     # whole tokens of the same model (16 layers, context 4096, full fp16 head over 128256 rows) on the host's cores:
