@@ -10,6 +10,7 @@
 #pragma once
 #include "attn_decode_kernels.h"
 #include "common.h"
+#include <atomic>
 #include <stdlib.h>
 
 namespace fx {
@@ -564,11 +565,11 @@ __global__ __launch_bounds__(NW * 64, WPE) void gemm_i8_dma_kernel(const int8_t*
 template <int BM, int BN, int EPI, int STAGES = 3, int WPE = 1, int BKB = 64, int NW = 4, int KSPLIT = 1>
 inline int launch_gemm_dma(const int8_t* a, const int8_t* w, int32_t* c, const float* s_x, const float* w_s,
                            const float* residual, float* y, int m, int k, int n, hipStream_t st, QkvEpiArgs qa = QkvEpiArgs()) {
-    static bool opted_in = false;             // more than the default 64 KiB of LDS per workgroup
-    if (!opted_in) {
+    static std::atomic<bool> opted_in{false};             // more than the default 64 KiB of LDS per workgroup
+    if (!opted_in.load(std::memory_order_acquire)) {   // idempotent: two threads racing here both set the same attribute
         FX_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_i8_dma_kernel<BM, BN, EPI, STAGES, WPE, BKB, NW, KSPLIT>),
                                    hipFuncAttributeMaxDynamicSharedMemorySize, gemm_dma_lds_bytes(BM, BN, STAGES, BKB, NW, KSPLIT)));
-        opted_in = true;
+        opted_in.store(true, std::memory_order_release);
     }
     const int tm = (m + BM - 1) / BM, tn = (n + BN - 1) / BN;
     gemm_i8_dma_kernel<BM, BN, EPI, STAGES, WPE, BKB, NW, KSPLIT><<<tm * tn, NW * 64, gemm_dma_lds_bytes(BM, BN, STAGES, BKB, NW, KSPLIT), st>>>(a, w, c, s_x, w_s, residual, y, m, k, n, tm, tn, qa);

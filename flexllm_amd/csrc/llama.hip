@@ -12,6 +12,7 @@
 #include "logits_kernels.h"
 #include "decode_mega.h"
 #include "prefill.h"
+#include <atomic>
 #include <vector>
 
 struct flexllm_llama {
@@ -200,13 +201,13 @@ static int launch_mega(flexllm_llama* m, int* token, const float* x_in, float* l
         const int w = e ? atoi(e) : 0;
         p.timeline_wg = w >= 0 && w < kMegaWG ? w : 0;
     }
-    static bool lds_opted_in = false;     // the kernels' LDS block exceeds the default 64 KiB per workgroup
-    if (!lds_opted_in) {
+    static std::atomic<bool> lds_opted_in{false};     // the kernels' LDS block exceeds the default 64 KiB per workgroup
+    if (!lds_opted_in.load(std::memory_order_acquire)) {   // idempotent: two threads racing here both set the same attribute
         FX_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(decode_mega_kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
                                    (int)sizeof(MegaLds)));
         FX_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(decode_mega_w4_kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
                                    (int)sizeof(MegaLds)));
-        lds_opted_in = true;
+        lds_opted_in.store(true, std::memory_order_release);
     }
     // An ordinary launch: one workgroup per CU fits by construction (mega_ok checks the CU count), and every barrier
     // and poll in the kernel is bounded, so work of other streams that delays some workgroups costs time, not a hang.
