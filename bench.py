@@ -205,6 +205,9 @@ def main():
     ap.add_argument("--copy-probe", action="store_true",
                     help="only run three 1 GiB device-to-device copies and exit: the transfer of known size that scales "
                          "the FETCH_SIZE / WRITE_SIZE counters")
+    ap.add_argument("--module-probe", action="store_true",
+                    help="only run the single-module legs (decode linear, Hadamard + quantisation, prefill linear stack, "
+                         "prefill attention, W4A4 linears) and exit: the short command the per-kernel counter runs use")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on one GPU only (no collectives, no sharding); use --gpus 1", file=sys.stderr)
@@ -224,6 +227,10 @@ def main():
             fx.check(lib.flexllm_rt_memcpy_d2d(C.c_void_p(dst.ptr), C.c_void_p(src.ptr), C.c_size_t(n), None))
         device_sync()
         print(json.dumps({"copy_probe_bytes": n, "copies": 3}))
+        return
+    if args.module_probe:
+        from flexllm_amd.device import Stream
+        print(json.dumps({"modules": module_legs(fx, lib, synth, ops, Stream(), Event)}))
         return
     cfg = llama.make_config()
     K, W = args.steps, args.warmup
