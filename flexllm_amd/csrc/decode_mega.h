@@ -1,4 +1,5 @@
-// One persistent kernel per decoded token: all 16 layers, the final norm and the fp16 lm_head.
+// One persistent kernel per decoded token: all 16 layers, the final norm and the output head (fp16 tied embedding for
+// the W8A8 model, int4 head for the W4A4 model: the kernel body is a template over the precision).
 //
 // Why: at batch 1 a decode step is ~100 dependent phases of 0.3-4 us of HBM streaming each; as separate
 // kernels every phase pays a launch plus a cold start, and the chip idles between them.  Here 256 workgroups
@@ -9,31 +10,38 @@
 //              4 attention dequant + per-token quant (redundant) -> o_proj rows + residual
 //              5 RMSNorm+quant (redundant) -> gate/up rows + SiLU*up
 //              6 Hadamard R4 + quant (redundant) -> down rows + residual
-//   then       final RMSNorm (redundant) -> lm_head rows, per-workgroup argmax candidates.
-// Where every workgroup needs what every other one produced (3->4, 4->5, 5->6, 6->1) the phases are separated
-// by a grid barrier built from device-scope relaxed atomics (two-level arrive, one broadcast flag).  Where the
-// consumers are few (1->2: a KV head's 32 workgroups need 384 of the 3072 q/k/v outputs; 2->3: the same 32
-// workgroups need each other's chunk statistics) there is no barrier: each value is stored as one 64-bit word
-// with the barrier epoch of its phase in the high half, and the consumers poll the words they need.  A slot is
-// rewritten a layer later, at least three grid barriers after its last reader.  The weights a workgroup needs
-// in the NEXT phase do not depend on the activations, so they are loaded into registers BEFORE waiting on
-// the barrier: HBM keeps streaming while the barrier's round trips are in flight.
+//   then       final RMSNorm (redundant) -> head rows, per-workgroup argmax candidates.
+// Hand-overs between workgroups, by what measured fastest for each:
+//   1->2, 2->3  few consumers (a KV head's 32 workgroups need 384 of the 3072 q/k/v outputs, then each other's chunk
+//               statistics): each value is one 64-bit word with the sequence number of the layer pass in its high
+//               half, and the consumers poll the words they need.
+//   4->5, 6->1  the residual stream, which every workgroup needs in full: tagged words as well (2048 words polled by
+//               every workgroup; a lane that has its values stops loading).  Faster than a grid barrier plus a load.
+//   3->4        int32 atomic adds into the attention accumulators, then a grid barrier (device-scope relaxed atomics,
+//               two-level arrive, one broadcast flag), then coherent loads.
+//   5->6        SiLU(gate)*up (8192 floats): coherent stores into a slice that no other layer pass of the launch uses,
+//               a grid barrier, then ORDINARY loads, which the 32 CUs of an XCD share through L2 (see MegaParams::h).
+// A tagged slot is rewritten a layer later, after at least one exchange that all its readers take part in as
+// producers, i.e. after they have finished with it.  The weights a workgroup needs in the NEXT phase do not depend on
+// the activations, so they are requested BEFORE waiting: HBM keeps streaming while the hand-over is in flight.
 //
 // Wave roles.  Vector-memory results return to a wave in issue order, so a wave with a long weight prefetch in
 // flight cannot see an activation load (or have a store acknowledged) until the prefetch has landed.  The
 // two big matrices are therefore owned by waves 4..7 ("stream waves"): they issue the gate/up rows a full
-// phase ahead (before the o_proj barrier) and the down rows before the gate/up barrier, and while such a
-// prefetch is in flight they touch global memory no further - activations reach them through LDS, and their
-// results leave through LDS.  Waves 0..3 load the activations, own the small q/k/v and o_proj rows and do
-// the global stores of those phases; only they drain their memory counter before arriving at the barrier.
+// phase ahead and the down rows before the gate/up barrier, one slice per phase, each right after the phase's
+// activation loads have landed.  Waves 0..3 own the small q/k/v and o_proj rows and do the global stores; only they
+// drain their memory counter before arriving at a barrier.
 //
-// Memory-model discipline (no cache flushes inside the kernel): every value that crosses workgroups between
-// barriers (x, x2, qkv, h, chunk statistics, attention accumulators) is written and read with device-scope
-// relaxed atomic stores/loads, which bypass the per-XCD L2 for coherence; each thread drains its outstanding
-// stores (s_waitcnt 0) before the workgroup arrives at the barrier.  Weights and the old KV cache are
-// read-only inside a step and use ordinary loads; the new token's K/V row is used from LDS by the workgroup
-// that owns its chunk and written to the cache for later steps (visible after the kernel boundary).
-// Every spin is bounded: on a timeout the kernel sets an error flag and runs to completion.
+// Memory-model discipline: every value that crosses workgroups inside a launch (x, x2, qkv, chunk statistics,
+// attention accumulators, h) is written with device-scope relaxed atomic stores/adds, which are performed at the
+// memory side (past the per-XCD L2), and - h apart - read with device-scope relaxed atomic loads; each thread drains
+// its outstanding stores (s_waitcnt vmcnt(0)) before its workgroup arrives at a barrier.  There is one fence: a
+// device-scope acquire at kernel start, which empties the XCD's L2 of clean lines so that h's ordinary loads cannot
+// hit a line of an earlier launch.  Weights and the old KV cache are read-only inside a step and use ordinary
+// loads; the new token's K/V row is used from LDS by the workgroup that owns its chunk and written to the cache for
+// later steps (that workgroup is also the only one that reads it back within the launch).
+// Every spin is bounded: on a time-out the kernel sets an error flag, every other wait sees the flag within 64
+// polls, and the launch ends after the current token.
 #pragma once
 #include "attn_decode_kernels.h"
 #include "gemv_i8.h"
