@@ -26,16 +26,26 @@ PMC_SUMMARY = os.path.join(ROOT, "profiles", "decode_mega_kernel_llama32_1b_ctx4
 MEGA_SOURCE = os.path.join(ROOT, "flexllm_amd", "csrc", "decode_mega.h")
 
 
+def kernel_source_hash():
+    """SHA-256 (first 16 hex digits) of the persistent kernel's source with // comments and white space removed: the
+    identity of the code that a counter summary was measured on."""
+    import hashlib
+    import re
+    src = open(MEGA_SOURCE, encoding="utf-8").read()
+    src = re.sub(r"//[^\n]*", "", src)
+    src = re.sub(r"\s+", "", src)
+    return hashlib.sha256(src.encode("utf-8")).hexdigest()[:16]
+
+
 def measured_traffic_per_token():
     """HBM bytes per generated token of the persistent decode kernel as the committed counter summary gives them
     (FETCH_SIZE / WRITE_SIZE per dispatch of an 8-token launch, each scaled by the same counter's reading for a 1 GiB
     device copy), or None when that summary was taken on another revision of the kernel: the summary records the
-    SHA-256 of the kernel's source file, and a figure measured on other code is not reported."""
-    import hashlib
+    hash of the kernel's source (kernel_source_hash), and a figure measured on other code is not reported."""
     import re
     try:
         txt = open(PMC_SUMMARY).read()
-        sha = hashlib.sha256(open(MEGA_SOURCE, "rb").read()).hexdigest()[:16]
+        sha = kernel_source_hash()
         m = re.search(r"kernel source sha256\[:16\]: ([0-9a-f]{16})", txt)
         if not m or m.group(1) != sha:
             return None
