@@ -198,8 +198,8 @@ __device__ __forceinline__ float block_sum(float v, float* red) {
 // round half away from zero of x/s with IEEE division, wrapped to 8 bits like (ap_int<8>)round(x/s).
 __device__ __forceinline__ int quant_round(float x, float s) { return (int)roundf(x / s); }
 
-// round(x / s) for a whole vector that shares s, without a division per element.  q~ = x * (1/s) is within
-// 3 * 2^-24 * |q| <= 2.3e-5 of the correctly rounded quotient (|q| <= 127.5), so both round to the same integer
+// round(x / s) for a whole vector that shares s, without a division per element.  q~ = x * rcp(s) is within
+// 4 * 2^-24 * |q| <= 3.1e-5 of the correctly rounded quotient (|q| <= 127.5), so both round to the same integer
 // unless q~ lies within 1e-4 of a tie (k + 0.5); `near_tie` collects those cases and the caller redoes them
 // with the exact expression.  Valid while 1/s is a normal number (`quant_fast_ok`).
 __device__ __forceinline__ bool quant_fast_ok(float s) { return s >= 0x1p-100f && s <= 0x1p100f; }
@@ -216,7 +216,7 @@ __device__ __forceinline__ void quant_vector(const float (&v)[N], float s, int (
         for (int i = 0; i < N; i++) n[i] = quant_round(v[i], s);
         return;
     }
-    const float rs = 1.0f / s;
+    const float rs = __builtin_amdgcn_rcpf(s);       // 1 ulp: the product below is then within 4 * 2^-24 * |q| of the quotient
     constexpr int G = N % 4 == 0 ? 4 : N;            // the exact path is taken per group: rare (about 2e-4 per element)
 #pragma unroll
     for (int g = 0; g < N / G; g++) {
@@ -237,6 +237,18 @@ __device__ __forceinline__ uint32_t pack4_i8(int a, int b, int c, int d) {
 // symmetric scale from a row's absmax: absmax/127, 0 -> 1
 __device__ __forceinline__ float sym_scale(float absmax, float scale_base) {
     float s = absmax / scale_base;
+    return s == 0.0f ? 1.0f : s;
+}
+// The same for a maximum that every lane of the wave holds (the result of a block-wide reduction), int8 range: the
+// division by 127 goes through the correctly rounded reciprocal and one exact residual step (`div_fast`), which gives
+// the IEEE quotient for every float32 in the guarded range (all 2^23 significands checked against the division on the
+// CPU; the sequence does not depend on the exponent while nothing under- or overflows), behind a scalar branch so that
+// the long division sequence is not issued as well.
+__device__ __forceinline__ float sym_scale_127_uniform(float absmax) {
+    constexpr float r127 = 1.0f / 127.0f;            // correctly rounded at compile time
+    float s;
+    if (__builtin_amdgcn_readfirstlane((int)(absmax >= 0x1p-60f && absmax <= 0x1p100f))) s = div_fast(absmax, 127.0f, r127);
+    else s = absmax / 127.0f;
     return s == 0.0f ? 1.0f : s;
 }
 

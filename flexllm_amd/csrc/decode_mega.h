@@ -304,7 +304,7 @@ __device__ __forceinline__ float norm_quant_2048(float (&v)[4], const float4& g,
     float amax = fmaxf(fmaxf(fabsf(v[0]), fabsf(v[1])), fmaxf(fabsf(v[2]), fabsf(v[3])));
     if (do_norm) amax = mega_block_max_h(amax, L.red_max, NoHook());
     else amax = mega_block_max_h(amax, L.red_max, hook);
-    const float sc = sym_scale(amax, 127.0f);
+    const float sc = sym_scale_127_uniform(amax);
     int n[4];
     quant_vector(v, sc, n);
     reinterpret_cast<uint32_t*>(L.xq)[t] = pack4_i8(n[0], n[1], n[2], n[3]);
@@ -1081,7 +1081,7 @@ __device__ __forceinline__ void decode_mega_body(const MegaParams& p) {
                 for (int q = 0; q < 4; q++) reinterpret_cast<uint16_t*>(L.xq)[q * 512 + t] = w16[q];   // nibble q*2048 + 4t + e
             } else {
                 amax = mega_block_max_h(amax, L.red_max, NoHook());
-                sx = sym_scale(amax, 127.0f);
+                sx = sym_scale_127_uniform(amax);
                 if (l == 1) fine();
                 int n16[16];
                 quant_vector(b2, sx, n16);

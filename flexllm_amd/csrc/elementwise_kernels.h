@@ -31,7 +31,7 @@ __global__ __launch_bounds__(kBlock) void quant_sym_kernel(const float* __restri
         }
     }
     amax = block_max<kNW>(amax, red);
-    const float sc = sym_scale(amax, 127.0f);
+    const float sc = sym_scale_127_uniform(amax);
     if (threadIdx.x == 0) s[row] = sc;
     uint32_t* qr = reinterpret_cast<uint32_t*>(q + (size_t)row * dim);
 #pragma unroll
@@ -123,7 +123,7 @@ __global__ __launch_bounds__(BLOCK) void rmsnorm_kernel(const float* __restrict_
     }
     if constexpr (QUANT) {
         amax = block_max<BLOCK / kWave>(amax, red);
-        const float sc = sym_scale(amax, 127.0f);
+        const float sc = sym_scale_127_uniform(amax);
         if (threadIdx.x == 0) s[row] = sc;
         uint32_t* qr = reinterpret_cast<uint32_t*>(q + (size_t)row * dim);
 #pragma unroll
@@ -215,7 +215,7 @@ static __global__ __launch_bounds__(kBlock) void head_quant_kernel(const float* 
     if (lane < nvec) v = xr[lane];
     float amax = fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w)));
     amax = wave_max(amax);
-    const float sc = sym_scale(amax, 127.0f);
+    const float sc = sym_scale_127_uniform(amax);
     if (lane == 0) s[row] = sc;
     if (lane < nvec)
         reinterpret_cast<uint32_t*>(q + (size_t)row * dim)[lane] =

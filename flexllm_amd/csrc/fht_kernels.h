@@ -161,7 +161,7 @@ __global__ __launch_bounds__(kFhtBlock) void fht_kernel(const float* __restrict_
         for (int r = 0; r < NR; r++) yr[r * 256 + t] = b[r];
     } else {
         amax = block_max<kFhtBlock / kWave>(amax, red);   // its leading barrier also retires the lds reads above
-        const float sc = sym_scale(amax, 127.0f);
+        const float sc = sym_scale_127_uniform(amax);
         if (t == 0) s[row] = sc;
         int8_t* lds_q = reinterpret_cast<int8_t*>(lds);
         {

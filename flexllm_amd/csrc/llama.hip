@@ -84,7 +84,7 @@ static __global__ __launch_bounds__(256) void dec_out_quant_kernel(const int32_t
         }
     }
     amax = block_max<4>(amax, red);
-    const float sc = sym_scale(amax, 127.0f);
+    const float sc = sym_scale_127_uniform(amax);
     if (threadIdx.x == 0) s[0] = sc;
 #pragma unroll
     for (int i = 0; i < VPT; i++) {
