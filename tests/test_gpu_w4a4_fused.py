@@ -184,3 +184,32 @@ def test_w4a4_16_layers_teacher_forced_at_position_4095_and_the_full_head():
         x = y_ref                                                   # teacher forcing
     errs = np.array(errs)
     assert errs.max() < 5e-2 and (errs > 1e-4).sum() <= 4 and np.median(errs) < 1e-5
+
+
+def test_w4a4_sampling_inside_the_kernel(small4):
+    """Ten tokens drawn with top-5 sampling inside the persistent kernel's W4A4 instance, host-supplied uniform numbers.
+    Each drawn id is what the oracle's sampler gives on the logits of that very step, recomputed with decode_hidden from
+    the previous id at the same position (bit for bit the same forward pass): this pins the per-workgroup candidate
+    selection over the int4 head's logits, the indexing of the uniform numbers and the feedback of the ids."""
+    fx, cfg, model, oracle, w = small4
+    L = cfg["layers"]
+    zero = np.zeros((L, cfg["max_pos"], cfg["kv_hidden"]), np.int8)
+    model.load_caches_token_major(zero, zero)
+    steps, k, tok0 = 10, 5, 29
+    rands = np.random.default_rng(8).uniform(0, 1, steps).astype(np.float32)
+    tok = fx.to_device(np.array([tok0], np.int32)); out = fx.zeros((steps,), np.int32)
+    model.decode_sample(tok, 0, steps, fx.to_device(rands), k, out)
+    model.check()
+    got = out.numpy().tolist()
+    model.load_caches_token_major(zero, zero)
+    ranks = []
+    for i in range(steps):
+        prev = tok0 if i == 0 else got[i - 1]
+        x = fx.ops.embed_f16(model._embed, fx.to_device(np.array([prev], np.int32)))
+        _, logits = model.decode_hidden(x, i, want_logits=True)
+        t_ref, idx, val, prob = oracle.sample_topk(logits.numpy(), k, float(rands[i]), 8)
+        assert np.abs(np.cumsum(prob.astype(np.float64)) - rands[i]).min() > 1e-5
+        assert got[i] == t_ref, "step %d" % i
+        ranks.append(int(np.nonzero(idx == t_ref)[0][0]))
+    assert len(set(ranks)) >= 2, ranks
+    assert int(tok.numpy()[0]) == got[-1]
