@@ -60,14 +60,6 @@ constexpr int kMegaSpinLimit = 1 << 20;   // polls of ~1 us each: a wait that ha
 constexpr int kMegaErrPeriod = 64;         // a spinning thread looks at the error flag every so many polls
 constexpr int kMegaMaxSteps = 64;  // tokens per launch in greedy mode (bounds the run time of one launch)
 
-// Layer table of the W4A4 variant: the same matrices with two 4-bit weights per byte along K (rows of K/2 bytes), and per
-// output row the sum of its dequantised weights, which the asymmetric activations' zero point multiplies.
-struct LayerW4 {
-    int8_t *wqkv, *wo, *wgu, *wd;
-    float *sqkv, *so, *sgu, *sd;
-    float *mqkv, *mo, *mgu, *md;
-};
-
 struct MegaParams {
     const void* layers;            // device array [layers] of LayerW (W8A8) or LayerW4 (W4A4)
     const uint8_t* head_w4;        // W4A4: int4 output head, nibble-packed [vocab][hidden/2], with per-row scale and row sum

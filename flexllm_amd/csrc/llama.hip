@@ -624,7 +624,6 @@ int flexllm_llama_decode_sample(flexllm_llama* m, int* token_io, int pos0, int s
 int flexllm_llama_generate(flexllm_llama* m, const int* prompt, int n_prompt, int steps, const float* rands, int top_k,
                            int* tokens_out, void* stream) {
     FX_REQUIRE(m && prompt && tokens_out, "llama_generate: null pointer");
-    FX_REQUIRE(!m->w4, "llama_generate: a W4A4 model has no fused prefill (its prefill runs stage by stage over the module entry points)");
     FX_REQUIRE(n_prompt >= 1 && steps >= 0 && n_prompt - 1 + steps <= m->cfg.max_pos,
                "llama_generate: prompt of %d tokens + %d steps exceed max_pos=%d", n_prompt, steps, m->cfg.max_pos);
     FX_REQUIRE(top_k == 0 || rands, "llama_generate: sampling (top_k=%d) needs the uniform numbers", top_k);
@@ -644,8 +643,11 @@ int flexllm_llama_generate(flexllm_llama* m, const int* prompt, int n_prompt, in
         FX_LAUNCH_CHECK();
         // rows s..rows-1 are zero padding: they write cache rows at positions >= s, which the decode steps below
         // overwrite one by one before any of them is read
-        int rc = llama_prefill_run(c, m->layers.data(), m->gamma, m->q_s, m->k_s, m->v_s, m->a_s, m->rope_sin, m->rope_cos,
-                                   m->k_cache, m->v_cache, m->cache_layer_bytes, &m->pws, m->gen_x, rows, nullptr, st);
+        int rc = m->w4 ? llama_prefill_run_w4a4(c, m->layers.data(), m->layers4.data(), m->gamma, m->q_s, m->k_s, m->v_s, m->a_s,
+                                                m->rope_sin, m->rope_cos, m->k_cache, m->v_cache, m->cache_layer_bytes,
+                                                &m->pws, m->gen_x, rows, nullptr, st)
+                       : llama_prefill_run(c, m->layers.data(), m->gamma, m->q_s, m->k_s, m->v_s, m->a_s, m->rope_sin, m->rope_cos,
+                                           m->k_cache, m->v_cache, m->cache_layer_bytes, &m->pws, m->gen_x, rows, nullptr, st);
         if (rc) return rc;
     }
     copy_int_kernel<<<1, 1, 0, st>>>(prompt + s, m->gen_token);
@@ -657,7 +659,10 @@ int flexllm_llama_generate(flexllm_llama* m, const int* prompt, int n_prompt, in
 
 int flexllm_llama_prefill_hidden(flexllm_llama* m, const float* x_in, int s, float* hidden_out, void* stream) {
     FX_REQUIRE(m && x_in, "llama_prefill_hidden: null pointer");
-    FX_REQUIRE(!m->w4, "llama_prefill_hidden: a W4A4 model has no fused prefill (its prefill runs stage by stage over the module entry points)");
+    if (m->w4)
+        return llama_prefill_run_w4a4(m->cfg, m->layers.data(), m->layers4.data(), m->gamma, m->q_s, m->k_s, m->v_s, m->a_s,
+                                      m->rope_sin, m->rope_cos, m->k_cache, m->v_cache, m->cache_layer_bytes, &m->pws, x_in, s,
+                                      hidden_out, as_stream(stream));
     return llama_prefill_run(m->cfg, m->layers.data(), m->gamma, m->q_s, m->k_s, m->v_s, m->a_s, m->rope_sin, m->rope_cos,
                              m->k_cache, m->v_cache, m->cache_layer_bytes, &m->pws, x_in, s, hidden_out, as_stream(stream));
 }

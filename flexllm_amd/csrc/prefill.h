@@ -9,8 +9,17 @@ struct LayerW {
     float *sqkv, *so, *sgu, *sd;
 };
 
+// Layer table of the W4A4 model: the same matrices with two 4-bit weights per byte along K (rows of K/2 bytes), and per
+// output row the sum of its dequantised weights, which the asymmetric activations' zero point multiplies.
+struct LayerW4 {
+    int8_t *wqkv, *wo, *wgu, *wd;
+    float *sqkv, *so, *sgu, *sd;
+    float *mqkv, *mo, *mgu, *md;
+};
+
 struct PrefillWorkspace {
     int tokens = 0;
+    bool w4 = false;        // sized for the W4A4 graph (one more fp32 scratch array)
     void* base = nullptr;
 };
 
@@ -27,5 +36,10 @@ int llama_prefill_run(const flexllm_llama_config& cfg, const LayerW* layers, con
                       const float* k_s, const float* v_s, const float* a_s, const float* rope_sin, const float* rope_cos,
                       int8_t* k_cache, int8_t* v_cache, size_t cache_layer_bytes, PrefillWorkspace* ws, const float* x_in,
                       int s, float* hidden_out, hipStream_t st);
+
+int llama_prefill_run_w4a4(const flexllm_llama_config& cfg, const LayerW* layers, const LayerW4* sums, const float* gamma,
+                           const float* q_s, const float* k_s, const float* v_s, const float* a_s, const float* rope_sin,
+                           const float* rope_cos, int8_t* k_cache, int8_t* v_cache, size_t cache_layer_bytes,
+                           PrefillWorkspace* ws, const float* x_in, int s, float* hidden_out, hipStream_t st);
 
 }  // namespace fx

@@ -12,21 +12,24 @@ struct PrefillBuffers {
     float *x, *x2, *qkv, *att, *gu;
     int8_t *xq, *q8;
     float* xs;
+    float *xb, *fh;         // W4A4 only: zero points per token; fp32 scratch [s][inter] (normalised rows, transformed rows)
 };
 
-static int prefill_workspace_get(PrefillWorkspace* ws, const flexllm_llama_config& c, int s, PrefillBuffers* b) {
+static int prefill_workspace_get(PrefillWorkspace* ws, const flexllm_llama_config& c, int s, PrefillBuffers* b, bool w4 = false) {
     const size_t H = c.hidden, KV = c.kv_hidden, I = c.inter;
     auto up = [](size_t v) { return (v + 255) & ~(size_t)255; };
     const size_t sz_x = up(sizeof(float) * s * H), sz_qkv = up(sizeof(float) * s * (H + 2 * KV));
     const size_t sz_gu = up(sizeof(float) * s * 2 * I), sz_xq = up((size_t)s * I), sz_q8 = up((size_t)s * H);
     const size_t sz_xs = up(sizeof(float) * s);
-    const size_t total = 3 * sz_x + sz_qkv + sz_gu + sz_xq + sz_q8 + sz_xs;
-    if (ws->tokens < s) {
+    const size_t sz_fh = w4 ? up(sizeof(float) * s * I) : 0;
+    const size_t total = 3 * sz_x + sz_qkv + sz_gu + sz_xq + sz_q8 + 2 * sz_xs + sz_fh;
+    if (ws->tokens < s || (w4 && !ws->w4)) {
         FX_HIP(hipDeviceSynchronize());
         prefill_workspace_free(ws);
         hipError_t e = hipMalloc(&ws->base, total);
         if (e != hipSuccess) { set_error("prefill workspace hipMalloc(%zu) failed: %s", total, hipGetErrorString(e)); return FLEXLLM_ENOMEM; }
         ws->tokens = s;
+        ws->w4 = w4;
     }
     char* p = (char*)ws->base;
     b->x = (float*)p; p += sz_x;
@@ -36,7 +39,9 @@ static int prefill_workspace_get(PrefillWorkspace* ws, const flexllm_llama_confi
     b->gu = (float*)p; p += sz_gu;
     b->xq = (int8_t*)p; p += sz_xq;
     b->q8 = (int8_t*)p; p += sz_q8;
-    b->xs = (float*)p;
+    b->xs = (float*)p; p += sz_xs;
+    b->xb = (float*)p; p += sz_xs;
+    b->fh = w4 ? (float*)p : nullptr;
     return FLEXLLM_OK;
 }
 
@@ -77,6 +82,55 @@ int llama_prefill_run(const flexllm_llama_config& c, const LayerW* layers, const
         if ((rc = launch_gemm_swiglu(b.xq, w.wgu, b.xs, w.sgu, b.gu, s, H, 2 * I, st))) return rc;     // b.gu = SiLU(gate)*up [s][I]
         fht_kernel<13, true, false><<<s, kFhtBlock, 0, st>>>(b.gu, nullptr, b.xq, b.xs, c.fht_scale);
         if ((rc = launch_gemm<kGemmDequant>(b.xq, w.wd, nullptr, b.xs, w.sd, b.x2, b.x, s, I, H, st))) return rc;
+    }
+    FX_LAUNCH_CHECK();
+    if (hidden_out) FX_HIP(hipMemcpyAsync(hidden_out, b.x, sizeof(float) * (size_t)s * H, hipMemcpyDeviceToDevice, st));
+    return FLEXLLM_OK;
+}
+
+// The W4A4 configuration (asymmetric uint4 activations x int4 weights, the stage order of SpinQuant_Prefilling.h:807-1050)
+// over the same kernels the module entry points use: the 4-bit values are held one per byte (layers: the matrices as
+// flexllm_llama_create keeps them, sums: the row sums of the dequantised weights) and multiplied on the int8 direct-load
+// MFMA kernel with the asymmetric dequantisation in its epilogue; RoPE, static quantisation and the cache stores run as
+// one kernel per token row, SiLU(gate)*up is applied by the Hadamard kernel as it loads the interleaved gate/up columns.
+int llama_prefill_run_w4a4(const flexllm_llama_config& c, const LayerW* layers, const LayerW4* sums, const float* gamma,
+                           const float* q_s_all, const float* k_s_all, const float* v_s_all, const float* a_s_all,
+                           const float* rope_sin, const float* rope_cos, int8_t* k_cache, int8_t* v_cache,
+                           size_t cache_layer_bytes, PrefillWorkspace* ws, const float* x_in, int s, float* hidden_out,
+                           hipStream_t st) {
+    FX_REQUIRE(s > 0 && s % kPfTile == 0 && s <= c.max_pos, "prefill: s=%d must be a positive multiple of 32, <= max_pos=%d", s, c.max_pos);
+    FX_REQUIRE(c.hidden == 2048 && c.inter == 8192, "prefill (W4A4): hidden=%d inter=%d (instantiated for 2048/8192)", c.hidden, c.inter);
+    PrefillBuffers b;
+    int rc = prefill_workspace_get(ws, c, s, &b, true);
+    if (rc) return rc;
+    const int H = c.hidden, KV = c.kv_hidden, I = c.inter;
+    uint8_t* xq = reinterpret_cast<uint8_t*>(b.xq);
+    FX_HIP(hipMemcpyAsync(b.x, x_in, sizeof(float) * (size_t)s * H, hipMemcpyDeviceToDevice, st));
+    for (int l = 0; l < c.layers; l++) {
+        const LayerW& w = layers[l];
+        const LayerW4& m4 = sums[l];
+        const float* q_s = q_s_all + (size_t)l * c.q_heads;
+        const float* k_s = k_s_all + (size_t)l * c.kv_heads;
+        const float* v_s = v_s_all + (size_t)l * c.kv_heads;
+        const float* a_s = a_s_all + (size_t)l * c.q_heads;
+        int8_t* kc = k_cache + (size_t)l * cache_layer_bytes;
+        int8_t* vc = v_cache + (size_t)l * cache_layer_bytes;
+        // attention block
+        rmsnorm_kernel<1, false, 512><<<s, 512, 0, st>>>(b.x, gamma + (size_t)(2 * l) * H, b.fh, nullptr, nullptr, H, c.eps);
+        quant_asym_kernel<2><<<s, kBlock, 0, st>>>(b.fh, xq, b.xs, b.xb, H, 15.0f, 15u);
+        if ((rc = launch_gemm_asym(b.xq, w.wqkv, b.xs, b.xb, w.sqkv, m4.mqkv, nullptr, b.qkv, s, H, H + 2 * KV, st))) return rc;
+        qkv_post_kernel<<<s, 256, 0, st>>>(b.qkv, rope_sin, rope_cos, q_s, k_s, v_s, b.q8, kc, vc, nullptr, 0, c.q_heads,
+                                           c.kv_heads, c.max_pos);
+        if ((rc = mha_prefill_launch(b.q8, kc, vc, q_s, k_s, v_s, a_s, b.att, nullptr, s, c.q_heads, c.kv_heads, c.max_pos, st))) return rc;
+        quant_asym_kernel<2><<<s, kBlock, 0, st>>>(b.att, xq, b.xs, b.xb, H, 15.0f, 15u);
+        if ((rc = launch_gemm_asym(b.xq, w.wo, b.xs, b.xb, w.so, m4.mo, b.x, b.x2, s, H, H, st))) return rc;
+        // feed-forward block
+        rmsnorm_kernel<1, false, 512><<<s, 512, 0, st>>>(b.x2, gamma + (size_t)(2 * l + 1) * H, b.fh, nullptr, nullptr, H, c.eps);
+        quant_asym_kernel<2><<<s, kBlock, 0, st>>>(b.fh, xq, b.xs, b.xb, H, 15.0f, 15u);
+        if ((rc = launch_gemm_asym(b.xq, w.wgu, b.xs, b.xb, w.sgu, m4.mgu, nullptr, b.gu, s, H, 2 * I, st))) return rc;   // interleaved (gate, up)
+        fht_kernel<13, false, true><<<s, kFhtBlock, 0, st>>>(b.gu, b.fh, nullptr, nullptr, c.fht_scale);
+        quant_asym_kernel<8><<<s, kBlock, 0, st>>>(b.fh, xq, b.xs, b.xb, I, 15.0f, 15u);
+        if ((rc = launch_gemm_asym(b.xq, w.wd, b.xs, b.xb, w.sd, m4.md, b.x2, b.x, s, I, H, st))) return rc;
     }
     FX_LAUNCH_CHECK();
     if (hidden_out) FX_HIP(hipMemcpyAsync(hidden_out, b.x, sizeof(float) * (size_t)s * H, hipMemcpyDeviceToDevice, st));

@@ -343,8 +343,10 @@ int flexllm_llama_create(flexllm_llama** out, const flexllm_llama_config* cfg, c
  * the dequantised weights (the generated headers' w_<proj>_sum), which the activations' zero point multiplies; the
  * head is int4 [vocab][hidden] one value per byte with per-row scale and row sum.  The library packs the matrices two
  * values per byte.  Decoding (flexllm_llama_decode_hidden / _decode_greedy / _decode_sample) runs in the persistent
- * kernel only, which then streams half the weight bytes per token; prefill of this configuration runs stage by stage
- * over the module entry points (flexllm_amd/llama_w4a4.py), and the entry points that prefill return an error. */
+ * kernel only, which then streams half the weight bytes per token.  flexllm_llama_prefill_hidden and
+ * flexllm_llama_generate run the configuration's prefill graph (SpinQuant_Prefilling.h:807-1050): per-token asymmetric
+ * uint4 quantisation, the 4-bit values multiplied one per byte on the int8 MFMA kernel with zero point x row sum in its
+ * epilogue, RoPE + static quantisation + cache stores, int8 attention, SiLU(gate)*up and the Hadamard transform. */
 typedef struct {
     flexllm_llama_weights base;
     const float* const* sumq; const float* const* sumk; const float* const* sumv; const float* const* sumo;
