@@ -760,9 +760,14 @@ __device__ __forceinline__ void decode_mega_body(const MegaParams& p) {
                 __syncthreads();
                 if (blk == 0 && part == 0) {
 #pragma unroll
-                    for (int g = 0; g < GROUP; g++)
-                        __hip_atomic_fetch_add(&p.o_acc[(a_h * GROUP + g) * kHd + d], tot[g] + L.osum[g][d], __ATOMIC_RELAXED,
+                    for (int i = 0; i < GROUP; i++) {
+                        // the 32 chunks of a KV head add into the same 256 words: each starts at another query head,
+                        // so that they do not all queue on the same 64-byte run at once
+                        const int g = (i + a_c) & (GROUP - 1);
+                        const int mine = g == 0 ? tot[0] : g == 1 ? tot[1] : g == 2 ? tot[2] : tot[3];
+                        __hip_atomic_fetch_add(&p.o_acc[(a_h * GROUP + g) * kHd + d], mine + L.osum[g][d], __ATOMIC_RELAXED,
                                                __HIP_MEMORY_SCOPE_AGENT);
+                    }
                 }
             } else {
                 gu_slice(2);
