@@ -71,7 +71,7 @@ def test_mha_prefill_dyn_per_channel_v_scale(fx, oracle):
 
 @pytest.mark.parametrize("length,qh,kvh", [(1, 8, 2), (5, 4, 4), (127, 32, 8), (129, 32, 8), (1000, 8, 2), (4096, 32, 8)])
 def test_mha_decode_dyn_vs_oracle(fx, oracle, length, qh, kvh):
-    """One query against `length` cached positions (4096: BASELINE's decode case), cache tail poisoned."""
+    """One query against `length` cached positions (4096: the benchmark's decode case), cache tail poisoned."""
     r = np.random.default_rng(200 + length)
     max_pos = ((length + 63) // 64) * 64 + 64
     q8 = r.integers(-127, 128, (qh, 64)).astype(np.int8); q8[:, 0] = 127
