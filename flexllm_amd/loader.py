@@ -13,8 +13,13 @@ What the reference's testbench reads (SpinQuant_Llama_32_1B/SpinQuant_Prefilling
 
 The reference tree ships none of these files, so the header syntax is taken from how the arrays are indexed: any C
 initialiser `name[d0][d1] = { ... }` (or one-dimensional) is accepted, numbers may carry an `f` suffix.  The rotary
-table (`parameters/RoPE_sin_cos.h`) is regenerated from the formula, and the output head is the embedding matrix
-in fp16 (tied), so `lm_head.bin` / `w_lm_head_lm_head.h` are not read.
+table (`parameters/RoPE_sin_cos.h`) is regenerated from the formula.  For the W8A8 model the output head is the
+embedding matrix in fp16 (tied) and `lm_head.bin` / `w_lm_head_lm_head.h` are not read; with w4a4=True the loader also
+returns the row sums (`sum<p>`) and the int4 output head (`lm_head.bin`, row-major int8 `[vocab][hidden]` holding -8..7,
+with `w_lm_head_lm_head_s[vocab]` and `w_lm_head_lm_head_sum[vocab]`, SpinQuant_Prefilling_Decoding_mem_opt_tb.cpp:
+187-192, 442, 655-660, 716-719): the dictionary `llama.Llama` turns into the W4A4 model.  A row sum is the sum of the
+row's DEQUANTISED weights (the zero point of the activations multiplies it directly, Modules/quant.h:147-152; the
+linear testbench accumulates qval * scale, Linear_Layer_Decoding_tb.cpp:171-188).
 
 `save_reference_parameters` writes the same files from a host weight dictionary, e.g. to hand a synthetic model to
 the reference's own testbench.
@@ -75,9 +80,10 @@ def _read_header_array(param_dir, fname, name, shape):
     return np.ascontiguousarray(arr.reshape(shape))
 
 
-def load_reference_parameters(param_dir, cfg, device=True):
+def load_reference_parameters(param_dir, cfg, device=True, w4a4=False):
     """Weight dictionary for `llama.Llama` from a reference `parameters/` directory.  device=False returns numpy
-    arrays (the layout of `llama.synth_weights(device=False)`)."""
+    arrays (the layout of `llama.synth_weights(device=False)`).  w4a4=True adds the row sums and the int4 output head
+    (the layout of `llama.synth_weights_w4a4`)."""
     L, H = cfg["layers"], cfg["hidden"]
     w = {}
     for key, stem in _PROJ_FILES.items():
@@ -93,6 +99,12 @@ def load_reference_parameters(param_dir, cfg, device=True):
         w["w" + key] = mats
         s = _read_header_array(param_dir, "w_%s_s_sum.h" % stem, "w_%s_s" % stem, (L, n))
         w["s" + key] = [np.ascontiguousarray(s[l]) for l in range(L)]
+        if w4a4:
+            sm = _read_header_array(param_dir, "w_%s_s_sum.h" % stem, "w_%s_sum" % stem, (L, n))
+            w["sum" + key] = [np.ascontiguousarray(sm[l]) for l in range(L)]
+            for l in range(L):
+                if mats[l].min() < -8 or mats[l].max() > 7:
+                    raise ParameterError("%s_L%02d.bin holds values outside -8..7: not an int4 export" % (stem, l))
     w["gamma"] = _read_header_array(param_dir, "w_rmsnorm.h", "RMSNorm_weight", (2 * L + 1, H))
     for key, (name, heads) in _STATIC.items():
         w[key] = _read_header_array(param_dir, name + ".h", name, (L, cfg[heads]))
@@ -104,6 +116,17 @@ def load_reference_parameters(param_dir, cfg, device=True):
     embed = np.memmap(path, dtype=np.float32, mode="r", shape=(cfg["vocab"], H))
     w["embed"] = np.asarray(embed).astype(np.float16).view(np.uint16)      # tied fp16 table (round to nearest even)
     w["rope_sin"], w["rope_cos"] = rope_table(cfg["max_pos"], cfg["head_dim"])
+    if w4a4:
+        path = os.path.join(param_dir, "lm_head.bin")
+        if not os.path.exists(path):
+            raise ParameterError("missing %s" % path)
+        if os.path.getsize(path) != cfg["vocab"] * H:
+            raise ParameterError("%s: %d bytes, expected %d x %d" % (path, os.path.getsize(path), cfg["vocab"], H))
+        w["head_w"] = np.fromfile(path, dtype=np.int8).reshape(cfg["vocab"], H)
+        if w["head_w"].min() < -8 or w["head_w"].max() > 7:
+            raise ParameterError("lm_head.bin holds values outside -8..7: not an int4 export")
+        w["head_s"] = _read_header_array(param_dir, "w_lm_head_lm_head.h", "w_lm_head_lm_head_s", (cfg["vocab"],))
+        w["head_sum"] = _read_header_array(param_dir, "w_lm_head_lm_head.h", "w_lm_head_lm_head_sum", (cfg["vocab"],))
     if not device:
         return w
     dev = {}
@@ -134,14 +157,18 @@ def _write_header(path, arrays):
 
 
 def save_reference_parameters(param_dir, cfg, w):
-    """Writes host weights `w` (layout of `llama.synth_weights(device=False)`) as a reference `parameters/` directory."""
+    """Writes host weights `w` (layout of `llama.synth_weights(device=False)`, or of `llama.synth_weights_w4a4` with its
+    row sums and int4 head) as a reference `parameters/` directory."""
     os.makedirs(param_dir, exist_ok=True)
     L = cfg["layers"]
     for key, stem in _PROJ_FILES.items():
         for l in range(L):
             np.ascontiguousarray(w["w" + key][l], dtype=np.int8).tofile(os.path.join(param_dir, "%s_L%02d.bin" % (stem, l)))
         s = np.stack([np.asarray(w["s" + key][l], dtype=np.float32) for l in range(L)])
-        sums = np.stack([np.asarray(w["w" + key][l], dtype=np.int64).sum(1).astype(np.float32) for l in range(L)])
+        if "sum" + key in w:
+            sums = np.stack([np.asarray(w["sum" + key][l], dtype=np.float32) for l in range(L)])
+        else:                                      # sum of the dequantised row: integer row sum times the row's scale
+            sums = np.stack([np.asarray(w["w" + key][l], dtype=np.int64).sum(1).astype(np.float32) for l in range(L)]) * s
         _write_header(os.path.join(param_dir, "w_%s_s_sum.h" % stem), [("w_%s_s" % stem, s), ("w_%s_sum" % stem, sums)])
     _write_header(os.path.join(param_dir, "w_rmsnorm.h"), [("RMSNorm_weight", w["gamma"])])
     for key, (name, _) in _STATIC.items():
@@ -149,3 +176,7 @@ def save_reference_parameters(param_dir, cfg, w):
     embed = np.asarray(w["embed"])
     embed = embed.view(np.float16) if embed.dtype == np.uint16 else embed
     embed.astype(np.float32).tofile(os.path.join(param_dir, "model_embed_tokens_fp32.bin"))
+    if "head_w" in w:
+        np.ascontiguousarray(w["head_w"], dtype=np.int8).tofile(os.path.join(param_dir, "lm_head.bin"))
+        _write_header(os.path.join(param_dir, "w_lm_head_lm_head.h"),
+                      [("w_lm_head_lm_head_s", np.asarray(w["head_s"], np.float32)), ("w_lm_head_lm_head_sum", np.asarray(w["head_sum"], np.float32))])

@@ -41,7 +41,29 @@ def test_round_trip_small_model(tmp_path):
     assert np.array_equal(r["embed"], w["embed"])          # fp16 -> fp32 file -> fp16 is the identity
     # the row sums the asymmetric 4-bit path reads are written as well
     sums = loader.parse_c_array(open(d + "/w_down_proj_s_sum.h").read(), "w_down_proj_sum")
-    assert np.array_equal(sums[1], w["wd"][1].astype(np.int64).sum(1).astype(np.float32))
+    # (the sum of the DEQUANTISED row: integer row sum times the row's scale)
+    assert np.array_equal(sums[1], w["wd"][1].astype(np.int64).sum(1).astype(np.float32) * w["sd"][1])
+
+
+def test_round_trip_w4a4_model(tmp_path):
+    """The W4A4 dictionary (int4 values one per byte, row sums, int4 output head) through the reference's files."""
+    cfg = llama.make_config(**SMALL)
+    w = llama.synth_weights_w4a4(cfg, seed=8, device=False)
+    d = str(tmp_path / "parameters")
+    loader.save_reference_parameters(d, cfg, w)
+    r = loader.load_reference_parameters(d, cfg, device=False, w4a4=True)
+    for key in [p + q for p in ("w", "s", "sum") for q in "qkvogud"]:
+        for l in range(cfg["layers"]):
+            assert r[key][l].dtype == w[key][l].dtype and np.array_equal(r[key][l], w[key][l]), (key, l)
+    for key in ("head_w", "head_s", "head_sum", "gamma", "q_s", "a_s"):
+        assert r[key].dtype == w[key].dtype and np.array_equal(r[key], w[key]), key
+    assert w["wq"][0].min() >= -8 and w["wq"][0].max() <= 7
+    # an int8 export is refused where int4 values are expected
+    w8 = llama.synth_weights(cfg, seed=7, device=False)
+    d8 = str(tmp_path / "parameters8")
+    loader.save_reference_parameters(d8, cfg, w8)
+    with pytest.raises(loader.ParameterError, match="-8..7"):
+        loader.load_reference_parameters(d8, cfg, device=False, w4a4=True)
 
 
 def test_missing_and_misshapen_files(tmp_path):
