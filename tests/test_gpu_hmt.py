@@ -102,3 +102,45 @@ def test_segment_loop_vs_oracle_on_the_real_layer_stack(fx, oracle, n_tok, seg_l
     stored = min(n_seg - 1, mem_num)                                            # the last segment stores no memory
     assert plug.mmem.numpy()[:stored].any(axis=1).all() and not plug.mmem.numpy()[stored:].any()
     model.close()
+
+
+def test_segment_loop_on_the_w4a4_layer_stack(fx, oracle):
+    """The plug-in around the W4A4 model (the reference's HMT unit wraps its 4-bit stack, HMT_SpinQuant_Unit.h): three
+    segments, oracle backbone = the oracle's W4A4 layer.  One 4-bit activation step is 1/15 of a row's range, so a
+    rounding tie that falls the other way moves a token by a few percent, and the plug-in is recurrent: the first
+    segment's rows are compared token by token (most agree to fp32 rounding), the later quantities within the bound of
+    such steps."""
+    from flexllm_amd import hmt, llama
+    cfg = llama.make_config(layers=1, vocab=512, max_pos=256)
+    host_w = llama.synth_weights_w4a4(cfg, seed=5, device=False)
+    dev_w = {k: ([fx.to_device(a) for a in v] if isinstance(v, list) else
+                 fx.to_device(v.view(np.float16) if k == "embed" else v)) for k, v in host_w.items()}
+    model = llama.Llama(cfg, dev_w)
+    assert model.w4a4
+    hidden = cfg["hidden"]
+    r = np.random.default_rng(78)
+    n_tok, seg_len, sum_len, rec, mem_num = 60, 24, 12, 4, 4
+    emb = r.standard_normal((n_tok, hidden)).astype(np.float32)
+    t_embed = r.standard_normal(hidden).astype(np.float32)
+    wq = (r.standard_normal((hidden, hidden)) / 45).astype(np.float32)
+    wk = (r.standard_normal((hidden, hidden)) / 45).astype(np.float32)
+
+    def backbone(x):
+        kc = np.zeros((cfg["max_pos"], cfg["kv_hidden"]), np.int8); vc = np.zeros_like(kc)
+        return oracle.w4a4_layer(cfg, host_w, 0, x, 0, kc, vc)
+
+    outs_ref, mmem_ref, kmem_ref, ps_ref = oracle.hmt_run(backbone, emb, t_embed, wq, wk, seg_len, sum_len, rec, mem_num,
+                                                          float(np.sqrt(hidden)), pad=32)
+    plug = hmt.Hmt(model, fx.to_device(wq), fx.to_device(wk), fx.to_device(t_embed), seg_len, sum_len, rec, mem_num)
+    outs, ps = plug.run(fx.to_device(emb))
+    model.check()
+    assert len(outs) == 3 and len(ps) == 2
+    e0 = np.abs(outs[0].numpy() - outs_ref[0]).max(axis=-1) / np.abs(outs_ref[0]).max()
+    print("first segment token errors: median %.2e max %.2e" % (np.median(e0), e0.max()), flush=True)
+    assert np.median(e0) < 1e-5 and e0.max() < 8e-2
+    for o, ref in zip(outs[1:], outs_ref[1:]):
+        assert o.shape == ref.shape and np.abs(o.numpy() - ref).max() <= 0.25 * np.abs(ref).max()
+    for pn, ref in zip(ps, ps_ref):
+        assert np.abs(pn.numpy() - ref).max() <= 0.25 * np.abs(ref).max()
+    assert plug.mmem.numpy()[:2].any(axis=1).all() and not plug.mmem.numpy()[2:].any()
+    model.close()
