@@ -56,6 +56,9 @@ constexpr int kMegaWG = 256;       // workgroups (persistent, one per CU)
 constexpr int kMegaT = 512;        // threads per workgroup
 constexpr int kMegaWaves = kMegaT / 64;
 constexpr int kMegaGroup = 32;     // workgroups per first-level barrier counter
+constexpr int kMegaFlagCopies = 8; // copies of the barrier's release flag, each on its own line: workgroup w polls copy w mod 8
+constexpr int kMegaFlagBase = 64 * (2 + kMegaWG / kMegaGroup);   // the flags follow the counters (in 32-bit words)
+constexpr int kMegaBarWords = kMegaFlagBase + 64 * kMegaFlagCopies;
 constexpr int kMegaSpinLimit = 1 << 20;   // polls of ~1 us each: a wait that has not ended after a second never will
 constexpr int kMegaErrPeriod = 64;         // a spinning thread looks at the error flag every so many polls
 constexpr int kMegaMaxSteps = 64;  // tokens per launch in greedy mode (bounds the run time of one launch)
@@ -192,10 +195,13 @@ __device__ __forceinline__ LayerW ldc_layer(const LayerW* p) {
 
 // Grid barrier from device-scope relaxed atomics: workgroup w adds 1 to group counter w/32 (8 counters on
 // separate 256-byte lines, so at most 32 atomics serialise on one address); the last arriver of a group adds 1
-// to the top counter, the last of those publishes the epoch in a flag that everybody polls.  (Polling the
-// group counters directly costs more: 256 pollers then contend with the arriving atomics on the same lines.)
+// to the top counter, the last of those publishes the epoch in the release flags.  There are eight copies of the
+// flag on eight lines and workgroup w polls copy w mod 8: a store into a line that 256 workgroups are polling queues
+// behind their loads at the memory side, behind 32 pollers it lands sooner (-0.2 us per barrier; 32 copies are no
+// better than 8).  (Polling the group counters directly costs more: 256 pollers then contend with the arriving
+// atomics on the same lines.  So does one level of 16 groups whose last arrivers set 16 flags in one polled line.)
 struct GridBarrier {
-    unsigned* mem;                              // [0] flag, [64] top counter, [128 + 64*g] group counters
+    unsigned* mem;                              // [64] top counter, [128 + 64*g] group counters, [kMegaFlagBase + 64*r] release flags
     unsigned epoch;
     int* err;
     bool dead = false;                          // thread 0 only: a wait timed out or the error flag was seen; later waits return at once
@@ -204,13 +210,19 @@ struct GridBarrier {
         if (drain) __builtin_amdgcn_s_waitcnt(0);          // this thread's stores have been acknowledged
         __syncthreads();
         epoch++;
-        if (threadIdx.x == 0) {
-            const int g = blockIdx.x / kMegaGroup;
-            const unsigned old = __hip_atomic_fetch_add(&mem[128 + 64 * g], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            if (old == epoch * kMegaGroup - 1) {
-                const unsigned o2 = __hip_atomic_fetch_add(&mem[64], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                if (o2 == epoch * (kMegaWG / kMegaGroup) - 1)
-                    __hip_atomic_store(&mem[0], epoch, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (threadIdx.x < 64) {
+            bool last = false;
+            if (threadIdx.x == 0) {
+                const int g = blockIdx.x / kMegaGroup;
+                const unsigned old = __hip_atomic_fetch_add(&mem[128 + 64 * g], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                if (old == epoch * kMegaGroup - 1) {
+                    const unsigned o2 = __hip_atomic_fetch_add(&mem[64], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    last = o2 == epoch * (kMegaWG / kMegaGroup) - 1;
+                }
+            }
+            if (__builtin_amdgcn_ballot_w64(last) != 0) {
+                for (int r = threadIdx.x; r < kMegaFlagCopies; r += 64)
+                    __hip_atomic_store(&mem[kMegaFlagBase + 64 * r], epoch, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             }
         }
     }
@@ -218,7 +230,8 @@ struct GridBarrier {
         if (threadIdx.x == 0 && !dead) {
             int it = 0;
             // signed distance so that the comparison survives counter wrap-around
-            while ((int)(__hip_atomic_load(&mem[0], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) - epoch) < 0) {
+            const unsigned* flag = &mem[kMegaFlagBase + 64 * (blockIdx.x % kMegaFlagCopies)];
+            while ((int)(__hip_atomic_load(flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) - epoch) < 0) {
                 if (spin_should_stop(++it, err)) { dead = true; break; }
             }
         }

@@ -345,8 +345,8 @@ int flexllm_llama_create(flexllm_llama** out, const flexllm_llama_config* cfg, c
     FX_TRY(dev_alloc(m, (void**)&m->am_i, sizeof(int) * kArgmaxParts));
     FX_TRY(dev_alloc(m, (void**)&m->layers_dev, sizeof(LayerW) * L));
     FX_TRY_HIP(hipMemcpy(m->layers_dev, m->layers.data(), sizeof(LayerW) * L, hipMemcpyHostToDevice));
-    FX_TRY(dev_alloc(m, (void**)&m->bar, sizeof(unsigned) * 64 * (2 + kMegaWG / kMegaGroup)));
-    FX_TRY_HIP(hipMemset(m->bar, 0, sizeof(unsigned) * 64 * (2 + kMegaWG / kMegaGroup)));
+    FX_TRY(dev_alloc(m, (void**)&m->bar, sizeof(unsigned) * kMegaBarWords));
+    FX_TRY_HIP(hipMemset(m->bar, 0, sizeof(unsigned) * kMegaBarWords));
     FX_TRY_HIP(hipMemset(m->state, 0, sizeof(int) * 8));
     FX_TRY_HIP(hipMemset(m->o_acc, 0, sizeof(int32_t) * H));
     FX_TRY_HIP(hipMemset(m->am_v, 0, sizeof(float) * kArgmaxParts));
@@ -497,7 +497,7 @@ int flexllm_llama_check(flexllm_llama* m) {
             return FLEXLLM_EINVAL;
         }
         // after a time-out the barrier counters and the attention accumulators hold partial counts: start them afresh
-        (void)hipMemset(m->bar, 0, sizeof(unsigned) * 64 * (2 + kMegaWG / kMegaGroup));
+        (void)hipMemset(m->bar, 0, sizeof(unsigned) * kMegaBarWords);
         (void)hipMemset(&m->state[2], 0, sizeof(int));
         (void)hipMemset(m->o_mega, 0, sizeof(int32_t) * (size_t)m->cfg.hidden);
         set_error("persistent decode kernel: a wait timed out (were all %d workgroups resident?)", kMegaWG);
