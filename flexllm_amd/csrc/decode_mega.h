@@ -82,7 +82,7 @@ struct MegaParams {
     float* h;
     float2* stats;                 // [q_heads][32] (one-kernel-per-stage path)
     unsigned long long* qkv_tag;   // [H + 2*KV]: q/k/v projection outputs, each with the epoch in its high word
-    unsigned long long* stats_tag; // [q_heads][32][2]: chunk max and chunk sum of exponentials, each with the epoch in its high word
+    unsigned long long* stats_tag; // [q_heads][2][32]: chunk maxima, then chunk sums of exponentials, each with the epoch in its high word
     unsigned long long* x_tag;     // [H]: the residual stream after a layer (down projection + residual), tagged with the layer's sequence number
     unsigned long long* x2_tag;    // [H]: the residual stream after attention (o projection + residual), tagged likewise
     int32_t* o_acc;                // [H]: attention accumulators (zero at launch, cleared again once read)
@@ -150,17 +150,35 @@ __device__ __forceinline__ void poll_tagged2(const unsigned long long* a, const 
     fb = __int_as_float((int)(unsigned)w1);
 }
 
-// Polls four consecutive tagged words (p 32-byte aligned per thread) until every active lane of the wave has seen `tag`
-// on all four; a lane that has its values stops loading (its later polls are masked out), so the traffic shrinks
-// as the data arrives.  Bounded like every wait here.
-__device__ __forceinline__ void poll_tagged4(const unsigned long long* p, unsigned tag, int* err, float (&v)[4]) {
+// Polls one tagged word per lane until it carries `tag` in every active lane of the wave (bounded likewise).
+__device__ __forceinline__ float poll_tagged1(const unsigned long long* a, unsigned tag, int* err) {
+    unsigned long long w0 = 0;
+    int it = 0;
+    for (;;) {
+        w0 = ld_u64(a);
+        if (__builtin_amdgcn_ballot_w64((unsigned)(w0 >> 32) != tag) == 0) break;
+        if (spin_should_stop(++it, err)) break;
+    }
+    return __int_as_float((int)(unsigned)w0);
+}
+
+// Polls the 2048 tagged words at `base` (the residual stream) with all eight waves until every word carries `tag`, and
+// leaves elements 4t..4t+3 in v.  Each load instruction of a wave covers 64 consecutive words, i.e. eight whole lines:
+// a line is asked for once per round and workgroup (four consecutive words per lane would touch every line with
+// four instructions), and what limits this hand-over is the number of poll requests the memory side has to serve.
+// The values then change places inside the wave through its own 1 KiB of LDS (`wave_lds`: 256 floats, no workgroup
+// barrier).  A lane that has its values stops loading (its later polls are masked out), so the traffic shrinks as the
+// data arrives.  Bounded like every wait here.
+__device__ __forceinline__ void poll_tagged4(const unsigned long long* base, unsigned tag, int* err, float* wave_lds, float (&v)[4]) {
+    const int lane = threadIdx.x & 63;
+    const unsigned long long* p = base + (threadIdx.x >> 6) * 256 + lane;
     unsigned long long w[4] = {0, 0, 0, 0};
     bool ok = false;
     int it = 0;
     for (;;) {
         if (!ok) {
 #pragma unroll
-            for (int i = 0; i < 4; i++) w[i] = ld_u64(p + i);
+            for (int i = 0; i < 4; i++) w[i] = ld_u64(p + 64 * i);
             ok = (unsigned)(w[0] >> 32) == tag && (unsigned)(w[1] >> 32) == tag && (unsigned)(w[2] >> 32) == tag &&
                  (unsigned)(w[3] >> 32) == tag;
         }
@@ -168,7 +186,10 @@ __device__ __forceinline__ void poll_tagged4(const unsigned long long* p, unsign
         if (spin_should_stop(++it, err)) break;
     }
 #pragma unroll
-    for (int i = 0; i < 4; i++) v[i] = __int_as_float((int)(unsigned)w[i]);
+    for (int i = 0; i < 4; i++) wave_lds[64 * i + lane] = __int_as_float((int)(unsigned)w[i]);
+    __builtin_amdgcn_wave_barrier();                 // same wave: its LDS accesses are performed in program order
+    const float4 mine = reinterpret_cast<const float4*>(wave_lds)[lane];
+    v[0] = mine.x; v[1] = mine.y; v[2] = mine.z; v[3] = mine.w;
 }
 
 // Read-only data at a wave-uniform address (layer table, per-row weight scales): the constant address space
@@ -602,7 +623,7 @@ __device__ __forceinline__ void decode_mega_body(const MegaParams& p) {
             }
             const float4 gam = reinterpret_cast<const float4*>(g0)[t];
             float v[4];
-            if (l > 0) poll_tagged4(&p.x_tag[4 * t], tag - 1u, bar.err, v);   // x of the previous layer, as it arrives
+            if (l > 0) poll_tagged4(p.x_tag, tag - 1u, bar.err, L.f + (t >> 6) * 256, v);   // x of the previous layer, as it arrives
             stamp();
             if (l == 0) {
                 if (p.x_in) { const float4 q = reinterpret_cast<const float4*>(p.x_in)[t]; v[0] = q.x; v[1] = q.y; v[2] = q.z; v[3] = q.w; }
@@ -673,10 +694,9 @@ __device__ __forceinline__ void decode_mega_body(const MegaParams& p) {
                     const int8_t b0 = (int8_t)static_q8(o0, div), b1 = (int8_t)static_q8(o1, div);
                     L.knew[k] = b0; L.knew[k + 32] = b1;
                     if (a_owner) { int8_t* dst = kc + k_index(a_h, pos, p.max_pos); dst[k] = b0; dst[k + 32] = b1; }
-                } else if (t < 224) {                                 // v of the new token
-                    const int d = t - 160;
-                    float tv, tv_again;
-                    poll_tagged2(&p.qkv_tag[H + KV + a_h * kHd + d], &p.qkv_tag[H + KV + a_h * kHd + d], tag, bar.err, tv, tv_again);
+                } else if (t >= 192 && t < 256) {                     // v of the new token: a wave of its own (two polls in
+                    const int d = t - 192;                            // one wave would run one after the other)
+                    const float tv = poll_tagged1(&p.qkv_tag[H + KV + a_h * kHd + d], tag, bar.err);
                     const int8_t b = (int8_t)static_q8(tv, 1.0f * vs1);
                     L.vnew[d] = b;
                     if (a_owner) vc[v_index(a_h, pos, d, p.max_pos)] = b;
@@ -702,9 +722,9 @@ __device__ __forceinline__ void decode_mega_body(const MegaParams& p) {
                     float sum = (a_c * kChunk + lane < len ? exp_f(s0 - m) : 0.0f) + (a_c * kChunk + lane + 64 < len ? exp_f(s1 - m) : 0.0f);
                     sum = wave_sum(sum);
                     if (lane == 0) {
-                        unsigned long long* slot = p.stats_tag + (size_t)((a_h * GROUP + wave) * 32 + a_c) * 2;
+                        unsigned long long* slot = p.stats_tag + (size_t)(a_h * GROUP + wave) * 64 + a_c;
                         st_tagged(slot, m, tag);
-                        st_tagged(slot + 1, sum, tag);
+                        st_tagged(slot + 32, sum, tag);
                     }
                 }
             } else {
@@ -720,12 +740,13 @@ __device__ __forceinline__ void decode_mega_body(const MegaParams& p) {
                 if (wave < GROUP) {
                     float m_c = -1e32f, l_c = 0.0f;
                     {
-                        const unsigned long long* slot = p.stats_tag + (size_t)((a_h * GROUP + wave) * 32 + min(lane, nchunks - 1)) * 2;
+                        // the maxima of a head's 32 chunks are consecutive words, then its sums: a poll is two loads of whole lines
+                        const unsigned long long* slot = p.stats_tag + (size_t)(a_h * GROUP + wave) * 64 + min(lane, nchunks - 1);
                         unsigned long long w0 = 0, w1 = 0;
                         int it = 0;
                         for (;;) {
                             w0 = ld_u64(slot);
-                            w1 = ld_u64(slot + 1);
+                            w1 = ld_u64(slot + 32);
                             const bool ok = (unsigned)(w0 >> 32) == tag && (unsigned)(w1 >> 32) == tag;
                             if (__builtin_amdgcn_ballot_w64(!ok) == 0) break;
                             if (spin_should_stop(++it, bar.err)) break;
@@ -870,7 +891,7 @@ __device__ __forceinline__ void decode_mega_body(const MegaParams& p) {
             }
             const float4 gam = reinterpret_cast<const float4*>(g1)[t];
             float v[4];
-            poll_tagged4(&p.x2_tag[4 * t], tag, bar.err, v);
+            poll_tagged4(p.x2_tag, tag, bar.err, L.f + (t >> 6) * 256, v);
             stamp();
             // every workgroup has published x2, so it has read the accumulators; the next parts are added a layer later,
             // by workgroups that have polled this workgroup's x, which wave 0 stores after this store has been acknowledged
@@ -1152,7 +1173,7 @@ __device__ __forceinline__ void decode_mega_body(const MegaParams& p) {
             };
             load_group(r);
             float v[4];
-            poll_tagged4(&p.x_tag[4 * t], seq0 + (unsigned)((step + 1) * p.n_layers), bar.err, v);
+            poll_tagged4(p.x_tag, seq0 + (unsigned)((step + 1) * p.n_layers), bar.err, L.f + (t >> 6) * 256, v);
             stamp();
             const float4 g = reinterpret_cast<const float4*>(p.gamma + (size_t)(2 * p.n_layers) * H)[t];
             const float2 sb = norm_quant_2048_u4(v, g, true, p.eps, L, NoHook());
@@ -1184,7 +1205,7 @@ __device__ __forceinline__ void decode_mega_body(const MegaParams& p) {
         };
         load_group(r);
         float v[4];
-        poll_tagged4(&p.x_tag[4 * t], seq0 + (unsigned)((step + 1) * p.n_layers), bar.err, v);
+        poll_tagged4(p.x_tag, seq0 + (unsigned)((step + 1) * p.n_layers), bar.err, L.f + (t >> 6) * 256, v);
         stamp();
         float ss = (v[0] * v[0] + v[1] * v[1]) + (v[2] * v[2] + v[3] * v[3]);
         ss = block_sum<kMegaWaves>(ss, L.red);
