@@ -94,6 +94,67 @@ __device__ __forceinline__ int pf_round4(const float (&e)[4], float kq, float cd
     return (int)(packed ^ 0x80808080u);
 }
 
+// The fast path of the probabilities.  The reference's exponential of a score is exp_f(fl(fl(tv*Q_s)*K_s) - max): two
+// roundings of its own per element that an exact result has to reproduce, ten instructions with the two-part exponent.
+// Almost no probability needs that: e~ = 2^(tv*c2 - m2) with c2 = fl(fl(Q_s*K_s)*log2 e), m2 = fl(max_int*c2) is one
+// conversion, one fused multiply-add and one 2^x, and differs from the exact value by a factor common to the row (the
+// roundings of max and m2: it cancels between the probability and the row sum, and the exact path's denominator is
+// the fast row sum times that factor, `pf_fast_row`) and per element by at most R = 2^-24 (3|max| + 9 X + 12) + 1e-6
+// relative, X = ln(kq / 0.4) bounding |score - max| of every probability that can reach 0.4 (float32 model of both
+// paths, tests/test_attention_fast_path_cpu.py: worst observed deviation 0.3 R).  So q~ = e~ * kq rounds like the reference's
+// expression unless it lies within win = 1e-4 + kq R of a tie; those groups of four are redone exactly (about 1e-4
+// of the elements).
+struct PfFastRow {
+    float c2, m2, imf;       // e~ = 2^(tv * c2 - m2), m2 = fl(imf * c2), imf = the row's integer maximum
+    float kq, win, cd;       // q~ = e~ * kq; redo within win of a tie, with the denominator cd
+};
+// With c2 below 2e-5 a masked score (-2^31) would not reach 2^-150, i.e. an e~ of exactly 0: such heads take the
+// exact path throughout.
+__device__ __forceinline__ bool pf_fast_ok(float c2, float as) { return quant_fast_ok(as) && c2 >= 2e-5f && c2 <= 1.0f; }
+__device__ __forceinline__ void pf_fast_row_begin(PfFastRow& f, int im, float c2) {
+    f.c2 = c2;
+    f.imf = (float)im;
+    f.m2 = f.imf * c2;
+}
+// total: the row's sum of e~.  mx = fl(fl(max_int*Q_s)*K_s) as the exact path forms it.
+__device__ __forceinline__ void pf_fast_row_finish(PfFastRow& f, float total, float sq, float sk, float mx, float as) {
+    const float t1 = f.imf * sq;                                         // mx == t1 * sk
+    const float r1 = __builtin_fmaf(f.imf, sq, -t1), r2 = __builtin_fmaf(t1, sk, -mx), rr = __builtin_fmaf(f.imf, f.c2, -f.m2);
+    const float offset = r2 + r1 * sk - rr * 0.693147182464599609375f;   // ln(exact exponential / e~), the row's common part
+    f.cd = 1.0f / (total * (1.0f + offset));
+    f.kq = (1.0f / total) * (1.0f / as);
+    const float x_max = fmaxf(0.0f, __logf(f.kq) + 0.92f);
+    const float rel = 5.9604645e-8f * (3.0f * fabsf(mx) + 9.0f * x_max + 12.0f) + 1e-6f;
+    f.win = 1e-4f + f.kq * rel;
+}
+__device__ __forceinline__ float pf_fast_exp(int tv, const PfFastRow& f) {
+    return __builtin_amdgcn_exp2f(__builtin_fmaf((float)tv, f.c2, -f.m2));   // a masked score (-2^31) gives 0
+}
+// Four e~ -> four probability bytes (biased by 128, as pf_round4).  exact(b): the exact exponential of element b, only
+// evaluated for a group near a tie.
+template <class Exact>
+__device__ __forceinline__ int pf_round4_fast(const float (&ef)[4], const PfFastRow& f, float as, Exact exact, unsigned& bytes) {
+    float qv[4];
+#pragma unroll
+    for (int b = 0; b < 4; b++) qv[b] = ef[b] * f.kq;
+    const float d0 = fabsf(__builtin_amdgcn_fractf(qv[0]) - 0.5f), d1 = fabsf(__builtin_amdgcn_fractf(qv[1]) - 0.5f);
+    const float d2 = fabsf(__builtin_amdgcn_fractf(qv[2]) - 0.5f), d3 = fabsf(__builtin_amdgcn_fractf(qv[3]) - 0.5f);
+    unsigned packed = 0;
+    if (fminf(fminf(d0, d1), fminf(d2, d3)) < f.win) {
+#pragma unroll
+        for (int b = 0; b < 4; b++) {
+            int v = (int)roundf((exact(b) * f.cd) / as);
+            v = v > 255 ? 255 : v;
+            packed |= (unsigned)v << (8 * b);
+        }
+    } else {
+#pragma unroll
+        for (int b = 0; b < 4; b++) packed = __builtin_amdgcn_cvt_pk_u8_f32(qv[b], b, packed);
+    }
+    bytes = packed;
+    return (int)(packed ^ 0x80808080u);
+}
+
 // Adds the waves' partial accumulators in LDS and writes the block's 32 x 64 outputs.
 __device__ __forceinline__ void pf_reduce_store(int (*lds_acc)[35], const i32x16& oacc0, const i32x16& oacc1, int vsum0, int vsum1,
                                                 bool has_tiles, const PfItem& it, float sa, float sv, float* __restrict__ o,
@@ -122,10 +183,10 @@ __device__ __forceinline__ void pf_reduce_store(int (*lds_acc)[35], const i32x16
 }
 
 // Rows of any length: three passes over the wave's key tiles, the scores recomputed in each (64-deep dot products on
-// the matrix cores).  Pass 0: integer row maximum (the dequantisation is monotonic).  Pass 1: the softmax denominator,
-// with a one-rounding exponent (2^(acc*c - m), c = Q_s*K_s*log2(e)): its error, a few 1e-7 relative on the terms that
-// matter, only moves the common factor 1/sum.  Pass 2: each probability from the accurate exponential of the
-// reference's own score expression, rounded as described above, and P.V.
+// the matrix cores).  Pass 0: integer row maximum (the dequantisation is monotonic).  Pass 1: the softmax denominator
+// from the one-rounding exponentials e~ (PfFastRow).  Pass 2: the probabilities from the same e~, rounded as described
+// there, the groups near a tie from the accurate exponential of the reference's own score expression; and P.V.  Heads
+// whose scales rule the fast path out (pf_fast_ok) take the accurate exponential for every probability.
 static __global__ __launch_bounds__(64 * kPfWaves) void pf_attention_kernel(const int8_t* __restrict__ q8, const int8_t* __restrict__ kc,
                                                                   const int8_t* __restrict__ vc, const float* __restrict__ q_s,
                                                                   const float* __restrict__ k_s, const float* __restrict__ v_s,
@@ -188,6 +249,9 @@ static __global__ __launch_bounds__(64 * kPfWaves) void pf_attention_kernel(cons
     // ---- pass 1: denominator ----
     const float c2 = sq * sk * 1.44269502162933349609375f;
     const float m2 = (float)im * c2;
+    const bool fast = pf_fast_ok(c2, as);                       // per head: uniform over the workgroup
+    PfFastRow fr;
+    pf_fast_row_begin(fr, im, c2);
     float lsum = 0.0f;
     {
         i32x4 kf0, kf1, nf0, nf1;
@@ -196,7 +260,10 @@ static __global__ __launch_bounds__(64 * kPfWaves) void pf_attention_kernel(cons
             if (kt + kPfWaves < ntiles) load_k((kt + kPfWaves) * kPfTile, nf0, nf1);
             int tv[16];
             int_tile(kt, kf0, kf1, tv);
-            if (kt == it.qb) {
+            if (fast) {                                        // the same e~ as in pass 2; masked keys come out as 0
+#pragma unroll
+                for (int r = 0; r < 16; r++) lsum += pf_fast_exp(tv[r], fr);
+            } else if (kt == it.qb) {
 #pragma unroll
                 for (int r = 0; r < 16; r++)
                     lsum += tv[r] == kPfMasked ? 0.0f : __builtin_amdgcn_exp2f(fminf(__builtin_fmaf((float)tv[r], c2, -m2), 0.0f));
@@ -216,6 +283,7 @@ static __global__ __launch_bounds__(64 * kPfWaves) void pf_attention_kernel(cons
     const float cd = 1.0f / total;
     const bool fast_q = quant_fast_ok(as);
     const float kq = cd * (1.0f / as);
+    if (fast) pf_fast_row_finish(fr, total, sq, sk, mx, as);
 
     // ---- pass 2: probabilities, partial P.V over this wave's tiles ----
     i32x16 oacc0 = zero16(), oacc1 = zero16();
@@ -237,6 +305,16 @@ static __global__ __launch_bounds__(64 * kPfWaves) void pf_attention_kernel(cons
             for (int a = 0; a < 4; a++) {
                 float e[4];
                 unsigned bytes;
+                if (fast) {
+#pragma unroll
+                    for (int b = 0; b < 4; b++) e[b] = pf_fast_exp(tv[a * 4 + b], fr);
+                    pf[a] = pf_round4_fast(e, fr, as, [&](int b) {
+                        const int ts = tv[a * 4 + b];
+                        return ts == kPfMasked ? 0.0f : exp_f<false>((float)ts * sq * sk - mx);
+                    }, bytes);
+                    if (p8_out) *reinterpret_cast<unsigned*>(p8_out + ((size_t)it.h * s + query) * s + k0 + 16 * g + a * 4) = bytes;
+                    continue;
+                }
                 if (kt == it.qb) {                             // uniform: only the diagonal tile has masked keys
 #pragma unroll
                     for (int b = 0; b < 4; b++)                // masked keys: exactly 0 whatever the scales
