@@ -893,10 +893,14 @@ __device__ __forceinline__ void decode_mega_body(const MegaParams& p) {
             float v[4];
             poll_tagged4(p.x2_tag, tag, bar.err, L.f + (t >> 6) * 256, v);
             stamp();
-            // every workgroup has published x2, so it has read the accumulators; the next parts are added a layer later,
-            // by workgroups that have polled this workgroup's x, which wave 0 stores after this store has been acknowledged
-            if (t < 8) st_i(&p.o_acc[wg * 8 + t], 0);
             auto down_row_0 = [&]() {
+                // Runs after the first workgroup barrier of the reduction below, i.e. once ALL eight waves have their
+                // share of x2: every workgroup has then published x2, so every workgroup has read the accumulators,
+                // and this workgroup's eight can be cleared.  (A wave's own poll only covers the 256 words of 32
+                // producers: clearing right behind it wiped accumulators that a slower workgroup had yet to read.)
+                // The next parts are added a layer later, by workgroups that have polled this workgroup's x, which
+                // the same threads store after this store has been acknowledged.
+                if (t < 8) st_i(&p.o_acc[wg * 8 + t], 0);
                 __builtin_amdgcn_s_waitcnt(0x0F70);                   // vmcnt(0): see gu_slice
                 if (is_s) {
                     if constexpr (W4) mega_row4_to_lds(w.wd, wg * 8 + sw * 2, lane, L.wd[sw * 2]);
