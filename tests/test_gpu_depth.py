@@ -297,3 +297,49 @@ def test_change_of_decode_schedule_in_mid_sequence(two_layer):
     for a, b in zip(sw.caches_token_major(), steady.caches_token_major()):
         assert np.array_equal(a, b)
     sw.close(); steady.close()
+
+
+@pytest.mark.parametrize("top_k", [0, 5], ids=["greedy", "top5"])
+def test_repeated_runs_are_identical_to_the_byte(two_layer, top_k):
+    """The same 80-token run (two launches, crossing the chunk boundary at position 128) 400 times on one model: token
+    ids and every cache byte identical each time, whether the rows the run writes are left in place, reloaded as zeros
+    or reloaded with their final values.  All arithmetic of the persistent kernel is order-independent (integer
+    accumulation, fixed reduction trees), so any difference is an exchange between workgroups gone wrong: this is the
+    check that showed the attention accumulators being cleared before a slow workgroup had read them (about 1 % of
+    such runs on some boxes, none on others)."""
+    import hashlib
+    fx, llama, oracle, cfg, dev_w, host_w = two_layer
+    steps, pos0, first = 80, 100, 333
+    r = np.random.default_rng(5)
+    kc = np.zeros((cfg["layers"], cfg["max_pos"], cfg["kv_hidden"]), np.int8); vc = np.zeros_like(kc)
+    kc[:, :pos0] = r.integers(-100, 101, (cfg["layers"], pos0, cfg["kv_hidden"]))
+    vc[:, :pos0] = r.integers(-100, 101, (cfg["layers"], pos0, cfg["kv_hidden"]))
+    rands = fx.to_device(r.uniform(0, 1, steps).astype(np.float32))
+    m = llama.Llama(cfg, dev_w)
+    out = fx.zeros((steps,), np.int32)
+
+    def run():
+        tok = fx.to_device(np.array([first], np.int32))
+        if top_k:
+            m.decode_sample(tok, pos0, steps, rands, top_k, out)
+        else:
+            m.decode_greedy(tok, pos0, steps, out, use_graph=0)
+        m.check()
+        k, v = m.caches_token_major()
+        return out.numpy().copy(), k, v
+
+    m.load_caches_token_major(kc, vc)
+    ids0, k0, v0 = run()
+    assert len(set(ids0.tolist())) > 10
+    want = hashlib.md5(ids0.tobytes() + k0.tobytes() + v0.tobytes()).hexdigest()
+    for rep in range(400):
+        if rep % 3 == 0:
+            m.load_caches_token_major(kc, vc)
+        elif rep % 3 == 1:
+            m.load_caches_token_major(k0, v0)
+        ids, k, v = run()
+        if hashlib.md5(ids.tobytes() + k.tobytes() + v.tobytes()).hexdigest() != want:
+            step = np.nonzero(ids != ids0)[0]
+            rows = np.nonzero((k != k0).any(axis=(0, 2)) | (v != v0).any(axis=(0, 2)))[0]
+            raise AssertionError("run %d differs: ids from step %s, cache rows %s" % (rep, step[:1], rows[:4]))
+    m.close()
