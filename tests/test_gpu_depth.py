@@ -185,6 +185,31 @@ def test_256_token_greedy_run_both_schedules(full):
     a.close(); b.close()
 
 
+def test_full_size_runs_are_identical_to_the_byte(full):
+    """48 greedy tokens of the full-size model up to the maximum context (every one of the 256 workgroups takes part
+    in the attention), thirty times: ids and cache bytes identical each time (see
+    test_repeated_runs_are_identical_to_the_byte)."""
+    import hashlib
+    fx, llama, oracle, cfg, dev_w, host_w = full
+    m = llama.Llama(cfg, dev_w)
+    lib = fx.lib()
+    fx.check(lib.flexllm_rt_fill_i8(C.c_void_p(m.k_cache.ptr), C.c_size_t(m.k_cache.size), C.c_uint64(921), -100, 100, None))
+    fx.check(lib.flexllm_rt_fill_i8(C.c_void_p(m.v_cache.ptr), C.c_size_t(m.v_cache.size), C.c_uint64(922), -100, 100, None))
+    steps, pos0 = 48, 4096 - 48
+    out = fx.zeros((steps,), np.int32)
+    seen = set()
+    for rep in range(30):
+        tok = fx.to_device(np.array([4242], np.int32))
+        m.decode_greedy(tok, pos0, steps, out, use_graph=0)
+        m.check()
+        h = hashlib.md5(out.numpy().tobytes())
+        h.update(m.k_cache.numpy().tobytes()); h.update(m.v_cache.numpy().tobytes())
+        seen.add(h.hexdigest())
+        assert len(seen) == 1, "run %d differs from the runs before it" % rep
+    assert len(set(out.numpy().tolist())) > 10
+    m.close()
+
+
 @pytest.fixture(scope="module")
 def two_layer():
     import flexllm_amd as fx
