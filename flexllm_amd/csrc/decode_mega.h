@@ -56,9 +56,9 @@ constexpr int kMegaWG = 256;       // workgroups (persistent, one per CU)
 constexpr int kMegaT = 512;        // threads per workgroup
 constexpr int kMegaWaves = kMegaT / 64;
 constexpr int kMegaGroup = 32;     // workgroups per first-level barrier counter
-constexpr int kMegaFlagCopies = 8; // copies of the barrier's release flag, each on its own line: workgroup w polls copy w mod 8
+constexpr int kMegaFlagCopies = 8; // copies of each of the barrier's release flags, each on its own line: workgroup w polls copy w mod 8
 constexpr int kMegaFlagBase = 64 * (2 + kMegaWG / kMegaGroup);   // the flags follow the counters (in 32-bit words)
-constexpr int kMegaBarWords = kMegaFlagBase + 64 * kMegaFlagCopies;
+constexpr int kMegaBarWords = kMegaFlagBase + 64 * kMegaFlagCopies * (kMegaWG / kMegaGroup);
 constexpr int kMegaSpinLimit = 1 << 20;   // polls of ~1 us each: a wait that has not ended after a second never will
 constexpr int kMegaErrPeriod = 64;         // a spinning thread looks at the error flag every so many polls
 constexpr int kMegaMaxSteps = 64;  // tokens per launch in greedy mode (bounds the run time of one launch)
@@ -215,17 +215,19 @@ __device__ __forceinline__ LayerW ldc_layer(const LayerW* p) {
 }
 
 // Grid barrier from device-scope relaxed atomics: workgroup w adds 1 to group counter w/32 (8 counters on
-// separate 256-byte lines, so at most 32 atomics serialise on one address); the last arriver of a group adds 1
-// to the top counter, the last of those publishes the epoch in the release flags.  There are eight copies of the
-// flag on eight lines and workgroup w polls copy w mod 8: a store into a line that 256 workgroups are polling queues
-// behind their loads at the memory side, behind 32 pollers it lands sooner (-0.2 us per barrier; 32 copies are no
-// better than 8).  (Polling the group counters directly costs more: 256 pollers then contend with the arriving
-// atomics on the same lines.  So does one level of 16 groups whose last arrivers set 16 flags in one polled line.)
+// separate 256-byte lines, so at most 32 atomics serialise on one address) and the last arriver of a group publishes
+// the epoch in the group's release flag; wave 0 of every workgroup polls the eight flags, one lane each.  Every flag
+// exists in eight copies on eight lines and workgroup w polls copy w mod 8 of each: a store into a line that 256
+// workgroups are polling queues behind their loads at the memory side, behind 32 pollers it lands sooner.  One
+// atomic round trip and one store-to-poll hand-over from the last arrival to the release (a top-level counter between
+// the groups and one flag adds a second round trip: +4 us per token; 16 groups of 16 or 4 of 64: +2).  (Polling the
+// group counters directly costs more: 256 pollers then contend with the arriving atomics on the same lines.  So do
+// the group flags without copies, 16 of them in one polled line.)
 struct GridBarrier {
-    unsigned* mem;                              // [64] top counter, [128 + 64*g] group counters, [kMegaFlagBase + 64*r] release flags
+    unsigned* mem;                              // [128 + 64*g] group counters, [kMegaFlagBase + 64*(8g + r)] copy r of group g's release flag
     unsigned epoch;
     int* err;
-    bool dead = false;                          // thread 0 only: a wait timed out or the error flag was seen; later waits return at once
+    bool dead = false;                          // wave 0 only: a wait timed out or the error flag was seen; later waits return at once
     // drain == false: the calling wave made no global store in this phase and may keep loads in flight
     __device__ __forceinline__ void arrive(bool drain = true) {
         if (drain) __builtin_amdgcn_s_waitcnt(0);          // this thread's stores have been acknowledged
@@ -233,26 +235,26 @@ struct GridBarrier {
         epoch++;
         if (threadIdx.x < 64) {
             bool last = false;
+            const int g = blockIdx.x / kMegaGroup;
             if (threadIdx.x == 0) {
-                const int g = blockIdx.x / kMegaGroup;
                 const unsigned old = __hip_atomic_fetch_add(&mem[128 + 64 * g], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                if (old == epoch * kMegaGroup - 1) {
-                    const unsigned o2 = __hip_atomic_fetch_add(&mem[64], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                    last = o2 == epoch * (kMegaWG / kMegaGroup) - 1;
-                }
+                last = old == epoch * kMegaGroup - 1;
             }
-            if (__builtin_amdgcn_ballot_w64(last) != 0) {
+            if (__builtin_amdgcn_ballot_w64(last) != 0) {        // the group is complete: its flag, in all copies
                 for (int r = threadIdx.x; r < kMegaFlagCopies; r += 64)
-                    __hip_atomic_store(&mem[kMegaFlagBase + 64 * r], epoch, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    __hip_atomic_store(&mem[kMegaFlagBase + 64 * (g * kMegaFlagCopies + r)], epoch, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             }
         }
     }
     __device__ __forceinline__ void wait() {
-        if (threadIdx.x == 0 && !dead) {
+        if (threadIdx.x < 64 && !dead) {
+            // lane j polls group j's flag, in this workgroup's copy
+            const unsigned* flag = &mem[kMegaFlagBase + 64 * ((threadIdx.x % (kMegaWG / kMegaGroup)) * kMegaFlagCopies + blockIdx.x % kMegaFlagCopies)];
             int it = 0;
-            // signed distance so that the comparison survives counter wrap-around
-            const unsigned* flag = &mem[kMegaFlagBase + 64 * (blockIdx.x % kMegaFlagCopies)];
-            while ((int)(__hip_atomic_load(flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) - epoch) < 0) {
+            for (;;) {
+                // signed distance so that the comparison survives counter wrap-around
+                const bool behind = (int)(__hip_atomic_load(flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) - epoch) < 0;
+                if (__builtin_amdgcn_ballot_w64(behind) == 0) break;
                 if (spin_should_stop(++it, err)) { dead = true; break; }
             }
         }
