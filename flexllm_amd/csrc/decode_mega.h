@@ -16,9 +16,12 @@
 //               statistics): each value is one 64-bit word with the sequence number of the layer pass in its high
 //               half, and the consumers poll the words they need.
 //   4->5, 6->1  the residual stream, which every workgroup needs in full: tagged words as well (2048 words polled by
-//               every workgroup; a lane that has its values stops loading).  Faster than a grid barrier plus a load.
-//   3->4        int32 atomic adds into the attention accumulators, then a grid barrier (device-scope relaxed atomics,
-//               two-level arrive, one broadcast flag), then coherent loads.
+//               every workgroup, each wave 256 of them in whole lines; a lane that has its values stops loading).
+//               Faster than a grid barrier plus a load.  A wave's poll says that 32 producers have published;
+//               "everybody has" holds for the workgroup only behind the workgroup barrier that follows the polls.
+//   3->4        int32 atomic adds into the attention accumulators, then a grid barrier (device-scope relaxed atomics:
+//               eight group counters, the last arriver of a group sets the group's release flag, everybody polls
+//               the eight flags), then coherent loads.
 //   5->6        SiLU(gate)*up (8192 floats): coherent stores into a slice that no other layer pass of the launch uses,
 //               a grid barrier, then ORDINARY loads, which the 32 CUs of an XCD share through L2 (see MegaParams::h).
 // A tagged slot is rewritten a layer later, after at least one exchange that all its readers take part in as
