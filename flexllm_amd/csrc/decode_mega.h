@@ -165,31 +165,35 @@ __device__ __forceinline__ float poll_tagged1(const unsigned long long* a, unsig
     return __int_as_float((int)(unsigned)w0);
 }
 
+typedef unsigned long long u64x2 __attribute__((ext_vector_type(2)));
 // Polls the 2048 tagged words at `base` (the residual stream) with all eight waves until every word carries `tag`, and
-// leaves elements 4t..4t+3 in v.  Each load instruction of a wave covers 64 consecutive words, i.e. eight whole lines:
-// a line is asked for once per round and workgroup (four consecutive words per lane would touch every line with
+// leaves elements 4t..4t+3 in v.  Each load instruction of a wave covers 128 consecutive words, i.e. sixteen whole
+// lines: a line is asked for once per round and workgroup (four consecutive words per lane would touch every line with
 // four instructions), and what limits this hand-over is the number of poll requests the memory side has to serve.
+// A lane's 16-byte load holds two tagged words of one 64-byte sector; each carries its own tag and was written by one
+// 8-byte store, so each is seen whole or not at all (the two need not be of the same moment).
 // The values then change places inside the wave through its own 1 KiB of LDS (`wave_lds`: 256 floats, no workgroup
 // barrier).  A lane that has its values stops loading (its later polls are masked out), so the traffic shrinks as the
 // data arrives.  Bounded like every wait here.
 __device__ __forceinline__ void poll_tagged4(const unsigned long long* base, unsigned tag, int* err, float* wave_lds, float (&v)[4]) {
     const int lane = threadIdx.x & 63;
-    const unsigned long long* p = base + (threadIdx.x >> 6) * 256 + lane;
-    unsigned long long w[4] = {0, 0, 0, 0};
+    const unsigned long long* p = base + (threadIdx.x >> 6) * 256 + 2 * lane;
+    u64x2 w0 = {0, 0}, w1 = {0, 0};
     bool ok = false;
     int it = 0;
     for (;;) {
         if (!ok) {
-#pragma unroll
-            for (int i = 0; i < 4; i++) w[i] = ld_u64(p + 64 * i);
-            ok = (unsigned)(w[0] >> 32) == tag && (unsigned)(w[1] >> 32) == tag && (unsigned)(w[2] >> 32) == tag &&
-                 (unsigned)(w[3] >> 32) == tag;
+            // two 16-byte loads per lane, 128 consecutive words per instruction; each 8-byte word inside is read whole
+            asm volatile("global_load_dwordx4 %0, %2, off sc1\n\tglobal_load_dwordx4 %1, %2, off offset:1024 sc1\n\ts_waitcnt vmcnt(0)"
+                         : "=&v"(w0), "=&v"(w1) : "v"(p) : "memory");
+            ok = (unsigned)(w0[0] >> 32) == tag && (unsigned)(w0[1] >> 32) == tag && (unsigned)(w1[0] >> 32) == tag &&
+                 (unsigned)(w1[1] >> 32) == tag;
         }
         if (__builtin_amdgcn_ballot_w64(!ok) == 0) break;
         if (spin_should_stop(++it, err)) break;
     }
-#pragma unroll
-    for (int i = 0; i < 4; i++) wave_lds[64 * i + lane] = __int_as_float((int)(unsigned)w[i]);
+    reinterpret_cast<float2*>(wave_lds)[lane] = make_float2(__int_as_float((int)(unsigned)w0[0]), __int_as_float((int)(unsigned)w0[1]));
+    reinterpret_cast<float2*>(wave_lds)[64 + lane] = make_float2(__int_as_float((int)(unsigned)w1[0]), __int_as_float((int)(unsigned)w1[1]));
     __builtin_amdgcn_wave_barrier();                 // same wave: its LDS accesses are performed in program order
     const float4 mine = reinterpret_cast<const float4*>(wave_lds)[lane];
     v[0] = mine.x; v[1] = mine.y; v[2] = mine.z; v[3] = mine.w;
