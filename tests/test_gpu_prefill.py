@@ -310,3 +310,40 @@ def test_full_size_prefill_prefix_invariance_and_decode_equivalence(fx):
         assert (d[0] != 0).mean() < 1e-3 and d[0].max() <= 1          # layer 0: ties only
         assert (d[1] != 0).mean() < 2e-2 and d[1].max() <= 3          # layer 1 inherits layer 0's flipped steps
     pre.close(); dec.close()
+
+
+@pytest.mark.parametrize("case", ["wide scores", "tiny scales", "peaky rows"])
+def test_mha_prefill_long_rows_fast_and_exact_paths(fx, oracle, case):
+    """Rows of more than 1024 keys (`pf_attention_kernel`) where the fast path of the probabilities is under strain or
+    switched off: scores spread over +-25 (large |max|: the widest window), scales so small that the kernel takes the
+    reference's expression for every probability (Q_s K_s log2 e < 2e-5), and rows dominated by one key (the factor
+    255/sum at its largest).  Same criteria as test_mha_prefill_vs_oracle."""
+    s, qh, kvh, hd = 1088, 4, 1, 64
+    r = np.random.default_rng({"wide scores": 31, "tiny scales": 32, "peaky rows": 33}[case])
+    q = r.standard_normal((s, qh, hd)).astype(np.float32)
+    k = r.standard_normal((s, kvh, hd)).astype(np.float32)
+    v = r.standard_normal((s, kvh, hd)).astype(np.float32)
+    q_s, k_s, v_s, a_s = mha_scales(qh, kvh)
+    if case == "wide scores":
+        q *= 6.0
+        q_s = (q_s * 6.0).astype(np.float32)
+    elif case == "tiny scales":
+        q_s = np.full(qh, 2e-5, np.float32); k_s = np.full(kvh, 0.05, np.float32)
+        q *= 0.005
+    else:
+        k[::97] *= 6.0                                            # a few keys that take nearly all of a row
+    ref = oracle.mha_prefill(q, k, v, q_s, k_s, v_s, a_s, want_p=True)
+    sc = fx.ops.Scales(q_s, k_s, v_s, a_s)
+    kc, vc = fx.ops.kv_cache(kvh, s)
+    fx.ops.kv_append_i8(fx.to_device(k), fx.to_device(v), kc, vc, sc, 0)
+    q8 = fx.ops.static_quant_i8(fx.to_device(q), fx.to_device(q_s), factor=8.0)
+    assert np.array_equal(q8.numpy(), ref["q8"])
+    o, p8 = fx.ops.mha_i8_prefill(q8, kc, vc, sc, want_p=True)
+    p = p8.numpy()
+    d = np.abs(p.astype(np.int32) - ref["p8"].astype(np.int32))
+    print(case, "probability bytes off by one:", int((d != 0).sum()), "of", int(s * (s + 1) // 2 * qh), "largest byte", int(ref["p8"].max()), flush=True)
+    assert d.max() <= 1 and (d != 0).mean() < 1e-4
+    group = qh // kvh
+    acc = np.stack([p[h].astype(np.float64) @ ref["v8"][:, h // group].astype(np.float64) for h in range(qh)], axis=1)
+    o_from_p = (acc.astype(np.float32) * a_s[None, :, None]) * np.repeat(v_s, group)[None, :, None]
+    assert np.array_equal(o.numpy(), o_from_p.astype(np.float32))
