@@ -499,9 +499,13 @@ __device__ __forceinline__ void decode_mega_body(const MegaParams& p) {
     const int sw = wave - 4;
     constexpr int H = 2048, KV = 512, QH = 32, KVH = 8, GROUP = 4;
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");   // see MegaParams::h
-    const int pos0 = p.state[0];
-    GridBarrier bar{p.bar, (unsigned)p.state[2], &p.state[3]};
-    const unsigned seq0 = (unsigned)p.state[4];
+    // The launch state was left by the previous launch (or a small kernel before this one).  It is read with coherent
+    // loads: the compiler would otherwise fetch it through the scalar cache, whose requests do not queue behind the
+    // invalidation above and could be served from a line of an earlier launch that survived in this XCD's L2.
+    const int pos0 = ld_i(&p.state[0]);
+    const int step_base = ld_i(&p.state[1]);
+    GridBarrier bar{p.bar, (unsigned)ld_i(&p.state[2]), &p.state[3]};
+    const unsigned seq0 = (unsigned)ld_i(&p.state[4]);
     int stamp_i = 0;
     // 'thread 0 of workgroup 0' from scalars and the hardware lane id: no per-thread value has to stay live for it
     auto is_t0 = [&]() { return wave == 0 && __builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u)) == 0; };
@@ -525,7 +529,7 @@ __device__ __forceinline__ void decode_mega_body(const MegaParams& p) {
 #else
     auto fine = [&]() {};
 #endif
-    int tok = p.x_in ? 0 : p.token[0];
+    int tok = p.x_in ? 0 : ld_i(&p.token[0]);
     if ((unsigned)tok >= (unsigned)p.vocab) {                      // never look up a row outside the table: report and use token 0
         if (wg == 0 && threadIdx.x == 0) st_i(&p.state[3], 2);
         tok = 0;
@@ -1278,7 +1282,7 @@ __device__ __forceinline__ void decode_mega_body(const MegaParams& p) {
             topk_block_select<kMegaT>(val, idx, p.top_k, L.tk_val, L.tk_idx);
             if (t == 0) {
                 float prob[kTopKMax];
-                const int sel = topk_sample_rank(L.tk_val, p.top_k, p.rands[p.state[1] + step], 1, prob);
+                const int sel = topk_sample_rank(L.tk_val, p.top_k, p.rands[step_base + step], 1, prob);
                 const int chosen = L.tk_idx[sel];
                 L.tk_tok = (unsigned)chosen < (unsigned)p.vocab ? chosen : 0;   // after a time-out the candidates may be anything
                 L.stop = bar.dead || ld_i(bar.err) == 1;
@@ -1286,7 +1290,7 @@ __device__ __forceinline__ void decode_mega_body(const MegaParams& p) {
             __syncthreads();
             tok = __builtin_amdgcn_readfirstlane(L.tk_tok);
             stop = __builtin_amdgcn_readfirstlane(L.stop);
-            if (wg == 0 && t == 0) p.tokens_out[p.state[1] + step] = tok;
+            if (wg == 0 && t == 0) p.tokens_out[step_base + step] = tok;
             __syncthreads();                                        // L.tk_* and L.f are reused by the next step
         } else if (greedy) {
             // every workgroup picks the winner among the kMegaWG candidates (largest value, then smallest index)
@@ -1310,7 +1314,7 @@ __device__ __forceinline__ void decode_mega_body(const MegaParams& p) {
                 if (L.bestv[i] > cv || (L.bestv[i] == cv && L.besti[i] < ci)) { cv = L.bestv[i]; ci = L.besti[i]; }
             tok = __builtin_amdgcn_readfirstlane((unsigned)ci < (unsigned)p.vocab ? ci : 0);   // after a time-out the candidates may be anything
             stop = __builtin_amdgcn_readfirstlane(L.stop);
-            if (wg == 0 && t == 0) p.tokens_out[p.state[1] + step] = tok;
+            if (wg == 0 && t == 0) p.tokens_out[step_base + step] = tok;
             __syncthreads();                                        // L.bestv/besti are reused by the next step
         }
     }
@@ -1319,7 +1323,7 @@ __device__ __forceinline__ void decode_mega_body(const MegaParams& p) {
     if (wg == 0 && is_t0()) {
         p.state[2] = (int)bar.epoch;
         p.state[4] = (int)(seq0 + (unsigned)(steps_done * p.n_layers));
-        if (greedy) { p.token[0] = tok; p.state[0] = pos0 + steps_done; p.state[1] += steps_done; }
+        if (greedy) { p.token[0] = tok; p.state[0] = pos0 + steps_done; p.state[1] = step_base + steps_done; }
     }
 #ifdef FX_MEGA_FINE_STAMPS
     if (p.timeline && is_t0()) p.timeline[p.n_layers * 12 + 2 + 64 + kMegaWG + wg] = wall_clock64();     // workgroup exit
