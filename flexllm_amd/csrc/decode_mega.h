@@ -741,6 +741,10 @@ __device__ __forceinline__ void decode_mega_body(const MegaParams& p) {
                     }
                 }
             } else {
+                // A workgroup without a key chunk keeps the pace of the others: its two slices issued at once, right
+                // behind phase 1, crowd the q/k/v and statistics hand-overs of the workgroups that have one (-10 us per
+                // token at half the maximum context).  The others need longer the more chunks exchange statistics.
+                __builtin_amdgcn_s_sleep(40);
                 gu_slice(1);
             }
             stamp();
@@ -817,6 +821,8 @@ __device__ __forceinline__ void decode_mega_body(const MegaParams& p) {
                     }
                 }
             } else {
+                __builtin_amdgcn_s_sleep(56);
+                for (int i = 0; i < min(nchunks, 8); i++) __builtin_amdgcn_s_sleep(5);
                 gu_slice(2);
             }
             stamp();
