@@ -14,6 +14,8 @@
 // P = min(255, round(p/A_s)) and accumulates P.V.  P is unsigned and the MFMA is signed x signed: (P-128).V is
 // accumulated and 128*colsum(V) over the same keys is added at the end, both exact in int32.
 #pragma once
+#include <type_traits>
+
 #include "attn_decode_kernels.h"
 
 namespace fx {
@@ -101,12 +103,14 @@ __device__ __forceinline__ int pf_round4(const float (&e)[4], float kq, float cd
 // roundings of max and m2: it cancels between the probability and the row sum, and the exact path's denominator is
 // the fast row sum times that factor, `pf_fast_row`) and per element by at most R = 2^-24 (3|max| + 9 X + 12) + 1e-6
 // relative, X = ln(kq / 0.4) bounding |score - max| of every probability that can reach 0.4 (float32 model of both
-// paths, tests/test_attention_fast_path_cpu.py: worst observed deviation 0.3 R).  So q~ = e~ * kq rounds like the reference's
-// expression unless it lies within win = 1e-4 + kq R of a tie; those groups of four are redone exactly (about 1e-4
-// of the elements).
+// paths, tests/test_attention_fast_path_cpu.py: worst observed deviation 0.3 R).  q~ = e~ * kq adds the roundings of
+// kq = fl(fl(1/sum) * fl(1/A_s)) and of the product, under 4e-7 relative.  So q~ rounds like the reference's expression
+// unless it lies within q~ * rel + 1e-6 of a tie, rel = R + 4e-7.  The check has two levels: one comparison for a group
+// of four against the widest window any of them can have (win, from q~ <= kq), and only in a group that fails it each
+// element against its own window; a group with an element inside its own window is redone exactly (a few in 1e5).
 struct PfFastRow {
     float c2, m2, imf;       // e~ = 2^(tv * c2 - m2), m2 = fl(imf * c2), imf = the row's integer maximum
-    float kq, win, cd;       // q~ = e~ * kq; redo within win of a tie, with the denominator cd
+    float kq, win, rel, cd;  // q~ = e~ * kq; windows as above; cd: the exact path's 1 / denominator
 };
 // With c2 below 2e-5 a masked score (-2^31) would not reach 2^-150, i.e. an e~ of exactly 0: such heads take the
 // exact path throughout.
@@ -124,14 +128,14 @@ __device__ __forceinline__ void pf_fast_row_finish(PfFastRow& f, float total, fl
     f.cd = 1.0f / (total * (1.0f + offset));
     f.kq = (1.0f / total) * (1.0f / as);
     const float x_max = fmaxf(0.0f, __logf(f.kq) + 0.92f);
-    const float rel = 5.9604645e-8f * (3.0f * fabsf(mx) + 9.0f * x_max + 12.0f) + 1e-6f;
-    f.win = 1e-4f + f.kq * rel;
+    f.rel = 5.9604645e-8f * (3.0f * fabsf(mx) + 9.0f * x_max + 12.0f) + 1.4e-6f;
+    f.win = 1e-6f + 1.01f * f.kq * f.rel;                                // e~ <= 1 up to its last bits: q~ <= 1.01 kq
 }
 __device__ __forceinline__ float pf_fast_exp(int tv, const PfFastRow& f) {
     return __builtin_amdgcn_exp2f(__builtin_fmaf((float)tv, f.c2, -f.m2));   // a masked score (-2^31) gives 0
 }
 // Four e~ -> four probability bytes (biased by 128, as pf_round4).  exact(b): the exact exponential of element b, only
-// evaluated for a group near a tie.
+// evaluated for a group with an element near a tie.
 template <class Exact>
 __device__ __forceinline__ int pf_round4_fast(const float (&ef)[4], const PfFastRow& f, float as, Exact exact, unsigned& bytes) {
     float qv[4];
@@ -140,7 +144,11 @@ __device__ __forceinline__ int pf_round4_fast(const float (&ef)[4], const PfFast
     const float d0 = fabsf(__builtin_amdgcn_fractf(qv[0]) - 0.5f), d1 = fabsf(__builtin_amdgcn_fractf(qv[1]) - 0.5f);
     const float d2 = fabsf(__builtin_amdgcn_fractf(qv[2]) - 0.5f), d3 = fabsf(__builtin_amdgcn_fractf(qv[3]) - 0.5f);
     unsigned packed = 0;
-    if (fminf(fminf(d0, d1), fminf(d2, d3)) < f.win) {
+    bool redo = fminf(fminf(d0, d1), fminf(d2, d3)) < f.win;
+    if (redo)
+        redo = d0 < __builtin_fmaf(qv[0], f.rel, 1e-6f) || d1 < __builtin_fmaf(qv[1], f.rel, 1e-6f) ||
+               d2 < __builtin_fmaf(qv[2], f.rel, 1e-6f) || d3 < __builtin_fmaf(qv[3], f.rel, 1e-6f);
+    if (redo) {
 #pragma unroll
         for (int b = 0; b < 4; b++) {
             int v = (int)roundf((exact(b) * f.cd) / as);
@@ -187,7 +195,11 @@ __device__ __forceinline__ void pf_reduce_store(int (*lds_acc)[35], const i32x16
 // from the one-rounding exponentials e~ (PfFastRow).  Pass 2: the probabilities from the same e~, rounded as described
 // there, the groups near a tie from the accurate exponential of the reference's own score expression; and P.V.  Heads
 // whose scales rule the fast path out (pf_fast_ok) take the accurate exponential for every probability.
-static __global__ __launch_bounds__(64 * kPfWaves) void pf_attention_kernel(const int8_t* __restrict__ q8, const int8_t* __restrict__ kc,
+// The choice between the two and the optional copy of the probability bytes (kStoreP) are made outside the tile loops,
+// and the K rows of the next tile are requested into the registers of the current one as soon as its scores are formed:
+// per probability the loops issue the arithmetic and little else.
+template <bool kStoreP>
+static __global__ __launch_bounds__(64 * kPfWaves, 4) void pf_attention_kernel(const int8_t* __restrict__ q8, const int8_t* __restrict__ kc,
                                                                   const int8_t* __restrict__ vc, const float* __restrict__ q_s,
                                                                   const float* __restrict__ k_s, const float* __restrict__ v_s,
                                                                   const float* __restrict__ a_s, float* __restrict__ o,
@@ -211,10 +223,11 @@ static __global__ __launch_bounds__(64 * kPfWaves) void pf_attention_kernel(cons
         kf1 = *reinterpret_cast<const i32x4*>(krow + 32 + g * 16);
     };
     // integer scores of one tile: register r is key k0 + 16g + r; keys beyond the query (diagonal tile only) are masked
-    auto int_tile = [&](int kt, const i32x4& kf0, const i32x4& kf1, int (&tv)[16]) {
+    auto int_tile = [&](int kt, const i32x4& kf0, const i32x4& kf1, int (&tv)[16], auto&& refill) {
         i32x16 acc = zero16();
         acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(kf0, qf0, acc, 0, 0, 0);
         acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(kf1, qf1, acc, 0, 0, 0);
+        refill();
         if (kt == it.qb) {
 #pragma unroll
             for (int r = 0; r < 16; r++) tv[r] = (it.q0 + 16 * g + r) <= query ? acc[r] : kPfMasked;
@@ -223,22 +236,26 @@ static __global__ __launch_bounds__(64 * kPfWaves) void pf_attention_kernel(cons
             for (int r = 0; r < 16; r++) tv[r] = acc[r];
         }
     };
+    // body(kt, kf0, kf1, refill) for this wave's tiles kt = wave, wave + kPfWaves, ...  One register set holds the K
+    // rows: the body calls refill() as soon as its two score products have been issued, which requests the next
+    // tile's rows into the same registers, and the arithmetic on the scores that follows covers their way from the
+    // cache.  No second set, nothing moved between trips.
+    auto for_tiles = [&](auto&& body) {
+        i32x4 kf0, kf1;
+        if (wave < ntiles) load_k(wave * kPfTile, kf0, kf1);
+        for (int kt = wave; kt < ntiles; kt += kPfWaves)
+            body(kt, kf0, kf1, [&] { if (kt + kPfWaves < ntiles) load_k((kt + kPfWaves) * kPfTile, kf0, kf1); });
+    };
 
     for (int i = threadIdx.x; i < 64 * 35; i += 64 * kPfWaves) (&lds_acc[0][0])[i] = 0;
     // ---- pass 0: integer row maximum ----
     int imax = kPfMasked;
-    {
-        i32x4 kf0, kf1, nf0, nf1;
-        if (wave < ntiles) load_k(wave * kPfTile, kf0, kf1);
-        for (int kt = wave; kt < ntiles; kt += kPfWaves) {
-            if (kt + kPfWaves < ntiles) load_k((kt + kPfWaves) * kPfTile, nf0, nf1);
-            int tv[16];
-            int_tile(kt, kf0, kf1, tv);
+    for_tiles([&](int kt, const i32x4& kf0, const i32x4& kf1, auto&& refill) {
+        int tv[16];
+        int_tile(kt, kf0, kf1, tv, refill);
 #pragma unroll
-            for (int r = 0; r < 16; r++) imax = max(imax, tv[r]);
-            kf0 = nf0; kf1 = nf1;
-        }
-    }
+        for (int r = 0; r < 16; r++) imax = max(imax, tv[r]);
+    });
     imax = max(imax, lane_xor_i<32>(imax));
     if (g == 0) lds_mi[wave][col] = imax;
     __syncthreads();
@@ -253,17 +270,18 @@ static __global__ __launch_bounds__(64 * kPfWaves) void pf_attention_kernel(cons
     PfFastRow fr;
     pf_fast_row_begin(fr, im, c2);
     float lsum = 0.0f;
-    {
-        i32x4 kf0, kf1, nf0, nf1;
-        if (wave < ntiles) load_k(wave * kPfTile, kf0, kf1);
-        for (int kt = wave; kt < ntiles; kt += kPfWaves) {
-            if (kt + kPfWaves < ntiles) load_k((kt + kPfWaves) * kPfTile, nf0, nf1);
+    if (fast) {
+        for_tiles([&](int kt, const i32x4& kf0, const i32x4& kf1, auto&& refill) {
             int tv[16];
-            int_tile(kt, kf0, kf1, tv);
-            if (fast) {                                        // the same e~ as in pass 2; masked keys come out as 0
+            int_tile(kt, kf0, kf1, tv, refill);
 #pragma unroll
-                for (int r = 0; r < 16; r++) lsum += pf_fast_exp(tv[r], fr);
-            } else if (kt == it.qb) {
+            for (int r = 0; r < 16; r++) lsum += pf_fast_exp(tv[r], fr);   // the same e~ as in pass 2; masked keys come out as 0
+        });
+    } else {
+        for_tiles([&](int kt, const i32x4& kf0, const i32x4& kf1, auto&& refill) {
+            int tv[16];
+            int_tile(kt, kf0, kf1, tv, refill);
+            if (kt == it.qb) {
 #pragma unroll
                 for (int r = 0; r < 16; r++)
                     lsum += tv[r] == kPfMasked ? 0.0f : __builtin_amdgcn_exp2f(fminf(__builtin_fmaf((float)tv[r], c2, -m2), 0.0f));
@@ -271,8 +289,7 @@ static __global__ __launch_bounds__(64 * kPfWaves) void pf_attention_kernel(cons
 #pragma unroll
                 for (int r = 0; r < 16; r++) lsum += __builtin_amdgcn_exp2f(fminf(__builtin_fmaf((float)tv[r], c2, -m2), 0.0f));
             }
-            kf0 = nf0; kf1 = nf1;
-        }
+        });
     }
     lsum = lsum + lane_xor_f<32>(lsum);
     if (g == 0) lds_l[wave][col] = lsum;
@@ -288,44 +305,42 @@ static __global__ __launch_bounds__(64 * kPfWaves) void pf_attention_kernel(cons
     // ---- pass 2: probabilities, partial P.V over this wave's tiles ----
     i32x16 oacc0 = zero16(), oacc1 = zero16();
     int vsum0 = 0, vsum1 = 0;
-    {
-        i32x4 kf0, kf1, nf0, nf1;
-        if (wave < ntiles) load_k(wave * kPfTile, kf0, kf1);
-        for (int kt = wave; kt < ntiles; kt += kPfWaves) {
+    uint8_t* const prow = kStoreP ? p8_out + ((size_t)it.h * s + query) * s + 16 * g : nullptr;
+    auto pass2 = [&](auto fast_c) {
+        constexpr bool kFast = decltype(fast_c)::value;
+        for_tiles([&](int kt, const i32x4& kf0, const i32x4& kf1, auto&& refill) {
             const int k0 = kt * kPfTile;
-            if (kt + kPfWaves < ntiles) load_k((kt + kPfWaves) * kPfTile, nf0, nf1);
             // B operand of P.V: V[key][d] for this lane's channels col, col+32 and its 16 consecutive keys
             const int8_t* vblk = vc + v_index(it.kvh, k0, 0, max_pos) + 16 * g;
             const i32x4 vf0 = *reinterpret_cast<const i32x4*>(vblk + (size_t)col * kVBlock);
             const i32x4 vf1 = *reinterpret_cast<const i32x4*>(vblk + (size_t)(col + 32) * kVBlock);
             int tv[16];
-            int_tile(kt, kf0, kf1, tv);
+            int_tile(kt, kf0, kf1, tv, refill);
             i32x4 pf;
+            unsigned bytes[4];
 #pragma unroll
             for (int a = 0; a < 4; a++) {
                 float e[4];
-                unsigned bytes;
-                if (fast) {
+                if constexpr (kFast) {
 #pragma unroll
                     for (int b = 0; b < 4; b++) e[b] = pf_fast_exp(tv[a * 4 + b], fr);
                     pf[a] = pf_round4_fast(e, fr, as, [&](int b) {
                         const int ts = tv[a * 4 + b];
                         return ts == kPfMasked ? 0.0f : exp_f<false>((float)ts * sq * sk - mx);
-                    }, bytes);
-                    if (p8_out) *reinterpret_cast<unsigned*>(p8_out + ((size_t)it.h * s + query) * s + k0 + 16 * g + a * 4) = bytes;
-                    continue;
-                }
-                if (kt == it.qb) {                             // uniform: only the diagonal tile has masked keys
-#pragma unroll
-                    for (int b = 0; b < 4; b++)                // masked keys: exactly 0 whatever the scales
-                        e[b] = tv[a * 4 + b] == kPfMasked ? 0.0f : exp_f<false>((float)tv[a * 4 + b] * sq * sk - mx);
+                    }, bytes[a]);
                 } else {
+                    if (kt == it.qb) {                         // uniform: only the diagonal tile has masked keys
 #pragma unroll
-                    for (int b = 0; b < 4; b++) e[b] = exp_f<false>((float)tv[a * 4 + b] * sq * sk - mx);
+                        for (int b = 0; b < 4; b++)            // masked keys: exactly 0 whatever the scales
+                            e[b] = tv[a * 4 + b] == kPfMasked ? 0.0f : exp_f<false>((float)tv[a * 4 + b] * sq * sk - mx);
+                    } else {
+#pragma unroll
+                        for (int b = 0; b < 4; b++) e[b] = exp_f<false>((float)tv[a * 4 + b] * sq * sk - mx);
+                    }
+                    pf[a] = pf_round4(e, kq, cd, as, fast_q, bytes[a]);
                 }
-                pf[a] = pf_round4(e, kq, cd, as, fast_q, bytes);
-                if (p8_out) *reinterpret_cast<unsigned*>(p8_out + ((size_t)it.h * s + query) * s + k0 + 16 * g + a * 4) = bytes;
             }
+            if constexpr (kStoreP) *reinterpret_cast<uint4*>(prow + k0) = make_uint4(bytes[0], bytes[1], bytes[2], bytes[3]);
 #pragma unroll
             for (int a = 0; a < 4; a++) {
                 vsum0 = __builtin_amdgcn_sdot4(0x01010101, vf0[a], vsum0, false);
@@ -333,9 +348,9 @@ static __global__ __launch_bounds__(64 * kPfWaves) void pf_attention_kernel(cons
             }
             oacc0 = __builtin_amdgcn_mfma_i32_32x32x32_i8(pf, vf0, oacc0, 0, 0, 0);
             oacc1 = __builtin_amdgcn_mfma_i32_32x32x32_i8(pf, vf1, oacc1, 0, 0, 0);
-            kf0 = nf0; kf1 = nf1;
-        }
-    }
+        });
+    };
+    if (fast) pass2(std::true_type{}); else pass2(std::false_type{});
     pf_reduce_store(lds_acc, oacc0, oacc1, vsum0, vsum1, wave < ntiles, it, a_s[it.h], v_s[it.kvh], o, q_heads);
 }
 
@@ -345,6 +360,7 @@ static __global__ __launch_bounds__(64 * kPfWaves) void pf_attention_kernel(cons
 // replace the integers in place, and the last pass only scales, rounds and multiplies with V.  This is also the
 // reference's own order (maximum, then exponentials and their sum, then probabilities from the same exponentials).
 constexpr int kPfCachedTiles = 4;
+template <bool kStoreP>
 static __global__ __launch_bounds__(64 * kPfWaves, 2) void pf_attention_cached_kernel(
     const int8_t* __restrict__ q8, const int8_t* __restrict__ kc, const int8_t* __restrict__ vc, const float* __restrict__ q_s,
     const float* __restrict__ k_s, const float* __restrict__ v_s, const float* __restrict__ a_s, float* __restrict__ o,
@@ -372,16 +388,19 @@ static __global__ __launch_bounds__(64 * kPfWaves, 2) void pf_attention_cached_k
     int tv[kPfCachedTiles][16];
     int imax = kPfMasked;
     {
-        i32x4 kf0, kf1, nf0, nf1;
-        if (wave < ntiles) load_k(wave * kPfTile, kf0, kf1);
+        // the K rows of all of this wave's tiles are requested at once: one trip to memory instead of one per tile (the
+        // registers they take are those that the scores of the later tiles fill afterwards)
+        i32x4 kf[kPfCachedTiles][2];
+#pragma unroll
+        for (int i = 0; i < kPfCachedTiles; i++)
+            if (wave + kPfWaves * i < ntiles) load_k((wave + kPfWaves * i) * kPfTile, kf[i][0], kf[i][1]);
 #pragma unroll
         for (int i = 0; i < kPfCachedTiles; i++) {
             const int kt = wave + kPfWaves * i;
             if (kt < ntiles) {
-                if (kt + kPfWaves < ntiles) load_k((kt + kPfWaves) * kPfTile, nf0, nf1);
                 i32x16 acc = zero16();
-                acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(kf0, qf0, acc, 0, 0, 0);
-                acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(kf1, qf1, acc, 0, 0, 0);
+                acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(kf[i][0], qf0, acc, 0, 0, 0);
+                acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(kf[i][1], qf1, acc, 0, 0, 0);
                 if (kt == it.qb) {                             // only the diagonal tile has keys beyond the query
 #pragma unroll
                     for (int r = 0; r < 16; r++) tv[i][r] = (it.q0 + 16 * g + r) <= query ? acc[r] : kPfMasked;
@@ -391,7 +410,6 @@ static __global__ __launch_bounds__(64 * kPfWaves, 2) void pf_attention_cached_k
                 }
 #pragma unroll
                 for (int r = 0; r < 16; r++) imax = max(imax, tv[i][r]);
-                kf0 = nf0; kf1 = nf1;
             }
         }
     }
@@ -404,12 +422,26 @@ static __global__ __launch_bounds__(64 * kPfWaves, 2) void pf_attention_cached_k
     const float mx = (float)im * sq * sk;                      // int -> float and the positive scales keep the order
 
     // ---- pass 1: exponentials with the final maximum, in place; row sum ----
+    // Heads whose scales allow it (pf_fast_ok) keep the one-rounding exponentials e~ of PfFastRow, the others the
+    // accurate ones.
+    const float c2 = sq * sk * 1.44269502162933349609375f;
+    // (a row block with at most one tile per wave gains nothing from them and stays on the accurate ones: measured)
+    const bool fast = pf_fast_ok(c2, as) && ntiles > kPfWaves;   // per head and workgroup: uniform
+    PfFastRow fr;
+    pf_fast_row_begin(fr, im, c2);
     float lsum = 0.0f;
 #pragma unroll
     for (int i = 0; i < kPfCachedTiles; i++) {
         const int kt = wave + kPfWaves * i;
         if (kt < ntiles) {
-            if (kt == it.qb) {                                 // uniform: only the diagonal tile has masked keys
+            if (fast) {                                        // a masked score (-2^31) gives an e~ of 0
+#pragma unroll
+                for (int r = 0; r < 16; r++) {
+                    const float e = pf_fast_exp(tv[i][r], fr);
+                    tv[i][r] = __float_as_int(e);
+                    lsum += e;
+                }
+            } else if (kt == it.qb) {                          // uniform: only the diagonal tile has masked keys
 #pragma unroll
                 for (int r = 0; r < 16; r++) {                 // they count as exp(-1e32 - max) = 0 whatever the scales
                     const float e = tv[i][r] == kPfMasked ? 0.0f : exp_f<false>((float)tv[i][r] * sq * sk - mx);
@@ -435,10 +467,17 @@ static __global__ __launch_bounds__(64 * kPfWaves, 2) void pf_attention_cached_k
     const float cd = 1.0f / total;
     const bool fast_q = quant_fast_ok(as);
     const float kq = cd * (1.0f / as);
+    float kqf = 0.0f, win = 0.0f;                              // fast path: q~ = e~ * kqf, the groups' window
+    if (fast) {
+        pf_fast_row_finish(fr, total, sq, sk, mx, as);
+        kqf = fr.kq;
+        win = fr.win;
+    }
 
     // ---- pass 2: probabilities from the kept exponentials, partial P.V ----
     i32x16 oacc0 = zero16(), oacc1 = zero16();
     int vsum0 = 0, vsum1 = 0;
+    unsigned near = 0;                                         // fast path: bit 4 i + a = group a of tile i may hold a rounding tie
 #pragma unroll
     for (int i = 0; i < kPfCachedTiles; i++) {
         const int kt = wave + kPfWaves * i;
@@ -448,14 +487,39 @@ static __global__ __launch_bounds__(64 * kPfWaves, 2) void pf_attention_cached_k
             const i32x4 vf0 = *reinterpret_cast<const i32x4*>(vblk + (size_t)col * kVBlock);
             const i32x4 vf1 = *reinterpret_cast<const i32x4*>(vblk + (size_t)(col + 32) * kVBlock);
             i32x4 pf;
+            unsigned bytes[4];
+            if (fast) {
+                // q~ = e~ * kq, rounded by the conversion.  A group of four with an element within the row's window
+                // of a tie (PfFastRow) is only noted here, one bit per group, and put right after the loop.
 #pragma unroll
-            for (int a = 0; a < 4; a++) {
-                const float e[4] = {__int_as_float(tv[i][a * 4]), __int_as_float(tv[i][a * 4 + 1]), __int_as_float(tv[i][a * 4 + 2]),
-                                    __int_as_float(tv[i][a * 4 + 3])};
-                unsigned bytes;
-                pf[a] = pf_round4(e, kq, cd, as, fast_q, bytes);
-                if (p8_out) *reinterpret_cast<unsigned*>(p8_out + ((size_t)it.h * s + query) * s + k0 + 16 * g + a * 4) = bytes;
+                for (int a = 0; a < 4; a++) {
+                    float qv[4];
+#pragma unroll
+                    for (int b = 0; b < 4; b++) qv[b] = __int_as_float(tv[i][a * 4 + b]) * kqf;
+                    const float d0 = fabsf(__builtin_amdgcn_fractf(qv[0]) - 0.5f), d1 = fabsf(__builtin_amdgcn_fractf(qv[1]) - 0.5f);
+                    const float d2 = fabsf(__builtin_amdgcn_fractf(qv[2]) - 0.5f), d3 = fabsf(__builtin_amdgcn_fractf(qv[3]) - 0.5f);
+                    if (fminf(fminf(d0, d1), fminf(d2, d3)) < win) {          // about one group in 10^4: each element's own window,
+                        const float rel = win * __builtin_amdgcn_rcpf(kqf) * 1.001f;   // with a factor that is not below PfFastRow's
+                        if (d0 < __builtin_fmaf(qv[0], rel, 1e-6f) || d1 < __builtin_fmaf(qv[1], rel, 1e-6f) ||
+                            d2 < __builtin_fmaf(qv[2], rel, 1e-6f) || d3 < __builtin_fmaf(qv[3], rel, 1e-6f))
+                            near |= 1u << (4 * i + a);
+                    }
+                    unsigned packed = 0;
+#pragma unroll
+                    for (int b = 0; b < 4; b++) packed = __builtin_amdgcn_cvt_pk_u8_f32(qv[b], b, packed);
+                    bytes[a] = packed;
+                    pf[a] = (int)(packed ^ 0x80808080u);
+                }
+            } else {
+#pragma unroll
+                for (int a = 0; a < 4; a++) {
+                    const float e[4] = {__int_as_float(tv[i][a * 4]), __int_as_float(tv[i][a * 4 + 1]), __int_as_float(tv[i][a * 4 + 2]),
+                                        __int_as_float(tv[i][a * 4 + 3])};
+                    pf[a] = pf_round4(e, kq, cd, as, fast_q, bytes[a]);
+                }
             }
+            if constexpr (kStoreP)
+                *reinterpret_cast<uint4*>(p8_out + ((size_t)it.h * s + query) * s + k0 + 16 * g) = make_uint4(bytes[0], bytes[1], bytes[2], bytes[3]);
 #pragma unroll
             for (int a = 0; a < 4; a++) {
                 vsum0 = __builtin_amdgcn_sdot4(0x01010101, vf0[a], vsum0, false);
@@ -463,6 +527,74 @@ static __global__ __launch_bounds__(64 * kPfWaves, 2) void pf_attention_cached_k
             }
             oacc0 = __builtin_amdgcn_mfma_i32_32x32x32_i8(pf, vf0, oacc0, 0, 0, 0);
             oacc1 = __builtin_amdgcn_mfma_i32_32x32x32_i8(pf, vf1, oacc1, 0, 0, 0);
+        }
+    }
+    // ---- the noted groups (fast path; a few tiles in a hundred have one in some lane) ----
+    // The integer scores are gone (the e~ took their registers), so a tile with a noted group in any lane is formed
+    // again by the whole wave (the matrix instruction works on all lanes): scores, the same e~ and fast bytes as above,
+    // and for the noted groups the bytes of pf_round4_fast.  P.V is linear in P: the difference of the two (a byte
+    // moves by one at most) times V is added to the accumulators, which is exact in int32.
+    // What this needs of the row (query operand, maximum, sum and what follows from them) is fetched and formed again
+    // here instead of being kept in registers through the loop above, which has none to spare.
+    if (fast && __builtin_amdgcn_ballot_w64(near != 0) != 0) {
+        int query2 = it.q0 + (int)(threadIdx.x & 31);
+        asm volatile("" : "+v"(query2) : : "memory");         // a value the compiler knows nothing about: really loaded again
+        const int8_t* qrow2 = q8 + ((size_t)query2 * q_heads + it.h) * kHd;
+        const i32x4 qf0 = *reinterpret_cast<const i32x4*>(qrow2 + g * 16);
+        const i32x4 qf1 = *reinterpret_cast<const i32x4*>(qrow2 + 32 + g * 16);
+        int im = lds_mi[0][col];
+        float total = lds_l[0][col];
+#pragma unroll
+        for (int w = 1; w < kPfWaves; w++) {
+            im = max(im, lds_mi[w][col]);
+            total += lds_l[w][col];
+        }
+        const float mx = (float)im * sq * sk;
+        PfFastRow fr;
+        pf_fast_row_begin(fr, im, sq * sk * 1.44269502162933349609375f);
+        pf_fast_row_finish(fr, total, sq, sk, mx, as);
+#pragma unroll
+        for (int i = 0; i < kPfCachedTiles; i++) {
+            const int kt = wave + kPfWaves * i;
+            const unsigned nb = (near >> (4 * i)) & 15u;
+            if (kt < ntiles && __builtin_amdgcn_ballot_w64(nb != 0) != 0) {
+                const int k0 = kt * kPfTile;
+                i32x4 kf0, kf1;
+                load_k(k0, kf0, kf1);
+                const int8_t* vblk = vc + v_index(it.kvh, k0, 0, max_pos) + 16 * g;
+                const i32x4 vf0 = *reinterpret_cast<const i32x4*>(vblk + (size_t)col * kVBlock);
+                const i32x4 vf1 = *reinterpret_cast<const i32x4*>(vblk + (size_t)(col + 32) * kVBlock);
+                i32x16 acc = zero16();
+                acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(kf0, qf0, acc, 0, 0, 0);
+                acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(kf1, qf1, acc, 0, 0, 0);
+                i32x4 dp = {0, 0, 0, 0};
+#pragma unroll
+                for (int a = 0; a < 4; a++) {
+                    if (nb >> a & 1) {
+                        int ts[4];
+                        float e[4];
+                        unsigned fastb = 0, exb;
+#pragma unroll
+                        for (int b = 0; b < 4; b++) {
+                            ts[b] = kt == it.qb && (it.q0 + 16 * g + a * 4 + b) > query ? kPfMasked : acc[a * 4 + b];
+                            e[b] = pf_fast_exp(ts[b], fr);
+                            fastb = __builtin_amdgcn_cvt_pk_u8_f32(e[b] * fr.kq, b, fastb);
+                        }
+                        pf_round4_fast(e, fr, as, [&](int b) {
+                            return ts[b] == kPfMasked ? 0.0f : exp_f<false>((float)ts[b] * sq * sk - mx);
+                        }, exb);
+                        unsigned d = 0;
+#pragma unroll
+                        for (int b = 0; b < 4; b++)
+                            d |= (((exb >> (8 * b)) & 255u) - ((fastb >> (8 * b)) & 255u) & 255u) << (8 * b);
+                        dp[a] = (int)d;
+                        if constexpr (kStoreP)
+                            *reinterpret_cast<unsigned*>(p8_out + ((size_t)it.h * s + query) * s + k0 + 16 * g + 4 * a) = exb;
+                    }
+                }
+                oacc0 = __builtin_amdgcn_mfma_i32_32x32x32_i8(dp, vf0, oacc0, 0, 0, 0);
+                oacc1 = __builtin_amdgcn_mfma_i32_32x32x32_i8(dp, vf1, oacc1, 0, 0, 0);
+            }
         }
     }
     pf_reduce_store(lds_acc, oacc0, oacc1, vsum0, vsum1, wave < ntiles, it, a_s[it.h], v_s[it.kvh], o, q_heads);
@@ -479,12 +611,14 @@ inline int mha_prefill_launch(const int8_t* q8, const int8_t* kc, const int8_t* 
         if (n_cu <= 0) n_cu = 256;
     }
     static const bool no_cached = getenv("FLEXLLM_ATTN_RECOMPUTE") != nullptr;      // forces the two-pass kernel (comparison runs)
-    if (s <= kPfTile * kPfWaves * kPfCachedTiles && !no_cached)
-        pf_attention_cached_kernel<<<(s / kPfTile) * q_heads, 64 * kPfWaves, 0, st>>>(q8, kc, vc, q_s, k_s, v_s, a_s, o, p8_out, s, q_heads,
-                                                                          q_heads / kv_heads, max_pos, n_cu);
-    else
-        pf_attention_kernel<<<(s / kPfTile) * q_heads, 64 * kPfWaves, 0, st>>>(q8, kc, vc, q_s, k_s, v_s, a_s, o, p8_out, s, q_heads,
-                                                                   q_heads / kv_heads, max_pos, n_cu);
+    const dim3 grid((s / kPfTile) * q_heads), block(64 * kPfWaves);
+    const int group = q_heads / kv_heads;
+    const bool cached = s <= kPfTile * kPfWaves * kPfCachedTiles && !no_cached;
+    // the copy of the probability bytes (p8_out, a test and inspection output) is compiled out of the usual instances
+    if (cached && p8_out) pf_attention_cached_kernel<true><<<grid, block, 0, st>>>(q8, kc, vc, q_s, k_s, v_s, a_s, o, p8_out, s, q_heads, group, max_pos, n_cu);
+    else if (cached) pf_attention_cached_kernel<false><<<grid, block, 0, st>>>(q8, kc, vc, q_s, k_s, v_s, a_s, o, p8_out, s, q_heads, group, max_pos, n_cu);
+    else if (p8_out) pf_attention_kernel<true><<<grid, block, 0, st>>>(q8, kc, vc, q_s, k_s, v_s, a_s, o, p8_out, s, q_heads, group, max_pos, n_cu);
+    else pf_attention_kernel<false><<<grid, block, 0, st>>>(q8, kc, vc, q_s, k_s, v_s, a_s, o, p8_out, s, q_heads, group, max_pos, n_cu);
     FX_LAUNCH_CHECK();
     return FLEXLLM_OK;
 }

@@ -2,8 +2,8 @@
 
 * exact: the reference's expression, exp(fl(fl(tv*Q_s)*K_s) - max) with the kernels' two-part exponential, times
   1/sum, divided by A_s, rounded half away (Modules/Softmax.h:456-635 as the oracle restates it);
-* fast: e~ = 2^(tv*c2 - m2), q~ = e~ * kq, rounded by the conversion instruction, taken unless q~ lies within the
-  row's window of a tie.
+* fast: e~ = 2^(tv*c2 - m2), q~ = e~ * kq, rounded by the conversion instruction, taken unless a q~ of its group of
+  four lies within its own window (proportional to q~) of a tie.
 
 The kernel's claim is that outside the window both give the same byte.  The model draws rows over a range of scales
 and score spreads, perturbs every hardware 2^x by up to one ulp either way, and checks exactly that, plus the size
@@ -57,11 +57,15 @@ def rows(seed, n_rows, n_keys, sq, sk, spread, a_s=f32(1.0 / 255)):
         cd = (f32(1) / (total * (f32(1) + offset)).astype(f32)).astype(f32)
         kq = ((f32(1) / total).astype(f32) * (f32(1) / a_s).astype(f32)).astype(f32)
         x_max = max(0.0, float(np.log(kq)) + 0.92)
-        rel = 5.9604645e-8 * (3.0 * abs(float(mx)) + 9.0 * x_max + 12.0) + 1e-6
-        win = 1e-4 + float(kq) * rel
+        rel = 5.9604645e-8 * (3.0 * abs(float(mx)) + 9.0 * x_max + 12.0) + 1.4e-6
+        win = 1e-6 + 1.01 * float(kq) * rel
         qf = (ef * kq).astype(f32)
         qe = ((e * cd).astype(f32) / a_s).astype(f32)
-        near = np.abs((qf - np.floor(qf)) - f32(0.5)) < win
+        d = np.abs((qf - np.floor(qf)) - f32(0.5))
+        assert float(qf.max()) <= 1.01 * float(kq)                  # the group check's window covers every element's own
+        near_el = d < fma(qf, f32(rel), f32(1e-6))                  # the element's own window
+        grp = (d.reshape(-1, 4).min(axis=1) < win) & near_el.reshape(-1, 4).any(axis=1)   # groups of four redone exactly
+        near = np.repeat(grp, 4)
         p_exact = np.minimum(255, np.floor(qe.astype(np.float64) + 0.5)).astype(np.int64)      # half away from zero
         p_fast = np.minimum(255, np.rint(qf.astype(np.float64))).astype(np.int64)              # nearest, ties to even
         outside += int(((p_exact != p_fast) & ~near).sum())
@@ -69,7 +73,7 @@ def rows(seed, n_rows, n_keys, sq, sk, spread, a_s=f32(1.0 / 255)):
         total_n += n_keys
         m = qe > 0.3
         if m.any():
-            worst = max(worst, float((np.abs(qf.astype(np.float64) - qe.astype(np.float64))[m] / (float(kq) * rel)).max()))
+            worst = max(worst, float((np.abs(qf.astype(np.float64) - qe.astype(np.float64))[m] / (qe.astype(np.float64)[m] * rel)).max()))
     return outside, redone / total_n, worst
 
 
@@ -80,4 +84,4 @@ def test_fast_probabilities_equal_the_exact_ones_outside_the_window():
             outside, share, worst = rows(100 + i, n_rows, n_keys, sq, sk, spread)
             assert outside == 0, (sq, sk, spread, n_keys)
             assert worst < 0.5, "deviation %.2f of the bound the window is built from" % worst
-            assert share < 2e-3, "share of elements redone exactly: %.1e" % share
+            assert share < (1e-3 if n_keys < 1024 else 5e-5), "share of elements redone exactly: %.1e" % share

@@ -312,13 +312,17 @@ def test_full_size_prefill_prefix_invariance_and_decode_equivalence(fx):
     pre.close(); dec.close()
 
 
+@pytest.mark.parametrize("s", [1088, 1024], ids=["rows over 1024 keys", "rows up to 1024 keys"])
 @pytest.mark.parametrize("case", ["wide scores", "tiny scales", "peaky rows"])
-def test_mha_prefill_long_rows_fast_and_exact_paths(fx, oracle, case):
-    """Rows of more than 1024 keys (`pf_attention_kernel`) where the fast path of the probabilities is under strain or
+def test_mha_prefill_long_rows_fast_and_exact_paths(fx, oracle, case, s):
+    """Rows of more than 1024 keys (`pf_attention_kernel`) and of up to 1024 keys (`pf_attention_cached_kernel`, whose
+    row blocks of more than 256 keys take the fast probabilities) where the fast path is under strain or
     switched off: scores spread over +-25 (large |max|: the widest window), scales so small that the kernel takes the
     reference's expression for every probability (Q_s K_s log2 e < 2e-5), and rows dominated by one key (the factor
-    255/sum at its largest).  Same criteria as test_mha_prefill_vs_oracle."""
-    s, qh, kvh, hd = 1088, 4, 1, 64
+    255/sum at its largest).  Same criteria as test_mha_prefill_vs_oracle; the output must be the product of the
+    probability bytes the kernel reports with V, bit for bit (this is what ties the groups that are put right after
+    the main loop to the accumulators), and the instance that does not report the bytes must give the same output."""
+    qh, kvh, hd = 4, 1, 64
     r = np.random.default_rng({"wide scores": 31, "tiny scales": 32, "peaky rows": 33}[case])
     q = r.standard_normal((s, qh, hd)).astype(np.float32)
     k = r.standard_normal((s, kvh, hd)).astype(np.float32)
@@ -347,3 +351,5 @@ def test_mha_prefill_long_rows_fast_and_exact_paths(fx, oracle, case):
     acc = np.stack([p[h].astype(np.float64) @ ref["v8"][:, h // group].astype(np.float64) for h in range(qh)], axis=1)
     o_from_p = (acc.astype(np.float32) * a_s[None, :, None]) * np.repeat(v_s, group)[None, :, None]
     assert np.array_equal(o.numpy(), o_from_p.astype(np.float32))
+    o2, _ = fx.ops.mha_i8_prefill(q8, kc, vc, sc, want_p=False)
+    assert np.array_equal(o2.numpy(), o.numpy())
