@@ -160,8 +160,8 @@ def module_legs(fx, lib, synth, ops, stream, Event):
         ops4 = 2 * 2 * QH * S * S * 64
         out["attention_prefill_S%d" % S] = {"us": round(us, 2), "GOP_full_S2": round(ops4 / 1e9, 2), "TOPs_full_S2": round(ops4 / us / 1e6, 1),
                                             "mfma_frac_full_S2": round(ops4 / us / 1e6 / INT8_PEAK_TOPS, 4),
-                                            "note": ("causal half computed, scores kept in registers between the two softmax passes"
-                                                     if S <= 1024 else "causal half computed, scores twice (two-pass softmax)")
+                                            "note": ("causal half computed, scores and then their exponentials kept in registers between the softmax passes"
+                                                     if S <= 1024 else "causal half computed, scores formed again in each of the three passes (maximum, sum, probabilities)")
                                                     + "; bound by the exponential and rounding per probability"}
         del q8, kc, vc, o
     # (5) W4A4 linears (the reference's shipped precision): decode GEMV 2048 -> 8192 on nibble-packed weights

@@ -29,8 +29,8 @@ __device__ __forceinline__ i32x16 zero16() {
     return z;
 }
 
-// grid (s/32 * q_heads), 64 * kPfWaves threads: the waves of a workgroup share one block of 32 queries and split
-// its key tiles round-robin (tile kt goes to wave kt % kPfWaves).  Row statistics are merged through LDS between the
+// grid (s/32 * q_heads), 64 * W threads (W = kPfWaves or kPfLongWaves): the waves of a workgroup share one block of 32
+// queries and split its key tiles round-robin (tile kt goes to wave kt % W).  Row statistics are merged through LDS between the
 // passes; the int32 P.V partial accumulators of the waves are added in LDS at the end (integer adds: exact).
 //
 // Work per query block grows linearly with its index (causal), and workgroups b, b+P, b+2P, ... (P = number of
@@ -46,7 +46,11 @@ __device__ __forceinline__ i32x16 zero16() {
 // exactly evaluated (e * cd) / A_s, so both round alike unless q~ lies within 1e-4 of a tie; those groups of four are
 // redone with the reference's own expression.  The conversion instruction rounds to nearest (ties to even, which only
 // differs from the reference's half-away rule AT a tie, i.e. in a group that is redone anyway) and saturates at 255.
-constexpr int kPfWaves = 8;        // waves per workgroup
+constexpr int kPfWaves = 8;        // waves per workgroup (rows of up to 1024 keys: four tiles of scores per wave in registers)
+// Rows of more than 1024 keys: four waves per workgroup.  What a wave does once (row constants, reductions, the merge of
+// the partial outputs) is a fifth of its instructions at eight tiles per pass; with four waves it is spread over twice
+// the tiles (S = 4096: 196 -> 180 us; two waves: no better, and worse for rows of 1536 keys).
+constexpr int kPfLongWaves = 4;
 constexpr int kPfMasked = -0x7fffffff - 1;
 
 struct PfItem {
@@ -164,6 +168,7 @@ __device__ __forceinline__ int pf_round4_fast(const float (&ef)[4], const PfFast
 }
 
 // Adds the waves' partial accumulators in LDS and writes the block's 32 x 64 outputs.
+template <int kW>
 __device__ __forceinline__ void pf_reduce_store(int (*lds_acc)[35], const i32x16& oacc0, const i32x16& oacc1, int vsum0, int vsum1,
                                                 bool has_tiles, const PfItem& it, float sa, float sv, float* __restrict__ o,
                                                 int q_heads) {
@@ -181,8 +186,8 @@ __device__ __forceinline__ void pf_reduce_store(int (*lds_acc)[35], const i32x16
     const int vs0 = lds_acc[lane][32] + lds_acc[lane ^ 32][32];
     const int vs1 = lds_acc[lane][33] + lds_acc[lane ^ 32][33];
 #pragma unroll
-    for (int rr = 0; rr < 16 / kPfWaves; rr++) {              // each wave writes its share of the 16 accumulator registers
-        const int r = wave * (16 / kPfWaves) + rr;
+    for (int rr = 0; rr < 16 / kW; rr++) {              // each wave writes its share of the 16 accumulator registers
+        const int r = wave * (16 / kW) + rr;
         const int row = it.q0 + (r >> 2) * 8 + it.g * 4 + (r & 3);          // accumulator row = query (standard 32x32 layout)
         float* orow = o + ((size_t)row * q_heads + it.h) * kHd;
         orow[it.col] = (float)(lds_acc[lane][r] + 128 * vs0) * sa * sv;
@@ -198,15 +203,15 @@ __device__ __forceinline__ void pf_reduce_store(int (*lds_acc)[35], const i32x16
 // The choice between the two and the optional copy of the probability bytes (kStoreP) are made outside the tile loops,
 // and the K rows of the next tile are requested into the registers of the current one as soon as its scores are formed:
 // per probability the loops issue the arithmetic and little else.
-template <bool kStoreP>
-static __global__ __launch_bounds__(64 * kPfWaves, 4) void pf_attention_kernel(const int8_t* __restrict__ q8, const int8_t* __restrict__ kc,
+template <bool kStoreP, int kW>
+static __global__ __launch_bounds__(64 * kW, 4) void pf_attention_kernel(const int8_t* __restrict__ q8, const int8_t* __restrict__ kc,
                                                                   const int8_t* __restrict__ vc, const float* __restrict__ q_s,
                                                                   const float* __restrict__ k_s, const float* __restrict__ v_s,
                                                                   const float* __restrict__ a_s, float* __restrict__ o,
                                                                   uint8_t* __restrict__ p8_out, int s, int q_heads, int group,
                                                                   int max_pos, int period) {
-    __shared__ int lds_mi[kPfWaves][32];
-    __shared__ float lds_l[kPfWaves][32];
+    __shared__ int lds_mi[kW][32];
+    __shared__ float lds_l[kW][32];
     __shared__ int lds_acc[64][35];            // [lane][16 acc0 | 16 acc1 | vsum0 | vsum1], odd pitch against bank conflicts
     const int wave = threadIdx.x >> 6;
     const PfItem it = pf_item(s, q_heads, group, period);
@@ -236,18 +241,18 @@ static __global__ __launch_bounds__(64 * kPfWaves, 4) void pf_attention_kernel(c
             for (int r = 0; r < 16; r++) tv[r] = acc[r];
         }
     };
-    // body(kt, kf0, kf1, refill) for this wave's tiles kt = wave, wave + kPfWaves, ...  One register set holds the K
+    // body(kt, kf0, kf1, refill) for this wave's tiles kt = wave, wave + kW, ...  One register set holds the K
     // rows: the body calls refill() as soon as its two score products have been issued, which requests the next
     // tile's rows into the same registers, and the arithmetic on the scores that follows covers their way from the
     // cache.  No second set, nothing moved between trips.
     auto for_tiles = [&](auto&& body) {
         i32x4 kf0, kf1;
         if (wave < ntiles) load_k(wave * kPfTile, kf0, kf1);
-        for (int kt = wave; kt < ntiles; kt += kPfWaves)
-            body(kt, kf0, kf1, [&] { if (kt + kPfWaves < ntiles) load_k((kt + kPfWaves) * kPfTile, kf0, kf1); });
+        for (int kt = wave; kt < ntiles; kt += kW)
+            body(kt, kf0, kf1, [&] { if (kt + kW < ntiles) load_k((kt + kW) * kPfTile, kf0, kf1); });
     };
 
-    for (int i = threadIdx.x; i < 64 * 35; i += 64 * kPfWaves) (&lds_acc[0][0])[i] = 0;
+    for (int i = threadIdx.x; i < 64 * 35; i += 64 * kW) (&lds_acc[0][0])[i] = 0;
     // ---- pass 0: integer row maximum ----
     int imax = kPfMasked;
     for_tiles([&](int kt, const i32x4& kf0, const i32x4& kf1, auto&& refill) {
@@ -261,7 +266,7 @@ static __global__ __launch_bounds__(64 * kPfWaves, 4) void pf_attention_kernel(c
     __syncthreads();
     int im = lds_mi[0][col];
 #pragma unroll
-    for (int w = 1; w < kPfWaves; w++) im = max(im, lds_mi[w][col]);
+    for (int w = 1; w < kW; w++) im = max(im, lds_mi[w][col]);
     const float mx = (float)im * sq * sk;                      // int -> float and the positive scales keep the order
     // ---- pass 1: denominator ----
     const float c2 = sq * sk * 1.44269502162933349609375f;
@@ -296,7 +301,7 @@ static __global__ __launch_bounds__(64 * kPfWaves, 4) void pf_attention_kernel(c
     __syncthreads();
     float total = lds_l[0][col];
 #pragma unroll
-    for (int w = 1; w < kPfWaves; w++) total += lds_l[w][col];
+    for (int w = 1; w < kW; w++) total += lds_l[w][col];
     const float cd = 1.0f / total;
     const bool fast_q = quant_fast_ok(as);
     const float kq = cd * (1.0f / as);
@@ -351,7 +356,7 @@ static __global__ __launch_bounds__(64 * kPfWaves, 4) void pf_attention_kernel(c
         });
     };
     if (fast) pass2(std::true_type{}); else pass2(std::false_type{});
-    pf_reduce_store(lds_acc, oacc0, oacc1, vsum0, vsum1, wave < ntiles, it, a_s[it.h], v_s[it.kvh], o, q_heads);
+    pf_reduce_store<kW>(lds_acc, oacc0, oacc1, vsum0, vsum1, wave < ntiles, it, a_s[it.h], v_s[it.kvh], o, q_heads);
 }
 
 // The same attention for rows of at most kPfWaves * kPfCachedTiles * 32 = 1024 keys, with every score tile of the
@@ -597,7 +602,7 @@ static __global__ __launch_bounds__(64 * kPfWaves, 2) void pf_attention_cached_k
             }
         }
     }
-    pf_reduce_store(lds_acc, oacc0, oacc1, vsum0, vsum1, wave < ntiles, it, a_s[it.h], v_s[it.kvh], o, q_heads);
+    pf_reduce_store<kPfWaves>(lds_acc, oacc0, oacc1, vsum0, vsum1, wave < ntiles, it, a_s[it.h], v_s[it.kvh], o, q_heads);
 }
 
 inline int mha_prefill_launch(const int8_t* q8, const int8_t* kc, const int8_t* vc, const float* q_s, const float* k_s,
@@ -612,13 +617,15 @@ inline int mha_prefill_launch(const int8_t* q8, const int8_t* kc, const int8_t* 
     }
     static const bool no_cached = getenv("FLEXLLM_ATTN_RECOMPUTE") != nullptr;      // forces the two-pass kernel (comparison runs)
     const dim3 grid((s / kPfTile) * q_heads), block(64 * kPfWaves);
+    constexpr int kLongW = kPfLongWaves;
+    const dim3 block_long(64 * kLongW);
     const int group = q_heads / kv_heads;
     const bool cached = s <= kPfTile * kPfWaves * kPfCachedTiles && !no_cached;
     // the copy of the probability bytes (p8_out, a test and inspection output) is compiled out of the usual instances
     if (cached && p8_out) pf_attention_cached_kernel<true><<<grid, block, 0, st>>>(q8, kc, vc, q_s, k_s, v_s, a_s, o, p8_out, s, q_heads, group, max_pos, n_cu);
     else if (cached) pf_attention_cached_kernel<false><<<grid, block, 0, st>>>(q8, kc, vc, q_s, k_s, v_s, a_s, o, p8_out, s, q_heads, group, max_pos, n_cu);
-    else if (p8_out) pf_attention_kernel<true><<<grid, block, 0, st>>>(q8, kc, vc, q_s, k_s, v_s, a_s, o, p8_out, s, q_heads, group, max_pos, n_cu);
-    else pf_attention_kernel<false><<<grid, block, 0, st>>>(q8, kc, vc, q_s, k_s, v_s, a_s, o, p8_out, s, q_heads, group, max_pos, n_cu);
+    else if (p8_out) pf_attention_kernel<true, kLongW><<<grid, block_long, 0, st>>>(q8, kc, vc, q_s, k_s, v_s, a_s, o, p8_out, s, q_heads, group, max_pos, n_cu);
+    else pf_attention_kernel<false, kLongW><<<grid, block_long, 0, st>>>(q8, kc, vc, q_s, k_s, v_s, a_s, o, p8_out, s, q_heads, group, max_pos, n_cu);
     FX_LAUNCH_CHECK();
     return FLEXLLM_OK;
 }
