@@ -172,7 +172,7 @@ template <int kW>
 __device__ __forceinline__ void pf_reduce_store(int (*lds_acc)[35], const i32x16& oacc0, const i32x16& oacc1, int vsum0, int vsum1,
                                                 bool has_tiles, const PfItem& it, float sa, float sv, float* __restrict__ o,
                                                 int q_heads) {
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     if (has_tiles) {
 #pragma unroll
         for (int r = 0; r < 16; r++) {
@@ -213,7 +213,7 @@ static __global__ __launch_bounds__(64 * kW, 4) void pf_attention_kernel(const i
     __shared__ int lds_mi[kW][32];
     __shared__ float lds_l[kW][32];
     __shared__ int lds_acc[64][35];            // [lane][16 acc0 | 16 acc1 | vsum0 | vsum1], odd pitch against bank conflicts
-    const int wave = threadIdx.x >> 6;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);   // uniform: loop control on the scalar unit
     const PfItem it = pf_item(s, q_heads, group, period);
     const int col = it.col, g = it.g, query = it.query, ntiles = it.ntiles;
     const float sq = q_s[it.h], sk = k_s[it.kvh], as = 1.0f * a_s[it.h];
@@ -222,11 +222,6 @@ static __global__ __launch_bounds__(64 * kW, 4) void pf_attention_kernel(const i
     const i32x4 qf0 = *reinterpret_cast<const i32x4*>(qrow + g * 16);
     const i32x4 qf1 = *reinterpret_cast<const i32x4*>(qrow + 32 + g * 16);
     const int krow_in_tile = pf_key_of_row(col);
-    auto load_k = [&](int k0, i32x4& kf0, i32x4& kf1) {
-        const int8_t* krow = kc + k_index(it.kvh, k0 + krow_in_tile, max_pos);
-        kf0 = *reinterpret_cast<const i32x4*>(krow + g * 16);
-        kf1 = *reinterpret_cast<const i32x4*>(krow + 32 + g * 16);
-    };
     // integer scores of one tile: register r is key k0 + 16g + r; keys beyond the query (diagonal tile only) are masked
     auto int_tile = [&](int kt, const i32x4& kf0, const i32x4& kf1, int (&tv)[16], auto&& refill) {
         i32x16 acc = zero16();
@@ -245,11 +240,18 @@ static __global__ __launch_bounds__(64 * kW, 4) void pf_attention_kernel(const i
     // rows: the body calls refill() as soon as its two score products have been issued, which requests the next
     // tile's rows into the same registers, and the arithmetic on the scores that follows covers their way from the
     // cache.  No second set, nothing moved between trips.
+    const int8_t* const krow0 = kc + k_index(it.kvh, wave * kPfTile + krow_in_tile, max_pos) + g * 16;   // this lane's row of the wave's first tile
     auto for_tiles = [&](auto&& body) {
         i32x4 kf0, kf1;
-        if (wave < ntiles) load_k(wave * kPfTile, kf0, kf1);
+        const int8_t* kp = krow0;                              // advanced by a constant per trip: one add, no index arithmetic
+        auto load = [&] {
+            kf0 = *reinterpret_cast<const i32x4*>(kp);
+            kf1 = *reinterpret_cast<const i32x4*>(kp + 32);
+            kp += (size_t)kW * kPfTile * kHd;
+        };
+        if (wave < ntiles) load();
         for (int kt = wave; kt < ntiles; kt += kW)
-            body(kt, kf0, kf1, [&] { if (kt + kW < ntiles) load_k((kt + kW) * kPfTile, kf0, kf1); });
+            body(kt, kf0, kf1, [&] { if (kt + kW < ntiles) load(); });
     };
 
     for (int i = threadIdx.x; i < 64 * 35; i += 64 * kW) (&lds_acc[0][0])[i] = 0;
@@ -373,7 +375,7 @@ static __global__ __launch_bounds__(64 * kPfWaves, 2) void pf_attention_cached_k
     __shared__ int lds_mi[kPfWaves][32];
     __shared__ float lds_l[kPfWaves][32];
     __shared__ int lds_acc[64][35];            // [lane][16 acc0 | 16 acc1 | vsum0 | vsum1], odd pitch against bank conflicts
-    const int wave = threadIdx.x >> 6;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);   // uniform: loop control on the scalar unit
     const PfItem it = pf_item(s, q_heads, group, period);
     const int col = it.col, g = it.g, query = it.query, ntiles = it.ntiles;   // ntiles <= kPfWaves * kPfCachedTiles (checked by the launcher)
     const float sq = q_s[it.h], sk = k_s[it.kvh], as = 1.0f * a_s[it.h];
