@@ -139,6 +139,53 @@ __global__ __launch_bounds__(BLOCK) void rmsnorm_kernel(const float* __restrict_
     }
 }
 
+// RMSNorm + per-row int8 quantisation of rows of 2048 values, one WAVE per row (prefill: a thousand rows or more at
+// once).  A row is eight 16-byte loads per lane, all in flight together, and the two reductions stay inside the wave:
+// no LDS, no workgroup barrier.  The arithmetic is that of rmsnorm_kernel<1, true, 512> to the bit: lane l holds the
+// values thread 64 w + l holds there (w = 0..7), the squares of each w are summed by the same wave butterfly, the
+// eight sums are added in the same order, and a maximum does not depend on the order.
+constexpr int kNormWaveRows = 4;                       // rows (waves) per workgroup
+static __global__ __launch_bounds__(64 * kNormWaveRows) void rmsnorm_quant_2048_wave_kernel(
+    const float* __restrict__ x, const float* __restrict__ gamma, int8_t* __restrict__ q, float* __restrict__ s, int rows, float eps) {
+    const int lane = threadIdx.x & 63;
+    const int row = blockIdx.x * kNormWaveRows + __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+    if (row >= rows) return;
+    const float4* xr = reinterpret_cast<const float4*>(x + (size_t)row * 2048);
+    const float4* gr = reinterpret_cast<const float4*>(gamma);
+    float4 v[8], g[8];
+#pragma unroll
+    for (int w = 0; w < 8; w++) v[w] = xr[w * 64 + lane];
+#pragma unroll
+    for (int w = 0; w < 8; w++) g[w] = gr[w * 64 + lane];
+    float ss = 0.0f;
+#pragma unroll
+    for (int w = 0; w < 8; w++) {
+        const float part = wave_sum((v[w].x * v[w].x + v[w].y * v[w].y) + (v[w].z * v[w].z + v[w].w * v[w].w));
+        ss = w == 0 ? part : ss + part;
+    }
+    const float rms = 1.0f / sqrtf(ss / 2048.0f + eps);
+    float amax = 0.0f;
+#pragma unroll
+    for (int w = 0; w < 8; w++) {
+        v[w].x = v[w].x * rms * g[w].x;
+        v[w].y = v[w].y * rms * g[w].y;
+        v[w].z = v[w].z * rms * g[w].z;
+        v[w].w = v[w].w * rms * g[w].w;
+        amax = fmaxf(amax, fmaxf(fmaxf(fabsf(v[w].x), fabsf(v[w].y)), fmaxf(fabsf(v[w].z), fabsf(v[w].w))));
+    }
+    amax = wave_max(amax);
+    const float sc = sym_scale_127_uniform(amax);
+    if (lane == 0) s[row] = sc;
+    uint32_t* qr = reinterpret_cast<uint32_t*>(q + (size_t)row * 2048);
+#pragma unroll
+    for (int w = 0; w < 8; w++) {
+        const float f[4] = {v[w].x, v[w].y, v[w].z, v[w].w};
+        int nq[4];
+        quant_vector(f, sc, nq);
+        qr[w * 64 + lane] = pack4_i8(nq[0], nq[1], nq[2], nq[3]);
+    }
+}
+
 // ------------------------------------------------------------------ elementwise
 static __global__ __launch_bounds__(kBlock) void dequant_kernel(const int32_t* __restrict__ acc, const float* __restrict__ s_x,
                                                          const float* __restrict__ b_x, const float* __restrict__ w_s,

@@ -45,6 +45,15 @@ static int prefill_workspace_get(PrefillWorkspace* ws, const flexllm_llama_confi
     return FLEXLLM_OK;
 }
 
+// RMSNorm + per-row quantisation of s rows of H = 2048 values: one wave per row (the same arithmetic as the
+// one-workgroup-per-row kernel, to the bit, without its two workgroup barriers).
+static inline void rmsnorm_quant_rows(const float* x, const float* gamma, int8_t* q, float* scale, int s, int H, float eps, hipStream_t st) {
+    if (H == 2048)
+        rmsnorm_quant_2048_wave_kernel<<<(s + kNormWaveRows - 1) / kNormWaveRows, 64 * kNormWaveRows, 0, st>>>(x, gamma, q, scale, s, eps);
+    else
+        rmsnorm_kernel<1, true, 512><<<s, 512, 0, st>>>(x, gamma, nullptr, q, scale, H, eps);
+}
+
 int llama_prefill_run(const flexllm_llama_config& c, const LayerW* layers, const float* gamma, const float* q_s_all,
                       const float* k_s_all, const float* v_s_all, const float* a_s_all, const float* rope_sin,
                       const float* rope_cos, int8_t* k_cache, int8_t* v_cache, size_t cache_layer_bytes,
@@ -66,7 +75,7 @@ int llama_prefill_run(const flexllm_llama_config& c, const LayerW* layers, const
         int8_t* kc = k_cache + (size_t)l * cache_layer_bytes;
         int8_t* vc = v_cache + (size_t)l * cache_layer_bytes;
         // attention block
-        rmsnorm_kernel<1, true, 512><<<s, 512, 0, st>>>(b.x, g0, nullptr, b.xq, b.xs, H, c.eps);
+        rmsnorm_quant_rows(b.x, g0, b.xq, b.xs, s, H, c.eps, st);
         {   // q/k/v projection with RoPE, static quantisation and the cache stores in the GEMM epilogue
             QkvEpiArgs qa;
             qa.sin_t = rope_sin; qa.cos_t = rope_cos; qa.q_s = q_s; qa.k_s = k_s; qa.v_s = v_s;
@@ -75,10 +84,10 @@ int llama_prefill_run(const flexllm_llama_config& c, const LayerW* layers, const
             if ((rc = launch_gemm_qkv(b.xq, w.wqkv, b.xs, w.sqkv, s, H, qa, st))) return rc;
         }
         if ((rc = mha_prefill_launch(b.q8, kc, vc, q_s, k_s, v_s, a_s, b.att, nullptr, s, c.q_heads, c.kv_heads, c.max_pos, st))) return rc;
-        quant_sym_kernel<2><<<s, kBlock, 0, st>>>(b.att, b.xq, b.xs, H);
+        quant_sym_kernel<2><<<s, kBlock, 0, st>>>(b.att, b.xq, b.xs, H);   // (one wave per row, as for the norm: measured no faster here)
         if ((rc = launch_gemm<kGemmDequant>(b.xq, w.wo, nullptr, b.xs, w.so, b.x, b.x2, s, H, H, st))) return rc;
         // feed-forward block
-        rmsnorm_kernel<1, true, 512><<<s, 512, 0, st>>>(b.x2, g1, nullptr, b.xq, b.xs, H, c.eps);
+        rmsnorm_quant_rows(b.x2, g1, b.xq, b.xs, s, H, c.eps, st);
         if ((rc = launch_gemm_swiglu(b.xq, w.wgu, b.xs, w.sgu, b.gu, s, H, 2 * I, st))) return rc;     // b.gu = SiLU(gate)*up [s][I]
         fht_kernel<13, true, false><<<s, kFhtBlock, 0, st>>>(b.gu, nullptr, b.xq, b.xs, c.fht_scale);
         if ((rc = launch_gemm<kGemmDequant>(b.xq, w.wd, nullptr, b.xs, w.sd, b.x2, b.x, s, I, H, st))) return rc;
