@@ -312,6 +312,38 @@ def test_full_size_prefill_prefix_invariance_and_decode_equivalence(fx):
     pre.close(); dec.close()
 
 
+@pytest.mark.parametrize("s,qh,kvh,spread,a_div", [(288, 6, 2, 3.0, 255.0), (544, 2, 2, 1.0, 255.0), (800, 6, 2, 2.0, 100.0),
+                                                   (1056, 2, 2, 3.0, 255.0), (1536, 4, 1, 2.0, 100.0)])
+def test_mha_prefill_other_shapes(fx, oracle, s, qh, kvh, spread, a_div):
+    """Lengths that are not multiples of 64 or of the eight-tile deal (row blocks with idle waves, a last cache block
+    half full), head groupings of 3 and 1 query heads per KV head, a probability scale other than 1/255 and wider
+    scores, on both attention kernels: probability bytes against the oracle, the output as the exact product of the
+    reported bytes with V, and the instance that does not report the bytes against the one that does."""
+    r = np.random.default_rng(4000 + s)
+    q = (r.standard_normal((s, qh, 64)) * spread).astype(np.float32)
+    k = r.standard_normal((s, kvh, 64)).astype(np.float32)
+    v = r.standard_normal((s, kvh, 64)).astype(np.float32)
+    q_s, k_s, v_s, _ = mha_scales(qh, kvh, seed=s)
+    q_s = (q_s * spread).astype(np.float32)
+    a_s = np.full(qh, 1.0 / a_div, np.float32)
+    ref = oracle.mha_prefill(q, k, v, q_s, k_s, v_s, a_s, want_p=True)
+    sc = fx.ops.Scales(q_s, k_s, v_s, a_s)
+    kc, vc = fx.ops.kv_cache(kvh, (s + 63) // 64 * 64)
+    fx.ops.kv_append_i8(fx.to_device(k), fx.to_device(v), kc, vc, sc, 0)
+    q8 = fx.ops.static_quant_i8(fx.to_device(q), fx.to_device(q_s), factor=8.0)
+    assert np.array_equal(q8.numpy(), ref["q8"])
+    o, p8 = fx.ops.mha_i8_prefill(q8, kc, vc, sc, want_p=True)
+    o2, _ = fx.ops.mha_i8_prefill(q8, kc, vc, sc, want_p=False)
+    p = p8.numpy()
+    d = np.abs(p.astype(np.int32) - ref["p8"].astype(np.int32))
+    assert d.max() <= 1 and (d != 0).mean() < 1e-4
+    group = qh // kvh
+    acc = np.stack([p[h].astype(np.float64) @ ref["v8"][:, h // group].astype(np.float64) for h in range(qh)], axis=1)
+    o_from_p = (acc.astype(np.float32) * a_s[None, :, None]) * np.repeat(v_s, group)[None, :, None]
+    assert np.array_equal(o.numpy(), o_from_p.astype(np.float32))
+    assert np.array_equal(o2.numpy(), o.numpy())
+
+
 @pytest.mark.parametrize("s", [1088, 1024], ids=["rows over 1024 keys", "rows up to 1024 keys"])
 @pytest.mark.parametrize("case", ["wide scores", "tiny scales", "peaky rows"])
 def test_mha_prefill_long_rows_fast_and_exact_paths(fx, oracle, case, s):
