@@ -148,11 +148,14 @@ __device__ __forceinline__ int pf_round4_fast(const float (&ef)[4], const PfFast
     const float d0 = fabsf(__builtin_amdgcn_fractf(qv[0]) - 0.5f), d1 = fabsf(__builtin_amdgcn_fractf(qv[1]) - 0.5f);
     const float d2 = fabsf(__builtin_amdgcn_fractf(qv[2]) - 0.5f), d3 = fabsf(__builtin_amdgcn_fractf(qv[3]) - 0.5f);
     unsigned packed = 0;
-    bool redo = fminf(fminf(d0, d1), fminf(d2, d3)) < f.win;
-    if (redo)
-        redo = d0 < __builtin_fmaf(qv[0], f.rel, 1e-6f) || d1 < __builtin_fmaf(qv[1], f.rel, 1e-6f) ||
-               d2 < __builtin_fmaf(qv[2], f.rel, 1e-6f) || d3 < __builtin_fmaf(qv[3], f.rel, 1e-6f);
-    if (redo) {
+    auto fast_bytes = [&] {
+#pragma unroll
+        for (int b = 0; b < 4; b++) packed = __builtin_amdgcn_cvt_pk_u8_f32(qv[b], b, packed);
+    };
+    if (!(fminf(fminf(d0, d1), fminf(d2, d3)) < f.win)) {     // the usual case: one comparison, one branch
+        fast_bytes();
+    } else if (d0 < __builtin_fmaf(qv[0], f.rel, 1e-6f) || d1 < __builtin_fmaf(qv[1], f.rel, 1e-6f) ||
+               d2 < __builtin_fmaf(qv[2], f.rel, 1e-6f) || d3 < __builtin_fmaf(qv[3], f.rel, 1e-6f)) {
 #pragma unroll
         for (int b = 0; b < 4; b++) {
             int v = (int)roundf((exact(b) * f.cd) / as);
@@ -160,8 +163,7 @@ __device__ __forceinline__ int pf_round4_fast(const float (&ef)[4], const PfFast
             packed |= (unsigned)v << (8 * b);
         }
     } else {
-#pragma unroll
-        for (int b = 0; b < 4; b++) packed = __builtin_amdgcn_cvt_pk_u8_f32(qv[b], b, packed);
+        fast_bytes();
     }
     bytes = packed;
     return (int)(packed ^ 0x80808080u);
