@@ -210,7 +210,7 @@ __host__ __device__ constexpr int gemm_dma_lds_bytes(int bm, int bn, int stages,
     return rings > epi ? rings : epi;
 }
 
-enum GemmDmaEpi { kDmaRaw = 0, kDmaDequant = 1, kDmaSwiglu = 2, kDmaQkv = 3, kDmaDequantAsym = 4 };
+enum GemmDmaEpi { kDmaRaw = 0, kDmaDequant = 1, kDmaSwiglu = 2, kDmaQkv = 3, kDmaDequantAsym = 4, kDmaSwigluAsym = 5 };
 
 // Arguments of the q/k/v epilogue: the 64-column tile of the fused [q | k | v] projection is one attention head,
 // so RoPE (pairs k, k+32), the static int8 quantisation and the store into q8 / the K cache / the transposed V
@@ -219,7 +219,7 @@ struct QkvEpiArgs {
     const float *sin_t, *cos_t, *q_s, *k_s, *v_s;
     int8_t *q8, *kc, *vc;
     int pos0, q_heads, kv_heads, max_pos;
-    const float *b_x, *w_sum;          // kDmaDequantAsym only: zero point per row, weight row sum (times its scale) per column
+    const float *b_x, *w_sum;          // kDmaDequantAsym / kDmaSwigluAsym only: zero point per row, weight row sum (times its scale) per column
 };
 
 __device__ __forceinline__ void gemm_dma_issue(const int8_t* base, unsigned voff, unsigned lds_dst) {
@@ -460,6 +460,8 @@ __global__ __launch_bounds__(NW * 64, WPE) void gemm_i8_dma_kernel(const int8_t*
         }
         return;
     }
+    constexpr bool kAsym = EPI == kDmaDequantAsym || EPI == kDmaSwigluAsym;      // + zero point x row sum of the dequantised weights
+    constexpr bool kPlain = EPI == kDmaDequant || EPI == kDmaDequantAsym;        // fp32 outputs (+ residual); else SiLU(gate) * up pairs
     constexpr int EP = 36;                                     // patch pitch in words (rows stay 16-byte aligned)
     int* patch = reinterpret_cast<int*>(gemm_smem) + wave * (32 * EP);
     const int pr = lane >> 3, pc = (lane & 7) * 4;             // row within a group of 8, first of this lane's 4 columns
@@ -467,8 +469,8 @@ __global__ __launch_bounds__(NW * 64, WPE) void gemm_i8_dma_kernel(const int8_t*
     // together with the stores issued before it (one counter covers both), once per group of rows.
     float sxv[TM][4];
     float4 wsv[TN];
-    float bxv[EPI == kDmaDequantAsym ? TM : 1][4];
-    float4 wsumv[EPI == kDmaDequantAsym ? TN : 1];
+    float bxv[kAsym ? TM : 1][4];
+    float4 wsumv[kAsym ? TN : 1];
     if constexpr (EPI != kDmaRaw) {
 #pragma unroll
         for (int i = 0; i < TM; i++)
@@ -480,7 +482,7 @@ __global__ __launch_bounds__(NW * 64, WPE) void gemm_i8_dma_kernel(const int8_t*
             wsv[j] = col < n ? *reinterpret_cast<const float4*>(w_s + col) : make_float4(0.0f, 0.0f, 0.0f, 0.0f);
         }
     }
-    if constexpr (EPI == kDmaDequantAsym) {
+    if constexpr (kAsym) {
 #pragma unroll
         for (int i = 0; i < TM; i++)
 #pragma unroll
@@ -499,7 +501,7 @@ __global__ __launch_bounds__(NW * 64, WPE) void gemm_i8_dma_kernel(const int8_t*
         for (int i = 0; i < TM; i++) {
             float4 rs[4];                                      // the tile's residual rows, in flight during the turn through LDS
             bool has_res = false;
-            if constexpr (EPI == kDmaDequant || EPI == kDmaDequantAsym) {
+            if constexpr (kPlain) {
                 has_res = residual != nullptr;
                 if (has_res) {
 #pragma unroll
@@ -538,12 +540,12 @@ __global__ __launch_bounds__(NW * 64, WPE) void gemm_i8_dma_kernel(const int8_t*
                     float4 o;
                     o.x = (float)v[0] * sx * ws.x; o.y = (float)v[1] * sx * ws.y;
                     o.z = (float)v[2] * sx * ws.z; o.w = (float)v[3] * sx * ws.w;
-                    if constexpr (EPI == kDmaDequantAsym) {      // + zero point x row sum of the dequantised weights
+                    if constexpr (kAsym) {
                         const float bx = bxv[i][p];
                         const float4 wq = wsumv[j];
                         o.x = o.x + bx * wq.x; o.y = o.y + bx * wq.y; o.z = o.z + bx * wq.z; o.w = o.w + bx * wq.w;
                     }
-                    if constexpr (EPI == kDmaDequant || EPI == kDmaDequantAsym) {
+                    if constexpr (kPlain) {
                         if (has_res) { o.x = o.x + rs[p].x; o.y = o.y + rs[p].y; o.z = o.z + rs[p].z; o.w = o.w + rs[p].w; }
                         if (ok) *reinterpret_cast<float4*>(y + (size_t)row * n + col) = o;
                     } else {
@@ -657,6 +659,29 @@ inline int launch_gemm_asym(const int8_t* a, const int8_t* w, const float* s_x, 
         return launch_gemm_dma<64, 64, DE, 4, 2, 128>(a, w, nullptr, s_x, w_s, residual, y, m, k, n, st, qa);
     }
     return launch_gemm_dma<64, 64, DE>(a, w, nullptr, s_x, w_s, residual, y, m, k, n, st, qa);
+}
+
+// The gate/up projection of the W4A4 graph (interleaved rows, asymmetric activations held one value per byte) with
+// SiLU(gate)*up in the epilogue: the asymmetric dequantisation of launch_gemm_asym followed by the product that the
+// Hadamard kernel would otherwise form from the interleaved fp32 columns - the same arithmetic, half the output.
+// Tiles as in launch_gemm_swiglu: 256x256 where its grid fills the CUs in whole rounds (1024 tokens: 44 us against
+// 50 us for the unfused 128x128 kernel, and the transform after it reads half as much), smaller ones otherwise.
+inline int launch_gemm_swiglu_asym(const int8_t* a, const int8_t* w_gu, const float* s_x, const float* b_x, const float* w_s_gu,
+                                   const float* w_sum_gu, float* h, int m, int k, int n2, hipStream_t st) {
+    FX_REQUIRE((size_t)m * k < (1ull << 31) && (size_t)n2 * k < (1ull << 31) && n2 % 4 == 0,
+               "linear_i8_gemm_swiglu_asym: m=%d k=%d n=%d outside the direct-load kernel's range", m, k, n2 / 2);
+    auto tiles = [&](int bm, int bn) { return ((m + bm - 1) / bm) * ((n2 + bn - 1) / bn); };
+    QkvEpiArgs qa = QkvEpiArgs();
+    qa.b_x = b_x; qa.w_sum = w_sum_gu;
+    constexpr int E = kDmaSwigluAsym;
+    if (k % 128 == 0) {
+        const int t256 = tiles(256, 256);
+        if (t256 >= 256 && (t256 % 256 == 0 || t256 >= 1024))
+            return launch_gemm_dma<256, 256, E, 2, 2, 128, 8>(a, w_gu, nullptr, s_x, w_s_gu, nullptr, h, m, k, n2, st, qa);
+        if (tiles(128, 128) >= 384) return launch_gemm_dma<128, 128, E, 2, 2, 128>(a, w_gu, nullptr, s_x, w_s_gu, nullptr, h, m, k, n2, st, qa);
+        return launch_gemm_dma<64, 64, E, 4, 2, 128>(a, w_gu, nullptr, s_x, w_s_gu, nullptr, h, m, k, n2, st, qa);
+    }
+    return launch_gemm_dma<64, 64, E>(a, w_gu, nullptr, s_x, w_s_gu, nullptr, h, m, k, n2, st, qa);
 }
 
 // W4A4 prefill GEMM on nibble-packed operands (register-staged kernel, nibbles widened on the way to LDS).

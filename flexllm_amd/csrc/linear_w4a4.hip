@@ -62,4 +62,13 @@ int flexllm_linear_i8_gemm_dequant_asym(const int8_t* a, const float* s_x, const
     return launch_gemm_asym(a, w, s_x, b_x, w_s, w_sum, residual, y, m, k, n, as_stream(stream));
 }
 
+int flexllm_linear_i8_gemm_swiglu_asym(const int8_t* a, const float* s_x, const float* b_x, const int8_t* w_gu, const float* w_s_gu,
+                                       const float* w_sum_gu, float* h, int m, int k, int n, void* stream) {
+    FX_REQUIRE(a && s_x && b_x && w_gu && w_s_gu && w_sum_gu && h, "linear_i8_gemm_swiglu_asym: null pointer");
+    FX_REQUIRE(k > 0 && k % kGemmBK == 0, "linear_i8_gemm_swiglu_asym: k=%d must be a multiple of 64", k);
+    FX_REQUIRE(m >= 0 && n >= 0 && n % 2 == 0, "linear_i8_gemm_swiglu_asym: m=%d n=%d (n must be even)", m, n);
+    if (m == 0 || n == 0) return FLEXLLM_OK;
+    return launch_gemm_swiglu_asym(a, w_gu, s_x, b_x, w_s_gu, w_sum_gu, h, m, k, 2 * n, as_stream(stream));
+}
+
 }  // extern "C"

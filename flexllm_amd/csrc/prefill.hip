@@ -101,7 +101,7 @@ int llama_prefill_run(const flexllm_llama_config& c, const LayerW* layers, const
 // over the same kernels the module entry points use: the 4-bit values are held one per byte (layers: the matrices as
 // flexllm_llama_create keeps them, sums: the row sums of the dequantised weights) and multiplied on the int8 direct-load
 // MFMA kernel with the asymmetric dequantisation in its epilogue; RoPE, static quantisation and the cache stores run as
-// one kernel per token row, SiLU(gate)*up is applied by the Hadamard kernel as it loads the interleaved gate/up columns.
+// one kernel per token row, SiLU(gate)*up is formed in the epilogue of the gate/up GEMM.
 int llama_prefill_run_w4a4(const flexllm_llama_config& c, const LayerW* layers, const LayerW4* sums, const float* gamma,
                            const float* q_s_all, const float* k_s_all, const float* v_s_all, const float* a_s_all,
                            const float* rope_sin, const float* rope_cos, int8_t* k_cache, int8_t* v_cache,
@@ -136,8 +136,9 @@ int llama_prefill_run_w4a4(const flexllm_llama_config& c, const LayerW* layers, 
         // feed-forward block
         rmsnorm_kernel<1, false, 512><<<s, 512, 0, st>>>(b.x2, gamma + (size_t)(2 * l + 1) * H, b.fh, nullptr, nullptr, H, c.eps);
         quant_asym_kernel<2><<<s, kBlock, 0, st>>>(b.fh, xq, b.xs, b.xb, H, 15.0f, 15u);
-        if ((rc = launch_gemm_asym(b.xq, w.wgu, b.xs, b.xb, w.sgu, m4.mgu, nullptr, b.gu, s, H, 2 * I, st))) return rc;   // interleaved (gate, up)
-        fht_kernel<13, false, true><<<s, kFhtBlock, 0, st>>>(b.gu, b.fh, nullptr, nullptr, c.fht_scale);
+        // gate/up with SiLU(gate)*up in the GEMM epilogue: b.gu = [s][I]
+        if ((rc = launch_gemm_swiglu_asym(b.xq, w.wgu, b.xs, b.xb, w.sgu, m4.mgu, b.gu, s, H, 2 * I, st))) return rc;
+        fht_kernel<13, false, false><<<s, kFhtBlock, 0, st>>>(b.gu, b.fh, nullptr, nullptr, c.fht_scale);
         quant_asym_kernel<8><<<s, kBlock, 0, st>>>(b.fh, xq, b.xs, b.xb, I, 15.0f, 15u);
         if ((rc = launch_gemm_asym(b.xq, w.wd, b.xs, b.xb, w.sd, m4.md, b.x2, b.x, s, I, H, st))) return rc;
     }

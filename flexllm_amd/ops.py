@@ -171,6 +171,17 @@ def linear_i8_gemm_dequant_asym(a, s_x, b_x, w, w_s, w_sum, residual=None, strea
     return y
 
 
+def linear_i8_gemm_swiglu_asym(a, s_x, b_x, w_gu, w_s_gu, w_sum_gu, stream=None):
+    """Gate/up projection of the W4A4 precision (operands one value per byte, interleaved gate/up rows) with
+    SiLU(gate) * up in the epilogue: h [m][n], n = w_gu.shape[0] // 2."""
+    m, k = a.shape
+    n = w_gu.shape[0] // 2
+    h = DeviceArray((m, n), np.float32)
+    check(lib().flexllm_linear_i8_gemm_swiglu_asym(_p(a), _p(s_x), _p(b_x), _p(w_gu), _p(w_s_gu), _p(w_sum_gu), _p(h), m, k, n,
+                                                   _s(stream)))
+    return h
+
+
 def lm_head_u4i4(n_vec, w4, w_s, w_sum, stream=None):
     """The reference's output head (SpinQuant_Decoding_mem_opt.h:363-365, config D6): the normalised hidden vector is
     quantised to asymmetric uint4, multiplied with the int4 head weights (nibble-packed [vocab_pad][hidden/2]) and

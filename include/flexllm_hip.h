@@ -159,6 +159,13 @@ int flexllm_linear_u4i4_gemm_dequant(const uint8_t* a4, const float* s_x, const 
  * k % 64 == 0, n % 4 == 0.  Replaces pref_Linear_Layer_i4xi4 + the asymmetric dequant like the entry point above. */
 int flexllm_linear_i8_gemm_dequant_asym(const int8_t* a, const float* s_x, const float* b_x, const int8_t* w, const float* w_s,
                                         const float* w_sum, const float* residual, float* y, int m, int k, int n, void* stream);
+/* The gate/up projection of the same precision with SiLU(gate) * up in the epilogue: w_gu [2n][k] with gate row i at
+ * 2i and up row i at 2i+1 (w_s_gu, w_sum_gu [2n] likewise), h [m][n] = up * SiLU(gate) of the dequantised pair - the
+ * values flexllm_linear_i8_gemm_dequant_asym followed by flexllm_swiglu_f32 give, bit for bit, with half the output
+ * traffic.  Replaces pref_Linear_Layer_i4xi4 (gate, up) + dequant + pref_Swish + pref_Gate_Layer
+ * (SpinQuant_Prefilling.h:938-1004).  k % 64 == 0. */
+int flexllm_linear_i8_gemm_swiglu_asym(const int8_t* a, const float* s_x, const float* b_x, const int8_t* w_gu, const float* w_s_gu,
+                                       const float* w_sum_gu, float* h, int m, int k, int n, void* stream);
 
 /* ---- FHT.h ---------------------------------------------------------------------------- */
 /* y = H_n x / scale (Sylvester order, butterfly stage order of the reference's omega network, so

@@ -87,6 +87,29 @@ def test_gemm_on_byte_held_operands_equals_the_packed_path(fx, oracle, m, k, n):
     assert np.array_equal(y2, oracle.dequant(np.full((m, n), -127 * 128 * k, np.int32), s_x, w_s, b_x=b_x, w_sum=w_sum))
 
 
+@pytest.mark.parametrize("m,k,n", [(1024, 2048, 8192), (512, 2048, 8192), (160, 2048, 192), (96, 64, 66), (32, 128, 2)])
+def test_gate_up_with_swiglu_in_the_epilogue_equals_the_two_step_route(fx, oracle, m, k, n):
+    """Gate/up projection of the W4A4 precision with SiLU(gate)*up in the GEMM epilogue (every tile variant its launcher
+    picks: 256x256 at the prefill shape, 128x128, 64x64, ragged edges) against the dequantising GEMM on the same
+    interleaved rows followed by the SwiGLU kernel: bit for bit; and the dequantised pairs against the oracle."""
+    a = rng.integers(0, 16, (m, k)).astype(np.uint8)
+    w = rng.integers(-8, 8, (2 * n, k)).astype(np.int8)                      # row 2i gate, row 2i+1 up
+    s_x = rng.uniform(0.01, 0.04, m).astype(np.float32); b_x = rng.uniform(-0.3, 0, m).astype(np.float32)
+    w_s = rng.uniform(0.01, 0.05, 2 * n).astype(np.float32)
+    w_sum = (w.sum(1, dtype=np.int64).astype(np.float32) * w_s).astype(np.float32)
+    da, dw = fx.to_device(a), fx.to_device(w)
+    dev = [fx.to_device(v) for v in (s_x, b_x, w_s, w_sum)]
+    h = fx.ops.linear_i8_gemm_swiglu_asym(da, dev[0], dev[1], dw, dev[2], dev[3]).numpy()
+    y = fx.ops.linear_i8_gemm_dequant_asym(da, dev[0], dev[1], dw, dev[2], dev[3]).numpy()
+    acc = a.astype(np.int32) @ w.astype(np.int32).T
+    assert np.array_equal(y, oracle.dequant(acc, s_x, w_s, b_x=b_x, w_sum=w_sum))
+    gate = np.ascontiguousarray(y[:, 0::2]); up = np.ascontiguousarray(y[:, 1::2])
+    h2 = fx.ops.swiglu_f32(fx.to_device(gate), fx.to_device(up)).numpy()
+    assert np.array_equal(h, h2)
+    ref = up.astype(np.float64) * (gate.astype(np.float64) / (1.0 + np.exp(-gate.astype(np.float64))))
+    assert np.abs(h - ref).max() <= 1e-6 * max(1.0, np.abs(ref).max())
+
+
 def test_w4a4_layer_like_the_reference_testbench(fx, oracle):
     """quant (asym uint4) -> linear -> dequant with zero point, decode and prefill shapes: bit-exact against the oracle
     chain, and within the testbench's own 1e-2 criterion of the fake-quant golden (…_tb.cpp:215-236)."""
