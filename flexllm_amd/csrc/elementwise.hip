@@ -101,6 +101,18 @@ int flexllm_rmsnorm_quant_i8(const float* x, const float* gamma, int8_t* q, floa
     return FLEXLLM_OK;
 }
 
+int flexllm_rmsnorm_quant_asym_u8(const float* x, const float* gamma, uint8_t* q, float* s, float* b, int bits, int rows, int dim,
+                                  float eps, void* stream) {
+    FX_REQUIRE(x && gamma && q && s && b, "rmsnorm_quant_asym: null pointer");
+    FX_REQUIRE(bits >= 2 && bits <= 8, "rmsnorm_quant_asym: bits=%d", bits);
+    FX_REQUIRE(rows >= 0 && dim == 2048, "rmsnorm_quant_asym: dim=%d (instantiated for rows of 2048 values)", dim);
+    if (rows == 0) return FLEXLLM_OK;
+    rmsnorm_quant_asym_2048_wave_kernel<<<(rows + kNormWaveRows - 1) / kNormWaveRows, 64 * kNormWaveRows, 0, as_stream(stream)>>>(
+        x, gamma, q, s, b, rows, eps, (float)((1 << bits) - 1), (1u << bits) - 1u);
+    FX_LAUNCH_CHECK();
+    return FLEXLLM_OK;
+}
+
 int flexllm_rope_f32(const float* x, float* y, const float* sin_t, const float* cos_t, int tokens, int heads,
                      int head_dim, int pos0, void* stream) {
     FX_REQUIRE(x && y && sin_t && cos_t, "rope: null pointer");

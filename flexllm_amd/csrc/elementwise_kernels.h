@@ -74,9 +74,14 @@ __global__ __launch_bounds__(kBlock) void quant_asym_kernel(const float* __restr
 #pragma unroll
     for (int i = 0; i < VPT; i++) {
         const int idx = threadIdx.x + i * kBlock;
-        if (idx < nvec)
-            qr[idx] = pack4_i8(quant_round(v[i].x - vmin, sc) & mask, quant_round(v[i].y - vmin, sc) & mask,
-                               quant_round(v[i].z - vmin, sc) & mask, quant_round(v[i].w - vmin, sc) & mask);
+        if (idx < nvec) {
+            // round((x - min) / s) through the reciprocal, with the division itself only next to a rounding tie: the
+            // same integers (quant_vector)
+            const float f[4] = {v[i].x - vmin, v[i].y - vmin, v[i].z - vmin, v[i].w - vmin};
+            int nq[4];
+            quant_vector(f, sc, nq);
+            qr[idx] = pack4_i8(nq[0] & mask, nq[1] & mask, nq[2] & mask, nq[3] & mask);
+        }
     }
 }
 
@@ -183,6 +188,54 @@ static __global__ __launch_bounds__(64 * kNormWaveRows) void rmsnorm_quant_2048_
         int nq[4];
         quant_vector(f, sc, nq);
         qr[w * 64 + lane] = pack4_i8(nq[0], nq[1], nq[2], nq[3]);
+    }
+}
+
+// The same for the W4A4 graph: RMSNorm of a row of 2048 values and its asymmetric quantisation to `levels` steps
+// (uint4: scale_base 15, mask 15), one wave per row - what rmsnorm_kernel<1, false, 512> followed by quant_asym_kernel
+// compute, to the bit (same sum of squares, maxima and minima do not depend on the order).
+static __global__ __launch_bounds__(64 * kNormWaveRows) void rmsnorm_quant_asym_2048_wave_kernel(
+    const float* __restrict__ x, const float* __restrict__ gamma, uint8_t* __restrict__ q, float* __restrict__ s,
+    float* __restrict__ b, int rows, float eps, float scale_base, unsigned mask) {
+    const int lane = threadIdx.x & 63;
+    const int row = blockIdx.x * kNormWaveRows + __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+    if (row >= rows) return;
+    const float4* xr = reinterpret_cast<const float4*>(x + (size_t)row * 2048);
+    const float4* gr = reinterpret_cast<const float4*>(gamma);
+    float4 v[8], g[8];
+#pragma unroll
+    for (int w = 0; w < 8; w++) v[w] = xr[w * 64 + lane];
+#pragma unroll
+    for (int w = 0; w < 8; w++) g[w] = gr[w * 64 + lane];
+    float ss = 0.0f;
+#pragma unroll
+    for (int w = 0; w < 8; w++) {
+        const float part = wave_sum((v[w].x * v[w].x + v[w].y * v[w].y) + (v[w].z * v[w].z + v[w].w * v[w].w));
+        ss = w == 0 ? part : ss + part;
+    }
+    const float rms = 1.0f / sqrtf(ss / 2048.0f + eps);
+    float vmax = -1e32f, vmin = 1e32f;
+#pragma unroll
+    for (int w = 0; w < 8; w++) {
+        v[w].x = v[w].x * rms * g[w].x;
+        v[w].y = v[w].y * rms * g[w].y;
+        v[w].z = v[w].z * rms * g[w].z;
+        v[w].w = v[w].w * rms * g[w].w;
+        vmax = fmaxf(vmax, fmaxf(fmaxf(v[w].x, v[w].y), fmaxf(v[w].z, v[w].w)));
+        vmin = fminf(vmin, fminf(fminf(v[w].x, v[w].y), fminf(v[w].z, v[w].w)));
+    }
+    vmax = wave_max(vmax);
+    vmin = wave_min(vmin);
+    float sc = (vmax - vmin) / scale_base;
+    if (sc == 0.0f) sc = 1.0f;
+    if (lane == 0) { s[row] = sc; b[row] = vmin; }
+    uint32_t* qr = reinterpret_cast<uint32_t*>(q + (size_t)row * 2048);
+#pragma unroll
+    for (int w = 0; w < 8; w++) {
+        const float f[4] = {v[w].x - vmin, v[w].y - vmin, v[w].z - vmin, v[w].w - vmin};
+        int nq[4];
+        quant_vector(f, sc, nq);
+        qr[w * 64 + lane] = pack4_i8(nq[0] & mask, nq[1] & mask, nq[2] & mask, nq[3] & mask);
     }
 }
 

@@ -25,9 +25,14 @@ namespace fx {
 
 constexpr int kFhtBlock = 256;
 
-template <int LOG2N, bool QUANT, bool SWIGLU = false>
+// QUANT: 0 = fp32 output y; 1 = per-row symmetric int8 (q, s); 2 = per-row asymmetric quantisation to scale_base steps
+// (uint4: 15), one value per byte, with the scale in s and the row minimum in zp - what quant_asym_kernel computes from
+// the fp32 output, to the bit.
+template <int LOG2N, int QUANT, bool SWIGLU = false>
 __global__ __launch_bounds__(kFhtBlock) void fht_kernel(const float* __restrict__ x, float* __restrict__ y,
-                                                        int8_t* __restrict__ q, float* __restrict__ s, float scale) {
+                                                        int8_t* __restrict__ q, float* __restrict__ s, float scale,
+                                                        float* __restrict__ zp = nullptr, float scale_base = 15.0f,
+                                                        unsigned mask = 15u) {
     constexpr int N = 1 << LOG2N;
     constexpr int NJ = N / 1024;   // float4 vectors per thread in layout A
     constexpr int NR = N / 256;    // floats per thread in layouts M and B
@@ -135,7 +140,7 @@ __global__ __launch_bounds__(kFhtBlock) void fht_kernel(const float* __restrict_
     }
 
     float amax = 0.0f;
-    if constexpr (!QUANT) {
+    if constexpr (QUANT == 0) {
 #pragma unroll
         for (int r = 0; r < NR; r++) b[r] = b[r] / scale;
     } else {
@@ -155,10 +160,34 @@ __global__ __launch_bounds__(kFhtBlock) void fht_kernel(const float* __restrict_
         }
         amax = amax / scale;
     }
-    if constexpr (!QUANT) {
+    if constexpr (QUANT == 0) {
         float* yr = y + row * N;
 #pragma unroll
         for (int r = 0; r < NR; r++) yr[r * 256 + t] = b[r];
+    } else if constexpr (QUANT == 2) {
+        // the quotients above are the fp32 outputs (correctly rounded either way); their extremes, then
+        // round((v - min) / s) & mask as quant_asym_kernel forms it
+        float vmax = b[0], vmin = b[0];
+#pragma unroll
+        for (int r = 1; r < NR; r++) { vmax = fmaxf(vmax, b[r]); vmin = fminf(vmin, b[r]); }
+        vmax = block_max<kFhtBlock / kWave>(vmax, red);   // its leading barrier also retires the lds reads above
+        vmin = block_min<kFhtBlock / kWave>(vmin, red);
+        float sc = (vmax - vmin) / scale_base;
+        if (sc == 0.0f) sc = 1.0f;
+        if (t == 0) { s[row] = sc; zp[row] = vmin; }
+        uint8_t* lds_q = reinterpret_cast<uint8_t*>(lds);
+        {
+            float d[NR];
+            int nq[NR];
+#pragma unroll
+            for (int r = 0; r < NR; r++) d[r] = b[r] - vmin;
+            quant_vector(d, sc, nq);
+#pragma unroll
+            for (int r = 0; r < NR; r++) lds_q[r * 256 + t] = (uint8_t)(nq[r] & mask);
+        }
+        __syncthreads();
+        i32x4* qr = reinterpret_cast<i32x4*>(q + row * N);
+        for (int c = t; c < N / 16; c += kFhtBlock) qr[c] = reinterpret_cast<const i32x4*>(lds_q)[c];
     } else {
         amax = block_max<kFhtBlock / kWave>(amax, red);   // its leading barrier also retires the lds reads above
         const float sc = sym_scale_127_uniform(amax);
@@ -176,13 +205,14 @@ __global__ __launch_bounds__(kFhtBlock) void fht_kernel(const float* __restrict_
     }
 }
 
-template <bool QUANT>
-static int launch_fht(const float* x, float* y, int8_t* q, float* s, int rows, int n, float scale, hipStream_t st) {
+template <int QUANT>
+static int launch_fht(const float* x, float* y, int8_t* q, float* s, int rows, int n, float scale, hipStream_t st,
+                      float* zp = nullptr, float scale_base = 15.0f, unsigned mask = 15u) {
     switch (n) {
-        case 1024: fht_kernel<10, QUANT><<<rows, kFhtBlock, 0, st>>>(x, y, q, s, scale); break;
-        case 2048: fht_kernel<11, QUANT><<<rows, kFhtBlock, 0, st>>>(x, y, q, s, scale); break;
-        case 4096: fht_kernel<12, QUANT><<<rows, kFhtBlock, 0, st>>>(x, y, q, s, scale); break;
-        case 8192: fht_kernel<13, QUANT><<<rows, kFhtBlock, 0, st>>>(x, y, q, s, scale); break;
+        case 1024: fht_kernel<10, QUANT><<<rows, kFhtBlock, 0, st>>>(x, y, q, s, scale, zp, scale_base, mask); break;
+        case 2048: fht_kernel<11, QUANT><<<rows, kFhtBlock, 0, st>>>(x, y, q, s, scale, zp, scale_base, mask); break;
+        case 4096: fht_kernel<12, QUANT><<<rows, kFhtBlock, 0, st>>>(x, y, q, s, scale, zp, scale_base, mask); break;
+        case 8192: fht_kernel<13, QUANT><<<rows, kFhtBlock, 0, st>>>(x, y, q, s, scale, zp, scale_base, mask); break;
         default:
             set_error("fht: n=%d must be a power of two in [1024, 8192]", n);
             return FLEXLLM_EINVAL;

@@ -125,8 +125,8 @@ int llama_prefill_run_w4a4(const flexllm_llama_config& c, const LayerW* layers, 
         int8_t* kc = k_cache + (size_t)l * cache_layer_bytes;
         int8_t* vc = v_cache + (size_t)l * cache_layer_bytes;
         // attention block
-        rmsnorm_kernel<1, false, 512><<<s, 512, 0, st>>>(b.x, gamma + (size_t)(2 * l) * H, b.fh, nullptr, nullptr, H, c.eps);
-        quant_asym_kernel<2><<<s, kBlock, 0, st>>>(b.fh, xq, b.xs, b.xb, H, 15.0f, 15u);
+        rmsnorm_quant_asym_2048_wave_kernel<<<(s + kNormWaveRows - 1) / kNormWaveRows, 64 * kNormWaveRows, 0, st>>>(
+            b.x, gamma + (size_t)(2 * l) * H, xq, b.xs, b.xb, s, c.eps, 15.0f, 15u);
         if ((rc = launch_gemm_asym(b.xq, w.wqkv, b.xs, b.xb, w.sqkv, m4.mqkv, nullptr, b.qkv, s, H, H + 2 * KV, st))) return rc;
         qkv_post_kernel<<<s, 256, 0, st>>>(b.qkv, rope_sin, rope_cos, q_s, k_s, v_s, b.q8, kc, vc, nullptr, 0, c.q_heads,
                                            c.kv_heads, c.max_pos);
@@ -134,12 +134,11 @@ int llama_prefill_run_w4a4(const flexllm_llama_config& c, const LayerW* layers, 
         quant_asym_kernel<2><<<s, kBlock, 0, st>>>(b.att, xq, b.xs, b.xb, H, 15.0f, 15u);
         if ((rc = launch_gemm_asym(b.xq, w.wo, b.xs, b.xb, w.so, m4.mo, b.x, b.x2, s, H, H, st))) return rc;
         // feed-forward block
-        rmsnorm_kernel<1, false, 512><<<s, 512, 0, st>>>(b.x2, gamma + (size_t)(2 * l + 1) * H, b.fh, nullptr, nullptr, H, c.eps);
-        quant_asym_kernel<2><<<s, kBlock, 0, st>>>(b.fh, xq, b.xs, b.xb, H, 15.0f, 15u);
+        rmsnorm_quant_asym_2048_wave_kernel<<<(s + kNormWaveRows - 1) / kNormWaveRows, 64 * kNormWaveRows, 0, st>>>(
+            b.x2, gamma + (size_t)(2 * l + 1) * H, xq, b.xs, b.xb, s, c.eps, 15.0f, 15u);
         // gate/up with SiLU(gate)*up in the GEMM epilogue: b.gu = [s][I]
         if ((rc = launch_gemm_swiglu_asym(b.xq, w.wgu, b.xs, b.xb, w.sgu, m4.mgu, b.gu, s, H, 2 * I, st))) return rc;
-        fht_kernel<13, false, false><<<s, kFhtBlock, 0, st>>>(b.gu, b.fh, nullptr, nullptr, c.fht_scale);
-        quant_asym_kernel<8><<<s, kBlock, 0, st>>>(b.fh, xq, b.xs, b.xb, I, 15.0f, 15u);
+        fht_kernel<13, 2, false><<<s, kFhtBlock, 0, st>>>(b.gu, nullptr, b.xq, b.xs, c.fht_scale, b.xb, 15.0f, 15u);   // transform + uint4 quantisation
         if ((rc = launch_gemm_asym(b.xq, w.wd, b.xs, b.xb, w.sd, m4.md, b.x2, b.x, s, I, H, st))) return rc;
     }
     FX_LAUNCH_CHECK();

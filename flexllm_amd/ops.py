@@ -205,7 +205,24 @@ def fht_quant_i8(x, scale=1.0, stream=None):
     return q, s
 
 
+def fht_quant_asym_u8(x, scale=1.0, bits=4, stream=None):
+    q = DeviceArray(x.shape, np.uint8)
+    s = DeviceArray(x.shape[:-1] or (1,), np.float32)
+    b = DeviceArray(x.shape[:-1] or (1,), np.float32)
+    check(lib().flexllm_fht_quant_asym_u8(_p(x), _p(q), _p(s), _p(b), bits, _rows(x), x.shape[-1], C.c_float(scale), _s(stream)))
+    return q, s, b
+
+
 # ---------------------------------------------------------------- LayerNorm.h
+def rmsnorm_quant_asym_u8(x, gamma, eps=1e-5, bits=4, stream=None):
+    q = DeviceArray(x.shape, np.uint8)
+    s = DeviceArray(x.shape[:-1] or (1,), np.float32)
+    b = DeviceArray(x.shape[:-1] or (1,), np.float32)
+    check(lib().flexllm_rmsnorm_quant_asym_u8(_p(x), _p(gamma), _p(q), _p(s), _p(b), bits, _rows(x), x.shape[-1], C.c_float(eps),
+                                              _s(stream)))
+    return q, s, b
+
+
 def rmsnorm_f32(x, gamma, eps=1e-5, stream=None):
     y = DeviceArray(x.shape, np.float32)
     check(lib().flexllm_rmsnorm_f32(_p(x), _p(gamma), _p(y), _rows(x), x.shape[-1], C.c_float(eps), _s(stream)))

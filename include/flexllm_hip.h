@@ -163,7 +163,7 @@ int flexllm_linear_i8_gemm_dequant_asym(const int8_t* a, const float* s_x, const
  * 2i and up row i at 2i+1 (w_s_gu, w_sum_gu [2n] likewise), h [m][n] = up * SiLU(gate) of the dequantised pair - the
  * values flexllm_linear_i8_gemm_dequant_asym followed by flexllm_swiglu_f32 give, bit for bit, with half the output
  * traffic.  Replaces pref_Linear_Layer_i4xi4 (gate, up) + dequant + pref_Swish + pref_Gate_Layer
- * (SpinQuant_Prefilling.h:938-1004).  k % 64 == 0. */
+ * (pref_Swish_Layer_ffn, pref_Gate_Layer_ffn: SpinQuant_Prefilling.h:649-670).  k % 64 == 0. */
 int flexllm_linear_i8_gemm_swiglu_asym(const int8_t* a, const float* s_x, const float* b_x, const int8_t* w_gu, const float* w_s_gu,
                                        const float* w_sum_gu, float* h, int m, int k, int n, void* stream);
 
@@ -174,6 +174,10 @@ int flexllm_linear_i8_gemm_swiglu_asym(const int8_t* a, const float* s_x, const 
 int flexllm_fht_f32(const float* x, float* y, int rows, int n, float scale, void* stream);
 /* FHT followed by flexllm_quant_sym_i8 on each transformed row, without the fp32 round trip. */
 int flexllm_fht_quant_i8(const float* x, int8_t* q, float* s, int rows, int n, float scale, void* stream);
+/* FHT followed by flexllm_quant_asym_u8 on each transformed row (the W4A4 graph's input of the down projection,
+ * pref_FHT_R4 + pref_quant_layer_ffn_down_fp32_int4, SpinQuant_Prefilling.h:673-700), without the fp32 round trip:
+ * the same bytes, scales and minima, bit for bit. */
+int flexllm_fht_quant_asym_u8(const float* x, uint8_t* q, float* s, float* b, int bits, int rows, int n, float scale, void* stream);
 
 /* ---- LayerNorm.h ---------------------------------------------------------------------- */
 /* RMSNorm: y = (x * (1/sqrt(mean(x^2)+eps))) * gamma.  Replaces pref_Layer_Norm
@@ -182,6 +186,11 @@ int flexllm_rmsnorm_f32(const float* x, const float* gamma, float* y, int rows, 
 /* RMSNorm followed by flexllm_quant_sym_i8 on each row. */
 int flexllm_rmsnorm_quant_i8(const float* x, const float* gamma, int8_t* q, float* s, int rows, int dim,
                              float eps, void* stream);
+/* RMSNorm followed by flexllm_quant_asym_u8 on each row (pref_Layer_Norm + pref_quant_layer_fp32_qint<4,true>,
+ * SpinQuant_Prefilling.h:78-90, 123-136), one wave per row; dim == 2048.  The sum of squares is taken in the order of the
+ * model graphs (512 partial sums of four squares, wave butterflies, eight wave sums in order). */
+int flexllm_rmsnorm_quant_asym_u8(const float* x, const float* gamma, uint8_t* q, float* s, float* b, int bits, int rows, int dim,
+                                  float eps, void* stream);
 
 /* ---- RoPE.h --------------------------------------------------------------------------- */
 /* Rotate-half RoPE from tables sin_t/cos_t [max_pos][head_dim/2]; x,y [tokens][heads][head_dim];

@@ -110,6 +110,42 @@ def test_gate_up_with_swiglu_in_the_epilogue_equals_the_two_step_route(fx, oracl
     assert np.abs(h - ref).max() <= 1e-6 * max(1.0, np.abs(ref).max())
 
 
+@pytest.mark.parametrize("n,rows", [(8192, 96), (2048, 33), (1024, 5)])
+def test_fht_with_asymmetric_quantisation_equals_the_two_step_route(fx, n, rows):
+    """Hadamard transform + asymmetric uint4 (and uint8) quantisation in one kernel against the transform followed by
+    the quantisation kernel: bytes, scales and minima bit for bit (the quotients by the transform's scale are correctly
+    rounded in both, and the rounding of (v - min) / s through the reciprocal gives the division's integers)."""
+    x = fx.to_device((rng.standard_normal((rows, n)) * rng.uniform(0.1, 3.0, (rows, 1))).astype(np.float32))
+    scale = float(np.sqrt(n))
+    y = fx.ops.fht_f32(x, scale)
+    for bits in (4, 8):
+        q2, s2, b2 = fx.ops.quant_asym_u8(y, bits=bits)
+        q1, s1, b1 = fx.ops.fht_quant_asym_u8(x, scale, bits=bits)
+        assert np.array_equal(s1.numpy(), s2.numpy()) and np.array_equal(b1.numpy(), b2.numpy())
+        assert np.array_equal(q1.numpy(), q2.numpy())
+        assert int(q1.numpy().max()) == (1 << bits) - 1 and int(q1.numpy().min()) == 0
+
+
+def test_rmsnorm_with_asymmetric_quantisation(fx, oracle):
+    """RMSNorm + asymmetric uint4 quantisation, one wave per row of 2048 values, against the oracle's norm and
+    quantiser: scale and minimum to fp32 rounding (the kernel sums the squares in the model graphs' order), bytes equal
+    but for single steps at rounding ties; and against the device's two-kernel route on the values that route produces."""
+    rows, dim = 200, 2048
+    x = (rng.standard_normal((rows, dim)) * rng.uniform(0.2, 4.0, (rows, 1))).astype(np.float32)
+    gamma = rng.uniform(0.5, 1.5, dim).astype(np.float32)
+    q, s, b = fx.ops.rmsnorm_quant_asym_u8(fx.to_device(x), fx.to_device(gamma))
+    q, s, b = q.numpy(), s.numpy(), b.numpy()
+    yn = oracle.rmsnorm_pref(x, gamma)
+    qr, sr, br = oracle.quant_asym(yn, 4)
+    assert np.abs(s - sr).max() <= 2e-6 * np.abs(sr).max() and np.abs(b - br).max() <= 2e-6 * np.abs(br).max()
+    d = np.abs(q.astype(np.int32) - qr.astype(np.int32))
+    assert d.max() <= 1 and (d != 0).mean() < 2e-3
+    q2, s2, b2 = fx.ops.quant_asym_u8(fx.ops.rmsnorm_f32(fx.to_device(x), fx.to_device(gamma)), bits=4)
+    d2 = np.abs(q.astype(np.int32) - q2.numpy().astype(np.int32))
+    assert d2.max() <= 1 and (d2 != 0).mean() < 2e-3
+    assert int(q.max()) == 15 and int(q.min()) == 0
+
+
 def test_w4a4_layer_like_the_reference_testbench(fx, oracle):
     """quant (asym uint4) -> linear -> dequant with zero point, decode and prefill shapes: bit-exact against the oracle
     chain, and within the testbench's own 1e-2 criterion of the fake-quant golden (…_tb.cpp:215-236)."""
