@@ -216,10 +216,12 @@ enum GemmDmaEpi { kDmaRaw = 0, kDmaDequant = 1, kDmaSwiglu = 2, kDmaQkv = 3, kDm
 // so RoPE (pairs k, k+32), the static int8 quantisation and the store into q8 / the K cache / the transposed V
 // cache blocks all happen on the tile (64 tokens x 64 channels; a V cache block is 64 positions x 64 channels).
 struct QkvEpiArgs {
-    const float *sin_t, *cos_t, *q_s, *k_s, *v_s;
-    int8_t *q8, *kc, *vc;
-    int pos0, q_heads, kv_heads, max_pos;
-    const float *b_x, *w_sum;          // kDmaDequantAsym / kDmaSwigluAsym only: zero point per row, weight row sum (times its scale) per column
+    const float *sin_t = nullptr, *cos_t = nullptr, *q_s = nullptr, *k_s = nullptr, *v_s = nullptr;
+    int8_t *q8 = nullptr, *kc = nullptr, *vc = nullptr;
+    int pos0 = 0, q_heads = 0, kv_heads = 0, max_pos = 0;
+    // asymmetric activations (kDmaDequantAsym / kDmaSwigluAsym; optional for kDmaQkv, null = symmetric): zero point per
+    // row, weight row sum (times its scale) per column
+    const float *b_x = nullptr, *w_sum = nullptr;
 };
 
 __device__ __forceinline__ void gemm_dma_issue(const int8_t* base, unsigned voff, unsigned lds_dst) {
@@ -414,10 +416,15 @@ __global__ __launch_bounds__(NW * 64, WPE) void gemm_i8_dma_kernel(const int8_t*
         {
             const int col = col0 + wn + (lane & 31);
             const float ws = w_s[col];
+            const bool asym = qa.b_x != nullptr;              // asymmetric activations: + zero point x row sum of the dequantised weights
+            const float wq = asym ? qa.w_sum[col] : 0.0f;
 #pragma unroll
             for (int r = 0; r < 16; r++) {
                 const int lr = wm + (r >> 2) * 8 + (lane >> 5) * 4 + (r & 3);
-                tile[lr * TP + wn + (lane & 31)] = (float)acc[0][0][r] * s_x[min(row0 + lr, m - 1)] * ws;
+                const int row = min(row0 + lr, m - 1);
+                float v = (float)acc[0][0][r] * s_x[row] * ws;
+                if (asym) v = v + qa.b_x[row] * wq;
+                tile[lr * TP + wn + (lane & 31)] = v;
             }
         }
         __syncthreads();

@@ -112,7 +112,7 @@ int llama_prefill_run_w4a4(const flexllm_llama_config& c, const LayerW* layers, 
     PrefillBuffers b;
     int rc = prefill_workspace_get(ws, c, s, &b, true);
     if (rc) return rc;
-    const int H = c.hidden, KV = c.kv_hidden, I = c.inter;
+    const int H = c.hidden, I = c.inter;
     uint8_t* xq = reinterpret_cast<uint8_t*>(b.xq);
     FX_HIP(hipMemcpyAsync(b.x, x_in, sizeof(float) * (size_t)s * H, hipMemcpyDeviceToDevice, st));
     for (int l = 0; l < c.layers; l++) {
@@ -127,9 +127,14 @@ int llama_prefill_run_w4a4(const flexllm_llama_config& c, const LayerW* layers, 
         // attention block
         rmsnorm_quant_asym_2048_wave_kernel<<<(s + kNormWaveRows - 1) / kNormWaveRows, 64 * kNormWaveRows, 0, st>>>(
             b.x, gamma + (size_t)(2 * l) * H, xq, b.xs, b.xb, s, c.eps, 15.0f, 15u);
-        if ((rc = launch_gemm_asym(b.xq, w.wqkv, b.xs, b.xb, w.sqkv, m4.mqkv, nullptr, b.qkv, s, H, H + 2 * KV, st))) return rc;
-        qkv_post_kernel<<<s, 256, 0, st>>>(b.qkv, rope_sin, rope_cos, q_s, k_s, v_s, b.q8, kc, vc, nullptr, 0, c.q_heads,
-                                           c.kv_heads, c.max_pos);
+        {   // q/k/v projection with the asymmetric dequantisation, RoPE, static quantisation and the cache stores in the GEMM epilogue
+            QkvEpiArgs qa;
+            qa.sin_t = rope_sin; qa.cos_t = rope_cos; qa.q_s = q_s; qa.k_s = k_s; qa.v_s = v_s;
+            qa.q8 = b.q8; qa.kc = kc; qa.vc = vc;
+            qa.pos0 = 0; qa.q_heads = c.q_heads; qa.kv_heads = c.kv_heads; qa.max_pos = c.max_pos;
+            qa.b_x = b.xb; qa.w_sum = m4.mqkv;
+            if ((rc = launch_gemm_qkv(b.xq, w.wqkv, b.xs, w.sqkv, s, H, qa, st))) return rc;
+        }
         if ((rc = mha_prefill_launch(b.q8, kc, vc, q_s, k_s, v_s, a_s, b.att, nullptr, s, c.q_heads, c.kv_heads, c.max_pos, st))) return rc;
         quant_asym_kernel<2><<<s, kBlock, 0, st>>>(b.att, xq, b.xs, b.xb, H, 15.0f, 15u);
         if ((rc = launch_gemm_asym(b.xq, w.wo, b.xs, b.xb, w.so, m4.mo, b.x, b.x2, s, H, H, st))) return rc;
