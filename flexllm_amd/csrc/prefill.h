@@ -19,7 +19,6 @@ struct LayerW4 {
 
 struct PrefillWorkspace {
     int tokens = 0;
-    bool w4 = false;        // sized for the W4A4 graph (one more fp32 scratch array)
     void* base = nullptr;
 };
 

@@ -9,39 +9,34 @@
 namespace fx {
 
 struct PrefillBuffers {
-    float *x, *x2, *qkv, *att, *gu;
-    int8_t *xq, *q8;
-    float* xs;
-    float *xb, *fh;         // W4A4 only: zero points per token; fp32 scratch [s][inter] (normalised rows, transformed rows)
+    float *x, *x2, *att;    // residual stream before / after the attention block, attention output: [s][hidden]
+    float* gu;              // SiLU(gate)*up [s][inter]
+    int8_t *xq, *q8;        // quantised input of the current linear layer [s][inter at most]; quantised, rotated q [s][hidden]
+    float *xs, *xb;         // per-token scales; per-token zero points (W4A4 graph)
 };
 
-static int prefill_workspace_get(PrefillWorkspace* ws, const flexllm_llama_config& c, int s, PrefillBuffers* b, bool w4 = false) {
-    const size_t H = c.hidden, KV = c.kv_hidden, I = c.inter;
+static int prefill_workspace_get(PrefillWorkspace* ws, const flexllm_llama_config& c, int s, PrefillBuffers* b) {
+    const size_t H = c.hidden, I = c.inter;
     auto up = [](size_t v) { return (v + 255) & ~(size_t)255; };
-    const size_t sz_x = up(sizeof(float) * s * H), sz_qkv = up(sizeof(float) * s * (H + 2 * KV));
-    const size_t sz_gu = up(sizeof(float) * s * 2 * I), sz_xq = up((size_t)s * I), sz_q8 = up((size_t)s * H);
+    const size_t sz_x = up(sizeof(float) * s * H), sz_gu = up(sizeof(float) * s * I), sz_xq = up((size_t)s * I), sz_q8 = up((size_t)s * H);
     const size_t sz_xs = up(sizeof(float) * s);
-    const size_t sz_fh = w4 ? up(sizeof(float) * s * I) : 0;
-    const size_t total = 3 * sz_x + sz_qkv + sz_gu + sz_xq + sz_q8 + 2 * sz_xs + sz_fh;
-    if (ws->tokens < s || (w4 && !ws->w4)) {
+    const size_t total = 3 * sz_x + sz_gu + sz_xq + sz_q8 + 2 * sz_xs;
+    if (ws->tokens < s) {
         FX_HIP(hipDeviceSynchronize());
         prefill_workspace_free(ws);
         hipError_t e = hipMalloc(&ws->base, total);
         if (e != hipSuccess) { set_error("prefill workspace hipMalloc(%zu) failed: %s", total, hipGetErrorString(e)); return FLEXLLM_ENOMEM; }
         ws->tokens = s;
-        ws->w4 = w4;
     }
     char* p = (char*)ws->base;
     b->x = (float*)p; p += sz_x;
     b->x2 = (float*)p; p += sz_x;
     b->att = (float*)p; p += sz_x;
-    b->qkv = (float*)p; p += sz_qkv;
     b->gu = (float*)p; p += sz_gu;
     b->xq = (int8_t*)p; p += sz_xq;
     b->q8 = (int8_t*)p; p += sz_q8;
     b->xs = (float*)p; p += sz_xs;
     b->xb = (float*)p; p += sz_xs;
-    b->fh = w4 ? (float*)p : nullptr;
     return FLEXLLM_OK;
 }
 
@@ -110,7 +105,7 @@ int llama_prefill_run_w4a4(const flexllm_llama_config& c, const LayerW* layers, 
     FX_REQUIRE(s > 0 && s % kPfTile == 0 && s <= c.max_pos, "prefill: s=%d must be a positive multiple of 32, <= max_pos=%d", s, c.max_pos);
     FX_REQUIRE(c.hidden == 2048 && c.inter == 8192, "prefill (W4A4): hidden=%d inter=%d (instantiated for 2048/8192)", c.hidden, c.inter);
     PrefillBuffers b;
-    int rc = prefill_workspace_get(ws, c, s, &b, true);
+    int rc = prefill_workspace_get(ws, c, s, &b);
     if (rc) return rc;
     const int H = c.hidden, I = c.inter;
     uint8_t* xq = reinterpret_cast<uint8_t*>(b.xq);
