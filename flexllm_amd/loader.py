@@ -12,12 +12,14 @@ What the reference's testbench reads (SpinQuant_Llama_32_1B/SpinQuant_Prefilling
     `V_s[layers][kv_heads]`, `A_s[layers][q_heads]` (SpinQuant_Llama_32_1B/MHA_i8xi8.h:11-14, :32, :63, :245)
 
 The reference tree ships none of these files, so the header syntax is taken from how the arrays are indexed: any C
-initialiser `name[d0][d1] = { ... }` (or one-dimensional) is accepted, numbers may carry an `f` suffix.  The rotary
+initialiser `name[d0][d1] = { ... }` (or one-dimensional) is accepted, numbers are C floating literals (decimal or
+hexadecimal, with or without an `f` suffix).  The rotary
 table (`parameters/RoPE_sin_cos.h`) is regenerated from the formula.  For the W8A8 model the output head is the
 embedding matrix in fp16 (tied) and `lm_head.bin` / `w_lm_head_lm_head.h` are not read; with w4a4=True the loader also
 returns the row sums (`sum<p>`) and the int4 output head (`lm_head.bin`, row-major int8 `[vocab][hidden]` holding -8..7,
 with `w_lm_head_lm_head_s[vocab]` and `w_lm_head_lm_head_sum[vocab]`, SpinQuant_Prefilling_Decoding_mem_opt_tb.cpp:
-187-192, 442, 655-660, 716-719): the dictionary `llama.Llama` turns into the W4A4 model.  A row sum is the sum of the
+187-192, 442, 655-660, 716-719; the file's row count is not pinned by anything the reference ships - the testbench
+reads the padded vocabulary's rows from it - so any whole number of rows >= vocab is accepted): the dictionary `llama.Llama` turns into the W4A4 model.  A row sum is the sum of the
 row's DEQUANTISED weights (the zero point of the activations multiplies it directly, Modules/quant.h:147-152; the
 linear testbench accumulates qval * scale, Linear_Layer_Decoding_tb.cpp:171-188).
 
@@ -36,7 +38,13 @@ _PROJ_FILES = dict(q="q_proj", k="k_proj", v="v_proj", o="o_proj", g="gate_proj"
 _PROJ_DIMS = dict(q=("hidden", "hidden"), k=("kv_hidden", "hidden"), v=("kv_hidden", "hidden"), o=("hidden", "hidden"),
                   g=("inter", "hidden"), u=("inter", "hidden"), d=("hidden", "inter"))
 _STATIC = dict(q_s=("Q_s", "q_heads"), k_s=("K_s", "kv_heads"), v_s=("V_s", "kv_heads"), a_s=("A_s", "q_heads"))
-_NUM = re.compile(r"[-+]?(?:\d+\.\d*|\.\d+|\d+)(?:[eE][-+]?\d+)?")
+# a C floating literal: hexadecimal (0x1.8p-3) or decimal, with an optional f/F/l/L suffix that is dropped
+_NUM = re.compile(r"[-+]?(?:0[xX](?:[0-9a-fA-F]+\.?[0-9a-fA-F]*|\.[0-9a-fA-F]+)(?:[pP][-+]?\d+)?"
+                  r"|(?:\d+\.\d*|\.\d+|\d+)(?:[eE][-+]?\d+)?)")
+
+
+def _c_float(tok):
+    return float.fromhex(tok) if "x" in tok or "X" in tok else float(tok)
 
 
 class ParameterError(ValueError):
@@ -59,8 +67,8 @@ def parse_c_array(text, name):
     if depth:
         raise ParameterError("array %s: unbalanced braces" % name)
     body = text[m.end():i - 1]
-    vals = np.array([float(v) for v in _NUM.findall(re.sub(r"(?<=[\d.])[fF]\b", "", body))], dtype=np.float64)
-    vals = vals.astype(np.float32)
+    with np.errstate(over="ignore"):
+        vals = np.array([_c_float(v) for v in _NUM.findall(body)], dtype=np.float64).astype(np.float32)
     if not all(d.isdigit() for d in dims):
         return vals                                # sizes given by macros or left open: flat, the caller knows the shape
     shape = [int(d) for d in dims]
@@ -69,13 +77,18 @@ def parse_c_array(text, name):
     return vals.reshape(shape)
 
 
-def _read_header_array(param_dir, fname, name, shape):
+def _read_header_array(param_dir, fname, name, shape, padded=False):
+    """padded=True accepts a one-dimensional array longer than `shape` (an export padded to the reference's
+    VOCAB_SIZE_PAD) and returns its first entries."""
     path = os.path.join(param_dir, fname)
     if not os.path.exists(path):
         raise ParameterError("missing %s" % path)
     with open(path) as f:
         arr = parse_c_array(f.read(), name)
-    if arr.size != int(np.prod(shape)):
+    want = int(np.prod(shape))
+    if padded and arr.size > want:
+        arr = arr.reshape(-1)[:want]
+    if arr.size != want:
         raise ParameterError("%s: %s has %d values, expected %s" % (path, name, arr.size, shape))
     return np.ascontiguousarray(arr.reshape(shape))
 
@@ -120,13 +133,17 @@ def load_reference_parameters(param_dir, cfg, device=True, w4a4=False):
         path = os.path.join(param_dir, "lm_head.bin")
         if not os.path.exists(path):
             raise ParameterError("missing %s" % path)
-        if os.path.getsize(path) != cfg["vocab"] * H:
-            raise ParameterError("%s: %d bytes, expected %d x %d" % (path, os.path.getsize(path), cfg["vocab"], H))
-        w["head_w"] = np.fromfile(path, dtype=np.int8).reshape(cfg["vocab"], H)
+        # The testbench reads VOCAB_SIZE_PAD (131072) rows from this file and VOCAB_SIZE (128256) scale pairs
+        # (:196-201, :716-719); no such file ships with the reference, so its row count is not pinned: any whole
+        # number of rows >= vocab is accepted and the first vocab rows are used, likewise for the two arrays.
+        size = os.path.getsize(path)
+        if size < cfg["vocab"] * H or size % H:
+            raise ParameterError("%s: %d bytes, expected at least %d whole rows of %d" % (path, size, cfg["vocab"], H))
+        w["head_w"] = np.ascontiguousarray(np.fromfile(path, dtype=np.int8, count=cfg["vocab"] * H).reshape(cfg["vocab"], H))
         if w["head_w"].min() < -8 or w["head_w"].max() > 7:
             raise ParameterError("lm_head.bin holds values outside -8..7: not an int4 export")
-        w["head_s"] = _read_header_array(param_dir, "w_lm_head_lm_head.h", "w_lm_head_lm_head_s", (cfg["vocab"],))
-        w["head_sum"] = _read_header_array(param_dir, "w_lm_head_lm_head.h", "w_lm_head_lm_head_sum", (cfg["vocab"],))
+        w["head_s"] = _read_header_array(param_dir, "w_lm_head_lm_head.h", "w_lm_head_lm_head_s", (cfg["vocab"],), padded=True)
+        w["head_sum"] = _read_header_array(param_dir, "w_lm_head_lm_head.h", "w_lm_head_lm_head_sum", (cfg["vocab"],), padded=True)
     if not device:
         return w
     dev = {}
