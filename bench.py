@@ -83,7 +83,104 @@ def _time(stream, Event, fn, reps):
     return e0.elapsed_ms(e1) * 1e3 / reps          # microseconds per call
 
 
-def module_legs(fx, lib, synth, ops, stream, Event):
+def measured_peaks(fx, lib, synth, stream, Event):
+    """What this GPU sustains on the two resources the rooflines are priced against, beside the published peaks:
+    HBM as a read-only stream over 4 GiB (16 times the memory-side cache) and as a 1 GiB device copy (read + write),
+    and the int8 matrix cores alone (no global memory) with zero and with pseudo-random operands, from registers and
+    re-read from LDS at every step, with the shader clock read inside the kernel under that load."""
+    P = lambda a: C.c_void_p(a.ptr)
+    out = {}
+    n = 1 << 32
+    buf = fx.empty((n,), np.int8)
+    fx.check(lib.flexllm_rt_fill_i8(P(buf), C.c_size_t(n), C.c_uint64(77), -100, 100, stream.handle))
+    wgs = 8192
+    sink = fx.empty((wgs * 4,), np.uint32)
+    us = _time(stream, Event, lambda i: lib.flexllm_probe_hbm_read(P(buf), C.c_size_t(n), wgs, P(sink), stream.handle), 5)
+    one = 1 << 30
+    us_c = _time(stream, Event, lambda i: lib.flexllm_rt_memcpy_d2d(C.c_void_p(buf.ptr + 2 * one), P(buf), C.c_size_t(one), stream.handle), 5)
+    out["hbm"] = {"published_GBs": HBM_PEAK_GBS, "read_stream_GBs": round(n / us / 1e3, 1), "read_stream_bytes": n,
+                  "copy_GBs_read_plus_write": round(2 * one / us_c / 1e3, 1), "copy_bytes": one,
+                  "note": "read_stream: non-temporal 16-byte loads over 4 GiB, read-only (the decode path's traffic is 99 % reads); "
+                          "copy: hipMemcpyAsync device to device of 1 GiB, bytes read + bytes written"}
+    del buf
+    iters, cus = 4000, 256
+    sink_i = fx.empty((cus * 256,), np.int32)
+    clocks = fx.zeros((2,), np.uint64)
+    mf = {"published_TOPs": INT8_PEAK_TOPS}
+    ops_launch = cus * 4 * iters * 16 * 65536.0
+    for name, rnd, lds in (("zeros_regs", 0, 0), ("random_regs", 1, 0), ("zeros_lds", 0, 1), ("random_lds", 1, 1)):
+        us = _time(stream, Event, lambda i: lib.flexllm_probe_mfma_i8(iters, rnd, lds, cus, P(sink_i), P(clocks), stream.handle), 3)
+        cyc, ticks = [int(v) for v in clocks.numpy()]
+        mf[name + "_TOPs"] = round(ops_launch / us / 1e6, 1)
+        mf[name + "_shader_clock_GHz"] = round(cyc / max(ticks, 1) * 0.1, 3)
+    mf["note"] = ("256 workgroups x 4 waves issuing v_mfma_i32_32x32x32_i8 back to back on 16 accumulator tiles per wave, no global "
+                  "memory; lds = the 8 operand fragments re-read from LDS for every 16 instructions; random operands draw more power "
+                  "than zeros and the clock drops accordingly; random_lds is what a GEMM's inner loop can reach at best")
+    out["mfma_i8"] = mf
+    return out
+
+
+def cpu_module_legs(oracle, cfg, n_threads):
+    """The CPU oracle (all OpenMP threads of the host) on the same module-level workloads as module_legs, so that each
+    GPU figure has the reference-semantics CPU figure beside it.  Bounded: the S = 4096 attention is timed on 4 of its
+    32 query heads."""
+    r = np.random.default_rng(5)
+    out = {}
+
+    def timed(fn, reps=1):
+        fn()
+        t0 = time.perf_counter()
+        for _ in range(reps):
+            fn()
+        return (time.perf_counter() - t0) / reps * 1e3
+
+    i8 = lambda *sh: r.integers(-127, 128, sh, dtype=np.int8)
+    K = N = 2048
+    x = r.standard_normal((1, K)).astype(np.float32); w = i8(N, K); ws = r.uniform(1e-3, 1e-2, N).astype(np.float32)
+    def lin1():
+        q, s = oracle.quant_sym(x)
+        oracle.dequant(oracle.linear_i8(q, w), s, ws)
+    out["linear_decode_2048x2048"] = {"ms_quant_gemv_dequant": round(timed(lin1, 20), 4)}
+    for n in (2048, 8192):
+        xf = r.standard_normal((1024, n)).astype(np.float32)
+        out["fht_quant_1024x%d" % n] = {"ms": round(timed(lambda: oracle.quant_sym(oracle.fht(xf, float(np.sqrt(n))))), 3)}
+    M, H, KV, I = 1024, 2048, 512, 8192
+    a = i8(M, H); a8 = i8(M, I); sx = r.uniform(0.01, 0.02, M).astype(np.float32)
+    res = r.standard_normal((M, H)).astype(np.float32)
+    scn = r.uniform(1e-4, 2e-4, 2 * I).astype(np.float32)
+    stack = {}
+    wq = i8(H + 2 * KV, H); stack["qkv"] = timed(lambda: oracle.dequant(oracle.linear_i8(a, wq), sx, scn[:H + 2 * KV]))
+    wo = i8(H, H); stack["o+res"] = timed(lambda: oracle.residual(oracle.dequant(oracle.linear_i8(a, wo), sx, scn[:H]), res))
+    wg = i8(2 * I, H)
+    def gu():
+        y = oracle.dequant(oracle.linear_i8(a, wg), sx, scn)
+        oracle.gate(y[:, 1::2], oracle.swish(y[:, 0::2]))
+    stack["gate_up+swiglu"] = timed(gu)
+    wd = i8(H, I); stack["down+res"] = timed(lambda: oracle.residual(oracle.dequant(oracle.linear_i8(a8, wd), sx, scn[:H]), res))
+    del wq, wo, wg, wd
+    stack = {k: round(v, 2) for k, v in stack.items()}
+    stack["total"] = round(sum(stack.values()), 2)
+    out["prefill_linear_stack_M1024"] = {"ms": stack}
+    sc = (np.full(32, 4e-3, np.float32), np.full(8, 0.03, np.float32), np.full(8, 0.03, np.float32), np.full(32, 1.0 / 255, np.float32))
+    S = 1024
+    q8 = i8(S, 32, 64); k8 = r.integers(-100, 101, (S, 8, 64), dtype=np.int8); v8 = r.integers(-100, 101, (S, 8, 64), dtype=np.int8)
+    out["attention_prefill_S1024"] = {"ms": round(timed(lambda: oracle.mha_prefill_i8(q8, k8, v8, *sc)), 2)}
+    S = 4096
+    q8 = i8(S, 4, 64); k8 = r.integers(-100, 101, (S, 1, 64), dtype=np.int8); v8 = r.integers(-100, 101, (S, 1, 64), dtype=np.int8)
+    sc4 = (sc[0][:4], sc[1][:1], sc[2][:1], sc[3][:4])
+    t0 = time.perf_counter(); oracle.mha_prefill_i8(q8, k8, v8, *sc4); t4 = (time.perf_counter() - t0) * 1e3
+    out["attention_prefill_S4096"] = {"ms_4_of_32_heads": round(t4, 1), "note": "one KV head with its 4 query heads: an eighth of the leg's work"}
+    K, N = 2048, 8192
+    w4 = r.integers(-8, 8, (N, K), dtype=np.int8); w4s = r.uniform(1e-3, 1e-2, N).astype(np.float32); w4m = r.uniform(-1, 1, N).astype(np.float32)
+    x1 = r.standard_normal((1, K)).astype(np.float32); xm = r.standard_normal((1024, K)).astype(np.float32)
+    out["w4a4_linear_decode_2048x8192"] = {"ms": round(timed(lambda: oracle.w4a4_linear(x1, w4, w4s, w4m), 10), 4)}
+    out["w4a4_linear_prefill_M1024_2048x8192"] = {"ms": round(timed(lambda: oracle.w4a4_linear(xm, w4, w4s, w4m)), 2)}
+    for v in out.values():
+        v["threads"] = n_threads
+    return out
+
+
+def module_legs(fx, lib, synth, ops, stream, Event, peaks=None):
     """Single-module timings on seeded synthetic inputs, weights cycled through rings larger than the 256 MB
     memory-side cache: (1) decode linear 2048x2048, (2) Hadamard + per-token quantisation of 1024 tokens,
     (3) the prefill linear stack of one layer at M=1024, (4) prefill attention at S=1024 and 4096, (5) the W4A4
@@ -143,6 +240,9 @@ def module_legs(fx, lib, synth, ops, stream, Event):
         tot_us += us; tot_ops += opsn
     stack["total"] = {"us": round(tot_us, 2), "GOP": round(tot_ops / 1e9, 2), "TOPs": round(tot_ops / tot_us / 1e6, 1),
                       "mfma_frac": round(tot_ops / tot_us / 1e6 / INT8_PEAK_TOPS, 4)}
+    if peaks:
+        for leg in stack.values():
+            leg["mfma_frac_of_measured_peak"] = round(leg["TOPs"] / peaks["mfma_i8"]["random_lds_TOPs"], 4)
     out["prefill_linear_stack_M1024"] = stack
     del wq, wo, wg, wd
     # (4) prefill attention, S = 1024 and the maximum context 4096, 32/8 heads, reading the int8 cache
@@ -215,6 +315,9 @@ def main():
     ap.add_argument("--copy-probe", action="store_true",
                     help="only run three 1 GiB device-to-device copies and exit: the transfer of known size that scales "
                          "the FETCH_SIZE / WRITE_SIZE counters")
+    ap.add_argument("--peaks-probe", action="store_true",
+                    help="only run the measured-peak probes (HBM read stream, device copy, matrix cores alone) and exit: the "
+                         "short command the profiler summary of the probes uses")
     ap.add_argument("--module-probe", action="store_true",
                     help="only run the single-module legs (decode linear, Hadamard + quantisation, prefill linear stack, "
                          "prefill attention, W4A4 linears) and exit: the short command the per-kernel counter runs use")
@@ -237,6 +340,10 @@ def main():
             fx.check(lib.flexllm_rt_memcpy_d2d(C.c_void_p(dst.ptr), C.c_void_p(src.ptr), C.c_size_t(n), None))
         device_sync()
         print(json.dumps({"copy_probe_bytes": n, "copies": 3}))
+        return
+    if args.peaks_probe:
+        from flexllm_amd.device import Stream
+        print(json.dumps({"peaks": measured_peaks(fx, lib, synth, Stream(), Event)}))
         return
     if args.module_probe:
         from flexllm_amd.device import Stream
@@ -341,8 +448,11 @@ def main():
 
     # ---- module-level legs: the other configurations the metric's source names, each against its roofline ----
     modules = None
+    peaks = None
     if not args.no_modules:
-        modules = module_legs(fx, lib, synth, ops, stream, Event)
+        # measured peaks of this GPU (HBM stream, matrix cores alone), beside the published ones
+        peaks = measured_peaks(fx, lib, synth, stream, Event)
+        modules = module_legs(fx, lib, synth, ops, stream, Event, peaks)
         if not args.no_prefill and cfg["max_pos"] >= 1024:
             # HMT plug-in at the reference's segment sizes (990 tokens, summary 495, recurrent 32, 64 memory slots):
             # one middle segment = stage 0 (512 rows) + retrieval + stage 1 (1024 rows) + memory update
@@ -459,6 +569,26 @@ def main():
                "single_core_value": round(n1 / t1, 4),
                "sample": "%d whole tokens (16 layers, context 4096, full head) on %d OpenMP threads in %.1f s; single thread: "
                          "%d tokens in %.1f s (C oracle, host reports %d cpus)" % (nN, n_threads, tN, n1, t1, os.cpu_count())}
+        del om, kc, vc
+        # the CPU figure beside the prefill leg: one full-size layer on 1024 tokens, measured (a 16-layer prefill is 16 of them)
+        if prefill_ms is not None:
+            cfg1 = llama.make_config(layers=1, vocab=256, max_pos=1024)
+            hw1 = {k: (v[:1] if isinstance(v, list) else v) for k, v in hw.items()}
+            hw1["embed"] = hw["embed"][:256]; hw1["rope_sin"] = hw["rope_sin"][:1024]; hw1["rope_cos"] = hw["rope_cos"][:1024]
+            hw1["gamma"] = np.ascontiguousarray(hw["gamma"][:3])
+            for n in ("q_s", "k_s", "v_s", "a_s"):
+                hw1[n] = np.ascontiguousarray(hw[n][:1])
+            om1 = oracle.OracleModel(cfg1, hw1)
+            k1, v1 = om1.new_caches()
+            xp = synth.host_normal_f32((1024, H), 906)
+            t0 = time.perf_counter(); om1.prefill(xp, k1, v1); t_layer = time.perf_counter() - t0
+            cpu["prefill_1024_one_layer_ms"] = round(t_layer * 1e3, 1)
+            cpu["prefill_1024_16_layers_ms_at_that_rate"] = round(16 * t_layer * 1e3, 1)
+        # and beside every module leg
+        if modules is not None:
+            for name, fig in cpu_module_legs(oracle, cfg, n_threads).items():
+                if name in modules:
+                    modules[name]["cpu_oracle"] = fig
 
     traffic_tok = measured_traffic_per_token()
     # prefill against the int8 MFMA roofline: 16 x (linear stack 2*M*sum(K*N) + attention 2*2*heads*S*S*64, full S^2)
@@ -470,6 +600,7 @@ def main():
         ops_total = L * (lin + att)
         prefill_roof = {"bound": "mfma", "ops": int(ops_total), "achieved": round(ops_total / (prefill_ms * 1e-3) / 1e12, 1),
                         "peak": INT8_PEAK_TOPS, "unit": "TOP/s", "frac": round(ops_total / (prefill_ms * 1e-3) / 1e12 / INT8_PEAK_TOPS, 4),
+                        "frac_of_measured_peak": None if not peaks else round(ops_total / (prefill_ms * 1e-3) / 1e12 / peaks["mfma_i8"]["random_lds_TOPs"], 4),
                         "note": "whole 1024-token prefill (16 layers: norms, quantisation, GEMMs, attention with the full S^2 counted, Hadamard)"}
     result = {
         "metric": "decode tok/s + prefill ms (1024 tok), Llama-3.2-1B W8A8, % HBM/MFMA roofline",
@@ -492,12 +623,14 @@ def main():
         "roofline": {"bound": "hbm", "kernel": "decode_mega_kernel (%d launches of <= %d tokens)" % (n_launch, TOKENS_PER_LAUNCH),
                      "achieved": round(bpt * K / (ev_ms * 1e-3) / 1e9, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(bpt * K / (ev_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
+                     "frac_of_measured_peak": None if not peaks else round(bpt * K / (ev_ms * 1e-3) / 1e9 / peaks["hbm"]["read_stream_GBs"], 4),
                      "traffic": int(traffic_tok * K / n_launch) if (traffic_tok and cfg["layers"] == 16 and pos_end == 4096) else None,
                      "bytes_per_launch": int(bpt * K / n_launch), "tokens_per_launch": round(K / n_launch, 2),
                      "avg_us": round(ev_ms / n_launch * 1e3, 2), "us_per_token": round(ev_ms / K * 1e3, 2)},
         "gemv_gate_up": {"kernel": "gemv_i8_kernel<2,4,swiglu> stand-alone (2048->2x8192), 16 distinct weight buffers",
                          "achieved_GBs": round(kern_gbs, 1), "hbm_frac": round(kern_gbs / HBM_PEAK_GBS, 4),
                          "bytes_per_launch": int(kern_bytes), "avg_us": round(kern_ms * 1e3, 3)},
+        "peaks": peaks,
         "modules": modules,
         "cpu_baseline": cpu,
     }

@@ -76,10 +76,11 @@ int flexllm_mha_i8_decode(const int8_t* q8, const int8_t* k_cache, const int8_t*
                "mha_decode: q_heads=%d kv_heads=%d (group size 1..4)", q_heads, kv_heads);
     FX_REQUIRE(len >= 1 && len <= kChunk * kMaxChunks && len <= max_pos && max_pos % kVBlock == 0,
                "mha_decode: len=%d max_pos=%d (1 <= len <= 8192, len <= max_pos, max_pos %% 64 == 0)", len, max_pos);
-    int rc = ensure_scratch(q_heads, len);
+    DecodeScratch ds;
+    int rc = decode_scratch_of_stream(as_stream(stream), q_heads, len, &ds);
     if (rc) return rc;
-    return mha_decode_launch(q8, k_cache, v_cache, sc->q_s, sc->k_s, sc->v_s, sc->a_s, o, p8_out, g_scratch.scores,
-                             g_scratch.stats, g_scratch.o_acc, len, q_heads, kv_heads, max_pos, as_stream(stream));
+    return mha_decode_launch(q8, k_cache, v_cache, sc->q_s, sc->k_s, sc->v_s, sc->a_s, o, p8_out, ds.scores, ds.stats,
+                             ds.o_acc, len, q_heads, kv_heads, max_pos, as_stream(stream));
 }
 
 int flexllm_mha_i8_decode_noalloc(const int8_t* q8, const int8_t* k_cache, const int8_t* v_cache, const flexllm_mha_scales* sc,

@@ -229,29 +229,22 @@ struct DecodeScratch {
     float* scores = nullptr;   // [q_heads][len]
     float2* stats = nullptr;   // [q_heads][kMaxChunks]
     int32_t* o_acc = nullptr;  // [q_heads][64]
-    size_t score_elems = 0;
-    int heads = 0;
 };
-inline DecodeScratch g_scratch;
-inline std::mutex g_scratch_mu;
 
-static int ensure_scratch(int q_heads, int len) {
-    std::lock_guard<std::mutex> lk(g_scratch_mu);
+// The calling stream's scratch (stream_scratch), carved into the three arrays.
+static int decode_scratch_of_stream(hipStream_t st, int q_heads, int len, DecodeScratch* out) {
+    const size_t heads = q_heads > 32 ? q_heads : 32;
     const size_t need = (size_t)q_heads * len;
-    if (need > g_scratch.score_elems || q_heads > g_scratch.heads) {
-        FX_HIP(hipDeviceSynchronize());
-        if (g_scratch.scores) (void)hipFree(g_scratch.scores);
-        if (g_scratch.stats) (void)hipFree(g_scratch.stats);
-        if (g_scratch.o_acc) (void)hipFree(g_scratch.o_acc);
-        g_scratch = DecodeScratch();
-        const int heads = q_heads > 32 ? q_heads : 32;
-        const size_t elems = need > (size_t)heads * 4096 ? need : (size_t)heads * 4096;
-        FX_HIP(hipMalloc(&g_scratch.scores, elems * sizeof(float)));
-        FX_HIP(hipMalloc(&g_scratch.stats, (size_t)heads * kMaxChunks * sizeof(float2)));
-        FX_HIP(hipMalloc(&g_scratch.o_acc, (size_t)heads * kHd * sizeof(int32_t)));
-        g_scratch.score_elems = elems;
-        g_scratch.heads = heads;
-    }
+    const size_t elems = need > heads * 4096 ? need : heads * 4096;
+    auto up = [](size_t v) { return (v + 255) & ~(size_t)255; };
+    const size_t b_scores = up(elems * sizeof(float)), b_stats = up(heads * kMaxChunks * sizeof(float2)), b_acc = up(heads * kHd * sizeof(int32_t));
+    void* base = nullptr;
+    int rc = stream_scratch(kScratchMhaDecode, st, b_scores + b_stats + b_acc, &base);
+    if (rc) return rc;
+    char* p = static_cast<char*>(base);
+    out->scores = reinterpret_cast<float*>(p);
+    out->stats = reinterpret_cast<float2*>(p + b_scores);
+    out->o_acc = reinterpret_cast<int32_t*>(p + b_scores + b_stats);
     return FLEXLLM_OK;
 }
 

@@ -301,40 +301,31 @@ static __global__ __launch_bounds__(256) void dec_out_dyn_kernel(const int32_t* 
     }
 }
 
-// library-owned scratch of the decode entry point (grown on demand, shared process-wide like flexllm_mha_i8_decode's)
+// scratch of the decode entry point: the calling stream's buffer (stream_scratch), carved into its arrays
 struct DynScratch {
     float* scores = nullptr;
     float2* stats = nullptr;
     float* pmax = nullptr;
     float* p_s = nullptr;
     int32_t* o_acc = nullptr;
-    size_t score_elems = 0;
-    int heads = 0;
 };
-static DynScratch g_dyn;
-static std::mutex g_dyn_mu;
 
-static int ensure_dyn_scratch(int q_heads, int len) {
-    std::lock_guard<std::mutex> lk(g_dyn_mu);
+static int dyn_scratch_of_stream(hipStream_t st, int q_heads, int len, DynScratch* out) {
+    const size_t heads = q_heads > 32 ? q_heads : 32;
     const size_t need = (size_t)q_heads * len;
-    if (need > g_dyn.score_elems || q_heads > g_dyn.heads) {
-        FX_HIP(hipDeviceSynchronize());
-        if (g_dyn.scores) (void)hipFree(g_dyn.scores);
-        if (g_dyn.stats) (void)hipFree(g_dyn.stats);
-        if (g_dyn.pmax) (void)hipFree(g_dyn.pmax);
-        if (g_dyn.p_s) (void)hipFree(g_dyn.p_s);
-        if (g_dyn.o_acc) (void)hipFree(g_dyn.o_acc);
-        g_dyn = DynScratch();
-        const int heads = q_heads > 32 ? q_heads : 32;
-        const size_t elems = need > (size_t)heads * 4096 ? need : (size_t)heads * 4096;
-        FX_HIP(hipMalloc(&g_dyn.scores, elems * sizeof(float)));
-        FX_HIP(hipMalloc(&g_dyn.stats, (size_t)heads * kMaxChunks * sizeof(float2)));
-        FX_HIP(hipMalloc(&g_dyn.pmax, (size_t)heads * kMaxChunks * sizeof(float)));
-        FX_HIP(hipMalloc(&g_dyn.p_s, (size_t)heads * sizeof(float)));
-        FX_HIP(hipMalloc(&g_dyn.o_acc, (size_t)heads * kHd * sizeof(int32_t)));
-        g_dyn.score_elems = elems;
-        g_dyn.heads = heads;
-    }
+    const size_t elems = need > heads * 4096 ? need : heads * 4096;
+    auto up = [](size_t v) { return (v + 255) & ~(size_t)255; };
+    const size_t b_scores = up(elems * sizeof(float)), b_stats = up(heads * kMaxChunks * sizeof(float2)),
+                 b_pmax = up(heads * kMaxChunks * sizeof(float)), b_ps = up(heads * sizeof(float)), b_acc = up(heads * kHd * sizeof(int32_t));
+    void* base = nullptr;
+    int rc = stream_scratch(kScratchMhaDecodeDyn, st, b_scores + b_stats + b_pmax + b_ps + b_acc, &base);
+    if (rc) return rc;
+    char* p = static_cast<char*>(base);
+    out->scores = reinterpret_cast<float*>(p); p += b_scores;
+    out->stats = reinterpret_cast<float2*>(p); p += b_stats;
+    out->pmax = reinterpret_cast<float*>(p); p += b_pmax;
+    out->p_s = reinterpret_cast<float*>(p); p += b_ps;
+    out->o_acc = reinterpret_cast<int32_t*>(p);
     return FLEXLLM_OK;
 }
 
@@ -376,18 +367,19 @@ int flexllm_mha_i8_decode_dyn(const int8_t* q8, const int8_t* k_cache, const int
                "mha_decode_dyn: q_heads=%d kv_heads=%d (group size 1..4)", q_heads, kv_heads);
     FX_REQUIRE(len >= 1 && len <= kChunk * kMaxChunks && len <= max_pos && max_pos % kVBlock == 0,
                "mha_decode_dyn: len=%d max_pos=%d (1 <= len <= 8192, len <= max_pos, max_pos %% 64 == 0)", len, max_pos);
-    int rc = ensure_dyn_scratch(q_heads, len);
-    if (rc) return rc;
     hipStream_t st = as_stream(stream);
+    DynScratch ds;
+    int rc = dyn_scratch_of_stream(st, q_heads, len, &ds);
+    if (rc) return rc;
     const DynScales d = {sc->q_s, sc->k_s, sc->v_s, sc->v_ch_s, sc->q_scale_div};
     const int group = q_heads / kv_heads;
     dim3 grid((len + kChunk - 1) / kChunk, kv_heads);
-    dec_scores_dyn_kernel<<<grid, 64 * group, 0, st>>>(q8, k_cache, d, g_dyn.scores, g_dyn.stats, g_dyn.o_acc, len, group, kv_heads, max_pos);
-    dec_pmax_dyn_kernel<<<grid, 64 * group, 0, st>>>(g_dyn.scores, g_dyn.stats, d, g_dyn.pmax, len, group, kv_heads);
-    float* p_s = p_s_out ? p_s_out : g_dyn.p_s;
-    dec_pv_dyn_kernel<<<grid, 64 * group, 0, st>>>(g_dyn.scores, g_dyn.pmax, v_cache, g_dyn.o_acc, p8_out, p_s, len, group, max_pos);
+    dec_scores_dyn_kernel<<<grid, 64 * group, 0, st>>>(q8, k_cache, d, ds.scores, ds.stats, ds.o_acc, len, group, kv_heads, max_pos);
+    dec_pmax_dyn_kernel<<<grid, 64 * group, 0, st>>>(ds.scores, ds.stats, d, ds.pmax, len, group, kv_heads);
+    float* p_s = p_s_out ? p_s_out : ds.p_s;
+    dec_pv_dyn_kernel<<<grid, 64 * group, 0, st>>>(ds.scores, ds.pmax, v_cache, ds.o_acc, p8_out, p_s, len, group, max_pos);
     const int n = q_heads * kHd;
-    dec_out_dyn_kernel<<<(n + 255) / 256, 256, 0, st>>>(g_dyn.o_acc, p_s, sc->v_ch_s, o, n, group);
+    dec_out_dyn_kernel<<<(n + 255) / 256, 256, 0, st>>>(ds.o_acc, p_s, sc->v_ch_s, o, n, group);
     FX_LAUNCH_CHECK();
     return FLEXLLM_OK;
 }

@@ -43,6 +43,16 @@ void set_error(const char* fmt, ...);
 
 inline hipStream_t as_stream(void* s) { return reinterpret_cast<hipStream_t>(s); }
 
+// Scratch of the stand-alone entry points that need device memory beyond their arguments (arg-max and top-k
+// candidates, decode attention's scores / statistics / accumulators).  One buffer per (device, stream, kind), at least
+// `bytes` long and 256-byte aligned, allocated on first use and grown on demand: work of one stream runs in order and
+// may share a buffer, calls on different streams get different buffers and may run at the same time (also from
+// several host threads).  Growing waits for the stream's earlier work before the old buffer is freed.  A buffer is
+// released when its stream is destroyed through flexllm_rt_stream_destroy, otherwise it lives until the process ends.
+enum ScratchKind { kScratchArgmax = 0, kScratchTopK = 1, kScratchMhaDecode = 2, kScratchMhaDecodeDyn = 3 };
+int stream_scratch(ScratchKind kind, hipStream_t st, size_t bytes, void** out);
+void stream_scratch_release(hipStream_t st);
+
 // ---------------------------------------------------------------- cross-lane exchange
 // Value held by lane (lane ^ MASK).  1,2: DPP quad_perm; 8: DPP row rotate by 8; 4: two DPP row shifts, each
 // writing the banks (groups of four lanes) it is right for; 16: ds_swizzle bit mode (no LDS traffic, crossbar

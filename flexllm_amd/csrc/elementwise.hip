@@ -86,7 +86,10 @@ int flexllm_rmsnorm_f32(const float* x, const float* gamma, float* y, int rows, 
     FX_REQUIRE(x && gamma && y, "rmsnorm: null pointer");
     FX_REQUIRE(rows >= 0 && dim > 0 && dim % 4 == 0 && dim <= 16384, "rmsnorm: dim=%d must be a multiple of 4, <= 16384", dim);
     if (rows == 0) return FLEXLLM_OK;
-    FX_DISPATCH_VPT(dim, (rmsnorm_kernel<VPT, false><<<rows, kBlock, 0, as_stream(stream)>>>(x, gamma, y, nullptr, nullptr, dim, eps)));
+    if (dim == 2048)      // the graphs' order of summation (see flexllm_rmsnorm_quant_i8)
+        rmsnorm_kernel<1, false, 512><<<rows, 512, 0, as_stream(stream)>>>(x, gamma, y, nullptr, nullptr, dim, eps);
+    else
+        FX_DISPATCH_VPT(dim, (rmsnorm_kernel<VPT, false><<<rows, kBlock, 0, as_stream(stream)>>>(x, gamma, y, nullptr, nullptr, dim, eps)));
     FX_LAUNCH_CHECK();
     return FLEXLLM_OK;
 }
@@ -96,7 +99,13 @@ int flexllm_rmsnorm_quant_i8(const float* x, const float* gamma, int8_t* q, floa
     FX_REQUIRE(x && gamma && q && s, "rmsnorm_quant: null pointer");
     FX_REQUIRE(rows >= 0 && dim > 0 && dim % 4 == 0 && dim <= 16384, "rmsnorm_quant: dim=%d must be a multiple of 4, <= 16384", dim);
     if (rows == 0) return FLEXLLM_OK;
-    FX_DISPATCH_VPT(dim, (rmsnorm_kernel<VPT, true><<<rows, kBlock, 0, as_stream(stream)>>>(x, gamma, nullptr, q, s, dim, eps)));
+    // Rows of 2048 values take the one-wave-per-row kernel of the layer graphs: one order of summation for the sum of
+    // squares on every path (this entry point, the prefill graph, both decode schedules), so that a stage-by-stage
+    // chain of entry points reproduces the graphs bit for bit.
+    if (dim == 2048)
+        rmsnorm_quant_2048_wave_kernel<<<(rows + kNormWaveRows - 1) / kNormWaveRows, 64 * kNormWaveRows, 0, as_stream(stream)>>>(x, gamma, q, s, rows, eps);
+    else
+        FX_DISPATCH_VPT(dim, (rmsnorm_kernel<VPT, true><<<rows, kBlock, 0, as_stream(stream)>>>(x, gamma, nullptr, q, s, dim, eps)));
     FX_LAUNCH_CHECK();
     return FLEXLLM_OK;
 }

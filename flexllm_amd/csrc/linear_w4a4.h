@@ -104,4 +104,11 @@ static __global__ __launch_bounds__(256) void pack_nibbles_kernel(const uint8_t*
         out[i] = (uint8_t)((in[2 * i] & 0xF) | ((in[2 * i + 1] & 0xF) << 4));
 }
 
+// counts the bytes of `in` that are not 4-bit two's-complement values (-8..7) held one per byte
+static __global__ __launch_bounds__(256) void nibble_range_kernel(const int8_t* __restrict__ in, size_t n, unsigned* __restrict__ bad) {
+    unsigned c = 0;
+    for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (size_t)gridDim.x * 256) c += in[i] < -8 || in[i] > 7;
+    if (c) atomicAdd(bad, c);
+}
+
 }  // namespace fx

@@ -397,10 +397,15 @@ int flexllm_llama_create_w4a4(flexllm_llama** out, const flexllm_llama_config* c
             return fail(FLEXLLM_EHIP);                                                 \
         }                                                                              \
     } while (0)
+    // Every matrix must hold 4-bit values: the prefill graph multiplies the bytes as they are, the persistent decode
+    // kernel their low nibbles, and the two would silently part on anything outside -8..7.
+    unsigned* bad = reinterpret_cast<unsigned*>(m->state) + 7;     // a word of the token state no kernel uses at create time
+    FX_TRY_HIP(hipMemset(bad, 0, sizeof(unsigned)));
     auto pack = [&](const int8_t* values, int8_t** packed, size_t n_values) -> int {
         int r = dev_alloc(m, (void**)packed, n_values / 2);
         if (r) return r;
         const size_t n_out = n_values / 2;
+        nibble_range_kernel<<<(int)((n_values + 255) / 256 < 4096 ? (n_values + 255) / 256 : 4096), 256>>>(values, n_values, bad);
         pack_nibbles_kernel<<<(int)((n_out + 255) / 256 < 4096 ? (n_out + 255) / 256 : 4096), 256>>>(
             reinterpret_cast<const uint8_t*>(values), reinterpret_cast<uint8_t*>(*packed), n_out);
         return FLEXLLM_OK;
@@ -439,6 +444,15 @@ int flexllm_llama_create_w4a4(flexllm_llama** out, const flexllm_llama_config* c
     FX_TRY_HIP(hipMemcpy(m->layers4_dev, m->layers4.data(), sizeof(LayerW4) * L, hipMemcpyHostToDevice));
     FX_TRY_HIP(hipDeviceSynchronize());
     FX_TRY_HIP(hipGetLastError());
+    {
+        unsigned n_bad = 0;
+        FX_TRY_HIP(hipMemcpy(&n_bad, bad, sizeof(unsigned), hipMemcpyDeviceToHost));
+        FX_TRY_HIP(hipMemset(bad, 0, sizeof(unsigned)));
+        if (n_bad) {
+            set_error("llama_create_w4a4: %u weight values lie outside -8..7 (not a 4-bit export)", n_bad);
+            return fail(FLEXLLM_EINVAL);
+        }
+    }
 #undef FX_TRY
 #undef FX_TRY_HIP
     m->w4 = true;

@@ -1,10 +1,7 @@
 // C ABI entry points; the kernels live in logits_kernels.h.
 #include "logits_kernels.h"
-#include <mutex>
 
 using namespace fx;
-
-static std::mutex g_logits_mu;      // guards the first-use allocation of the stand-alone entry points' scratch
 
 extern "C" {
 
@@ -24,14 +21,12 @@ int flexllm_lm_head_f16(const uint16_t* embed, const float* n, float* logits, in
 
 int flexllm_argmax_f32(const float* x, int n, int* result, void* stream) {
     FX_REQUIRE(x && result && n > 0, "argmax: bad arguments");
-    {   // the first call allocates; concurrent first calls from several threads must not both do it
-        std::lock_guard<std::mutex> lk(g_logits_mu);
-        if (!g_pv) {
-            FX_HIP(hipMalloc(&g_pv, kArgmaxParts * sizeof(float)));
-            FX_HIP(hipMalloc(&g_pi, kArgmaxParts * sizeof(int)));
-        }
-    }
-    return argmax_launch(x, n, result, g_pv, g_pi, as_stream(stream));
+    // per-workgroup candidates in the calling stream's scratch: [kArgmaxParts] values, then [kArgmaxParts] indices
+    void* base = nullptr;
+    int rc = stream_scratch(kScratchArgmax, as_stream(stream), kArgmaxParts * (sizeof(float) + sizeof(int)), &base);
+    if (rc) return rc;
+    float* pv = static_cast<float*>(base);
+    return argmax_launch(x, n, result, pv, reinterpret_cast<int*>(pv + kArgmaxParts), as_stream(stream));
 }
 
 int flexllm_sample_topk_f32(const float* logits, int n, int top_k, const float* rand, int enable_sub_max, int* token,
@@ -40,15 +35,13 @@ int flexllm_sample_topk_f32(const float* logits, int n, int top_k, const float* 
     FX_REQUIRE(n > 0 && top_k >= 1 && top_k <= kTopKMax && top_k <= n, "sample_topk: n=%d top_k=%d (1..%d)", n, top_k, kTopKMax);
     TopKOut out = {token, top_idx, top_val, top_prob, nullptr, nullptr, nullptr};
     if (n >= 4096) {
-        {
-            std::lock_guard<std::mutex> lk(g_logits_mu);
-            if (!g_tv) {
-                FX_HIP(hipMalloc(&g_tv, kTopKParts * kTopKMax * sizeof(float)));
-                FX_HIP(hipMalloc(&g_ti, kTopKParts * kTopKMax * sizeof(int)));
-            }
-        }
-        topk_partial_kernel<<<kTopKParts, kTopKPartThreads, 0, as_stream(stream)>>>(logits, n, top_k, g_tv, g_ti);
-        topk_sample_kernel<256><<<1, 256, 0, as_stream(stream)>>>(g_tv, g_ti, kTopKParts * top_k, top_k, rand, 0, enable_sub_max, out);
+        void* base = nullptr;                      // the calling stream's scratch: candidate values, then their indices
+        int rc = stream_scratch(kScratchTopK, as_stream(stream), (size_t)kTopKParts * kTopKMax * (sizeof(float) + sizeof(int)), &base);
+        if (rc) return rc;
+        float* tv = static_cast<float*>(base);
+        int* ti = reinterpret_cast<int*>(tv + kTopKParts * kTopKMax);
+        topk_partial_kernel<<<kTopKParts, kTopKPartThreads, 0, as_stream(stream)>>>(logits, n, top_k, tv, ti);
+        topk_sample_kernel<256><<<1, 256, 0, as_stream(stream)>>>(tv, ti, kTopKParts * top_k, top_k, rand, 0, enable_sub_max, out);
     } else {
         topk_sample_kernel<kTopKThreads><<<1, kTopKThreads, 0, as_stream(stream)>>>(logits, nullptr, n, top_k, rand, 0, enable_sub_max, out);
     }

@@ -312,12 +312,8 @@ static __global__ __launch_bounds__(THREADS) void topk_sample_kernel(const float
 }
 
 constexpr int kArgmaxParts = 256;
-// Process-wide candidate buffers of the stand-alone arg-max and sampling entry points (allocated on first use;
-// calls that overlap on different streams would share them, a model object owns buffers of its own).
-inline float* g_pv = nullptr;
-inline int* g_pi = nullptr;
-inline float* g_tv = nullptr;
-inline int* g_ti = nullptr;
+// (the stand-alone arg-max and sampling entry points keep their candidate buffers in the calling stream's scratch,
+// a model object owns buffers of its own)
 
 inline int argmax_launch(const float* x, int n, int* result, float* pv, int* pi, hipStream_t st) {
     argmax_partial_kernel<<<kArgmaxParts, 256, 0, st>>>(x, n, pv, pi);

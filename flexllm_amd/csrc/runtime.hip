@@ -1,8 +1,11 @@
 // Error plumbing, thin runtime helpers for FFI hosts, and the counter-based fill kernels.
 #include "common.h"
 #include <hip/hip_fp16.h>
+#include <map>
+#include <mutex>
 #include <stdarg.h>
 #include <string.h>
+#include <tuple>
 
 namespace fx {
 static thread_local char g_err[512] = "";
@@ -11,6 +14,50 @@ void set_error(const char* fmt, ...) {
     va_start(ap, fmt);
     vsnprintf(g_err, sizeof(g_err), fmt, ap);
     va_end(ap);
+}
+
+namespace {
+struct ScratchBuf { void* ptr = nullptr; size_t bytes = 0; };
+std::mutex g_scratch_mu;
+std::map<std::tuple<int, hipStream_t, int>, ScratchBuf> g_scratch_map;
+}  // namespace
+
+int stream_scratch(ScratchKind kind, hipStream_t st, size_t bytes, void** out) {
+    int dev = 0;
+    FX_HIP(hipGetDevice(&dev));
+    std::lock_guard<std::mutex> lk(g_scratch_mu);
+    ScratchBuf& b = g_scratch_map[std::make_tuple(dev, st, (int)kind)];
+    if (b.bytes < bytes) {
+        if (b.ptr) {
+            FX_HIP(hipStreamSynchronize(st));          // kernels queued earlier on this stream may still use the old buffer
+            (void)hipFree(b.ptr);
+            b = ScratchBuf();
+        }
+        const size_t want = (bytes + 255) & ~(size_t)255;
+        hipError_t e = hipMalloc(&b.ptr, want);
+        if (e != hipSuccess) {
+            b = ScratchBuf();
+            set_error("scratch hipMalloc(%zu) failed: %s", want, hipGetErrorString(e));
+            return e == hipErrorOutOfMemory ? FLEXLLM_ENOMEM : FLEXLLM_EHIP;
+        }
+        b.bytes = want;
+    }
+    *out = b.ptr;
+    return FLEXLLM_OK;
+}
+
+void stream_scratch_release(hipStream_t st) {
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess) return;
+    std::lock_guard<std::mutex> lk(g_scratch_mu);
+    for (auto it = g_scratch_map.begin(); it != g_scratch_map.end();) {
+        if (std::get<0>(it->first) == dev && std::get<1>(it->first) == st) {
+            if (it->second.ptr) (void)hipFree(it->second.ptr);
+            it = g_scratch_map.erase(it);
+        } else {
+            ++it;
+        }
+    }
 }
 
 // SplitMix64 of (seed, index): the same sequence as flexllm_amd.synth.splitmix64 on the host.
@@ -65,6 +112,11 @@ int flexllm_rt_malloc(void** dptr, size_t bytes) {
     FX_HIP(e);
     return FLEXLLM_OK;
 }
+int flexllm_rt_mem_info(size_t* free_bytes, size_t* total_bytes) {
+    FX_REQUIRE(free_bytes && total_bytes, "mem_info: null pointer");
+    FX_HIP(hipMemGetInfo(free_bytes, total_bytes));
+    return FLEXLLM_OK;
+}
 int flexllm_rt_free(void* dptr) { FX_HIP(hipFree(dptr)); return FLEXLLM_OK; }
 int flexllm_rt_memcpy_h2d(void* dst, const void* src, size_t bytes, void* stream) {
     FX_HIP(hipMemcpyAsync(dst, src, bytes, hipMemcpyHostToDevice, as_stream(stream)));
@@ -91,7 +143,12 @@ int flexllm_rt_stream_create(void** stream) {
     *stream = s;
     return FLEXLLM_OK;
 }
-int flexllm_rt_stream_destroy(void* stream) { FX_HIP(hipStreamDestroy(as_stream(stream))); return FLEXLLM_OK; }
+int flexllm_rt_stream_destroy(void* stream) {
+    FX_HIP(hipStreamSynchronize(as_stream(stream)));
+    stream_scratch_release(as_stream(stream));         // the stand-alone entry points' scratch of this stream
+    FX_HIP(hipStreamDestroy(as_stream(stream)));
+    return FLEXLLM_OK;
+}
 int flexllm_rt_stream_sync(void* stream) { FX_HIP(hipStreamSynchronize(as_stream(stream))); return FLEXLLM_OK; }
 int flexllm_rt_device_sync(void) { FX_HIP(hipDeviceSynchronize()); return FLEXLLM_OK; }
 int flexllm_rt_event_create(void** event) {

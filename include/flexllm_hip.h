@@ -14,11 +14,14 @@
  *    their inputs.  fp32 results follow the reference's operation order except for
  *    reductions over a row (sum of squares, sum of exponentials), whose association
  *    differs; those agree to <=1e-3 relative.
- *  - Three stand-alone entry points keep small scratch buffers that the library allocates on first use and shares
- *    process-wide: flexllm_argmax_f32, flexllm_sample_topk_f32 (rows of 4096 logits and more) and
- *    flexllm_mha_i8_decode.  Calls to one of them that may run at the same time on different streams must be
- *    serialised by the caller.  A flexllm_llama object owns all of its buffers; use one object from one stream at a
- *    time.
+ *  - Four stand-alone entry points need scratch memory beyond their arguments: flexllm_argmax_f32,
+ *    flexllm_sample_topk_f32 (rows of 4096 logits and more), flexllm_mha_i8_decode and flexllm_mha_i8_decode_dyn.
+ *    The library keeps one buffer per (device, stream, entry point), allocated on the first call on that stream
+ *    and grown on demand (growing waits for the stream's earlier work).  Calls on different streams therefore never
+ *    share scratch and may run at the same time, from one host thread or several; calls on one stream run in
+ *    stream order.  flexllm_rt_stream_destroy releases a stream's buffers; buffers of streams created elsewhere
+ *    live until the process ends.  A flexllm_llama object owns all of its buffers; use one object from one
+ *    stream at a time.
  *
  * Reference citations are relative to the reference tree root.
  */
@@ -44,6 +47,8 @@ int flexllm_rt_device_count(int* count);
 int flexllm_rt_device_name(char* buf, int buflen);
 int flexllm_rt_malloc(void** dptr, size_t bytes);
 int flexllm_rt_free(void* dptr);
+/* Free and total device memory of the current device in bytes (hipMemGetInfo). */
+int flexllm_rt_mem_info(size_t* free_bytes, size_t* total_bytes);
 int flexllm_rt_memcpy_h2d(void* dst, const void* src, size_t bytes, void* stream);
 int flexllm_rt_memcpy_d2h(void* dst, const void* src, size_t bytes, void* stream);
 int flexllm_rt_memcpy_d2d(void* dst, const void* src, size_t bytes, void* stream);
@@ -63,6 +68,20 @@ int flexllm_rt_event_elapsed_ms(void* start, void* stop, float* ms);
 int flexllm_rt_fill_i8(int8_t* dst, size_t n, uint64_t seed, int lo, int hi, void* stream);
 int flexllm_rt_fill_uniform_f32(float* dst, size_t n, uint64_t seed, float lo, float hi, void* stream);
 int flexllm_rt_fill_uniform_f16(uint16_t* dst, size_t n, uint64_t seed, float lo, float hi, void* stream);
+
+/* ---- measurement probes (no counterpart in the reference: they exist so that a benchmark can print the rate this GPU
+ *      sustains next to the published peak a roofline is priced against) ------------------------------------------- */
+/* Matrix cores alone: `workgroups` x 4 waves, each issuing iters x 16 v_mfma_i32_32x32x32_i8 on a 4x4 grid of
+ * accumulator tiles = workgroups * 4 * iters * 16 * 65536 int8 operations per launch.  random_operands: pseudo-random
+ * operand bytes (else zeros, which draw less power and run at a higher clock); from_lds: the eight operand fragments
+ * are re-read from LDS at every step, as in a GEMM's main loop (else they stay in registers).  sink: device
+ * [workgroups * 256] int32 (written, keeps the work alive); clocks: optional device [2] uint64 = {shader-clock cycles,
+ * 100 MHz wall-clock ticks} of one wave's loop, i.e. the shader clock under this load. */
+int flexllm_probe_mfma_i8(int iters, int random_operands, int from_lds, int workgroups, int* sink, unsigned long long* clocks,
+                          void* stream);
+/* Read-only stream over `bytes` (a multiple of 16) of device memory with non-temporal 16-byte loads; sink: device
+ * [workgroups * 4] uint32. */
+int flexllm_probe_hbm_read(const void* src, size_t bytes, int workgroups, unsigned* sink, void* stream);
 
 /* ---- quant.h ------------------------------------------------------------------------ */
 /* Per-token symmetric int8 quantisation: s=absmax/127 (0 -> 1), q=round_half_away(x/s).

@@ -332,17 +332,11 @@ void fxo_causal_mask(const float* x, int rows, int heads, int dim, float* y) {
 
 /* ------------------------------------------------- MHA_i8xi8.h whole attention */
 
-void fxo_mha_prefill(const float* q, const float* k, const float* v, int s, int q_heads, int kv_heads,
-                     int hd, const fxo_mha_scales* sc, int8_t* q8_out, int8_t* k8_out, int8_t* v8_out,
-                     uint8_t* p8_out, float* o) {
+/* The attention proper on already quantised tensors.  p8_in != NULL replaces the probabilities this function would
+ * compute (a test feeds the device's own probability bytes back to isolate the P.V stage behind a rounding tie). */
+void fxo_mha_prefill_i8(const int8_t* q8, const int8_t* k8, const int8_t* v8, int s, int q_heads, int kv_heads,
+                        int hd, const fxo_mha_scales* sc, const uint8_t* p8_in, uint8_t* p8_out, float* o) {
     const int group = q_heads / kv_heads;
-    int8_t* q8 = (int8_t*)malloc((size_t)s * q_heads * hd);
-    int8_t* k8 = (int8_t*)malloc((size_t)s * kv_heads * hd);
-    int8_t* v8 = (int8_t*)malloc((size_t)s * kv_heads * hd);
-    /* MHA_i8xi8.h:40-42 (q, with sqrt(head_dim) folded in), :71-73 (k), :285-287 (v) */
-    fxo_static_quant(q, s, q_heads, hd, sc->q_s, sqrtf((float)hd), 1, 8, q8);
-    fxo_static_quant(k, s, kv_heads, hd, sc->k_s, 1.0f, 1, 8, k8);
-    fxo_static_quant(v, s, kv_heads, hd, sc->v_s, 1.0f, 1, 8, v8);
 #pragma omp parallel
     {
     float* row = (float*)malloc(sizeof(float) * s);
@@ -353,18 +347,22 @@ void fxo_mha_prefill(const float* q, const float* k, const float* v, int s, int 
         for (int i = 0; i < s; i++) {
             const int kh = h / group;                                     /* MHA.h:96-106 */
             const int8_t* qi = q8 + ((size_t)i * q_heads + h) * hd;
-            for (int j = 0; j < s; j++) {
-                const int8_t* kj = k8 + ((size_t)j * kv_heads + kh) * hd;
-                int32_t acc = 0;                                          /* MHA.h:189-243 */
-                for (int d = 0; d < hd; d++) acc += (int32_t)qi[d] * (int32_t)kj[d];
-                float a = (float)acc * sc->q_s[h] * sc->k_s[kh];          /* MHA_i8xi8.h:154 -> quant.h:315 */
-                row[j] = (j <= i) ? a : (float)-1e32;                     /* MHA.h:262-267 */
-            }
-            softmax_row(row, s, prob);                                    /* MHA_i8xi8.h:231 */
-            for (int j = 0; j < s; j++) {                                 /* MHA_i8xi8.h:254: unsigned, base 256 */
-                float t = prob[j] / (1.0f * sc->a_s[h]);
-                int rt = (int)roundf(t);
-                p8[j] = (uint8_t)(rt > 255 ? 255 : rt);
+            if (p8_in) {
+                memcpy(p8, p8_in + ((size_t)h * s + i) * s, (size_t)s);
+            } else {
+                for (int j = 0; j < s; j++) {
+                    const int8_t* kj = k8 + ((size_t)j * kv_heads + kh) * hd;
+                    int32_t acc = 0;                                      /* MHA.h:189-243 */
+                    for (int d = 0; d < hd; d++) acc += (int32_t)qi[d] * (int32_t)kj[d];
+                    float a = (float)acc * sc->q_s[h] * sc->k_s[kh];      /* MHA_i8xi8.h:154 -> quant.h:315 */
+                    row[j] = (j <= i) ? a : (float)-1e32;                 /* MHA.h:262-267 */
+                }
+                softmax_row(row, s, prob);                                /* MHA_i8xi8.h:231 */
+                for (int j = 0; j < s; j++) {                             /* MHA_i8xi8.h:254: unsigned, base 256 */
+                    float t = prob[j] / (1.0f * sc->a_s[h]);
+                    int rt = (int)roundf(t);
+                    p8[j] = (uint8_t)(rt > 255 ? 255 : rt);
+                }
             }
             if (p8_out) memcpy(p8_out + ((size_t)h * s + i) * s, p8, (size_t)s);
             if (o)
@@ -378,6 +376,19 @@ void fxo_mha_prefill(const float* q, const float* k, const float* v, int s, int 
     }
     free(row); free(prob); free(p8);
     }
+}
+
+void fxo_mha_prefill(const float* q, const float* k, const float* v, int s, int q_heads, int kv_heads,
+                     int hd, const fxo_mha_scales* sc, int8_t* q8_out, int8_t* k8_out, int8_t* v8_out,
+                     uint8_t* p8_out, float* o) {
+    int8_t* q8 = (int8_t*)malloc((size_t)s * q_heads * hd);
+    int8_t* k8 = (int8_t*)malloc((size_t)s * kv_heads * hd);
+    int8_t* v8 = (int8_t*)malloc((size_t)s * kv_heads * hd);
+    /* MHA_i8xi8.h:40-42 (q, with sqrt(head_dim) folded in), :71-73 (k), :285-287 (v) */
+    fxo_static_quant(q, s, q_heads, hd, sc->q_s, sqrtf((float)hd), 1, 8, q8);
+    fxo_static_quant(k, s, kv_heads, hd, sc->k_s, 1.0f, 1, 8, k8);
+    fxo_static_quant(v, s, kv_heads, hd, sc->v_s, 1.0f, 1, 8, v8);
+    fxo_mha_prefill_i8(q8, k8, v8, s, q_heads, kv_heads, hd, sc, NULL, p8_out, o);
     if (q8_out) memcpy(q8_out, q8, (size_t)s * q_heads * hd);
     if (k8_out) memcpy(k8_out, k8, (size_t)s * kv_heads * hd);
     if (v8_out) memcpy(v8_out, v8, (size_t)s * kv_heads * hd);

@@ -108,6 +108,11 @@ typedef struct {
 void fxo_mha_prefill(const float* q, const float* k, const float* v, int s, int q_heads, int kv_heads,
                      int head_dim, const fxo_mha_scales* sc, int8_t* q8, int8_t* k8, int8_t* v8,
                      uint8_t* p8, float* o);
+/* The same attention from the int8 tensors (q8 [s][q_heads][64], k8, v8 [s][kv_heads][64]); with p8_in the given
+ * probability bytes [q_heads][s][s] take the place of the computed ones in P.V (fxo_mha_prefill is the static
+ * quantisation followed by this function, so the checks that pin one pin the other). */
+void fxo_mha_prefill_i8(const int8_t* q8, const int8_t* k8, const int8_t* v8, int s, int q_heads, int kv_heads,
+                        int head_dim, const fxo_mha_scales* sc, const uint8_t* p8_in, uint8_t* p8_out, float* o);
 /* Decode attention of MHA_i8xi8.h:1027-1114 for one layer, one query against len cached keys
  * (the new token's k/v already appended). q8 [q_heads][64], caches [len][kv_heads][64]. */
 void fxo_mha_decode(const int8_t* q8, const int8_t* k_cache, const int8_t* v_cache, int len,

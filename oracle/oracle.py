@@ -324,6 +324,21 @@ def mha_prefill(q, k, v, q_s, k_s, v_s, a_s, want_p=False):
     return dict(q8=q8, k8=k8, v8=v8, p8=p8, o=o)
 
 
+def mha_prefill_i8(q8, k8, v8, q_s, k_s, v_s, a_s, p8_in=None, want_p=False):
+    """Attention from int8 tensors q8 [s][qh][64], k8/v8 [s][kvh][64]; p8_in [qh][s][s] replaces the computed
+    probabilities in P.V."""
+    q8 = np.ascontiguousarray(q8, np.int8); k8 = np.ascontiguousarray(k8, np.int8); v8 = np.ascontiguousarray(v8, np.int8)
+    s, qh, hd = q8.shape
+    kvh = k8.shape[1]
+    sc, keep = _scales(q_s, k_s, v_s, a_s)
+    p_in = np.ascontiguousarray(p8_in, np.uint8) if p8_in is not None else None
+    assert p_in is None or p_in.shape == (qh, s, s)
+    p8 = np.empty((qh, s, s), np.uint8) if want_p else None
+    o = np.empty((s, qh, hd), np.float32)
+    lib().fxo_mha_prefill_i8(_p(q8), _p(k8), _p(v8), s, qh, kvh, hd, C.byref(sc), _p(p_in), _p(p8), _p(o))
+    return (o, p8) if want_p else o
+
+
 def mha_decode(q8, k_cache, v_cache, q_s, k_s, v_s, a_s, want_p=False):
     """q8 [qh][hd] int8, caches [len][kvh][hd] int8 -> (o [qh][hd] fp32, p8 [qh][len])."""
     q8 = np.ascontiguousarray(q8, np.int8)

@@ -393,3 +393,37 @@ def test_sample_topk(fx, oracle, n, k):
     y = np.full(n, -3.0, np.float32); y[[n - 1, 5, n // 2]] = 9.0
     tok, idx, val, prob = fx.ops.sample_topk_f32(fx.to_device(y), min(k, 3) if k >= 3 else 1, 0.0)
     assert list(idx) == sorted([n - 1, 5, n // 2])[:len(idx)] and np.all(val == 9.0) and tok == 5
+
+
+def test_stand_alone_scratch_is_per_stream(fx, oracle):
+    """flexllm_mha_i8_decode, flexllm_argmax_f32 and flexllm_sample_topk_f32 keep their scratch per (device, stream):
+    calls issued back to back on two streams with no synchronisation between them (so that they may overlap on the
+    device) give what each gives alone, also after a stream's scratch had to grow."""
+    rng = np.random.default_rng(314)
+    qh, kvh, max_pos = 32, 8, 4096
+    sc = fx.ops.Scales(rng.uniform(0.003, 0.005, qh).astype(np.float32), rng.uniform(0.02, 0.04, kvh).astype(np.float32),
+                       rng.uniform(0.02, 0.04, kvh).astype(np.float32), np.full(qh, 1.0 / 255, np.float32))
+    cases = []
+    for length in (4096, 3000):
+        q8 = fx.to_device(rng.integers(-128, 128, (qh, 64)).astype(np.int8))
+        kc, vc = fx.ops.kv_cache(kvh, max_pos)
+        fx.ops.kv_store_i8(fx.to_device(rng.integers(-60, 60, (length, kvh, 64)).astype(np.int8)),
+                           fx.to_device(rng.integers(-128, 128, (length, kvh, 64)).astype(np.int8)), kc, vc, 0)
+        o_ref, _ = fx.ops.mha_i8_decode(q8, kc, vc, sc, length)
+        logits = fx.to_device(rng.standard_normal(128256).astype(np.float32))
+        cases.append((q8, kc, vc, length, o_ref.numpy(), logits, int(np.argmax(logits.numpy()))))
+    streams = [fx.Stream(), fx.Stream()]
+    fx.ops.mha_i8_decode(cases[0][0], cases[0][1], cases[0][2], sc, 64, stream=streams[0])    # a small scratch first: the long call must grow it
+    for rep in range(20):
+        outs = []
+        for (q8, kc, vc, length, o_ref, logits, am), st in zip(cases, streams):
+            o, _ = fx.ops.mha_i8_decode(q8, kc, vc, sc, length, stream=st)
+            outs.append((o, fx.ops.argmax_f32(logits, stream=st)))
+        for st in streams:
+            st.sync()
+        for (q8, kc, vc, length, o_ref, logits, am), (o, r) in zip(cases, outs):
+            assert np.array_equal(o.numpy(), o_ref), "repetition %d" % rep
+            assert int(r.numpy()[0]) == am
+    tok_a = fx.ops.sample_topk_f32(cases[0][5], 5, 0.3, stream=streams[0])[0]
+    tok_b = fx.ops.sample_topk_f32(cases[1][5], 5, 0.3, stream=streams[1])[0]
+    assert tok_a == oracle.sample_topk(cases[0][5].numpy(), 5, 0.3, 8)[0] and tok_b == oracle.sample_topk(cases[1][5].numpy(), 5, 0.3, 8)[0]

@@ -51,10 +51,11 @@ def test_gemm_all_tile_shapes_and_extremes(fx):
     assert np.all(fx.ops.linear_i8_gemm(fx.to_device(a), fx.to_device(w)).numpy() == 8192 * 128 * 128)
 
 
-@pytest.mark.parametrize("m,k,n", [(4096, 2048, 2048), (2048, 128, 4096), (2000, 384, 4100), (3072, 256, 2048)])
+@pytest.mark.parametrize("m,k,n", [(4096, 2048, 2048), (2048, 128, 4096), (2000, 384, 4100), (3072, 256, 2048), (1024, 2048, 2048)])
 def test_gemm_long_prefill_shapes(fx, oracle, m, k, n):
     """Shapes with 384..767 tiles of 128x128 (the o projection of a 4096-token prefill, shallow ones, a ragged one):
-    the 128x128 variant with two stages of 128-byte rows.  Raw int32 and dequantised + residual, float64 BLAS as the
+    the 128x128 variant with two stages of 128-byte rows; and the o projection of a 1024-token prefill (1024 x 2048 ->
+    2048, the narrow-tile instance the layer graph runs at that length).  Raw int32 and dequantised + residual, float64 BLAS as the
     exact reference (|sum| < 2^31)."""
     a = rng.integers(-128, 128, (m, k)).astype(np.int8)
     w = rng.integers(-128, 128, (n, k)).astype(np.int8)

@@ -287,3 +287,22 @@ def test_w4a4_sampling_inside_the_kernel(small4):
         ranks.append(int(np.nonzero(idx == t_ref)[0][0]))
     assert len(set(ranks)) >= 2, ranks
     assert int(tok.numpy()[0]) == got[-1]
+
+
+@pytest.mark.parametrize("where", ["wd", "head_w"])
+def test_w4a4_create_refuses_values_outside_the_4_bit_range(small4, where):
+    """The prefill graph multiplies the byte-held matrices as they are, the persistent decode kernel their low nibbles:
+    an export holding a value outside -8..7 would make the two disagree silently, so the model is refused at creation."""
+    fx, cfg, model, oracle, host_w = small4
+    from flexllm_amd import llama
+    w = dict(host_w)
+    if where == "wd":
+        bad = host_w["wd"][1].copy(); bad[17, 4000] = 9
+        w["wd"] = [host_w["wd"][0], bad]
+    else:
+        bad = host_w["head_w"].copy(); bad[-1, -1] = -9
+        w["head_w"] = bad
+    with pytest.raises(Exception, match="outside -8..7"):
+        llama.Llama(cfg, to_dev(fx, w))
+    m = llama.Llama(cfg, to_dev(fx, host_w))           # the unmodified export is still accepted afterwards
+    m.close()
