@@ -54,6 +54,18 @@ def lib():
         _lib = C.CDLL(LIB_PATH)
         _lib.flexllm_last_error.restype = C.c_char_p
         _lib.flexllm_build_info.restype = C.c_char_p
+        # Every entry point with a size_t parameter is typed: an untyped Python int is passed as a 32-bit C int, which
+        # would silently cut a size of 4 GiB to zero.
+        vp, sz, i, u64, f = C.c_void_p, C.c_size_t, C.c_int, C.c_uint64, C.c_float
+        for name, args in (("flexllm_rt_malloc", [vp, sz]), ("flexllm_rt_mem_info", [vp, vp]),
+                           ("flexllm_rt_memcpy_h2d", [vp, vp, sz, vp]), ("flexllm_rt_memcpy_d2h", [vp, vp, sz, vp]),
+                           ("flexllm_rt_memcpy_d2d", [vp, vp, sz, vp]), ("flexllm_rt_memset", [vp, i, sz, vp]),
+                           ("flexllm_rt_fill_i8", [vp, sz, u64, i, i, vp]), ("flexllm_rt_fill_uniform_f32", [vp, sz, u64, f, f, vp]),
+                           ("flexllm_rt_fill_uniform_f16", [vp, sz, u64, f, f, vp]),
+                           ("flexllm_probe_hbm_read", [vp, sz, i, vp, vp]), ("flexllm_pack_nibbles", [vp, vp, sz, vp]),
+                           ("flexllm_swish_f32", [vp, vp, sz, vp]), ("flexllm_swiglu_f32", [vp, vp, vp, sz, vp]),
+                           ("flexllm_residual_add_f32", [vp, vp, vp, sz, vp])):
+            getattr(_lib, name).argtypes = args
     return _lib
 
 

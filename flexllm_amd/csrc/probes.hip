@@ -64,10 +64,12 @@ __global__ __launch_bounds__(256) void probe_hbm_read_kernel(const i32x4* __rest
     const size_t stride = (size_t)gridDim.x * 256;
     size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
     unsigned acc = 0;
-    for (; i + 3 * stride < n16; i += 4 * stride) {          // four independent loads in flight per thread
-        const i32x4 a = __builtin_nontemporal_load(src + i), b = __builtin_nontemporal_load(src + i + stride);
-        const i32x4 c = __builtin_nontemporal_load(src + i + 2 * stride), d = __builtin_nontemporal_load(src + i + 3 * stride);
-        acc ^= (unsigned)((a[0] ^ a[1] ^ a[2] ^ a[3]) ^ (b[0] ^ b[1] ^ b[2] ^ b[3]) ^ (c[0] ^ c[1] ^ c[2] ^ c[3]) ^ (d[0] ^ d[1] ^ d[2] ^ d[3]));
+    for (; i + 7 * stride < n16; i += 8 * stride) {          // eight independent loads in flight per thread
+        i32x4 v[8];
+#pragma unroll
+        for (int u = 0; u < 8; u++) v[u] = __builtin_nontemporal_load(src + i + u * stride);
+#pragma unroll
+        for (int u = 0; u < 8; u++) acc ^= (unsigned)(v[u][0] ^ v[u][1] ^ v[u][2] ^ v[u][3]);
     }
     for (; i < n16; i += stride) {
         const i32x4 a = __builtin_nontemporal_load(src + i);

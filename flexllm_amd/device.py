@@ -68,7 +68,7 @@ class DeviceArray:
         self.dtype = np.dtype(dtype)
         self.nbytes = int(np.prod(self.shape, dtype=np.int64)) * self.dtype.itemsize
         p = C.c_void_p()
-        check(lib().flexllm_rt_malloc(C.byref(p), max(self.nbytes, 1)))
+        check(lib().flexllm_rt_malloc(C.byref(p), C.c_size_t(max(self.nbytes, 1))))     # size_t: an untyped int would be cut to 32 bits
         self.ptr = p.value
         self._owner = True
 
@@ -79,18 +79,18 @@ class DeviceArray:
     def copy_from(self, host):
         host = np.ascontiguousarray(host, dtype=self.dtype)
         assert host.nbytes == self.nbytes, (host.shape, self.shape)
-        check(lib().flexllm_rt_memcpy_h2d(C.c_void_p(self.ptr), host.ctypes.data_as(C.c_void_p), self.nbytes, None))
+        check(lib().flexllm_rt_memcpy_h2d(C.c_void_p(self.ptr), host.ctypes.data_as(C.c_void_p), C.c_size_t(self.nbytes), None))
         return self
 
     def numpy(self):
         device_sync()
         out = np.empty(self.shape, self.dtype)
         if self.nbytes:
-            check(lib().flexllm_rt_memcpy_d2h(out.ctypes.data_as(C.c_void_p), C.c_void_p(self.ptr), self.nbytes, None))
+            check(lib().flexllm_rt_memcpy_d2h(out.ctypes.data_as(C.c_void_p), C.c_void_p(self.ptr), C.c_size_t(self.nbytes), None))
         return out
 
     def zero_(self, stream=None):
-        check(lib().flexllm_rt_memset(C.c_void_p(self.ptr), 0, self.nbytes, _s(stream)))
+        check(lib().flexllm_rt_memset(C.c_void_p(self.ptr), 0, C.c_size_t(self.nbytes), _s(stream)))
         return self
 
     def view(self, offset_bytes, shape, dtype=None):

@@ -291,6 +291,21 @@ void dec_Linear_Layer_i4xi4(IS& input_seq, const DeviceWeight4& weight, OS& outp
     check(flexllm_linear_u4i4_gemv(dx.get(), weight.w4.get(), dc.get(), input_dim, output_dim, nullptr));
     fill_dec(output_seq, dc.download(), output_dim, block_parallel);
 }
+// Modules/Linear_Layer.h:293-301 (is_uint_input = true), the weight stream replaced by a resident DeviceWeight4: seq_len
+// tokens of unsigned 4-bit activations in the prefill packing -> int32 accumulators in the same packing
+template <int io_parallel, int weight_parallel, int max_input_dim = 2048, int max_log2_input_dim = 11, int max_output_dim = 2048,
+          int max_seq_len = 1024, bool is_uint_input = false, class IS, class OS>
+void pref_Linear_Layer_i4xi4(IS& input_seq, const DeviceWeight4& weight, OS& output_seq, int seq_len = max_seq_len,
+                             int input_dim = max_input_dim, int output_dim = max_output_dim) {
+    static_assert(is_uint_input, "the W4A4 path has unsigned (asymmetric) activations");
+    auto a = drain_pref<uint8_t>(input_seq, seq_len, input_dim, io_parallel);
+    std::vector<uint8_t> a4(a.size() / 2);
+    for (size_t i = 0; i < a4.size(); i++) a4[i] = (uint8_t)((a[2 * i] & 0xF) | ((a[2 * i + 1] & 0xF) << 4));
+    DeviceArray<uint8_t> da(a4);
+    DeviceArray<int32_t> dc((size_t)seq_len * output_dim);
+    check(flexllm_linear_u4i4_gemm(da.get(), weight.w4.get(), dc.get(), seq_len, input_dim, output_dim, nullptr));
+    fill_pref(output_seq, dc.download(), seq_len, output_dim, io_parallel);
+}
 // Modules/Linear_Layer.h:612-617 / :1103-1108
 template <int io_parallel, int io_hidden_dim, int max_seq_len = 1024, class IA, class IB, class OS>
 void pref_Gate_Layer_fp32xfp32(IA& input_seq, IB& gate_seq, OS& output_seq, int seq_len = max_seq_len) {
@@ -759,6 +774,100 @@ void MHA_i8xi8_decoding_layer(const std::vector<VF>& q_mmap, const std::vector<V
         const int per = H / BP;
         for (int j = 0; j < H; j++) o_mmap[(size_t)t * per + j % per][j / per] = o[j];
     }
+}
+
+// ======================================================================================= Linear_Layer_test.h tops
+// QuantWrapper_Linear_Layer_q_Decoding_tb (SpinQuant_Llama_32_1B/Linear_Layer_test.h:332-364) for ONE layer, with the
+// testbench's own buffers: input_mmap / output_mmap in the decode packing [t*dim/BP + j % (dim/BP)][j / (dim/BP)],
+// quant_weight_mmaps = the BP lane buffers of packed int4 weight words exactly as Linear_Layer_Decoding_tb.cpp:176-186
+// fills them, weight_s_sum_mmap[n] = {scale, row sum of the dequantised weights}.  Per token: asymmetric uint4
+// quantisation, int4 GEMV, dequantisation with zero point x row sum.
+template <int BP, int WP, int input_dim, int output_dim, class VF, class VW, class VS>
+void QuantWrapper_Linear_Layer_q_Decoding_layer(const std::vector<VF>& input_mmap, std::vector<VW>* quant_weight_mmaps,
+                                                const std::vector<VS>& weight_s_sum_mmap, std::vector<VF>& output_mmap,
+                                                int dec_seq_len) {
+    std::vector<int8_t> row_major((size_t)output_dim * input_dim);
+    unpack_weight_int4_decode<WP, BP>(quant_weight_mmaps, output_dim, input_dim, row_major.data());
+    DeviceWeight4 weight(row_major.data(), output_dim, input_dim);
+    std::vector<float> ws(output_dim), wsum(output_dim);
+    for (int n = 0; n < output_dim; n++) { ws[n] = weight_s_sum_mmap[n][0]; wsum[n] = weight_s_sum_mmap[n][1]; }
+    DeviceArray<float> dws(ws), dwsum(wsum), dx(input_dim), ds(1), db(1), dy(output_dim);
+    DeviceArray<uint8_t> dq(input_dim), dq4(input_dim / 2);
+    const int per_in = input_dim / BP, per_out = output_dim / BP;
+    std::vector<float> x(input_dim);
+    for (int t = 0; t < dec_seq_len; t++) {
+        for (int j = 0; j < input_dim; j++) x[j] = input_mmap[(size_t)t * per_in + j % per_in][j / per_in];
+        dx.upload(x);
+        check(flexllm_quant_asym_u8(dx.get(), dq.get(), ds.get(), db.get(), 4, 1, input_dim, nullptr));
+        check(flexllm_pack_nibbles(dq.get(), dq4.get(), (size_t)input_dim, nullptr));
+        check(flexllm_linear_u4i4_gemv_dequant(dq4.get(), ds.get(), db.get(), weight.w4.get(), dws.get(), dwsum.get(), nullptr,
+                                               dy.get(), input_dim, output_dim, nullptr));
+        const auto y = dy.download();
+        for (int j = 0; j < output_dim; j++) output_mmap[(size_t)t * per_out + j % per_out][j / per_out] = y[j];
+    }
+}
+// QuantWrapper_Linear_Layer_q_Prefilling_tb (Linear_Layer_test.h:145-175) for ONE layer: input_mmap / output_mmap in the
+// prefill packing [(t/TP)*dim + j][t % TP], quant_weight_mmap the packed words of Linear_Layer_Prefilling_tb.cpp:
+// 226-231 (WP output channels per word group, the vector may be wider than WP/2 bytes: the read-parallel padding).
+template <int TP, int WP, int input_dim, int output_dim, class VF, class VW, class VS>
+void QuantWrapper_Linear_Layer_q_Prefilling_layer(const std::vector<VF>& input_mmap, const std::vector<VW>& quant_weight_mmap,
+                                                  const std::vector<VS>& weight_s_sum_mmap, std::vector<VF>& output_mmap, int seq_len) {
+    std::vector<int8_t> row_major((size_t)output_dim * input_dim);
+    unpack_weight_int4_prefill<WP>(quant_weight_mmap, output_dim, input_dim, row_major.data());
+    DeviceWeight4 weight(row_major.data(), output_dim, input_dim);
+    std::vector<float> ws(output_dim), wsum(output_dim), x((size_t)seq_len * input_dim);
+    for (int n = 0; n < output_dim; n++) { ws[n] = weight_s_sum_mmap[n][0]; wsum[n] = weight_s_sum_mmap[n][1]; }
+    for (int t = 0; t < seq_len; t++)
+        for (int j = 0; j < input_dim; j++) x[(size_t)t * input_dim + j] = input_mmap[(size_t)(t / TP) * input_dim + j][t % TP];
+    DeviceArray<float> dx(x), dws(ws), dwsum(wsum), ds(seq_len), db(seq_len), dy((size_t)seq_len * output_dim);
+    DeviceArray<uint8_t> dq(x.size()), dq4(x.size() / 2);
+    check(flexllm_quant_asym_u8(dx.get(), dq.get(), ds.get(), db.get(), 4, seq_len, input_dim, nullptr));
+    check(flexllm_pack_nibbles(dq.get(), dq4.get(), x.size(), nullptr));
+    check(flexllm_linear_u4i4_gemm_dequant(dq4.get(), ds.get(), db.get(), weight.w4.get(), dws.get(), dwsum.get(), nullptr, dy.get(),
+                                           seq_len, input_dim, output_dim, nullptr));
+    const auto y = dy.download();
+    for (int t = 0; t < seq_len; t++)
+        for (int j = 0; j < output_dim; j++) output_mmap[(size_t)(t / TP) * output_dim + j][t % TP] = y[(size_t)t * output_dim + j];
+}
+
+// ======================================================================================= Logits.h
+// The logits stream is block-partitioned like every decode stream: lane i of read m carries logit
+// i*(logits_num/block_parallel_samp) + m (Modules/Logits.h:98).
+// Modules/Logits.h:34-40: the top_k largest logits in descending order (strict '>' on insertion, so an equal value
+// queues behind the one found first), softmax over them, top_k packs {index, probability}.
+template <typename T, int block_parallel_samp, int max_logits_num, int top_k, int max_hidden_dim = 2048, int block_logits_num = 2048,
+          int inner_block_parallel = 1, bool enable_softmax = true, bool enable_sub_max = true, class IS, class OS>
+void dec_Logits_Max_K_Layer(IS& logits_stream, OS& max_logits_stream, int logits_num = max_logits_num) {
+    static_assert(std::is_same<T, float>::value && enable_softmax, "fp32 logits, probabilities on the output");
+    auto logits = drain_dec<float>(logits_stream, logits_num, block_parallel_samp);
+    DeviceArray<float> dl(logits), dr(std::vector<float>{0.0f}), dval(top_k), dprob(top_k);
+    DeviceArray<int> dtok(1), didx(top_k);
+    check(flexllm_sample_topk_f32(dl.get(), logits_num, top_k, dr.get(), enable_sub_max ? 1 : 0, dtok.get(), didx.get(), dval.get(),
+                                  dprob.get(), nullptr));
+    const auto idx = didx.download();
+    const auto prob = dprob.download();
+    for (int k = 0; k < top_k; k++) {
+        typename OS::value_type out_pack;
+        out_pack[0] = (T)idx[k];
+        out_pack[1] = prob[k];
+        max_logits_stream.write(out_pack);
+    }
+}
+// Modules/Logits.h:145-155: top-k selection and softmax as above, a draw with the host-supplied uniform number rand_seed
+// (the smallest k with rand_seed < cdf[k], else the last), and the sampled token's embedding row read from vocab_lib
+// (fp32 rows in the decode packing, row t at vocab_lib[t*dim/BPE ...], Modules/data_io.h:348-363) onto the stream.
+template <typename T, int block_parallel_samp, int max_logits_num, int top_k, int block_parallel_embed, int max_hidden_dim = 2048,
+          int block_logits_num = 2048, int inner_block_parallel = 1, bool enable_sub_max = true, class IS, class VE, class OS>
+void dec_Sampling_Embedding_Layer(IS& logits_stream, const std::vector<VE>& vocab_lib, OS& new_embedding_stream, T rand_seed,
+                                  int& sampled_idx, int logits_num = max_logits_num, int io_hidden_dim = max_hidden_dim) {
+    static_assert(std::is_same<T, float>::value, "fp32 logits");
+    auto logits = drain_dec<float>(logits_stream, logits_num, block_parallel_samp);
+    DeviceArray<float> dl(logits), dr(std::vector<float>{(float)rand_seed});
+    DeviceArray<int> dtok(1);
+    check(flexllm_sample_topk_f32(dl.get(), logits_num, top_k, dr.get(), enable_sub_max ? 1 : 0, dtok.get(), nullptr, nullptr, nullptr, nullptr));
+    sampled_idx = dtok.download()[0];
+    const size_t per = (size_t)io_hidden_dim / block_parallel_embed;
+    for (size_t i = 0; i < per; i++) new_embedding_stream.write(vocab_lib[(size_t)sampled_idx * per + i]);
 }
 
 }  // namespace fxhost

@@ -10,6 +10,9 @@
 //                                     launched through fxhost::invoke(top, "hip", mmaps..., scalars...) on the reference's
 //                                     own cache line layouts, and stage by stage through the dec_MHA_* module functions
 //   layout adapters               <-> the packed int4 weight words and the KV-cache line layouts of the testbenches
+//   QuantWrapper linear tops      <-> SpinQuant_Llama_32_1B/Linear_Layer_test.h:145-175, :332-364 launched through
+//                                     fxhost::invoke on the testbenches' packed int4 weight words
+//   Logits                        <-> Modules/Logits.h:34-279 (top-k layer, sampling + embedding feedback)
 //   FHT / RMSNorm / Swish / residual / softmax / RoPE against float64 closed forms
 #include <algorithm>
 #include <array>
@@ -688,6 +691,190 @@ static void adapters_test() {
     verdict("layout adapters (packed int4 weight words, prefill KV-cache lines; the decode lines are exercised by the MHA test)", ok);
 }
 
+
+// The linear testbench tops launched the way the testbenches launch them - fxhost::invoke(top, "hip", mmaps..., length) -
+// on the testbenches' own buffers: activations in the stream packings and the packed int4 weight words written with
+// the index formulas of Linear_Layer_Decoding_tb.cpp:176-186 and Linear_Layer_Prefilling_tb.cpp:226-231 (not through
+// this build's pack adapters).  Checked against the quantised golden of the testbench (q_out * s_x * s_w + b_x * sum_w,
+// :236-249) to fp32 rounding and against its fake-quant golden at its own 1e-2.
+template <bool DECODE>
+static void QuantWrapper_Linear_Layer_q_tops_test() {
+    constexpr int K = HIDDEN_DIM, N = HIDDEN_DIM, BP = T_BLOCK_PARALLEL, TP = TOKEN_PARALLEL;
+    constexpr int WP = DECODE ? DEC_W_PARALLEL : 24, WPR = DECODE ? DEC_W_PARALLEL : 32;   // prefill: PRE_QKVO_W_PARALLEL = 24, read width 32
+    const int T = DECODE ? 8 : 64;
+    std::default_random_engine gen(42);
+    std::uniform_real_distribution<float> dist(-1.0, 1.0);
+    using VF = vec<float, DECODE ? BP : TP>;
+    using VW = vec<int8_t, WPR / 2>;
+    using VS = vec<float, 2>;
+    std::vector<float> x((size_t)T * K), fq((size_t)T * K), in_s(T), in_b(T), w_fq((size_t)N * K);
+    std::vector<int> q_in((size_t)T * K), q_w((size_t)N * K);
+    std::vector<VF> input_mmap(DECODE ? (size_t)T * K / BP : (size_t)T / TP * K), output_mmap(DECODE ? (size_t)T * N / BP : (size_t)T / TP * N);
+    for (int i = 0; i < T; i++) {
+        float vmax = -1e30f, vmin = 1e30f;
+        for (int j = 0; j < K; j++) {
+            const float val = dist(gen);
+            x[(size_t)i * K + j] = val; vmax = std::max(vmax, val); vmin = std::min(vmin, val);
+            if (DECODE) input_mmap[(size_t)i * (K / BP) + j % (K / BP)][j / (K / BP)] = val;
+            else input_mmap[(size_t)(i / TP) * K + j][i % TP] = val;
+        }
+        float scale = (vmax - vmin) / 15.0f;
+        if (scale == 0) scale = 1.0f;
+        in_s[i] = scale; in_b[i] = vmin;
+        for (int j = 0; j < K; j++) {
+            const int q = (int)std::round((x[(size_t)i * K + j] - vmin) / scale);
+            q_in[(size_t)i * K + j] = q;
+            fq[(size_t)i * K + j] = q * scale + vmin;
+        }
+    }
+    std::vector<VS> weight_s_sum_mmap(N);
+    std::vector<VW> lanes[BP], flat;
+    if (DECODE) for (int I = 0; I < BP; I++) lanes[I].assign((size_t)(N / BP + WP - 1) / WP * K, VW());
+    else flat.assign((size_t)((N + WP - 1) / WP) * K, VW());
+    for (int n = 0; n < N; n++) {
+        float w_max = 0;
+        for (int j = 0; j < K; j++) { w_fq[(size_t)n * K + j] = dist(gen); w_max = std::max(w_max, std::abs(w_fq[(size_t)n * K + j])); }
+        float scale = w_max / 7.0f;
+        if (scale == 0) scale = 1.0f;
+        weight_s_sum_mmap[n][0] = scale; weight_s_sum_mmap[n][1] = 0;
+        for (int j = 0; j < K; j++) {
+            int qval = (int)std::round(w_fq[(size_t)n * K + j] / scale);
+            qval = std::max(-8, std::min(7, qval));
+            w_fq[(size_t)n * K + j] = qval * scale;
+            q_w[(size_t)n * K + j] = qval;
+            weight_s_sum_mmap[n][1] += w_fq[(size_t)n * K + j];
+            // the packed word this value lives in, by the testbench's formula
+            int8_t* slot;
+            int nib;
+            if (DECODE) { const int I = n / (N / BP), i = n % (N / BP); slot = &lanes[I][(size_t)(i / WP) * K + j][(i / 2) % (WP / 2)]; nib = i % 2; }
+            else { slot = &flat[(size_t)((n / 2) / (WP / 2)) * K + j][(n / 2) % (WP / 2)]; nib = n % 2; }
+            const unsigned old = (uint8_t)*slot, v = (unsigned)qval & 0xF;
+            *slot = (int8_t)(nib ? ((old & 0x0F) | (v << 4)) : ((old & 0xF0) | v));
+        }
+    }
+    std::cout << "kernel begins running!\n";
+    int64_t ns;
+    if constexpr (DECODE)
+        ns = invoke(QuantWrapper_Linear_Layer_q_Decoding_layer<BP, WP, K, N, VF, VW, VS>, "hip", read_only_mmap(input_mmap),
+                    read_only_mmaps(lanes), read_only_mmap(weight_s_sum_mmap), write_only_mmap(output_mmap), T);
+    else
+        ns = invoke(QuantWrapper_Linear_Layer_q_Prefilling_layer<TP, WP, K, N, VF, VW, VS>, "hip", read_only_mmap(input_mmap),
+                    read_only_mmap(flat), read_only_mmap(weight_s_sum_mmap), write_only_mmap(output_mmap), T);
+    std::cout << "kernel time: " << ns * 1e-9 << " s" << std::endl;
+    bool correct = true;
+    double worst_q = 0;
+    for (int i = 0; i < T && correct; i++)
+        for (int j = 0; j < N; j++) {
+            long long acc = 0;
+            double gold_fq = 0;
+            for (int k = 0; k < K; k++) {
+                acc += (long long)q_in[(size_t)i * K + k] * q_w[(size_t)j * K + k];
+                gold_fq += (double)fq[(size_t)i * K + k] * w_fq[(size_t)j * K + k];
+            }
+            const float gold_q = (float)acc * in_s[i] * weight_s_sum_mmap[j][0] + in_b[i] * weight_s_sum_mmap[j][1];
+            const float my = DECODE ? output_mmap[(size_t)i * (N / BP) + j % (N / BP)][j / (N / BP)] : output_mmap[(size_t)(i / TP) * N + j][i % TP];
+            worst_q = std::max(worst_q, (double)std::abs(my - gold_q));
+            if (std::abs(my - gold_q) > 1e-5 * std::abs(gold_q) + 1e-5 || std::abs(my - gold_fq) > 1e-2 * std::abs(gold_fq) + 1e-3) {
+                correct = false;
+                std::cout << "Mismatch at (" << i << ", " << j << "): My: " << my << ", Ref_q: " << gold_q << ", Ref_fq: " << gold_fq << std::endl;
+                break;
+            }
+        }
+    verdict(DECODE ? "QuantWrapper linear top (decode) through invoke on the testbench's packed int4 weight lanes"
+                   : "QuantWrapper linear top (prefill, weight parallel 24 in words of 32) through invoke on the testbench's packed int4 weight words", correct);
+}
+
+// pref_Linear_Layer_i4xi4 as a module: uint4 activations in the prefill packing x resident int4 weights -> exact int32
+static void pref_Linear_Layer_i4xi4_test() {
+    constexpr int S = 32, K = 256, N = 96, TP = TOKEN_PARALLEL;
+    std::default_random_engine gen(5);
+    std::uniform_int_distribution<int> da(0, 15), dw(-8, 7);
+    std::vector<int> a((size_t)S * K), w((size_t)N * K);
+    std::vector<int8_t> w8((size_t)N * K);
+    for (auto& v : a) v = da(gen);
+    for (size_t i = 0; i < w.size(); i++) { w[i] = dw(gen); w8[i] = (int8_t)w[i]; }
+    stream<vec<uint8_t, TP>> in;
+    stream<vec<int32_t, TP>> out;
+    for (int M = 0; M < S / TP; M++)
+        for (int k = 0; k < K; k++) { vec<uint8_t, TP> p; for (int m = 0; m < TP; m++) p[m] = (uint8_t)a[(size_t)(M * TP + m) * K + k]; in.write(p); }
+    DeviceWeight4 weight(w8.data(), N, K);
+    pref_Linear_Layer_i4xi4<TP, 24, K, 8, N, S, true>(in, weight, out, S, K, N);
+    bool ok = true;
+    for (int M = 0; M < S / TP; M++)
+        for (int n = 0; n < N; n++) {
+            const auto p = out.read();
+            for (int m = 0; m < TP; m++) {
+                int acc = 0;
+                for (int k = 0; k < K; k++) acc += a[(size_t)(M * TP + m) * K + k] * w[(size_t)n * K + k];
+                if (p[m] != acc) ok = false;
+            }
+        }
+    verdict("pref_Linear_Layer_i4xi4 (uint4 x int4, prefill stream packing, exact int32)", ok && out.empty());
+}
+
+// Modules/Logits.h: top-k layer and the sampling + embedding layer on block-partitioned logit streams
+static void Logits_test() {
+    constexpr int BPS = 8, V = 128256, TOPK = 5;
+    std::default_random_engine gen(11);
+    std::normal_distribution<float> nd(0.0f, 2.0f);
+    std::vector<float> logits(V);
+    for (auto& v : logits) v = nd(gen);
+    logits[777] = logits[90001];                                   // an exact tie somewhere in the body of the distribution
+    std::vector<int> order(V);
+    for (int i = 0; i < V; i++) order[i] = i;
+    std::partial_sort(order.begin(), order.begin() + TOPK, order.end(), [&](int a, int b) { return logits[a] > logits[b] || (logits[a] == logits[b] && a < b); });
+    double e[TOPK], sum = 0;
+    for (int k = 0; k < TOPK; k++) { e[k] = std::exp((double)logits[order[k]] - (double)logits[order[0]]); sum += e[k]; }
+    auto feed = [&](stream<vec<float, BPS>>& s, const std::vector<float>& l, int n) {
+        for (int m = 0; m < n / BPS; m++) { vec<float, BPS> p; for (int i = 0; i < BPS; i++) p[i] = l[(size_t)i * (n / BPS) + m]; s.write(p); }
+    };
+    bool ok = true;
+    {
+        stream<vec<float, BPS>> ls;
+        stream<vec<float, 2>> out;
+        feed(ls, logits, V);
+        dec_Logits_Max_K_Layer<float, BPS, V, TOPK>(ls, out, V);
+        for (int k = 0; k < TOPK; k++) {
+            const auto p = out.read();
+            if ((int)p[0] != order[k] || std::abs(p[1] - e[k] / sum) > 1e-5) { ok = false; std::cout << "top-k " << k << ": My: " << p[0] << " " << p[1] << ", Ref: " << order[k] << " " << e[k] / sum << std::endl; }
+        }
+        ok = ok && out.empty();
+    }
+    {   // sampling + embedding feedback on a small vocabulary (the table is a host buffer here), several uniform numbers
+        constexpr int V2 = 4096, HID = 256, BPE = 8;
+        std::vector<float> l2(logits.begin(), logits.begin() + V2);
+        std::vector<int> o2(V2);
+        for (int i = 0; i < V2; i++) o2[i] = i;
+        std::partial_sort(o2.begin(), o2.begin() + TOPK, o2.end(), [&](int a, int b) { return l2[a] > l2[b] || (l2[a] == l2[b] && a < b); });
+        float pr[TOPK], part[2] = {0, 0};
+        for (int k = 0; k < TOPK; k++) { pr[k] = std::exp(l2[o2[k]] - l2[o2[0]]); part[k % 2] += pr[k]; }   // Logits.h:231-246, float like the reference
+        const float tot = part[0] + part[1];
+        float cdf[TOPK];
+        for (int k = 0; k < TOPK; k++) { pr[k] /= tot; cdf[k] = k ? pr[k] + cdf[k - 1] : pr[0]; }
+        std::vector<vec<float, BPE>> vocab_lib((size_t)V2 * HID / BPE);
+        for (size_t i = 0; i < vocab_lib.size(); i++) for (int j = 0; j < BPE; j++) vocab_lib[i][j] = (float)(i * BPE + j) * 0.25f;
+        for (float r : {0.0f, 0.37f, 0.62f, 0.81f, 0.93f, 0.9999f}) {
+            bool near_edge = false;
+            for (int k = 0; k < TOPK; k++) near_edge = near_edge || std::abs(cdf[k] - r) < 1e-5f;
+            if (near_edge) continue;                                 // the device's expf against glibc's at a boundary
+            int sel = TOPK - 1;
+            for (int k = TOPK - 1; k >= 0; k--) if (r < cdf[k]) sel = k;
+            stream<vec<float, BPS>> ls;
+            stream<vec<float, BPE>> emb;
+            feed(ls, l2, V2);
+            int sampled_idx = -1;
+            dec_Sampling_Embedding_Layer<float, BPS, V2, TOPK, BPE, HID>(ls, vocab_lib, emb, r, sampled_idx, V2, HID);
+            if (sampled_idx != o2[sel]) { ok = false; std::cout << "rand " << r << ": My: " << sampled_idx << ", Ref: " << o2[sel] << std::endl; }
+            for (int i = 0; i < HID / BPE && sampled_idx >= 0; i++) {
+                const auto p = emb.read();
+                for (int j = 0; j < BPE; j++) if (p[j] != vocab_lib[(size_t)sampled_idx * (HID / BPE) + i][j]) ok = false;
+            }
+            ok = ok && emb.empty();
+        }
+    }
+    verdict("Logits (top-k layer on 128256 logits; sampling + embedding feedback)", ok);
+}
+
 int main() {
     try {
         QuantWrapper_Linear_Layer_q_decoding_test();
@@ -699,6 +886,10 @@ int main() {
         dec_MHA_test();
         pref_MHA_modules_test();
         adapters_test();
+        QuantWrapper_Linear_Layer_q_tops_test<true>();
+        QuantWrapper_Linear_Layer_q_tops_test<false>();
+        pref_Linear_Layer_i4xi4_test();
+        Logits_test();
     } catch (const std::exception& e) {
         std::cerr << "harness error: " << e.what() << std::endl;
         return 2;

@@ -69,3 +69,26 @@ def test_product_code_never_touches_the_oracle():
             if f.endswith((".py", ".hip", ".h", ".cpp")):
                 text = open(os.path.join(dirpath, f), errors="ignore").read()
                 assert "oracle" not in text.lower(), "%s mentions the oracle" % os.path.join(dirpath, f)
+
+
+def test_size_t_parameters_are_typed_in_the_binding():
+    """An untyped Python int reaches C as a 32-bit int: a 4 GiB size would arrive as zero.  Every entry point that
+    declares a size_t parameter in the header must therefore carry argtypes with c_size_t in that position."""
+    import ctypes as C
+    import re
+    from flexllm_amd import _lib
+    lib = _lib.lib()
+    header = open(os.path.join(ROOT, "include", "flexllm_hip.h")).read()
+    header = re.sub(r"/\*.*?\*/", " ", header, flags=re.S)
+    found = 0
+    for m in re.finditer(r"\bint\s+(flexllm_\w+)\s*\(([^)]*)\)\s*;", header):
+        name, params = m.group(1), [p.strip() for p in m.group(2).split(",")]
+        pos = [k for k, p in enumerate(params) if re.match(r"size_t\s+\w+$", p)]
+        if not pos:
+            continue
+        found += 1
+        at = getattr(lib, name).argtypes
+        assert at is not None and len(at) == len(params), name
+        for k in pos:
+            assert at[k] is C.c_size_t, (name, k)
+    assert found >= 10
