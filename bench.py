@@ -94,13 +94,13 @@ def measured_peaks(fx, lib, synth, stream, Event):
     buf = fx.empty((n,), np.int8)
     fx.check(lib.flexllm_rt_fill_i8(P(buf), C.c_size_t(n), C.c_uint64(77), -100, 100, stream.handle))
     sink = fx.empty((16384 * 4,), np.uint32)
-    us, wgs = min((_time(stream, Event, lambda i: lib.flexllm_probe_hbm_read(P(buf), C.c_size_t(n), g, P(sink), stream.handle), 4), g)
-                  for g in (1024, 2048, 4096, 8192, 16384))                 # the best grid size is reported
+    us, wgs, nt = min((_time(stream, Event, lambda i: lib.flexllm_probe_hbm_read(P(buf), C.c_size_t(n), g, t, P(sink), stream.handle), 4), g, t)
+                      for g in (256, 512, 1024, 2048, 4096) for t in (0, 1))       # the best grid size and load kind are reported
     one = 1 << 30
     us_c = _time(stream, Event, lambda i: lib.flexllm_rt_memcpy_d2d(C.c_void_p(buf.ptr + 2 * one), P(buf), C.c_size_t(one), stream.handle), 5)
-    out["hbm"] = {"published_GBs": HBM_PEAK_GBS, "read_stream_GBs": round(n / us / 1e3, 1), "read_stream_bytes": n, "read_stream_workgroups": wgs,
+    out["hbm"] = {"published_GBs": HBM_PEAK_GBS, "read_stream_GBs": round(n / us / 1e3, 1), "read_stream_bytes": n, "read_stream_workgroups": wgs, "read_stream_non_temporal": bool(nt),
                   "copy_GBs_read_plus_write": round(2 * one / us_c / 1e3, 1), "copy_bytes": one,
-                  "note": "read_stream: non-temporal 16-byte loads over 4 GiB, read-only (the decode path's traffic is 99 % reads); "
+                  "note": "read_stream: 16-byte loads over 4 GiB in contiguous 32 KiB blocks per workgroup, read-only (the decode path's traffic is 99 % reads); "
                           "copy: hipMemcpyAsync device to device of 1 GiB, bytes read + bytes written"}
     del buf
     iters, cus = 4000, 256

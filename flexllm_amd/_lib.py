@@ -62,7 +62,7 @@ def lib():
                            ("flexllm_rt_memcpy_d2d", [vp, vp, sz, vp]), ("flexllm_rt_memset", [vp, i, sz, vp]),
                            ("flexllm_rt_fill_i8", [vp, sz, u64, i, i, vp]), ("flexllm_rt_fill_uniform_f32", [vp, sz, u64, f, f, vp]),
                            ("flexllm_rt_fill_uniform_f16", [vp, sz, u64, f, f, vp]),
-                           ("flexllm_probe_hbm_read", [vp, sz, i, vp, vp]), ("flexllm_pack_nibbles", [vp, vp, sz, vp]),
+                           ("flexllm_probe_hbm_read", [vp, sz, i, i, vp, vp]), ("flexllm_pack_nibbles", [vp, vp, sz, vp]),
                            ("flexllm_swish_f32", [vp, vp, sz, vp]), ("flexllm_swiglu_f32", [vp, vp, vp, sz, vp]),
                            ("flexllm_residual_add_f32", [vp, vp, vp, sz, vp])):
             getattr(_lib, name).argtypes = args

@@ -58,21 +58,24 @@ __global__ __launch_bounds__(256) void probe_mfma_i8_kernel(int* __restrict__ si
     if (clocks && blockIdx.x == 0 && threadIdx.x == 0) { clocks[0] = c1 - c0; clocks[1] = w1 - w0; }
 }
 
-// HBM read stream: every thread reads 16-byte words with a grid stride and folds them into one word; a wave writes
-// one word.  Read-only traffic of `n16` 16-byte words, nothing else.
+// HBM read stream: a workgroup reads contiguous blocks of 32 KiB (eight 16-byte loads in flight per thread, a wave's
+// load covers 1 KiB of contiguous memory), blocks dealt to the workgroups round-robin; every word is folded into one
+// word per wave.  Read-only traffic of `n16` 16-byte words, nothing else.
+template <bool NT>
 __global__ __launch_bounds__(256) void probe_hbm_read_kernel(const i32x4* __restrict__ src, size_t n16, unsigned* __restrict__ sink) {
-    const size_t stride = (size_t)gridDim.x * 256;
-    size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    constexpr size_t kBlock16 = 8 * 256;                     // 16-byte words per block
     unsigned acc = 0;
-    for (; i + 7 * stride < n16; i += 8 * stride) {          // eight independent loads in flight per thread
+    const size_t n_blocks = n16 / kBlock16;
+    for (size_t b = blockIdx.x; b < n_blocks; b += gridDim.x) {
+        const i32x4* p = src + b * kBlock16 + threadIdx.x;
         i32x4 v[8];
 #pragma unroll
-        for (int u = 0; u < 8; u++) v[u] = __builtin_nontemporal_load(src + i + u * stride);
+        for (int u = 0; u < 8; u++) v[u] = NT ? __builtin_nontemporal_load(p + u * 256) : p[u * 256];
 #pragma unroll
         for (int u = 0; u < 8; u++) acc ^= (unsigned)(v[u][0] ^ v[u][1] ^ v[u][2] ^ v[u][3]);
     }
-    for (; i < n16; i += stride) {
-        const i32x4 a = __builtin_nontemporal_load(src + i);
+    for (size_t i = n_blocks * kBlock16 + (size_t)blockIdx.x * 256 + threadIdx.x; i < n16; i += (size_t)gridDim.x * 256) {
+        const i32x4 a = src[i];
         acc ^= (unsigned)(a[0] ^ a[1] ^ a[2] ^ a[3]);
     }
 #pragma unroll
@@ -97,10 +100,13 @@ int flexllm_probe_mfma_i8(int iters, int random_operands, int from_lds, int work
     return FLEXLLM_OK;
 }
 
-int flexllm_probe_hbm_read(const void* src, size_t bytes, int workgroups, unsigned* sink, void* stream) {
+int flexllm_probe_hbm_read(const void* src, size_t bytes, int workgroups, int non_temporal, unsigned* sink, void* stream) {
     FX_REQUIRE(src && sink && bytes % 16 == 0 && workgroups > 0 && workgroups <= 65536, "probe_hbm_read: bytes=%zu workgroups=%d", bytes, workgroups);
     FX_REQUIRE((reinterpret_cast<uintptr_t>(src) & 15) == 0, "probe_hbm_read: src must be 16-byte aligned");
-    probe_hbm_read_kernel<<<workgroups, 256, 0, as_stream(stream)>>>(static_cast<const i32x4*>(src), bytes / 16, sink);
+    if (non_temporal)
+        probe_hbm_read_kernel<true><<<workgroups, 256, 0, as_stream(stream)>>>(static_cast<const i32x4*>(src), bytes / 16, sink);
+    else
+        probe_hbm_read_kernel<false><<<workgroups, 256, 0, as_stream(stream)>>>(static_cast<const i32x4*>(src), bytes / 16, sink);
     FX_LAUNCH_CHECK();
     return FLEXLLM_OK;
 }

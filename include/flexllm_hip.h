@@ -79,9 +79,9 @@ int flexllm_rt_fill_uniform_f16(uint16_t* dst, size_t n, uint64_t seed, float lo
  * 100 MHz wall-clock ticks} of one wave's loop, i.e. the shader clock under this load. */
 int flexllm_probe_mfma_i8(int iters, int random_operands, int from_lds, int workgroups, int* sink, unsigned long long* clocks,
                           void* stream);
-/* Read-only stream over `bytes` (a multiple of 16) of device memory with non-temporal 16-byte loads; sink: device
- * [workgroups * 4] uint32. */
-int flexllm_probe_hbm_read(const void* src, size_t bytes, int workgroups, unsigned* sink, void* stream);
+/* Read-only stream over `bytes` (a multiple of 16) of device memory with 16-byte loads (non_temporal: with the
+ * non-temporal hint), contiguous 32 KiB blocks per workgroup; sink: device [workgroups * 4] uint32. */
+int flexllm_probe_hbm_read(const void* src, size_t bytes, int workgroups, int non_temporal, unsigned* sink, void* stream);
 
 /* ---- quant.h ------------------------------------------------------------------------ */
 /* Per-token symmetric int8 quantisation: s=absmax/127 (0 -> 1), q=round_half_away(x/s).
