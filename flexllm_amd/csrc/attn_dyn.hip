@@ -9,10 +9,11 @@
 //     o[d]  = float(sum_j P8[j] * v8[j][d]) * s_p  (* v_ch_s[kvh][d], the reference library's per-channel V scale).
 // P is signed here (0..127), so the MFMA / dot products need no offset trick.
 //
-// Prefill: the tiling of attn_prefill.h (32 queries x one head per workgroup, four waves split the key tiles,
-// S^T = K.Q^T so that the probabilities land in the A-operand layout of P.V), in three passes over the wave's tiles
-// because the row needs two global quantities before a probability can be rounded: the softmax denominator and the
-// maximum of p'.  Scores are recomputed in every pass (64-deep dot products on the matrix cores: cheap).
+// Prefill: the tiling of attn_prefill.h (32 queries x one head per workgroup, eight waves split the key tiles,
+// S^T = K.Q^T so that the probabilities land in the A-operand layout of P.V).  The row needs two global quantities
+// before a probability can be rounded: the softmax denominator and the maximum of p'.  Rows of up to 1024 keys keep
+// their scores in registers between those steps (pf_attention_dyn_cached_kernel); longer rows go over the wave's tiles in
+// three passes and form the scores again in each (64-deep dot products on the matrix cores: cheap).
 // Decode: the chunked kernels of attn_decode_kernels.h with one more kernel for the row maximum of p'.
 #include "attn_prefill.h"
 #include "gemv_i8.h"
@@ -24,59 +25,67 @@ struct DynScales {
     float q_div;
 };
 
+// Rows of any length: three passes over the wave's tiles, the scores formed again in each.  The K rows are loaded in the
+// permuted order of attn_prefill.h (a lane's 16 values are 16 consecutive keys); the tile's K and V scales are fetched by
+// the wave's lanes (one key each), parked in a wave-private corner of LDS and read back as four 16-byte words per lane.
+template <bool kStoreP>
 static __global__ __launch_bounds__(64 * kPfWaves) void pf_attention_dyn_kernel(
     const int8_t* __restrict__ q8, const int8_t* __restrict__ kc, const int8_t* __restrict__ vc, DynScales sc,
     float* __restrict__ o, int8_t* __restrict__ p8_out, float* __restrict__ p_s_out, int s, int q_heads, int kv_heads,
     int max_pos, int period) {
     __shared__ float lds_m[kPfWaves][32], lds_l[kPfWaves][32], lds_pm[kPfWaves][32], lds_sp[32];
     __shared__ int lds_acc[64][33];            // [lane][16 acc0 | 16 acc1], odd pitch against bank conflicts
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    __shared__ __attribute__((aligned(16))) float lds_sc[kPfWaves][2][kPfTile];   // per wave: K scales, V scales of the current tile
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int group = q_heads / kv_heads;
-    const int n_items = (int)gridDim.x, nqb = s / kPfTile;
-    const int round = (int)blockIdx.x / period, c = (int)blockIdx.x % period;
-    const int in_round = min(period, n_items - round * period);
-    const int item = round * period + ((round & 1) ? in_round - 1 - c : c);   // items in order of decreasing length, dealt in snake order
-    const int qb = nqb - 1 - item / q_heads;
-    const int q0 = qb * kPfTile;
-    const int h = item % q_heads, kvh = h / group;
-    const int col = lane & 31, g = lane >> 5;
-    const int query = q0 + col;
+    const PfItem it = pf_item(s, q_heads, group, period);
+    const int col = it.col, g = it.g, query = it.query, ntiles = it.ntiles, kvh = it.kvh, h = it.h;
     const float sq = sc.q_s[(size_t)query * q_heads + h] / sc.q_div;
 
     const int8_t* qrow = q8 + ((size_t)query * q_heads + h) * kHd;
     const i32x4 qf0 = *reinterpret_cast<const i32x4*>(qrow + g * 16);
     const i32x4 qf1 = *reinterpret_cast<const i32x4*>(qrow + 32 + g * 16);
-
-    auto load_k = [&](int k0, i32x4& kf0, i32x4& kf1) {
-        const int8_t* krow = kc + k_index(kvh, k0 + col, max_pos);
-        kf0 = *reinterpret_cast<const i32x4*>(krow + g * 16);
-        kf1 = *reinterpret_cast<const i32x4*>(krow + 32 + g * 16);
-    };
-    // scores of one tile: register r = 4a+b of this lane is (query, key k0 + 8a + 4g + b); the key's scale comes from
-    // the lane that loaded it (lane key-in-tile holds K_s of that key)
-    auto score_tile = [&](int k0, const i32x4& kf0, const i32x4& kf1, float ks_lane, float (&scv)[16]) {
+    const int krow_in_tile = pf_key_of_row(col);
+    const float* scale_tab = g == 0 ? sc.k_s : sc.v_s;        // lanes 0..31 fetch the K scales of the tile's keys, lanes 32..63 the V scales
+    // scores of tile kt (register r = key k0 + 16 g + r, masked beyond the query) and, on request, the V scales of the same keys
+    auto tile = [&](int kt, float (&scv)[16], float (&vs)[16], bool want_vs) {
+        const int k0 = kt * kPfTile;
+        const int8_t* krow = kc + k_index(kvh, k0 + krow_in_tile, max_pos);
+        const i32x4 kf0 = *reinterpret_cast<const i32x4*>(krow + g * 16);
+        const i32x4 kf1 = *reinterpret_cast<const i32x4*>(krow + 32 + g * 16);
+        lds_sc[wave][g][col] = scale_tab[(size_t)(k0 + col) * kv_heads + kvh];
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();                       // the corner is private to the wave: its LDS accesses complete in order
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
         i32x16 acc = zero16();
         acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(kf0, qf0, acc, 0, 0, 0);
         acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(kf1, qf1, acc, 0, 0, 0);
 #pragma unroll
-        for (int r = 0; r < 16; r++) {
-            const int kin = (r >> 2) * 8 + g * 4 + (r & 3);
-            const float ks = __shfl(ks_lane, kin);
-            const float v = (float)acc[r] * sq * ks;
-            scv[r] = (k0 + kin <= query) ? v : -1e32f;
+        for (int a = 0; a < 4; a++) {
+            const float4 ks4 = *reinterpret_cast<const float4*>(&lds_sc[wave][0][16 * g + 4 * a]);
+            const float ks[4] = {ks4.x, ks4.y, ks4.z, ks4.w};
+            if (want_vs) {
+                const float4 vs4 = *reinterpret_cast<const float4*>(&lds_sc[wave][1][16 * g + 4 * a]);
+                vs[4 * a] = vs4.x; vs[4 * a + 1] = vs4.y; vs[4 * a + 2] = vs4.z; vs[4 * a + 3] = vs4.w;
+            }
+#pragma unroll
+            for (int b = 0; b < 4; b++) {
+                const float v = (float)acc[4 * a + b] * sq * ks[b];
+                scv[4 * a + b] = (k0 + 16 * g + 4 * a + b <= query) ? v : -1e32f;
+            }
         }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();                       // reads of this tile's scales before the next tile's writes
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
     };
-    auto tile_scale = [&](const float* tab, int k0) { return tab[(size_t)(k0 + col) * kv_heads + kvh]; };
 
-    const int ntiles = qb + 1;
     for (int i = threadIdx.x; i < 64 * 33; i += 64 * kPfWaves) (&lds_acc[0][0])[i] = 0;
+    float scv[16], vs[16];
     // ---- pass 1: row maximum and sum of exponentials over this wave's tiles ----
     float m_run = -1e32f, l_run = 0.0f;
     for (int kt = wave; kt < ntiles; kt += kPfWaves) {
-        i32x4 kf0, kf1;
-        load_k(kt * kPfTile, kf0, kf1);
-        float scv[16];
-        score_tile(kt * kPfTile, kf0, kf1, tile_scale(sc.k_s, kt * kPfTile), scv);
+        tile(kt, scv, vs, false);
         float mt = scv[0];
 #pragma unroll
         for (int r = 1; r < 16; r++) mt = fmaxf(mt, scv[r]);
@@ -105,16 +114,9 @@ static __global__ __launch_bounds__(64 * kPfWaves) void pf_attention_dyn_kernel(
     // ---- pass 2: row maximum of p' = p * V_s[key] ----
     float pm = 0.0f;
     for (int kt = wave; kt < ntiles; kt += kPfWaves) {
-        i32x4 kf0, kf1;
-        load_k(kt * kPfTile, kf0, kf1);
-        float scv[16];
-        score_tile(kt * kPfTile, kf0, kf1, tile_scale(sc.k_s, kt * kPfTile), scv);
-        const float vs_lane = tile_scale(sc.v_s, kt * kPfTile);
+        tile(kt, scv, vs, true);
 #pragma unroll
-        for (int r = 0; r < 16; r++) {
-            const float vs = __shfl(vs_lane, (r >> 2) * 8 + g * 4 + (r & 3));
-            pm = fmaxf(pm, exp_f<false>(scv[r] - mx) * cd * vs);          // masked keys give exactly 0
-        }
+        for (int r = 0; r < 16; r++) pm = fmaxf(pm, exp_f<false>(scv[r] - mx) * cd * vs[r]);          // masked keys give exactly 0
     }
     pm = fmaxf(pm, lane_xor_f<32>(pm));
     if (g == 0) lds_pm[wave][col] = pm;
@@ -130,35 +132,24 @@ static __global__ __launch_bounds__(64 * kPfWaves) void pf_attention_dyn_kernel(
 
     // ---- pass 3: probabilities, partial P.V over this wave's tiles ----
     i32x16 oacc0 = zero16(), oacc1 = zero16();
+    int8_t* const prow = kStoreP ? p8_out + ((size_t)h * s + query) * s + 16 * g : nullptr;
     for (int kt = wave; kt < ntiles; kt += kPfWaves) {
         const int k0 = kt * kPfTile;
-        i32x4 kf0, kf1;
-        load_k(k0, kf0, kf1);
-        const int8_t* vblk = vc + v_index(kvh, k0, 0, max_pos);
-        i32x4 vf0, vf1;
-#pragma unroll
-        for (int a = 0; a < 4; a++) {
-            vf0[a] = *reinterpret_cast<const int*>(vblk + (size_t)col * kVBlock + a * 8 + g * 4);
-            vf1[a] = *reinterpret_cast<const int*>(vblk + (size_t)(col + 32) * kVBlock + a * 8 + g * 4);
-        }
-        float scv[16];
-        score_tile(k0, kf0, kf1, tile_scale(sc.k_s, k0), scv);
-        const float vs_lane = tile_scale(sc.v_s, k0);
+        const int8_t* vblk = vc + v_index(kvh, k0, 0, max_pos) + 16 * g;
+        const i32x4 vf0 = *reinterpret_cast<const i32x4*>(vblk + (size_t)col * kVBlock);
+        const i32x4 vf1 = *reinterpret_cast<const i32x4*>(vblk + (size_t)(col + 32) * kVBlock);
+        tile(kt, scv, vs, true);
         i32x4 pf;
 #pragma unroll
         for (int a = 0; a < 4; a++) {
-            uint32_t packed = 0;
+            float f[4];
 #pragma unroll
-            for (int b = 0; b < 4; b++) {
-                const int kin = a * 8 + g * 4 + b;
-                const float vs = __shfl(vs_lane, kin);
-                const float pp = exp_f<false>(scv[a * 4 + b] - mx) * cd * vs;
-                const int pq = (int)roundf(pp / sp);                      // 0..127 by construction of sp
-                if (p8_out) p8_out[((size_t)h * s + query) * s + k0 + kin] = (int8_t)pq;
-                packed |= (uint32_t)(pq & 0xff) << (8 * b);
-            }
-            pf[a] = (int)packed;
+            for (int b = 0; b < 4; b++) f[b] = exp_f<false>(scv[4 * a + b] - mx) * cd * vs[4 * a + b];
+            int nq[4];
+            quant_vector(f, sp, nq);                                       // 0..127 by construction of sp
+            pf[a] = (int)pack4_i8(nq[0], nq[1], nq[2], nq[3]);
         }
+        if constexpr (kStoreP) *reinterpret_cast<i32x4*>(prow + k0) = pf;
         oacc0 = __builtin_amdgcn_mfma_i32_32x32x32_i8(pf, vf0, oacc0, 0, 0, 0);
         oacc1 = __builtin_amdgcn_mfma_i32_32x32x32_i8(pf, vf1, oacc1, 0, 0, 0);
     }
@@ -175,7 +166,173 @@ static __global__ __launch_bounds__(64 * kPfWaves) void pf_attention_dyn_kernel(
     for (int rr = 0; rr < 16 / kPfWaves; rr++) {              // accumulator register r holds query row 8a + 4g + b, channel col
         const int r = wave * (16 / kPfWaves) + rr;
         const int qi = (r >> 2) * 8 + g * 4 + (r & 3);
-        float* orow = o + ((size_t)(q0 + qi) * q_heads + h) * kHd;
+        float* orow = o + ((size_t)(it.q0 + qi) * q_heads + h) * kHd;
+        const float spq = lds_sp[qi];
+        const float t0 = (float)lds_acc[lane][r] * spq, t1 = (float)lds_acc[lane][16 + r] * spq;
+        orow[col] = sc.v_ch_s ? t0 * vch0 : t0;
+        orow[col + 32] = sc.v_ch_s ? t1 * vch1 : t1;
+    }
+}
+
+// Rows of at most kPfWaves * kPfCachedTiles * 32 = 1024 keys: the structure of pf_attention_cached_kernel.  Every score
+// tile of a wave stays in registers through all the row-wide steps, so each score is formed once and each exponential
+// is taken once: scores (kept) and their maximum; exponentials with the final maximum (in place) and their sum;
+// p' = e * (1/sum) * V_s[key] (in place) and its maximum; rounding and P.V.  The K rows are loaded in the permuted order
+// of attn_prefill.h, which makes a lane's 16 values 16 consecutive keys: their K and V scales are four 16-byte reads
+// from a per-workgroup table in LDS (the scales of the row block's keys, staged once), the probability bytes leave as
+// one 16-byte store, and V's operand is one 16-byte load per channel.  round(p' / s_p) goes through the reciprocal with
+// the IEEE division only next to a rounding tie (quant_vector), like the per-row quantisers.
+template <bool kStoreP>
+static __global__ __launch_bounds__(64 * kPfWaves, 2) void pf_attention_dyn_cached_kernel(
+    const int8_t* __restrict__ q8, const int8_t* __restrict__ kc, const int8_t* __restrict__ vc, DynScales sc,
+    float* __restrict__ o, int8_t* __restrict__ p8_out, float* __restrict__ p_s_out, int s, int q_heads, int kv_heads,
+    int max_pos, int period) {
+    __shared__ float lds_m[kPfWaves][32], lds_l[kPfWaves][32], lds_pm[kPfWaves][32], lds_sp[32];
+    __shared__ int lds_acc[64][33];            // [lane][16 acc0 | 16 acc1], odd pitch against bank conflicts
+    __shared__ __attribute__((aligned(16))) float lds_ks[kPfWaves * kPfCachedTiles * kPfTile], lds_vs[kPfWaves * kPfCachedTiles * kPfTile];
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int group = q_heads / kv_heads;
+    const PfItem it = pf_item(s, q_heads, group, period);
+    const int col = it.col, g = it.g, query = it.query, ntiles = it.ntiles, kvh = it.kvh, h = it.h;   // ntiles <= 32 (launcher)
+    const float sq = sc.q_s[(size_t)query * q_heads + h] / sc.q_div;
+
+    const int8_t* qrow = q8 + ((size_t)query * q_heads + h) * kHd;
+    const i32x4 qf0 = *reinterpret_cast<const i32x4*>(qrow + g * 16);
+    const i32x4 qf1 = *reinterpret_cast<const i32x4*>(qrow + 32 + g * 16);
+    const int krow_in_tile = pf_key_of_row(col);
+    // the K rows of all of this wave's tiles are requested at once
+    i32x4 kf[kPfCachedTiles][2];
+#pragma unroll
+    for (int i = 0; i < kPfCachedTiles; i++)
+        if (wave + kPfWaves * i < ntiles) {
+            const int8_t* krow = kc + k_index(kvh, (wave + kPfWaves * i) * kPfTile + krow_in_tile, max_pos);
+            kf[i][0] = *reinterpret_cast<const i32x4*>(krow + g * 16);
+            kf[i][1] = *reinterpret_cast<const i32x4*>(krow + 32 + g * 16);
+        }
+    for (int j = threadIdx.x; j < ntiles * kPfTile; j += 64 * kPfWaves) {
+        lds_ks[j] = sc.k_s[(size_t)j * kv_heads + kvh];
+        lds_vs[j] = sc.v_s[(size_t)j * kv_heads + kvh];
+    }
+    for (int i = threadIdx.x; i < 64 * 33; i += 64 * kPfWaves) (&lds_acc[0][0])[i] = 0;
+    __syncthreads();
+
+    // ---- scores of this wave's tiles (kept), row maximum: register r of a lane is key k0 + 16 g + r ----
+    float sv[kPfCachedTiles][16];
+    float m_run = -1e32f;
+#pragma unroll
+    for (int i = 0; i < kPfCachedTiles; i++) {
+        const int kt = wave + kPfWaves * i;
+        if (kt < ntiles) {
+            i32x16 acc = zero16();
+            acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(kf[i][0], qf0, acc, 0, 0, 0);
+            acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(kf[i][1], qf1, acc, 0, 0, 0);
+            const int key0 = kt * kPfTile + 16 * g;
+#pragma unroll
+            for (int a = 0; a < 4; a++) {
+                const float4 ks4 = *reinterpret_cast<const float4*>(&lds_ks[key0 + 4 * a]);
+                const float ks[4] = {ks4.x, ks4.y, ks4.z, ks4.w};
+#pragma unroll
+                for (int b = 0; b < 4; b++) {
+                    const float v = (float)acc[4 * a + b] * sq * ks[b];
+                    sv[i][4 * a + b] = (key0 + 4 * a + b <= query) ? v : -1e32f;
+                    m_run = fmaxf(m_run, sv[i][4 * a + b]);
+                }
+            }
+        }
+    }
+    m_run = fmaxf(m_run, lane_xor_f<32>(m_run));
+    if (g == 0) lds_m[wave][col] = m_run;
+    __syncthreads();
+    float mx = lds_m[0][col];
+#pragma unroll
+    for (int w = 1; w < kPfWaves; w++) mx = fmaxf(mx, lds_m[w][col]);
+    // ---- exponentials (in place) and their sum ----
+    float l_run = 0.0f;
+#pragma unroll
+    for (int i = 0; i < kPfCachedTiles; i++)
+        if (wave + kPfWaves * i < ntiles) {
+#pragma unroll
+            for (int r = 0; r < 16; r++) {
+                sv[i][r] = exp_f<false>(sv[i][r] - mx);                 // masked keys give exactly 0
+                l_run += sv[i][r];
+            }
+        }
+    l_run = l_run + lane_xor_f<32>(l_run);
+    if (g == 0) lds_l[wave][col] = l_run;
+    __syncthreads();
+    float total = lds_l[0][col];
+#pragma unroll
+    for (int w = 1; w < kPfWaves; w++) total += lds_l[w][col];
+    const float cd = 1.0f / total;
+    // ---- p' = p * V_s[key] (in place) and its maximum ----
+    float pm = 0.0f;
+#pragma unroll
+    for (int i = 0; i < kPfCachedTiles; i++) {
+        const int kt = wave + kPfWaves * i;
+        if (kt < ntiles) {
+            const int key0 = kt * kPfTile + 16 * g;
+#pragma unroll
+            for (int a = 0; a < 4; a++) {
+                const float4 vs4 = *reinterpret_cast<const float4*>(&lds_vs[key0 + 4 * a]);
+                const float vs[4] = {vs4.x, vs4.y, vs4.z, vs4.w};
+#pragma unroll
+                for (int b = 0; b < 4; b++) {
+                    sv[i][4 * a + b] = sv[i][4 * a + b] * cd * vs[b];
+                    pm = fmaxf(pm, sv[i][4 * a + b]);
+                }
+            }
+        }
+    }
+    pm = fmaxf(pm, lane_xor_f<32>(pm));
+    if (g == 0) lds_pm[wave][col] = pm;
+    __syncthreads();
+    float pmax = lds_pm[0][col];
+#pragma unroll
+    for (int w = 1; w < kPfWaves; w++) pmax = fmaxf(pmax, lds_pm[w][col]);
+    const float sp = sym_scale(pmax, 127.0f);
+    if (wave == 0 && g == 0) {
+        lds_sp[col] = sp;
+        if (p_s_out) p_s_out[(size_t)query * q_heads + h] = sp;
+    }
+    // ---- probabilities, partial P.V over this wave's tiles ----
+    i32x16 oacc0 = zero16(), oacc1 = zero16();
+    int8_t* const prow = kStoreP ? p8_out + ((size_t)h * s + query) * s + 16 * g : nullptr;
+#pragma unroll
+    for (int i = 0; i < kPfCachedTiles; i++) {
+        const int kt = wave + kPfWaves * i;
+        if (kt < ntiles) {
+            const int k0 = kt * kPfTile;
+            const int8_t* vblk = vc + v_index(kvh, k0, 0, max_pos) + 16 * g;
+            const i32x4 vf0 = *reinterpret_cast<const i32x4*>(vblk + (size_t)col * kVBlock);
+            const i32x4 vf1 = *reinterpret_cast<const i32x4*>(vblk + (size_t)(col + 32) * kVBlock);
+            i32x4 pf;
+#pragma unroll
+            for (int a = 0; a < 4; a++) {
+                const float f[4] = {sv[i][4 * a], sv[i][4 * a + 1], sv[i][4 * a + 2], sv[i][4 * a + 3]};
+                int nq[4];
+                quant_vector(f, sp, nq);                                   // 0..127 by construction of sp
+                pf[a] = (int)pack4_i8(nq[0], nq[1], nq[2], nq[3]);
+            }
+            if constexpr (kStoreP) *reinterpret_cast<i32x4*>(prow + k0) = pf;
+            oacc0 = __builtin_amdgcn_mfma_i32_32x32x32_i8(pf, vf0, oacc0, 0, 0, 0);
+            oacc1 = __builtin_amdgcn_mfma_i32_32x32x32_i8(pf, vf1, oacc1, 0, 0, 0);
+        }
+    }
+    if (wave < ntiles) {
+#pragma unroll
+        for (int r = 0; r < 16; r++) {
+            atomicAdd(&lds_acc[lane][r], oacc0[r]);
+            atomicAdd(&lds_acc[lane][16 + r], oacc1[r]);
+        }
+    }
+    __syncthreads();
+    const float vch0 = sc.v_ch_s ? sc.v_ch_s[kvh * kHd + col] : 1.0f, vch1 = sc.v_ch_s ? sc.v_ch_s[kvh * kHd + col + 32] : 1.0f;
+#pragma unroll
+    for (int rr = 0; rr < 16 / kPfWaves; rr++) {              // accumulator register r holds query row 8a + 4g + b, channel col
+        const int r = wave * (16 / kPfWaves) + rr;
+        const int qi = (r >> 2) * 8 + g * 4 + (r & 3);
+        float* orow = o + ((size_t)(it.q0 + qi) * q_heads + h) * kHd;
         const float spq = lds_sp[qi];
         const float t0 = (float)lds_acc[lane][r] * spq, t1 = (float)lds_acc[lane][16 + r] * spq;
         orow[col] = sc.v_ch_s ? t0 * vch0 : t0;
@@ -350,8 +507,21 @@ int flexllm_mha_i8_prefill_dyn(const int8_t* q8, const int8_t* k_cache, const in
     FX_HIP(hipDeviceGetAttribute(&n_cu, hipDeviceAttributeMultiprocessorCount, dev));
     if (n_cu <= 0) n_cu = 256;
     const DynScales d = {sc->q_s, sc->k_s, sc->v_s, sc->v_ch_s, sc->q_scale_div};
-    pf_attention_dyn_kernel<<<(s / kPfTile) * q_heads, 64 * kPfWaves, 0, as_stream(stream)>>>(q8, k_cache, v_cache, d, o, p8_out, p_s_out, s,
-                                                                                          q_heads, kv_heads, max_pos, n_cu);
+    const int grid = (s / kPfTile) * q_heads;
+    if (s <= kPfWaves * kPfCachedTiles * kPfTile) {            // every row fits the registers of eight waves
+        if (p8_out)
+            pf_attention_dyn_cached_kernel<true><<<grid, 64 * kPfWaves, 0, as_stream(stream)>>>(q8, k_cache, v_cache, d, o, p8_out, p_s_out, s,
+                                                                                                q_heads, kv_heads, max_pos, n_cu);
+        else
+            pf_attention_dyn_cached_kernel<false><<<grid, 64 * kPfWaves, 0, as_stream(stream)>>>(q8, k_cache, v_cache, d, o, nullptr, p_s_out, s,
+                                                                                                 q_heads, kv_heads, max_pos, n_cu);
+    } else if (p8_out) {
+        pf_attention_dyn_kernel<true><<<grid, 64 * kPfWaves, 0, as_stream(stream)>>>(q8, k_cache, v_cache, d, o, p8_out, p_s_out, s, q_heads,
+                                                                                     kv_heads, max_pos, n_cu);
+    } else {
+        pf_attention_dyn_kernel<false><<<grid, 64 * kPfWaves, 0, as_stream(stream)>>>(q8, k_cache, v_cache, d, o, nullptr, p_s_out, s, q_heads,
+                                                                                      kv_heads, max_pos, n_cu);
+    }
     FX_LAUNCH_CHECK();
     return FLEXLLM_OK;
 }
