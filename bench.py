@@ -200,8 +200,13 @@ def module_legs(fx, lib, synth, ops, stream, Event, peaks=None):
     def leg1b(i):
         lib.flexllm_linear_i8_gemv_dequant(P(xq), P(xs), P(ring[i % len(ring)]), P(w_s), None, P(y), K, N, stream.handle)
     us_b = _time(stream, Event, leg1b, 160)
+    def leg1c(i):
+        lib.flexllm_quant_linear_i8_gemv_dequant(P(x), P(ring[i % len(ring)]), P(w_s), None, P(y), None, None, K, N, stream.handle)
+    us_c = _time(stream, Event, leg1c, 160)
     b1 = N * K + 4 * N + 4 * K + 4 * N
     out["linear_decode_2048x2048"] = {"bytes": b1, "us_quant_gemv_dequant": round(us, 2), "us_gemv_dequant": round(us_b, 2),
+                                      "us_fused_one_launch": round(us_c, 2), "GBs_fused": round(b1 / us_c / 1e3, 1),
+                                      "hbm_frac_fused": round(b1 / us_c / 1e3 / HBM_PEAK_GBS, 4),
                                       "GBs_gemv": round(b1 / us_b / 1e3, 1), "hbm_frac_gemv": round(b1 / us_b / 1e3 / HBM_PEAK_GBS, 4)}
     del ring
     # (2) FHT / sqrt(n) -> per-token int8, 1024 tokens
@@ -264,6 +269,25 @@ def module_legs(fx, lib, synth, ops, stream, Event, peaks=None):
                                                      if S <= 1024 else "causal half computed, scores formed again in each of the three passes (maximum, sum, probabilities)")
                                                     + "; bound by the exponential and rounding per probability"}
         del q8, kc, vc, o
+    # (4b) the same attention with dynamic per-(token, head) scales (the variant the metric's source names for the module
+    # test): S = 1024, 32/8 heads; rows of up to 1024 keys keep their scores in registers
+    S = 1024
+    q8 = synth.device_i8((S, QH, 64), 9410)
+    kc, vc = ops.kv_cache(KVH, S)
+    lib.flexllm_rt_fill_i8(P(kc), C.c_size_t(kc.size), C.c_uint64(9411), -100, 100, stream.handle)
+    lib.flexllm_rt_fill_i8(P(vc), C.c_size_t(vc.size), C.c_uint64(9412), -100, 100, stream.handle)
+    dq = synth.device_uniform_f32((S, QH), 9413, 0.003, 0.005); dk = synth.device_uniform_f32((S, KVH), 9414, 0.02, 0.04)
+    dv = synth.device_uniform_f32((S, KVH), 9415, 0.02, 0.04)
+    dsc = ops._dyn_scales(dq, dk, dv, None, 8.0)
+    o = fx.empty((S, QH, 64), np.float32); ps = fx.empty((S, QH), np.float32)
+    def leg4b(i):
+        lib.flexllm_mha_i8_prefill_dyn(P(q8), P(kc), P(vc), C.byref(dsc), P(o), None, P(ps), S, QH, KVH, 64, S, stream.handle)
+    us = _time(stream, Event, leg4b, 20)
+    ops4 = 2 * 2 * QH * S * S * 64
+    out["attention_prefill_dyn_S1024"] = {"us": round(us, 2), "GOP_full_S2": round(ops4 / 1e9, 2), "TOPs_full_S2": round(ops4 / us / 1e6, 1),
+                                          "mfma_frac_full_S2": round(ops4 / us / 1e6 / INT8_PEAK_TOPS, 4),
+                                          "note": "per-(token, head) Q/K/V scales, V's scale folded into int8 probabilities (own formulation: no reference counterpart for the P.V side)"}
+    del q8, kc, vc, o
     # (5) W4A4 linears (the reference's shipped precision): decode GEMV 2048 -> 8192 on nibble-packed weights
     # (half the bytes of the int8 path) and the prefill GEMM at M = 1024
     K, N = 2048, 8192

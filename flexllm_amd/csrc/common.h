@@ -209,7 +209,8 @@ __device__ __forceinline__ float block_sum(float v, float* red) {
 __device__ __forceinline__ int quant_round(float x, float s) { return (int)roundf(x / s); }
 
 // round(x / s) for a whole vector that shares s, without a division per element.  q~ = x * rcp(s) is within
-// 4 * 2^-24 * |q| <= 3.1e-5 of the correctly rounded quotient (|q| <= 127.5), so both round to the same integer
+// 4 * 2^-24 * |q| <= 3.1e-5 of the correctly rounded quotient for |q| <= 127.5 (symmetric int8), <= 6.1e-5 for
+// |q| <= 255 (the asymmetric uint8 use: still inside the window, with a margin of 1.6), so both round to the same integer
 // unless q~ lies within 1e-4 of a tie (k + 0.5); `near_tie` collects those cases and the caller redoes them
 // with the exact expression.  Valid while 1/s is a normal number (`quant_fast_ok`).
 __device__ __forceinline__ bool quant_fast_ok(float s) { return s >= 0x1p-100f && s <= 0x1p100f; }

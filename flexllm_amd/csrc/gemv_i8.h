@@ -116,6 +116,84 @@ __global__ __launch_bounds__(kGemvBlock) void gemv_i8_kernel(const int8_t* __res
     }
 }
 
+// The whole decode linear of one token in one launch: per-token symmetric int8 quantisation of the fp32 activation,
+// GEMV, dequantisation (+ residual).  Every wave quantises the activation for itself, straight into the register
+// layout the row products read (lane l holds the 16-value chunks l, l+64, ...): eight 16-byte loads per chunk pair, a
+// wave-wide maximum, the library's quantiser arithmetic (sym_scale_127_uniform, quant_vector: the bytes and the scale
+// are those of quant_sym_kernel) - no LDS, no workgroup barrier, no second kernel.
+template <int NCH, int U>
+__global__ __launch_bounds__(kGemvBlock) void gemv_f32_i8_kernel(const float* __restrict__ x, const int8_t* __restrict__ w,
+                                                                 const float* __restrict__ w_s, const float* __restrict__ residual,
+                                                                 float* __restrict__ y, float* __restrict__ s_x_out,
+                                                                 int8_t* __restrict__ q_out, int k, int n, int rows_per_wave) {
+    const int lane = threadIdx.x & 63;
+    const int gw = blockIdx.x * kGemvWaves + (threadIdx.x >> 6);
+    const int row0 = gw * rows_per_wave;
+    if (row0 >= n) return;
+    const int nrows = min(rows_per_wave, n - row0);
+    const int nchunks = k >> 4;
+    // the first two weight rows of this wave are requested before anything else: they do not depend on the activation,
+    // and the quantisation below (a trip to the cache, a wave-wide maximum, a division) runs while they are on their way
+    i32x4 wv[2][NCH];
+#pragma unroll
+    for (int u = 0; u < 2; u++) {
+        const i32x4* wr = reinterpret_cast<const i32x4*>(w + (size_t)(row0 + min(u, nrows - 1)) * k);
+#pragma unroll
+        for (int i = 0; i < NCH; i++) {
+            const int c = lane + 64 * i;
+            wv[u][i] = c < nchunks ? __builtin_nontemporal_load(wr + c) : i32x4{0, 0, 0, 0};
+        }
+    }
+    float4 xf[NCH][4];
+    float amax = 0.0f;
+#pragma unroll
+    for (int i = 0; i < NCH; i++) {
+        const int c = lane + 64 * i;
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            xf[i][j] = c < nchunks ? reinterpret_cast<const float4*>(x)[4 * c + j] : make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+            amax = fmaxf(amax, fmaxf(fmaxf(fabsf(xf[i][j].x), fabsf(xf[i][j].y)), fmaxf(fabsf(xf[i][j].z), fabsf(xf[i][j].w))));
+        }
+    }
+    amax = wave_max(amax);
+    const float sx = sym_scale_127_uniform(amax);
+    i32x4 xr[NCH];
+#pragma unroll
+    for (int i = 0; i < NCH; i++)
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            const float f[4] = {xf[i][j].x, xf[i][j].y, xf[i][j].z, xf[i][j].w};
+            int nq[4];
+            quant_vector(f, sx, nq);
+            xr[i][j] = (int)pack4_i8(nq[0], nq[1], nq[2], nq[3]);
+        }
+    if (gw == 0) {                                             // the quantised activation and its scale, on request
+        if (s_x_out && lane == 0) s_x_out[0] = sx;
+        if (q_out) {
+#pragma unroll
+            for (int i = 0; i < NCH; i++)
+                if (lane + 64 * i < nchunks) reinterpret_cast<i32x4*>(q_out)[lane + 64 * i] = xr[i];
+        }
+    }
+    auto epi = [&](int row, int sum) {
+        if (lane == 0) {
+            float v = (float)sum * sx * w_s[row];
+            if (residual) v = v + residual[row];
+            y[row] = v;
+        }
+    };
+#pragma unroll
+    for (int u = 0; u < 2; u++) {
+        if (u < nrows) {
+            int acc = 0;
+#pragma unroll
+            for (int i = 0; i < NCH; i++) acc = dot16(wv[u][i], xr[i], acc);
+            epi(row0 + u, wave_sum_i(acc));
+        }
+    }
+    if (nrows > 2) wave_gemv_rows<NCH, U>(w, xr, k, nchunks, row0 + 2, nrows - 2, lane, epi);
+}
+
 // Picks rows per wave so that the chip holds ~8 waves per CU while each wave still streams several KiB.
 static inline int pick_rows_per_wave(int k, int n) {
     const int target_waves = 256 * 8;  // 256 CUs x 8 waves
@@ -139,6 +217,19 @@ inline int launch_gemv(const int8_t* x, const int8_t* w, int32_t* acc, const flo
     else if (nch <= 8) FX_GEMV_CASE(8, 2);
     else FX_GEMV_CASE(16, 2);
 #undef FX_GEMV_CASE
+    FX_LAUNCH_CHECK();
+    return FLEXLLM_OK;
+}
+
+inline int launch_gemv_f32(const float* x, const int8_t* w, const float* w_s, const float* residual, float* y, float* s_x_out,
+                           int8_t* q_out, int k, int n, hipStream_t st) {
+    const int nch = (k / 16 + 63) / 64;
+    const int rpw = pick_rows_per_wave(k, n);
+    const int waves = (n + rpw - 1) / rpw;
+    const int grid = (waves + kGemvWaves - 1) / kGemvWaves;
+    if (nch <= 1) gemv_f32_i8_kernel<1, 4><<<grid, kGemvBlock, 0, st>>>(x, w, w_s, residual, y, s_x_out, q_out, k, n, rpw);
+    else if (nch <= 2) gemv_f32_i8_kernel<2, 4><<<grid, kGemvBlock, 0, st>>>(x, w, w_s, residual, y, s_x_out, q_out, k, n, rpw);
+    else gemv_f32_i8_kernel<4, 2><<<grid, kGemvBlock, 0, st>>>(x, w, w_s, residual, y, s_x_out, q_out, k, n, rpw);
     FX_LAUNCH_CHECK();
     return FLEXLLM_OK;
 }

@@ -60,6 +60,15 @@ int flexllm_linear_i8_gemv_dequant(const int8_t* x, const float* s_x, const int8
     return launch_gemv<kEpiDequant>(x, w, nullptr, s_x, w_s, residual, y, k, n, as_stream(stream));
 }
 
+int flexllm_quant_linear_i8_gemv_dequant(const float* x, const int8_t* w, const float* w_s, const float* residual, float* y,
+                                         float* s_x_out, int8_t* q_out, int k, int n, void* stream) {
+    FX_REQUIRE(x && w && w_s && y, "quant_linear_i8_gemv_dequant: null pointer");
+    FX_REQUIRE(k > 0 && k % 16 == 0 && k <= 4096, "quant_linear_i8_gemv_dequant: k=%d must be a multiple of 16, <= 4096", k);
+    FX_REQUIRE(n >= 0, "quant_linear_i8_gemv_dequant: n=%d", n);
+    if (n == 0) return FLEXLLM_OK;
+    return launch_gemv_f32(x, w, w_s, residual, y, s_x_out, q_out, k, n, as_stream(stream));
+}
+
 int flexllm_linear_i8_gemv_swiglu(const int8_t* x, const float* s_x, const int8_t* w_gu, const float* w_s_gu, float* y,
                                   int k, int n, void* stream) {
     FX_REQUIRE(x && s_x && w_gu && w_s_gu && y, "linear_i8_gemv_swiglu: null pointer");

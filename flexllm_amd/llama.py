@@ -93,8 +93,9 @@ def synth_weights_w4a4(cfg, seed=1, device=False, embed_range=1.7):
 
 class Llama:
     """Device model object.  `weights` holds DeviceArrays (see synth_weights(device=True)); with the keys of
-    synth_weights_w4a4 (`sum<p>`, `head_w`, ...) it is the W4A4 model (flexllm_llama_create_w4a4), which decodes in the
-    persistent kernel and has no fused prefill."""
+    synth_weights_w4a4 (`sum<p>`, `head_w`, ...) it is the W4A4 model (flexllm_llama_create_w4a4): it decodes in the
+    persistent kernel's W4A4 instance, and prefill_hidden / generate run the W4A4 prefill graph (uint4 activations x int4
+    weights held one per byte on the int8 MFMA kernel, asymmetric dequantisation in the epilogues)."""
 
     def __init__(self, cfg, weights):
         self.cfg = cfg

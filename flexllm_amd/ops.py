@@ -87,6 +87,17 @@ def linear_i8_gemv_dequant(x, s_x, w, w_s, residual=None, stream=None, out=None)
     return y
 
 
+def quant_linear_i8_gemv_dequant(x, w, w_s, residual=None, want_q=False, stream=None, out=None):
+    """One token's whole decode linear in one launch: quantise x fp32 [k] per token (symmetric int8), GEMV, dequantise
+    (+ residual).  Returns y, or (y, q int8 [k], s_x [1]) with want_q."""
+    n, k = w.shape
+    y = out if out is not None else DeviceArray((n,), np.float32)
+    q = DeviceArray((k,), np.int8) if want_q else None
+    s = DeviceArray((1,), np.float32) if want_q else None
+    check(lib().flexllm_quant_linear_i8_gemv_dequant(_p(x), _p(w), _p(w_s), _p(residual), _p(y), _p(s), _p(q), k, n, _s(stream)))
+    return (y, q, s) if want_q else y
+
+
 def linear_i8_gemv_swiglu(x, s_x, w_gu, w_s_gu, stream=None, out=None):
     """x int8 [k], w_gu int8 [2n][k] (rows interleaved gate, up) -> y fp32 [n] = up * silu(gate)."""
     k = x.shape[-1]

@@ -122,6 +122,13 @@ int flexllm_linear_i8_gemv(const int8_t* x, const int8_t* w, int32_t* acc, int k
  * (+ dec_Residual_Layer, Modules/Residual_Layer.h:69-87). */
 int flexllm_linear_i8_gemv_dequant(const int8_t* x, const float* s_x, const int8_t* w, const float* w_s,
                                    const float* residual, float* y, int k, int n, void* stream);
+/* The whole decode linear of one token in one launch: per-token symmetric int8 quantisation of x fp32 [k] (the bytes and
+ * the scale of flexllm_quant_sym_i8), GEMV, dequantisation (+ residual) - what the reference's quantised linear wrapper
+ * chains per token: dec_quant_layer_fp32_qint -> dec_Linear_Layer -> dec_dequant_layer_qint_fp32_bandwidth
+ * (SpinQuant_Llama_32_1B/Linear_Layer_test.h:332-364).  Optional outputs: s_x_out [1] the activation scale, q_out [k] the
+ * quantised activation.  k % 16 == 0, k <= 4096. */
+int flexllm_quant_linear_i8_gemv_dequant(const float* x, const int8_t* w, const float* w_s, const float* residual, float* y,
+                                         float* s_x_out, int8_t* q_out, int k, int n, void* stream);
 /* Fused gate/up projection + SwiGLU: w_gu is int8 [2n][k] with rows interleaved (row 2i = gate_i, row 2i+1 = up_i),
  * w_s_gu the matching 2n scales; y[i] = up_i * (gate_i/(1+exp(-gate_i))), gate_i/up_i dequantised as above.
  * = two GEMVs + dec_Swish (Modules/Swish.h:26-41) + dec_Gate_Layer_fp32xfp32 (Modules/Linear_Layer.h:1103-1121). */
@@ -306,7 +313,11 @@ int flexllm_mha_i8_prefill(const int8_t* q8, const int8_t* k_cache, const int8_t
  * is folded into the probabilities before they are quantised with the same symmetric quantiser:
  * p'[j] = softmax(a)[j] * V_s[j][kvh], s_p = max_j p'[j] / 127, P8 = round(p'/s_p) (int8, 0..127),
  * o[d] = float(sum_j P8[j]*v8[j][d]) * s_p, times v_ch_s[kvh][d] when the reference library's per-channel V scale
- * (Modules/MHA.h:713-738) is given.  K and V are read from the cache layouts of flexllm_kv_store_i8. */
+ * (Modules/MHA.h:713-738) is given.  K and V are read from the cache layouts of flexllm_kv_store_i8.
+ * PARITY: the q.K side (per-token scale streams) has a reference counterpart; the P.V side does not - the reference
+ * keeps V's scale static per channel and has no per-token V path, so folding V_s into the probabilities and the int8
+ * probabilities 0..127 are this library's own formulation: parity of that stage and of the output is unpinned by the
+ * reference (the CPU checker restates the same formulation; it is pinned against a float64 fake-quant golden only). */
 typedef struct {
     const float* q_s;      /* prefill: [s][q_heads]; decode: [q_heads]: the quantiser's scales of q */
     const float* k_s;      /* [max_pos][kv_heads]: K scale cache, one scale per position and KV head */
@@ -377,7 +388,9 @@ int flexllm_llama_create(flexllm_llama** out, const flexllm_llama_config* cfg, c
  * and the fp16 embedding table that turns a token id into the layer input; sum<p>[l] is the per-output-row sum of
  * the dequantised weights (the generated headers' w_<proj>_sum), which the activations' zero point multiplies; the
  * head is int4 [vocab][hidden] one value per byte with per-row scale and row sum.  The library packs the matrices two
- * values per byte.  Decoding (flexllm_llama_decode_hidden / _decode_greedy / _decode_sample) runs in the persistent
+ * values per byte for the decode kernel and keeps the byte-held copy for the prefill GEMMs (1.5 x the packed weight
+ * memory); a value outside -8..7 anywhere in the matrices or the head is refused with FLEXLLM_EINVAL, because the two
+ * copies would otherwise disagree (the packed one keeps the low nibble).  Decoding (flexllm_llama_decode_hidden / _decode_greedy / _decode_sample) runs in the persistent
  * kernel only, which then streams half the weight bytes per token.  flexllm_llama_prefill_hidden and
  * flexllm_llama_generate run the configuration's prefill graph (SpinQuant_Prefilling.h:807-1050): per-token asymmetric
  * uint4 quantisation, the 4-bit values multiplied one per byte on the int8 MFMA kernel with zero point x row sum in its

@@ -427,3 +427,30 @@ def test_stand_alone_scratch_is_per_stream(fx, oracle):
     tok_a = fx.ops.sample_topk_f32(cases[0][5], 5, 0.3, stream=streams[0])[0]
     tok_b = fx.ops.sample_topk_f32(cases[1][5], 5, 0.3, stream=streams[1])[0]
     assert tok_a == oracle.sample_topk(cases[0][5].numpy(), 5, 0.3, 8)[0] and tok_b == oracle.sample_topk(cases[1][5].numpy(), 5, 0.3, 8)[0]
+
+
+@pytest.mark.parametrize("k,n", [(2048, 2048), (4096, 512), (64, 37), (2048, 8192), (1024, 2)])
+def test_fused_quant_gemv_dequant_decode_linear(fx, oracle, k, n):
+    """flexllm_quant_linear_i8_gemv_dequant - the decode linear of BASELINE's first configuration in one launch (fp32
+    activation ~N(0,1) with outliers -> per-token int8 -> GEMV against uniform int8 weights -> dequantisation with
+    per-channel scales): quantised bytes, scale and outputs bit for bit against the oracle's chain and against the
+    two-kernel route on the device; a zero activation takes scale 1."""
+    r = np.random.default_rng(1000 + k + n)
+    x = outliers(r.standard_normal((1, k)).astype(np.float32))[0]
+    w = r.integers(-127, 128, (n, k)).astype(np.int8)
+    w_s = r.uniform(1e-3, 1e-2, n).astype(np.float32)
+    res = r.standard_normal(n).astype(np.float32)
+    dw, dws = fx.to_device(w), fx.to_device(w_s)
+    for xv in (x, np.zeros(k, np.float32)):
+        dx = fx.to_device(xv)
+        y, q, s = fx.ops.quant_linear_i8_gemv_dequant(dx, dw, dws, want_q=True)
+        q_ref, s_ref = oracle.quant_sym(xv[None, :])
+        assert np.array_equal(q.numpy(), q_ref[0]) and np.array_equal(s.numpy(), s_ref.reshape(1))
+        y_ref = oracle.dequant(oracle.linear_i8(q_ref, w), s_ref, w_s)[0]
+        assert np.array_equal(y.numpy(), y_ref)
+        y_res = fx.ops.quant_linear_i8_gemv_dequant(dx, dw, dws, residual=fx.to_device(res))
+        assert np.array_equal(y_res.numpy(), oracle.residual(y_ref, res))
+        q2, s2 = fx.ops.quant_sym_i8(fx.to_device(xv[None, :]))
+        y2 = fx.ops.linear_i8_gemv_dequant(q2.view(0, (k,)), s2, dw, dws)
+        assert np.array_equal(y.numpy(), y2.numpy())
+    assert float(s.numpy()[0]) == 1.0 and not y.numpy().any()
