@@ -431,7 +431,7 @@ def test_stand_alone_scratch_is_per_stream(fx, oracle):
 
 @pytest.mark.parametrize("k,n", [(2048, 2048), (4096, 512), (64, 37), (2048, 8192), (1024, 2)])
 def test_fused_quant_gemv_dequant_decode_linear(fx, oracle, k, n):
-    """flexllm_quant_linear_i8_gemv_dequant - the decode linear of BASELINE's first configuration in one launch (fp32
+    """flexllm_quant_linear_i8_gemv_dequant - the benchmark's single decode linear (1 x 2048 against 2048 x 2048) in one launch (fp32
     activation ~N(0,1) with outliers -> per-token int8 -> GEMV against uniform int8 weights -> dequantisation with
     per-channel scales): quantised bytes, scale and outputs bit for bit against the oracle's chain and against the
     two-kernel route on the device; a zero activation takes scale 1."""
