@@ -380,6 +380,8 @@ def main():
     # own row always wins the tied head and the loop would feed the same id back for ever)
     dev_w = llama.synth_weights(cfg, seed=1, device=True, embed_range=0.03)
     model = llama.Llama(cfg, dev_w)
+    exchange_info = model.exchange_info()
+    exchange_info["near_us"], exchange_info["far_us"] = round(exchange_info["near_us"], 3), round(exchange_info["far_us"], 3)
     model.set_decode_mode(args.decode_mode)
     # cache pre-filled with seeded int8 values directly in cache layout, as the reference's decode harness does
     C_fill = lib.flexllm_rt_fill_i8
@@ -637,7 +639,10 @@ def main():
                    "layers": cfg["layers"], "context": pos_end, "device": fx.device.device_name()},
         "decode": {"bytes_per_token": int(bpt), "achieved_GBs": round(token_gbs, 1),
                    "hbm_frac": round(token_gbs / HBM_PEAK_GBS, 4), "event_ms_per_step": round(ev_ms / K, 5),
-                   "last_tokens": timed_tokens[-4:].tolist(), "distinct_tokens": int(len(set(timed_tokens.tolist())))},
+                   "last_tokens": timed_tokens[-4:].tolist(), "distinct_tokens": int(len(set(timed_tokens.tolist()))),
+                   # where the words that workgroups hand to each other live: one copy per I/O die when the
+                   # calibration at model creation could tell the dies' memory apart
+                   "exchange_memory": exchange_info},
         "prefill_ms_1024": None if prefill_ms is None else round(prefill_ms, 3),
         "prefill_ms_4096": None if prefill_ms_4096 is None else round(prefill_ms_4096, 3),
         "prefill_roofline": prefill_roof,

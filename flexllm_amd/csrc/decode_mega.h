@@ -59,9 +59,10 @@ constexpr int kMegaWG = 256;       // workgroups (persistent, one per CU)
 constexpr int kMegaT = 512;        // threads per workgroup
 constexpr int kMegaWaves = kMegaT / 64;
 constexpr int kMegaGroup = 32;     // workgroups per first-level barrier counter
-constexpr int kMegaFlagCopies = 8; // copies of each of the barrier's release flags, each on its own line: workgroup w polls copy w mod 8
-constexpr int kMegaFlagBase = 64 * (2 + kMegaWG / kMegaGroup);   // the flags follow the counters (in 32-bit words)
-constexpr int kMegaBarWords = kMegaFlagBase + 64 * kMegaFlagCopies * (kMegaWG / kMegaGroup);
+constexpr int kMegaGroups = kMegaWG / kMegaGroup;   // 8 first-level groups: workgroup w belongs to group w mod 8, the XCD it runs on
+constexpr int kMegaFlagCopies = 8; // copies of each of the barrier's release flags: workgroup w polls copy w mod 8
+constexpr int kMegaFlagBase = 64 * kMegaGroups;     // the flags follow the counters (in 32-bit words); flag (group g, copy r) at + 16 * (8 r + g)
+constexpr int kMegaBarWords = kMegaFlagBase + 16 * kMegaFlagCopies * kMegaGroups;   // per die: 6 KiB
 constexpr int kMegaSpinLimit = 1 << 20;   // polls of ~1 us each: a wait that has not ended after a second never will
 constexpr int kMegaErrPeriod = 64;         // a spinning thread looks at the error flag every so many polls
 constexpr int kMegaMaxSteps = 64;  // tokens per launch in greedy mode (bounds the run time of one launch)
@@ -84,13 +85,22 @@ struct MegaParams {
     // follows its write-through store) fetches it, the others hit in L2.
     float* h;
     float2* stats;                 // [q_heads][32] (one-kernel-per-stage path)
-    unsigned long long* qkv_tag;   // [H + 2*KV]: q/k/v projection outputs, each with the epoch in its high word
-    unsigned long long* stats_tag; // [q_heads][2][32]: chunk maxima, then chunk sums of exponentials, each with the epoch in its high word
-    unsigned long long* x_tag;     // [H]: the residual stream after a layer (down projection + residual), tagged with the layer's sequence number
-    unsigned long long* x2_tag;    // [H]: the residual stream after attention (o projection + residual), tagged likewise
-    int32_t* o_acc;                // [H]: attention accumulators (zero at launch, cleared again once read)
+    // The words that cross workgroups inside a launch live in 8 KiB blocks of one arena, every array once per I/O die:
+    // copy d is in memory attached to die d and is READ by the workgroups of that die's XCDs, while producers store
+    // into both copies (a hand-over through the other die's memory takes 0.2-0.7 us longer).  Byte k of
+    // xblk[d][k / 8] is the arena block that holds block k of die d's copy (kXb* below); when the placement of memory is
+    // not known both dies name the same blocks.  Tagged arrays start as 0xFF..FF, accumulators and the barrier as 0.
+    //   qkv    [H + 2 KV] tagged words = 3 blocks: q/k/v projection outputs, each with the layer pass's sequence number in its high word
+    //   stats  [q_heads][2][32] tagged words = 2 blocks of 16 heads: chunk maxima, then chunk sums of exponentials
+    //   x      [H] tagged words = 2 blocks: the residual stream after a layer (down projection + residual)
+    //   x2     [H] tagged words = 2 blocks: the residual stream after attention (o projection + residual)
+    //   o_acc  [H] int32 = 1 block: attention accumulators (zero at launch, cleared again once read).  One copy only (die 0's entry):
+    //          adding every part twice costs more than the reads across the dies (measured)
+    //   bar    1 block: grid barrier, see GridBarrier
+    char* xarena;
+    unsigned long long xblk[2][2];
+    unsigned die_mask;             // bit x = the I/O die of XCD x
     int* state;                    // [0] pos, [1] step, [2] barrier epoch base, [3] error flag, [4] layer sequence number base
-    unsigned* bar;                 // [0] flag, [64] top counter, [128+64g] group counters
     int* token;                    // current token id (device), used when x_in == NULL; greedy mode leaves the last token here
     int* tokens_out;               // greedy mode: generated ids are written to tokens_out[state[1] + step]; NULL otherwise
     int n_steps;                   // tokens per launch (> 1 only in greedy mode)
@@ -125,6 +135,14 @@ __device__ __forceinline__ void st_i(int* p, int v) { __hip_atomic_store(p, v, _
 // A float that carries the epoch it was written in: one 64-bit store, so a reader that sees the tag sees the value.
 __device__ __forceinline__ void st_tagged(unsigned long long* p, float v, unsigned tag) {
     __hip_atomic_store(p, ((unsigned long long)tag << 32) | (unsigned)__float_as_int(v), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+// Block k of die `die`'s copy of the exchange arrays (MegaParams::xblk): a few scalar operations when die and k are uniform.
+// The kernel keeps the table in scalars of its own, read from the arguments once and made opaque: values the compiler
+// knows to be kernel arguments are fetched again from memory wherever registers are short, a scalar load and a wait in
+// every phase.
+constexpr int kXbQkv = 0, kXbStats = 3, kXbX = 5, kXbX2 = 7, kXbOacc = 9, kXbBar = 10, kXbCount = 11;
+__device__ __forceinline__ char* xblock_of(char* base, unsigned long long w0, unsigned long long w1, int k) {
+    return base + (size_t)((unsigned)((k < 8 ? w0 : w1) >> (8 * (k & 7))) & 0xFFu) * 8192u;
 }
 __device__ __forceinline__ unsigned long long ld_u64(const unsigned long long* p) {
     return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -221,20 +239,26 @@ __device__ __forceinline__ LayerW ldc_layer(const LayerW* p) {
     return w;
 }
 
-// Grid barrier from device-scope relaxed atomics: workgroup w adds 1 to group counter w/32 (8 counters on
+// Grid barrier from device-scope relaxed atomics: workgroup w adds 1 to the counter of group w mod 8 (8 counters on
 // separate 256-byte lines, so at most 32 atomics serialise on one address) and the last arriver of a group publishes
 // the epoch in the group's release flag; wave 0 of every workgroup polls the eight flags, one lane each.  Every flag
-// exists in eight copies on eight lines and workgroup w polls copy w mod 8 of each: a store into a line that 256
-// workgroups are polling queues behind their loads at the memory side, behind 32 pollers it lands sooner.  One
-// atomic round trip and one store-to-poll hand-over from the last arrival to the release (a top-level counter between
-// the groups and one flag adds a second round trip: +4 us per token; 16 groups of 16 or 4 of 64: +2).  (Polling the
-// group counters directly costs more: 256 pollers then contend with the arriving atomics on the same lines.  So do
-// the group flags without copies, 16 of them in one polled line.)
+// exists in eight copies and workgroup w polls copy w mod 8 of each: a store into a line that 256 workgroups are
+// polling queues behind their loads at the memory side, behind 32 pollers it lands sooner.  One atomic round trip and
+// one store-to-poll hand-over from the last arrival to the release (a top-level counter between the groups and one
+// flag adds a second round trip: +4 us per token; 16 groups of 16 or 4 of 64: +2).  (Polling the group counters
+// directly costs more: 256 pollers then contend with the arriving atomics on the same lines.  A barrier without
+// atomics - every workgroup stores the epoch into a word of its own in each of the eight copies and polls all 256
+// words of its copy - costs more as well: +1 us per layer.)
+// Workgroups are dealt to the XCDs round-robin, so group g and the pollers of copy g are the 32 workgroups of XCD g:
+// its counter and its flag copies live in memory of that XCD's die (mem[die]).  Which block a word is in follows from
+// the static index and die_mask alone, never from where a workgroup really runs: writers and pollers always agree.
 struct GridBarrier {
-    unsigned* mem;                              // [128 + 64*g] group counters, [kMegaFlagBase + 64*(8g + r)] copy r of group g's release flag
+    unsigned* mem[2];                           // per die: [64 g] group counters, [kMegaFlagBase + 16 (8 r + g)] copy r of group g's release flag
+    unsigned die_mask;
     unsigned epoch;
     int* err;
     bool dead = false;                          // wave 0 only: a wait timed out or the error flag was seen; later waits return at once
+    __device__ __forceinline__ unsigned* block_of(int xcd) const { return ((die_mask >> xcd) & 1u) ? mem[1] : mem[0]; }
     // drain == false: the calling wave made no global store in this phase and may keep loads in flight
     __device__ __forceinline__ void arrive(bool drain = true) {
         if (drain) __builtin_amdgcn_s_waitcnt(0);          // this thread's stores have been acknowledged
@@ -242,21 +266,23 @@ struct GridBarrier {
         epoch++;
         if (threadIdx.x < 64) {
             bool last = false;
-            const int g = blockIdx.x / kMegaGroup;
+            const int g = blockIdx.x % kMegaGroups;
             if (threadIdx.x == 0) {
-                const unsigned old = __hip_atomic_fetch_add(&mem[128 + 64 * g], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                const unsigned old = __hip_atomic_fetch_add(&block_of(g)[64 * g], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                 last = old == epoch * kMegaGroup - 1;
             }
             if (__builtin_amdgcn_ballot_w64(last) != 0) {        // the group is complete: its flag, in all copies
-                for (int r = threadIdx.x; r < kMegaFlagCopies; r += 64)
-                    __hip_atomic_store(&mem[kMegaFlagBase + 64 * (g * kMegaFlagCopies + r)], epoch, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                const int r = threadIdx.x;
+                if (r < kMegaFlagCopies)
+                    __hip_atomic_store(&block_of(r)[kMegaFlagBase + 16 * (kMegaGroups * r + g)], epoch, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             }
         }
     }
     __device__ __forceinline__ void wait() {
         if (threadIdx.x < 64 && !dead) {
             // lane j polls group j's flag, in this workgroup's copy
-            const unsigned* flag = &mem[kMegaFlagBase + 64 * ((threadIdx.x % (kMegaWG / kMegaGroup)) * kMegaFlagCopies + blockIdx.x % kMegaFlagCopies)];
+            const int r = blockIdx.x % kMegaFlagCopies;
+            const unsigned* flag = &block_of(r)[kMegaFlagBase + 16 * (kMegaGroups * r + threadIdx.x % kMegaGroups)];
             int it = 0;
             for (;;) {
                 // signed distance so that the comparison survives counter wrap-around
@@ -498,13 +524,20 @@ __device__ __forceinline__ void decode_mega_body(const MegaParams& p) {
     const bool is_s = wave >= 4;                        // stream wave (see the file comment)
     const int sw = wave - 4;
     constexpr int H = 2048, KV = 512, QH = 32, KVH = 8, GROUP = 4;
+    char* xbase = p.xarena;
+    unsigned long long xw00 = p.xblk[0][0], xw01 = p.xblk[0][1], xw10 = p.xblk[1][0], xw11 = p.xblk[1][1];
+    asm volatile("" : "+s"(xbase), "+s"(xw00), "+s"(xw01), "+s"(xw10), "+s"(xw11));
+    struct XT {} xt;                                             // (tag for the two accessors below)
+    auto xblock = [&](XT, int die_, int k) -> char* { return xblock_of(xbase, die_ ? xw10 : xw00, die_ ? xw11 : xw01, k); };
+    auto xwords = [&](XT, int die_, int k) -> unsigned long long* { return reinterpret_cast<unsigned long long*>(xblock(xt, die_, k)); };
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");   // see MegaParams::h
     // The launch state was left by the previous launch (or a small kernel before this one).  It is read with coherent
     // loads: the compiler would otherwise fetch it through the scalar cache, whose requests do not queue behind the
     // invalidation above and could be served from a line of an earlier launch that survived in this XCD's L2.
     const int pos0 = ld_i(&p.state[0]);
     const int step_base = ld_i(&p.state[1]);
-    GridBarrier bar{p.bar, (unsigned)ld_i(&p.state[2]), &p.state[3]};
+    GridBarrier bar{{reinterpret_cast<unsigned*>(xblock(xt, 0, kXbBar)), reinterpret_cast<unsigned*>(xblock(xt, 1, kXbBar))}, p.die_mask,
+                    (unsigned)ld_i(&p.state[2]), &p.state[3]};
     const unsigned seq0 = (unsigned)ld_i(&p.state[4]);
     int stamp_i = 0;
     // 'thread 0 of workgroup 0' from scalars and the hardware lane id: no per-thread value has to stay live for it
@@ -547,6 +580,20 @@ __device__ __forceinline__ void decode_mega_body(const MegaParams& p) {
 
     // attention work item of this workgroup
     const int a_h = wg / 32, a_c = wg % 32;
+    // The die this workgroup really runs on: it only chooses which copy to READ, and both copies hold the same words.
+    int die;
+    {
+        unsigned xcc;
+        asm volatile("s_getreg_b32 %0, hwreg(HW_REG_XCC_ID)" : "=s"(xcc));
+        die = (int)((p.die_mask >> (xcc & 7u)) & 1u);
+    }
+    // this wave's 256 words of its die's copy, as poll_tagged4 addresses them (base + wave * 256)
+    auto my_copy = [&](int xb) -> const unsigned long long* { return xwords(xt, die, xb + (wave >> 2)) - (wave >> 2) * 1024; };
+    // the eight values of this workgroup go to both copies: threads 0..7 write copy 0, threads 8..15 copy 1
+    auto publish8 = [&](int xb, const float* v8, unsigned tag_) {
+        const int t_ = threadIdx.x;
+        if (t_ < 16) st_tagged(xwords(xt, t_ >> 3, xb + (wg >> 7)) + (wg & 127) * 8 + (t_ & 7), v8[t_ & 7], tag_);
+    };
     const bool a_active = a_c * kChunk < len && a_c * kChunk < p.max_pos;
     const bool a_owner = a_active && (pos / kChunk == a_c);       // this chunk holds the new token
     const int nchunks = (len + kChunk - 1) / kChunk;              // active chunks per head: the parts every accumulator receives
@@ -636,7 +683,7 @@ __device__ __forceinline__ void decode_mega_body(const MegaParams& p) {
             }
             const float4 gam = reinterpret_cast<const float4*>(g0)[t];
             float v[4];
-            if (l > 0) poll_tagged4(p.x_tag, tag - 1u, bar.err, L.f + (t >> 6) * 256, v);   // x of the previous layer, as it arrives
+            if (l > 0) poll_tagged4(my_copy(kXbX), tag - 1u, bar.err, L.f + (t >> 6) * 256, v);   // x of the previous layer, as it arrives
             stamp();
             if (l == 0) {
                 if (p.x_in) { const float4 q = reinterpret_cast<const float4*>(p.x_in)[t]; v[0] = q.x; v[1] = q.y; v[2] = q.z; v[3] = q.w; }
@@ -660,7 +707,7 @@ __device__ __forceinline__ void decode_mega_body(const MegaParams& p) {
                     } else {
                         out = (float)mega_dot_row<2>(wr[j], L.xq, lane) * sx * wsc[j];
                     }
-                    if (lane == 0) st_tagged(&p.qkv_tag[r], out, tag);
+                    if (lane < 2) st_tagged(xwords(xt, lane, kXbQkv + (r >> 10)) + (r & 1023), out, tag);   // lane 0 -> copy 0, lane 1 -> copy 1
                 }
             }
             stamp();
@@ -693,7 +740,8 @@ __device__ __forceinline__ void decode_mega_body(const MegaParams& p) {
                 if (t < 128) {                                        // q: 4 heads x 32 pairs
                     const int g = t >> 5, k = t & 31, qh = a_h * GROUP + g;
                     float t0, t1;
-                    poll_tagged2(&p.qkv_tag[qh * kHd + k], &p.qkv_tag[qh * kHd + k + 32], tag, bar.err, t0, t1);
+                    const unsigned long long* src = xwords(xt, die, kXbQkv + (a_h >> 2)) + (qh * kHd & 1023) + k;   // 16 heads per block
+                    poll_tagged2(src, src + 32, tag, bar.err, t0, t1);
                     const float o0 = t0 * cs[k] - t1 * sn[k], o1 = t0 * sn[k] + t1 * cs[k];
                     const float div = 8.0f * (g == 0 ? qs4[0] : g == 1 ? qs4[1] : g == 2 ? qs4[2] : qs4[3]);
                     L.q8[g][k] = (int8_t)static_q8(o0, div);
@@ -701,7 +749,8 @@ __device__ __forceinline__ void decode_mega_body(const MegaParams& p) {
                 } else if (t < 160) {                                 // k of the new token: 32 pairs
                     const int k = t - 128;
                     float t0, t1;
-                    poll_tagged2(&p.qkv_tag[H + a_h * kHd + k], &p.qkv_tag[H + a_h * kHd + k + 32], tag, bar.err, t0, t1);
+                    const unsigned long long* src = xwords(xt, die, kXbQkv + 2) + a_h * kHd + k;       // block 2: k, then v
+                    poll_tagged2(src, src + 32, tag, bar.err, t0, t1);
                     const float o0 = t0 * cs[k] - t1 * sn[k], o1 = t0 * sn[k] + t1 * cs[k];
                     const float div = 1.0f * ks1;
                     const int8_t b0 = (int8_t)static_q8(o0, div), b1 = (int8_t)static_q8(o1, div);
@@ -709,7 +758,7 @@ __device__ __forceinline__ void decode_mega_body(const MegaParams& p) {
                     if (a_owner) { int8_t* dst = kc + k_index(a_h, pos, p.max_pos); dst[k] = b0; dst[k + 32] = b1; }
                 } else if (t >= 192 && t < 256) {                     // v of the new token: a wave of its own (two polls in
                     const int d = t - 192;                            // one wave would run one after the other)
-                    const float tv = poll_tagged1(&p.qkv_tag[H + KV + a_h * kHd + d], tag, bar.err);
+                    const float tv = poll_tagged1(xwords(xt, die, kXbQkv + 2) + KV + a_h * kHd + d, tag, bar.err);
                     const int8_t b = (int8_t)static_q8(tv, 1.0f * vs1);
                     L.vnew[d] = b;
                     if (a_owner) vc[v_index(a_h, pos, d, p.max_pos)] = b;
@@ -734,8 +783,8 @@ __device__ __forceinline__ void decode_mega_body(const MegaParams& p) {
                     const float m = wave_max(fmaxf(s0, s1));
                     float sum = (a_c * kChunk + lane < len ? exp_f(s0 - m) : 0.0f) + (a_c * kChunk + lane + 64 < len ? exp_f(s1 - m) : 0.0f);
                     sum = wave_sum(sum);
-                    if (lane == 0) {
-                        unsigned long long* slot = p.stats_tag + (size_t)(a_h * GROUP + wave) * 64 + a_c;
+                    if (lane < 2) {                                   // lane 0 -> copy 0, lane 1 -> copy 1
+                        unsigned long long* slot = xwords(xt, lane, kXbStats + (a_h >> 2)) + (size_t)((a_h & 3) * GROUP + wave) * 64 + a_c;
                         st_tagged(slot, m, tag);
                         st_tagged(slot + 32, sum, tag);
                     }
@@ -758,7 +807,7 @@ __device__ __forceinline__ void decode_mega_body(const MegaParams& p) {
                     float m_c = -1e32f, l_c = 0.0f;
                     {
                         // the maxima of a head's 32 chunks are consecutive words, then its sums: a poll is two loads of whole lines
-                        const unsigned long long* slot = p.stats_tag + (size_t)(a_h * GROUP + wave) * 64 + min(lane, nchunks - 1);
+                        const unsigned long long* slot = xwords(xt, die, kXbStats + (a_h >> 2)) + (size_t)((a_h & 3) * GROUP + wave) * 64 + min(lane, nchunks - 1);
                         unsigned long long w0 = 0, w1 = 0;
                         int it = 0;
                         for (;;) {
@@ -816,8 +865,8 @@ __device__ __forceinline__ void decode_mega_body(const MegaParams& p) {
                         // so that they do not all queue on the same 64-byte run at once
                         const int g = (i + a_c) & (GROUP - 1);
                         const int mine = g == 0 ? tot[0] : g == 1 ? tot[1] : g == 2 ? tot[2] : tot[3];
-                        __hip_atomic_fetch_add(&p.o_acc[(a_h * GROUP + g) * kHd + d], mine + L.osum[g][d], __ATOMIC_RELAXED,
-                                               __HIP_MEMORY_SCOPE_AGENT);
+                        __hip_atomic_fetch_add(reinterpret_cast<int*>(xblock(xt, 0, kXbOacc)) + (a_h * GROUP + g) * kHd + d, mine + L.osum[g][d],
+                                               __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                     }
                 }
             } else {
@@ -854,7 +903,7 @@ __device__ __forceinline__ void decode_mega_body(const MegaParams& p) {
             stamp();
 #pragma unroll
             for (int i = 0; i < 2; i++) {
-                const unsigned long long w2 = ld_u64(reinterpret_cast<const unsigned long long*>(p.o_acc + 4 * t + 2 * i));
+                const unsigned long long w2 = ld_u64(reinterpret_cast<const unsigned long long*>(reinterpret_cast<const int*>(xblock(xt, 0, kXbOacc)) + 4 * t + 2 * i));
                 v[2 * i] = (float)(int)(unsigned)w2 * osa * osv;
                 v[2 * i + 1] = (float)(int)(unsigned)(w2 >> 32) * osa * osv;
             }
@@ -888,7 +937,7 @@ __device__ __forceinline__ void decode_mega_body(const MegaParams& p) {
             // the workgroup's eight outputs leave as one 32-byte store: eight single-lane stores from four waves into
             // the same sector take longer to be acknowledged, and the barrier waits for that
             __syncthreads();
-            if (t < 8) st_tagged(&p.x2_tag[wg * 8 + t], L.res8[t], tag);
+            publish8(kXbX2, L.res8, tag);
             stamp();
             // no grid barrier: the consumers poll the tagged words
         }
@@ -910,7 +959,7 @@ __device__ __forceinline__ void decode_mega_body(const MegaParams& p) {
             }
             const float4 gam = reinterpret_cast<const float4*>(g1)[t];
             float v[4];
-            poll_tagged4(p.x2_tag, tag, bar.err, L.f + (t >> 6) * 256, v);
+            poll_tagged4(my_copy(kXbX2), tag, bar.err, L.f + (t >> 6) * 256, v);
             stamp();
             auto down_row_0 = [&]() {
                 // Runs after the first workgroup barrier of the reduction below, i.e. once ALL eight waves have their
@@ -919,7 +968,7 @@ __device__ __forceinline__ void decode_mega_body(const MegaParams& p) {
                 // producers: clearing right behind it wiped accumulators that a slower workgroup had yet to read.)
                 // The next parts are added a layer later, by workgroups that have polled this workgroup's x, which
                 // the same threads store after this store has been acknowledged.
-                if (t < 8) st_i(&p.o_acc[wg * 8 + t], 0);
+                if (t < 8) st_i(reinterpret_cast<int*>(xblock(xt, 0, kXbOacc)) + wg * 8 + t, 0);
                 __builtin_amdgcn_s_waitcnt(0x0F70);                   // vmcnt(0): see gu_slice
                 if (is_s) {
                     if constexpr (W4) mega_row4_to_lds(w.wd, wg * 8 + sw * 2, lane, L.wd[sw * 2]);
@@ -1155,10 +1204,10 @@ __device__ __forceinline__ void decode_mega_body(const MegaParams& p) {
                 if (lane == 0) L.res8[drow - wg * 8] = (float)a0 * sx * dsc + xres;
             }
             __syncthreads();
-            if (t < 8) {
+            if (t < 16) {
                 __builtin_amdgcn_s_waitcnt(0x0F70);                  // vmcnt(0): the accumulator reset of phase 5 has landed
-                st_tagged(&p.x_tag[wg * 8 + t], L.res8[t], tag);     // one 64-byte store, as in phase 4
-                if (l == p.n_layers - 1) st_f(&p.x[wg * 8 + t], L.res8[t]);   // the hidden state the host reads back
+                publish8(kXbX, L.res8, tag);                      // one 64-byte store per copy, as in phase 4
+                if (t < 8 && l == p.n_layers - 1) st_f(&p.x[wg * 8 + t], L.res8[t]);   // the hidden state the host reads back
             }
             if (l == 1) fine();
             if (l == 1) fine();
@@ -1196,7 +1245,7 @@ __device__ __forceinline__ void decode_mega_body(const MegaParams& p) {
             };
             load_group(r);
             float v[4];
-            poll_tagged4(p.x_tag, seq0 + (unsigned)((step + 1) * p.n_layers), bar.err, L.f + (t >> 6) * 256, v);
+            poll_tagged4(my_copy(kXbX), seq0 + (unsigned)((step + 1) * p.n_layers), bar.err, L.f + (t >> 6) * 256, v);
             stamp();
             const float4 g = reinterpret_cast<const float4*>(p.gamma + (size_t)(2 * p.n_layers) * H)[t];
             const float2 sb = norm_quant_2048_u4(v, g, true, p.eps, L, NoHook());
@@ -1228,7 +1277,7 @@ __device__ __forceinline__ void decode_mega_body(const MegaParams& p) {
         };
         load_group(r);
         float v[4];
-        poll_tagged4(p.x_tag, seq0 + (unsigned)((step + 1) * p.n_layers), bar.err, L.f + (t >> 6) * 256, v);
+        poll_tagged4(my_copy(kXbX), seq0 + (unsigned)((step + 1) * p.n_layers), bar.err, L.f + (t >> 6) * 256, v);
         stamp();
         float ss = (v[0] * v[0] + v[1] * v[1]) + (v[2] * v[2] + v[3] * v[3]);
         ss = block_sum<kMegaWaves>(ss, L.red);

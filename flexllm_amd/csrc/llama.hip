@@ -11,6 +11,7 @@
 #include "gemv_i8.h"
 #include "logits_kernels.h"
 #include "decode_mega.h"
+#include "die_arena.h"
 #include "prefill.h"
 #include <atomic>
 #include <vector>
@@ -30,10 +31,11 @@ struct flexllm_llama {
     float* xs = nullptr;
     float* scores = nullptr;
     float2* stats = nullptr;
-    unsigned long long* qkv_tag = nullptr;     // persistent kernel: q/k/v outputs tagged with the barrier epoch
-    unsigned long long* stats_tag = nullptr;   // persistent kernel: chunk statistics tagged with the layer sequence number
-    int32_t* o_mega = nullptr;                 // persistent kernel: its own attention accumulators (zero whenever it is not running)
-    unsigned long long *x_tag = nullptr, *x2_tag = nullptr;   // persistent kernel: the residual stream after a layer / after attention, tagged likewise
+    // Persistent kernel: the words its workgroups hand to each other, one copy per I/O die, in 8 KiB blocks of `arena`
+    // ([die][block]; see die_arena.h).  Tagged arrays start as 0xFF..FF (never a live tag), accumulators and barrier as 0.
+    fx::DieArena arena;
+    unsigned long long xblk[2][2] = {};        // MegaParams::xblk: which arena block holds block k of die d's copy
+    void* xptr[2][fx::kXbCount] = {};          // the same as pointers (host-side resets)
     int32_t* o_acc = nullptr;
     int* state = nullptr;           // [0] position of the token being processed, [1] step index
     float* am_v = nullptr;
@@ -56,7 +58,6 @@ struct flexllm_llama {
     fx::LayerW4* layers4_dev = nullptr;
     uint8_t* head_w4 = nullptr;
     float *head_s = nullptr, *head_sum = nullptr;
-    unsigned* bar = nullptr;            // grid-barrier counters of the persistent kernel
     bool mega_ok = false;               // shapes match the persistent kernel's compile-time constants
     int decode_mode = 0;                // 0: persistent kernel when possible, 1: one kernel per stage
     long long* timeline = nullptr;      // stage stamps of the persistent kernel (debug aid)
@@ -190,7 +191,11 @@ static int launch_mega(flexllm_llama* m, int* token, const float* x_in, float* l
     p.embed = reinterpret_cast<const __half*>(m->embed);
     p.k_cache = m->k_cache; p.v_cache = m->v_cache; p.cache_layer_bytes = m->cache_layer_bytes;
     p.x = m->x; p.x2 = m->x2; p.qkv = m->qkv; p.h = m->h; p.logits = logits ? logits : m->logits;
-    p.stats = m->stats; p.stats_tag = m->stats_tag; p.qkv_tag = m->qkv_tag; p.x_tag = m->x_tag; p.x2_tag = m->x2_tag; p.o_acc = m->o_mega; p.state = m->state; p.bar = m->bar;
+    p.stats = m->stats; p.state = m->state;
+    p.xarena = m->arena.base;
+    for (int d = 0; d < 2; d++)
+        for (int i = 0; i < 2; i++) p.xblk[d][i] = m->xblk[d][i];
+    p.die_mask = m->arena.die_mask;
     p.token = token; p.tokens_out = tokens_out; p.n_steps = steps; p.x_in = x_in; p.am_v = m->am_v; p.am_i = m->am_i;
     p.n_layers = c.layers; p.max_pos = c.max_pos; p.vocab = c.vocab; p.want_head = want_head;
     p.top_k = top_k; p.rands = rands; p.cand_v = m->topk_val; p.cand_i = m->topk_idx;
@@ -326,16 +331,25 @@ int flexllm_llama_create(flexllm_llama** out, const flexllm_llama_config* cfg, c
     FX_TRY(dev_alloc(m, (void**)&m->scores, sizeof(float) * (size_t)c.q_heads * c.max_pos));
     FX_TRY(dev_alloc(m, (void**)&m->stats, sizeof(float2) * (size_t)c.q_heads * kMaxChunks));
     FX_TRY(dev_alloc(m, (void**)&m->o_acc, sizeof(int32_t) * H));
-    FX_TRY(dev_alloc(m, (void**)&m->qkv_tag, sizeof(unsigned long long) * (size_t)(H + 2 * KV)));
-    FX_TRY_HIP(hipMemset(m->qkv_tag, 0xFF, sizeof(unsigned long long) * (size_t)(H + 2 * KV)));   // tag 0xFFFFFFFF: never a live epoch (the first is 0)
-    FX_TRY(dev_alloc(m, (void**)&m->stats_tag, sizeof(unsigned long long) * 2 * (size_t)c.q_heads * kMaxChunks));
-    FX_TRY_HIP(hipMemset(m->stats_tag, 0xFF, sizeof(unsigned long long) * 2 * (size_t)c.q_heads * kMaxChunks));
-    FX_TRY(dev_alloc(m, (void**)&m->x_tag, sizeof(unsigned long long) * (size_t)H));
-    FX_TRY_HIP(hipMemset(m->x_tag, 0xFF, sizeof(unsigned long long) * (size_t)H));
-    FX_TRY(dev_alloc(m, (void**)&m->x2_tag, sizeof(unsigned long long) * (size_t)H));
-    FX_TRY_HIP(hipMemset(m->x2_tag, 0xFF, sizeof(unsigned long long) * (size_t)H));
-    FX_TRY(dev_alloc(m, (void**)&m->o_mega, sizeof(int32_t) * (size_t)H));
-    FX_TRY_HIP(hipMemset(m->o_mega, 0, sizeof(int32_t) * (size_t)H));
+    {
+        // the exchange words of the persistent kernel: 11 blocks per die (FLEXLLM_DIE_COPIES=0: one copy, no calibration)
+        const char* e = getenv("FLEXLLM_DIE_COPIES");
+        void* raw = nullptr;
+        const int rc_arena = die_arena_create(m->arena, 48, !(e && atoi(e) == 0), &raw);
+        if (raw) m->owned.push_back(raw);
+        FX_TRY(rc_arena);
+        static_assert(sizeof(unsigned long long) * 1024 == kDieBlock && sizeof(int32_t) * 2048 == kDieBlock && sizeof(unsigned) * kMegaBarWords <= kDieBlock,
+                      "the exchange arrays are cut into 8 KiB blocks");
+        for (int k = 0; k < kXbCount; k++) {
+            void* pr[2];
+            if (!m->arena.take_pair(pr, k < kXbOacc ? 0xFF : 0)) { set_error("llama_create: the exchange arena is used up"); return fail(FLEXLLM_EHIP); }
+            for (int d = 0; d < 2; d++) {
+                m->xptr[d][k] = pr[d];
+                const unsigned long long idx = (unsigned long long)((static_cast<char*>(pr[d]) - m->arena.base) / kDieBlock);
+                m->xblk[d][k / 8] |= idx << (8 * (k % 8));
+            }
+        }
+    }
     FX_TRY(dev_alloc(m, (void**)&m->state, sizeof(int) * 8));
     FX_TRY(dev_alloc(m, (void**)&m->am_v, sizeof(float) * kArgmaxParts));
     // per-workgroup sampling candidates: of the persistent kernel's workgroups or of the stand-alone first stage
@@ -345,8 +359,6 @@ int flexllm_llama_create(flexllm_llama** out, const flexllm_llama_config* cfg, c
     FX_TRY(dev_alloc(m, (void**)&m->am_i, sizeof(int) * kArgmaxParts));
     FX_TRY(dev_alloc(m, (void**)&m->layers_dev, sizeof(LayerW) * L));
     FX_TRY_HIP(hipMemcpy(m->layers_dev, m->layers.data(), sizeof(LayerW) * L, hipMemcpyHostToDevice));
-    FX_TRY(dev_alloc(m, (void**)&m->bar, sizeof(unsigned) * kMegaBarWords));
-    FX_TRY_HIP(hipMemset(m->bar, 0, sizeof(unsigned) * kMegaBarWords));
     FX_TRY_HIP(hipMemset(m->state, 0, sizeof(int) * 8));
     FX_TRY_HIP(hipMemset(m->o_acc, 0, sizeof(int32_t) * H));
     FX_TRY_HIP(hipMemset(m->am_v, 0, sizeof(float) * kArgmaxParts));
@@ -482,6 +494,15 @@ int flexllm_llama_set_decode_mode(flexllm_llama* m, int mode) {
     return FLEXLLM_OK;
 }
 
+int flexllm_llama_exchange_info(const flexllm_llama* m, int* two_copies, unsigned* die_mask, float* near_us, float* far_us) {
+    FX_REQUIRE(m && two_copies && die_mask && near_us && far_us, "llama_exchange_info: null pointer");
+    *two_copies = m->arena.calibrated ? 1 : 0;
+    *die_mask = m->arena.die_mask;
+    *near_us = m->arena.near_us;
+    *far_us = m->arena.far_us;
+    return FLEXLLM_OK;
+}
+
 int flexllm_llama_stage_timeline(flexllm_llama* m, long long* host_out, int max_entries) {
     FX_REQUIRE(m && host_out && max_entries > 0, "llama_stage_timeline: bad arguments");
     // stage stamps, fine stamps, per-workgroup entry and exit, one layer's stamps of every workgroup (debug builds)
@@ -511,9 +532,9 @@ int flexllm_llama_check(flexllm_llama* m) {
             return FLEXLLM_EINVAL;
         }
         // after a time-out the barrier counters and the attention accumulators hold partial counts: start them afresh
-        (void)hipMemset(m->bar, 0, sizeof(unsigned) * kMegaBarWords);
+        for (int d = 0; d < 2; d++) (void)hipMemset(m->xptr[d][kXbBar], 0, kDieBlock);
         (void)hipMemset(&m->state[2], 0, sizeof(int));
-        (void)hipMemset(m->o_mega, 0, sizeof(int32_t) * (size_t)m->cfg.hidden);
+        for (int d = 0; d < 2; d++) (void)hipMemset(m->xptr[d][kXbOacc], 0, kDieBlock);
         set_error("persistent decode kernel: a wait timed out (were all %d workgroups resident?)", kMegaWG);
         return FLEXLLM_EHIP;
     }

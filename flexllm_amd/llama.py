@@ -204,6 +204,14 @@ class Llama:
         """0: persistent one-kernel-per-token schedule (default), 1: one kernel per stage."""
         check(lib().flexllm_llama_set_decode_mode(self.handle, int(mode)))
 
+    def exchange_info(self):
+        """How the persistent decode kernel's exchange memory was placed at creation: {"two_copies": bool (one copy of
+        every exchanged array per I/O die, each in that die's memory), "die_mask": int (bit x = die of XCD x),
+        "near_us", "far_us": measured exchange round through own-die / other-die memory}."""
+        two, mask, near, far = C.c_int(0), C.c_uint(0), C.c_float(0.0), C.c_float(0.0)
+        check(lib().flexllm_llama_exchange_info(self.handle, C.byref(two), C.byref(mask), C.byref(near), C.byref(far)))
+        return {"two_copies": bool(two.value), "die_mask": int(mask.value), "near_us": float(near.value), "far_us": float(far.value)}
+
     def check(self):
         """Synchronise and raise if the persistent decode kernel reported a barrier time-out."""
         check(lib().flexllm_llama_check(self.handle))

@@ -413,6 +413,18 @@ int flexllm_llama_set_decode_mode(flexllm_llama* m, int mode);
  * stamps of the last persistent decode step: per layer 6 x (stage start after the barrier, stage end before the
  * next arrive), then the head's start and end. */
 int flexllm_llama_stage_timeline(flexllm_llama* m, long long* host_out, int max_entries);
+/* How the persistent decode kernel's exchange memory was placed when the model was created (no counterpart in the
+ * reference).  The GPU is two I/O dies with four XCDs and half of the HBM each; a word handed from one workgroup to
+ * another through memory of the other die takes longer, and memory alternates between the dies in 8 KiB blocks.
+ * flexllm_llama_create measures which die each block of a small arena belongs to (about 10 ms) and keeps every
+ * exchanged array once per die: producers store into both copies, consumers poll their own die's.
+ *   *two_copies  1 when the measurement succeeded; 0 when the arrays exist once (fewer than 256 CUs, workgroups not
+ *                dealt round-robin to eight XCDs, no clear difference between the blocks, or FLEXLLM_DIE_COPIES=0
+ *                in the environment when the model was created).  Results are the same either way.
+ *   *die_mask    bit x = the die of XCD x
+ *   *near_us, *far_us   mean time of one exchange round among the 32 workgroups of an XCD through memory of their
+ *                own die / of the other die, as measured (0 when two_copies is 0) */
+int flexllm_llama_exchange_info(const flexllm_llama* m, int* two_copies, unsigned* die_mask, float* near_us, float* far_us);
 /* Synchronises the device and reports what a decode run flagged on the device: a grid barrier of the persistent
  * kernel that timed out (FLEXLLM_EHIP), or an input token id outside the vocabulary (FLEXLLM_EINVAL; token 0 was
  * used in its place, no row outside the embedding table is ever read).  Clears the flag. */

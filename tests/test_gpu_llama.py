@@ -296,3 +296,31 @@ def test_generate_with_sampling():
     _, idx0, _, _ = oracle.sample_topk(logits0, k, float(rands[0]), 8)
     assert got[0] in idx0.tolist()
     model.close()
+
+
+def test_exchange_memory_per_die_changes_no_bit(monkeypatch):
+    """The persistent kernel keeps the words its workgroups hand to each other once per I/O die, in memory that a
+    calibration at creation found attached to that die; with FLEXLLM_DIE_COPIES=0 they exist once.  Placement is a
+    matter of speed only: tokens, hidden state and caches of a 40-token greedy run are identical bit for bit."""
+    import flexllm_amd as fx
+    from flexllm_amd import llama
+    cfg = llama.make_config(layers=3, vocab=4096, max_pos=256)
+    dev_w = llama.synth_weights(cfg, seed=5, device=True)
+    runs = []
+    for copies in ("1", "0"):
+        monkeypatch.setenv("FLEXLLM_DIE_COPIES", copies)
+        model = llama.Llama(cfg, dev_w)
+        info = model.exchange_info()
+        print("FLEXLLM_DIE_COPIES=%s:" % copies, info, flush=True)
+        if copies == "0":
+            assert not info["two_copies"]
+        elif info["two_copies"]:                     # the measurement found two dies of four XCDs
+            assert bin(info["die_mask"]).count("1") == 4 and not info["die_mask"] & 1
+            assert 0.0 < info["near_us"] < info["far_us"]
+        tok = fx.to_device(np.array([77], np.int32)); out = fx.zeros((40,), np.int32)
+        model.decode_greedy(tok, 0, 40, out, use_graph=False)
+        model.check()
+        runs.append((out.numpy().copy(), model.k_cache.numpy().copy(), model.v_cache.numpy().copy()))
+        model.close()
+    assert np.array_equal(runs[0][0], runs[1][0])
+    assert np.array_equal(runs[0][1], runs[1][1]) and np.array_equal(runs[0][2], runs[1][2])
