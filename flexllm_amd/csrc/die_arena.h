@@ -55,6 +55,43 @@ static __global__ __launch_bounds__(64) void die_probe_kernel(unsigned long long
     if (lane == 0) out[wg] = wall_clock64() - t0;
 }
 
+// Pure host arithmetic of the calibration.  us[b * 8 + x] = exchange round of XCD x's workgroups through block b.
+// XCDs of one die see the same blocks as near, so the sign of the correlation with XCD 0 over the blocks splits them
+// into the two dies (*die_mask: bit x = die of XCD x, XCD 0 on die 0); a block belongs to the die whose four XCDs are at
+// least 4 % faster on average (die_of_block[b] = 0 or 1), otherwise to none (-1).  Returns false - no usable picture -
+// unless each die has exactly four XCDs and at least four blocks.
+static bool die_classify(const float* us, int n_blocks, unsigned* die_mask, int* die_of_block, float* near_us, float* far_us) {
+    if (n_blocks < 8) return false;
+    double mean[8] = {0};
+    for (int b = 0; b < n_blocks; b++)
+        for (int x = 0; x < 8; x++) mean[x] += us[(size_t)b * 8 + x] / n_blocks;
+    unsigned mask = 0;
+    int on_die1 = 0;
+    for (int x = 1; x < 8; x++) {
+        double c = 0.0;
+        for (int b = 0; b < n_blocks; b++) c += (us[(size_t)b * 8] - mean[0]) * (us[(size_t)b * 8 + x] - mean[x]);
+        if (c < 0.0) { mask |= 1u << x; on_die1++; }
+    }
+    if (on_die1 != 4) return false;
+    double near_sum = 0.0, far_sum = 0.0;
+    int count[2] = {0, 0};
+    for (int b = 0; b < n_blocks; b++) {
+        double s[2] = {0.0, 0.0};
+        for (int x = 0; x < 8; x++) s[(mask >> x) & 1] += us[(size_t)b * 8 + x] / 4.0;
+        const int die = s[0] < s[1] ? 0 : 1;
+        if (!(s[1 - die] >= 1.04 * s[die])) { die_of_block[b] = -1; continue; }     // no clear difference (or not a number)
+        die_of_block[b] = die;
+        count[die]++;
+        near_sum += s[die];
+        far_sum += s[1 - die];
+    }
+    if (count[0] < 4 || count[1] < 4) return false;
+    *die_mask = mask;
+    *near_us = (float)(near_sum / (count[0] + count[1]));
+    *far_us = (float)(far_sum / (count[0] + count[1]));
+    return true;
+}
+
 struct DieArena {
     char* base = nullptr;                  // 8 KiB aligned
     int n_blocks = 0;
@@ -128,37 +165,12 @@ static int die_arena_create(DieArena& a, int n_blocks, bool want_calibration, vo
             float& slot = t[(size_t)b * 8 + w % 8];
             slot = us > slot ? us : slot;
         }
-    // XCDs of one die see the same blocks as near: the sign of the correlation with XCD 0 over the blocks
-    float mean[8] = {0};
-    for (int b = 0; b < n_blocks; b++)
-        for (int x = 0; x < 8; x++) mean[x] += t[(size_t)b * 8 + x] / n_blocks;
+    std::vector<int> die_of(n_blocks);
     unsigned mask = 0;
-    int on_die1 = 0;
-    for (int x = 1; x < 8; x++) {
-        float c = 0.0f;
-        for (int b = 0; b < n_blocks; b++) c += (t[(size_t)b * 8] - mean[0]) * (t[(size_t)b * 8 + x] - mean[x]);
-        if (c < 0.0f) { mask |= 1u << x; on_die1++; }
-    }
-    if (on_die1 != 4) return FLEXLLM_OK;                            // not two dies of four XCDs: single copy
-    std::vector<int> blocks[2];
-    double near_sum = 0.0, far_sum = 0.0;
-    int classified = 0;
-    for (int b = 0; b < n_blocks; b++) {
-        float s[2] = {0.0f, 0.0f};
-        for (int x = 0; x < 8; x++) s[(mask >> x) & 1] += t[(size_t)b * 8 + x] / 4.0f;
-        const int die = s[0] < s[1] ? 0 : 1;
-        if (s[1 - die] < 1.04f * s[die]) continue;                  // no clear difference: leave the block unused
-        blocks[die].push_back(b);
-        near_sum += s[die];
-        far_sum += s[1 - die];
-        classified++;
-    }
-    if (blocks[0].size() < 4 || blocks[1].size() < 4) return FLEXLLM_OK;
-    a.blocks[0] = blocks[0];
-    a.blocks[1] = blocks[1];
+    if (!die_classify(t.data(), n_blocks, &mask, die_of.data(), &a.near_us, &a.far_us)) return FLEXLLM_OK;   // no clear picture: single copy
+    for (int b = 0; b < n_blocks; b++)
+        if (die_of[b] >= 0) a.blocks[die_of[b]].push_back(b);
     a.die_mask = mask;
-    a.near_us = (float)(near_sum / classified);
-    a.far_us = (float)(far_sum / classified);
     a.calibrated = true;
     return FLEXLLM_OK;
 }

@@ -494,6 +494,14 @@ int flexllm_llama_set_decode_mode(flexllm_llama* m, int mode) {
     return FLEXLLM_OK;
 }
 
+int flexllm_die_classify(const float* us, int n_blocks, int* usable, unsigned* die_mask, int* die_of_block, float* near_us, float* far_us) {
+    FX_REQUIRE(us && usable && die_mask && die_of_block && near_us && far_us && n_blocks > 0, "die_classify: bad arguments");
+    *die_mask = 0; *near_us = 0.0f; *far_us = 0.0f;
+    for (int b = 0; b < n_blocks; b++) die_of_block[b] = -1;
+    *usable = die_classify(us, n_blocks, die_mask, die_of_block, near_us, far_us) ? 1 : 0;
+    return FLEXLLM_OK;
+}
+
 int flexllm_llama_exchange_info(const flexllm_llama* m, int* two_copies, unsigned* die_mask, float* near_us, float* far_us) {
     FX_REQUIRE(m && two_copies && die_mask && near_us && far_us, "llama_exchange_info: null pointer");
     *two_copies = m->arena.calibrated ? 1 : 0;

@@ -425,6 +425,12 @@ int flexllm_llama_stage_timeline(flexllm_llama* m, long long* host_out, int max_
  *   *near_us, *far_us   mean time of one exchange round among the 32 workgroups of an XCD through memory of their
  *                own die / of the other die, as measured (0 when two_copies is 0) */
 int flexllm_llama_exchange_info(const flexllm_llama* m, int* two_copies, unsigned* die_mask, float* near_us, float* far_us);
+/* The arithmetic of that measurement, on the host alone (no GPU needed; exported so that it can be checked on made-up
+ * timings).  us[b * 8 + x] = exchange round of XCD x's workgroups through block b, microseconds.  XCDs whose timings
+ * correlate with XCD 0's over the blocks are die 0 (*die_mask: bit x = die of XCD x); die_of_block[b] = the die whose
+ * four XCDs are at least 4 % faster through block b, or -1.  *usable = 0 - and the library would keep one copy - unless
+ * each die has four XCDs and at least four blocks; *near_us / *far_us = mean round through own-die / other-die blocks. */
+int flexllm_die_classify(const float* us, int n_blocks, int* usable, unsigned* die_mask, int* die_of_block, float* near_us, float* far_us);
 /* Synchronises the device and reports what a decode run flagged on the device: a grid barrier of the persistent
  * kernel that timed out (FLEXLLM_EHIP), or an input token id outside the vocabulary (FLEXLLM_EINVAL; token 0 was
  * used in its place, no row outside the embedding table is ever read).  Clears the flag. */

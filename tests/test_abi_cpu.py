@@ -92,3 +92,44 @@ def test_size_t_parameters_are_typed_in_the_binding():
         for k in pos:
             assert at[k] is C.c_size_t, (name, k)
     assert found >= 10
+
+
+def test_die_classification_of_made_up_timings():
+    """The host arithmetic behind the per-die placement of the decode kernel's exchange words (no GPU involved): blocks
+    alternate between two dies, XCDs {0, 2, 5, 7} sit on one die and {1, 3, 4, 6} on the other, with 3 % noise; one block
+    shows no difference and stays unused.  Degenerate inputs (no contrast, three XCDs on a die, NaN) are not usable."""
+    import ctypes as C
+    import numpy as np
+    from flexllm_amd import _lib
+    lib = _lib.lib()
+    rng = np.random.default_rng(4)
+    n = 48
+    die_of_xcd = np.array([0, 1, 0, 1, 1, 0, 1, 0])
+    true_die = (np.arange(n) // 2 + np.arange(n) // 16) % 2          # 16 KiB stripes whose polarity flips further up
+    us = np.where(true_die[:, None] == die_of_xcd[None, :], 1.0, 1.6) * (1.0 + 0.03 * rng.standard_normal((n, 8)))
+    us[7, :] = 1.3                                                    # a block with no clear owner
+    us = np.ascontiguousarray(us, np.float32)
+
+    def classify(t):
+        usable, mask, near, far = C.c_int(-1), C.c_uint(0), C.c_float(0), C.c_float(0)
+        die = (C.c_int * len(t))()
+        rc = lib.flexllm_die_classify(t.ctypes.data_as(C.POINTER(C.c_float)), len(t), C.byref(usable), C.byref(mask), die,
+                                      C.byref(near), C.byref(far))
+        assert rc == 0
+        return usable.value, mask.value, np.array(die[:]), near.value, far.value
+
+    usable, mask, die, near, far = classify(us)
+    assert usable == 1
+    assert mask == sum(1 << x for x in range(8) if die_of_xcd[x] != die_of_xcd[0])
+    expect = np.where(true_die == die_of_xcd[0], 0, 1)
+    expect[7] = -1
+    assert np.array_equal(die, expect)
+    assert 0.9 < near < 1.1 and 1.5 < far < 1.7
+    flat = np.ones((n, 8), np.float32) * (1.0 + 0.01 * rng.standard_normal((n, 8)).astype(np.float32))
+    assert classify(flat)[0] == 0                                     # no contrast: at most noise, never four clear blocks per die
+    lop = us.copy(); lop[:, 5] = us[:, 1]                             # XCD 5 behaves like the other die: 3 + 5
+    assert classify(lop)[0] == 0
+    bad = us.copy(); bad[:, :] = np.nan
+    u, _, d, _, _ = classify(bad)
+    assert u == 0 and (d == -1).all()
+    assert classify(us[:6])[0] == 0                                   # too few blocks
