@@ -24,6 +24,8 @@
 //               the eight flags), then coherent loads.
 //   5->6        SiLU(gate)*up (8192 floats): coherent stores into a slice that no other layer pass of the launch uses,
 //               a grid barrier, then ORDINARY loads, which the 32 CUs of an XCD share through L2 (see MegaParams::h).
+// The tagged arrays and the barrier's words exist once per I/O die, in memory attached to that die (MegaParams::xblk):
+// producers store into both copies, consumers poll their own die's.
 // A tagged slot is rewritten a layer later, after at least one exchange that all its readers take part in as
 // producers, i.e. after they have finished with it.  The weights a workgroup needs in the NEXT phase do not depend on
 // the activations, so they are requested BEFORE waiting: HBM keeps streaming while the hand-over is in flight.
