@@ -120,6 +120,7 @@ struct DieArena {
 // want_calibration == false skips the measurement (single-copy operation).
 static int die_arena_create(DieArena& a, int n_blocks, bool want_calibration, void** raw) {
     a = DieArena();
+    FX_REQUIRE(n_blocks >= 8 && n_blocks <= 255, "die arena: %d blocks (users keep block indices in a byte)", n_blocks);
     FX_HIP(hipMalloc(raw, (size_t)(n_blocks + 1) * kDieBlock));
     a.base = reinterpret_cast<char*>((reinterpret_cast<uintptr_t>(*raw) + kDieBlock - 1) & ~(uintptr_t)(kDieBlock - 1));
     a.n_blocks = n_blocks;
