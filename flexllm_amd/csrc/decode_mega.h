@@ -318,6 +318,9 @@ struct MegaLds {
     int tk_idx[kTopKMax];
     int tk_tok;
     int stop;                                          // set by thread 0 at the end of a step when the error flag is up: the launch ends there
+#ifdef FX_MEGA_ALL_STAMPS
+    long long dbg[12];                                 // debug build: the stamps of one layer, stored to memory at the layer's end
+#endif
     __attribute__((aligned(16))) int8_t wd[8][8192];   // this workgroup's 8 down rows, filled by global->LDS direct loads (64 KiB);
                                                        // the odd rows first hold gate/up rows 12..15 of their stream wave
     __attribute__((aligned(16))) int8_t gu2[4][8192];  // gate/up rows 8..11 of each stream wave (32 KiB)
@@ -545,12 +548,15 @@ __device__ __forceinline__ void decode_mega_body(const MegaParams& p) {
     // 'thread 0 of workgroup 0' from scalars and the hardware lane id: no per-thread value has to stay live for it
     auto is_t0 = [&]() { return wave == 0 && __builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u)) == 0; };
 #ifdef FX_MEGA_ALL_STAMPS
-    // debug build: every workgroup records the 12 stamps of one layer (the eighth) behind the other timeline entries
+    // debug build: every workgroup records the 12 stamps of one layer (the eighth) behind the other timeline entries.
+    // They wait in LDS until the layer's last one: a store per stamp would sit in front of the next wait for the
+    // vector-memory counter and stretch exactly the intervals under study (by up to 1 us).  No other stamps in this build.
     int cur_layer = 0;
     auto stamp = [&]() {
-        if (p.timeline && is_t0()) {
-            if (wg == p.timeline_wg) p.timeline[stamp_i] = wall_clock64();
-            if (cur_layer == 8) p.timeline[p.n_layers * 12 + 2 + 64 + 2 * kMegaWG + wg * 12 + stamp_i % 12] = wall_clock64();
+        if (p.timeline && is_t0() && cur_layer == 8) {
+            L.dbg[stamp_i % 12] = wall_clock64();
+            if (stamp_i % 12 == 11)
+                for (int i = 0; i < 12; i++) p.timeline[p.n_layers * 12 + 2 + 64 + 2 * kMegaWG + wg * 12 + i] = L.dbg[i];
         }
         stamp_i++;
     };
