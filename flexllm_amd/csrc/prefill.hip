@@ -58,8 +58,11 @@ int llama_prefill_run(const flexllm_llama_config& c, const LayerW* layers, const
     int rc = prefill_workspace_get(ws, c, s, &b);
     if (rc) return rc;
     const int H = c.hidden, I = c.inter;
-    FX_HIP(hipMemcpyAsync(b.x, x_in, sizeof(float) * (size_t)s * H, hipMemcpyDeviceToDevice, st));
+    // The first layer reads the caller's x_in and the last one writes the caller's hidden_out directly (x_in is last read
+    // by the first layer's o projection, so the two may be one buffer): no copies in or out.
+    const float* xin = x_in;
     for (int l = 0; l < c.layers; l++) {
+        float* const xout = (l == c.layers - 1 && hidden_out) ? hidden_out : b.x;
         const LayerW& w = layers[l];
         const float* g0 = gamma + (size_t)(2 * l) * H;
         const float* g1 = gamma + (size_t)(2 * l + 1) * H;
@@ -70,7 +73,7 @@ int llama_prefill_run(const flexllm_llama_config& c, const LayerW* layers, const
         int8_t* kc = k_cache + (size_t)l * cache_layer_bytes;
         int8_t* vc = v_cache + (size_t)l * cache_layer_bytes;
         // attention block
-        rmsnorm_quant_rows(b.x, g0, b.xq, b.xs, s, H, c.eps, st);
+        rmsnorm_quant_rows(xin, g0, b.xq, b.xs, s, H, c.eps, st);
         {   // q/k/v projection with RoPE, static quantisation and the cache stores in the GEMM epilogue
             QkvEpiArgs qa;
             qa.sin_t = rope_sin; qa.cos_t = rope_cos; qa.q_s = q_s; qa.k_s = k_s; qa.v_s = v_s;
@@ -80,15 +83,15 @@ int llama_prefill_run(const flexllm_llama_config& c, const LayerW* layers, const
         }
         if ((rc = mha_prefill_launch(b.q8, kc, vc, q_s, k_s, v_s, a_s, b.att, nullptr, s, c.q_heads, c.kv_heads, c.max_pos, st))) return rc;
         quant_sym_kernel<2><<<s, kBlock, 0, st>>>(b.att, b.xq, b.xs, H);   // (one wave per row, as for the norm: measured no faster here)
-        if ((rc = launch_gemm<kGemmDequant>(b.xq, w.wo, nullptr, b.xs, w.so, b.x, b.x2, s, H, H, st))) return rc;
+        if ((rc = launch_gemm<kGemmDequant>(b.xq, w.wo, nullptr, b.xs, w.so, xin, b.x2, s, H, H, st))) return rc;
         // feed-forward block
         rmsnorm_quant_rows(b.x2, g1, b.xq, b.xs, s, H, c.eps, st);
         if ((rc = launch_gemm_swiglu(b.xq, w.wgu, b.xs, w.sgu, b.gu, s, H, 2 * I, st))) return rc;     // b.gu = SiLU(gate)*up [s][I]
         fht_kernel<13, true, false><<<s, kFhtBlock, 0, st>>>(b.gu, nullptr, b.xq, b.xs, c.fht_scale);
-        if ((rc = launch_gemm<kGemmDequant>(b.xq, w.wd, nullptr, b.xs, w.sd, b.x2, b.x, s, I, H, st))) return rc;
+        if ((rc = launch_gemm<kGemmDequant>(b.xq, w.wd, nullptr, b.xs, w.sd, b.x2, xout, s, I, H, st))) return rc;
+        xin = xout;
     }
     FX_LAUNCH_CHECK();
-    if (hidden_out) FX_HIP(hipMemcpyAsync(hidden_out, b.x, sizeof(float) * (size_t)s * H, hipMemcpyDeviceToDevice, st));
     return FLEXLLM_OK;
 }
 
@@ -109,8 +112,9 @@ int llama_prefill_run_w4a4(const flexllm_llama_config& c, const LayerW* layers, 
     if (rc) return rc;
     const int H = c.hidden, I = c.inter;
     uint8_t* xq = reinterpret_cast<uint8_t*>(b.xq);
-    FX_HIP(hipMemcpyAsync(b.x, x_in, sizeof(float) * (size_t)s * H, hipMemcpyDeviceToDevice, st));
+    const float* xin = x_in;                                   // no copies in or out, as in llama_prefill_run
     for (int l = 0; l < c.layers; l++) {
+        float* const xout = (l == c.layers - 1 && hidden_out) ? hidden_out : b.x;
         const LayerW& w = layers[l];
         const LayerW4& m4 = sums[l];
         const float* q_s = q_s_all + (size_t)l * c.q_heads;
@@ -121,7 +125,7 @@ int llama_prefill_run_w4a4(const flexllm_llama_config& c, const LayerW* layers, 
         int8_t* vc = v_cache + (size_t)l * cache_layer_bytes;
         // attention block
         rmsnorm_quant_asym_2048_wave_kernel<<<(s + kNormWaveRows - 1) / kNormWaveRows, 64 * kNormWaveRows, 0, st>>>(
-            b.x, gamma + (size_t)(2 * l) * H, xq, b.xs, b.xb, s, c.eps, 15.0f, 15u);
+            xin, gamma + (size_t)(2 * l) * H, xq, b.xs, b.xb, s, c.eps, 15.0f, 15u);
         {   // q/k/v projection with the asymmetric dequantisation, RoPE, static quantisation and the cache stores in the GEMM epilogue
             QkvEpiArgs qa;
             qa.sin_t = rope_sin; qa.cos_t = rope_cos; qa.q_s = q_s; qa.k_s = k_s; qa.v_s = v_s;
@@ -132,17 +136,17 @@ int llama_prefill_run_w4a4(const flexllm_llama_config& c, const LayerW* layers, 
         }
         if ((rc = mha_prefill_launch(b.q8, kc, vc, q_s, k_s, v_s, a_s, b.att, nullptr, s, c.q_heads, c.kv_heads, c.max_pos, st))) return rc;
         quant_asym_kernel<2><<<s, kBlock, 0, st>>>(b.att, xq, b.xs, b.xb, H, 15.0f, 15u);
-        if ((rc = launch_gemm_asym(b.xq, w.wo, b.xs, b.xb, w.so, m4.mo, b.x, b.x2, s, H, H, st))) return rc;
+        if ((rc = launch_gemm_asym(b.xq, w.wo, b.xs, b.xb, w.so, m4.mo, xin, b.x2, s, H, H, st))) return rc;
         // feed-forward block
         rmsnorm_quant_asym_2048_wave_kernel<<<(s + kNormWaveRows - 1) / kNormWaveRows, 64 * kNormWaveRows, 0, st>>>(
             b.x2, gamma + (size_t)(2 * l + 1) * H, xq, b.xs, b.xb, s, c.eps, 15.0f, 15u);
         // gate/up with SiLU(gate)*up in the GEMM epilogue: b.gu = [s][I]
         if ((rc = launch_gemm_swiglu_asym(b.xq, w.wgu, b.xs, b.xb, w.sgu, m4.mgu, b.gu, s, H, 2 * I, st))) return rc;
         fht_kernel<13, 2, false><<<s, kFhtBlock, 0, st>>>(b.gu, nullptr, b.xq, b.xs, c.fht_scale, b.xb, 15.0f, 15u);   // transform + uint4 quantisation
-        if ((rc = launch_gemm_asym(b.xq, w.wd, b.xs, b.xb, w.sd, m4.md, b.x2, b.x, s, I, H, st))) return rc;
+        if ((rc = launch_gemm_asym(b.xq, w.wd, b.xs, b.xb, w.sd, m4.md, b.x2, xout, s, I, H, st))) return rc;
+        xin = xout;
     }
     FX_LAUNCH_CHECK();
-    if (hidden_out) FX_HIP(hipMemcpyAsync(hidden_out, b.x, sizeof(float) * (size_t)s * H, hipMemcpyDeviceToDevice, st));
     return FLEXLLM_OK;
 }
 
